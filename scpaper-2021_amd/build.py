@@ -1,0 +1,76 @@
+"""Build recipe of the native library (HIP kernels + C ABI + C++ host layer).
+
+    python scpaper-2021_amd/build.py            # compile everything for gfx950
+
+hipcc cross-compiles for gfx950 without a GPU.  Objects go to
+``scpaper-2021_amd/build/`` and the shared library to
+``scpaper-2021_amd/lib/libet_hip.so`` (both ignored by git; the library
+travels with the source tree to the GPU machine).
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import os
+import shutil
+import subprocess
+import sys
+from pathlib import Path
+
+PKG = Path(__file__).resolve().parent
+ROOT = PKG.parent
+BUILD = PKG / "build"
+LIBDIR = PKG / "lib"
+LIB = LIBDIR / "libet_hip.so"
+
+ARCH = "gfx950"
+HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+
+COMMON = ["-O3", "-std=c++17", "-fPIC", "-I", str(ROOT / "include"), "-Wall", "-Wno-unused-function"]
+# Packed-fp32 code generation is switched off for device code.
+DEVICE = [f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+          "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument"]
+
+
+def sources() -> list[Path]:
+    return sorted((PKG / "csrc").glob("*.hip")) + sorted((PKG / "host").glob("*.cpp"))
+
+
+def _compile(src: Path) -> Path:
+    obj = BUILD / (src.name + ".o")
+    cmd = [HIPCC, *COMMON]
+    if src.suffix == ".hip":
+        cmd += DEVICE
+    cmd += ["-c", str(src), "-o", str(obj)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    # hipcc's host pass does not know the packed-fp32 feature name; that
+    # warning is expected and dropped here.
+    noise = ("is not a recognized feature for this target", "'-packed-fp32-ops'")
+    err = "\n".join(l for l in res.stderr.splitlines() if not any(n in l for n in noise))
+    if res.returncode != 0:
+        raise RuntimeError(f"compile failed: {' '.join(cmd)}\n{err}")
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    return obj
+
+
+def build_all(jobs: int | None = None, verbose: bool = True) -> Path:
+    """Compile every source for gfx950 and link the shared library."""
+    BUILD.mkdir(exist_ok=True)
+    LIBDIR.mkdir(exist_ok=True)
+    srcs = sources()
+    jobs = jobs or min(8, len(srcs))
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = list(pool.map(_compile, srcs))
+    tmp = LIB.with_suffix(".so.tmp")
+    cmd = [HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", *map(str, objs), "-o", str(tmp)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed: {' '.join(cmd)}\n{res.stderr}")
+    os.replace(tmp, LIB)
+    if verbose:
+        print(f"built {LIB} from {len(srcs)} sources")
+    return LIB
+
+
+if __name__ == "__main__":
+    build_all()

@@ -1,0 +1,291 @@
+// Fused multi-head self-attention for gfx950: scores, mask, softmax and P*V in
+// one kernel; the score matrix lives in registers only.
+//
+// Grid (query strip, head, sequence).  A workgroup stages one block of up to
+// 128 keys of its head in LDS — K as [key][hd] and V transposed as [hd][key]
+// — and each wave owns 16 query rows.  Both contractions are computed
+// transposed so that no register shuffle is needed between them:
+//   S^T = K * Q^T : MFMA A = K rows (from LDS), B = Q rows (registers);
+//                   lane (r = lane%16, g = lane/16) ends with the scores of
+//                   query r against keys 16*kb + 4g..4g+3 of every key block.
+//   O^T = V^T * P^T: the contraction index of v_mfma_f32_16x16x32_f16 is
+//                   mapped so that the 8 values a lane must supply as the B
+//                   operand are exactly the 2x4 probabilities it already holds
+//                   (key blocks 2s and 2s+1); the A operand reads the same
+//                   keys of V^T from LDS as two 8-byte loads.
+// Softmax is the running-max form over key blocks (one block when S <= 128):
+// fp32 scores, exp2 with log2(e) folded into the scale, row max/sum reduced
+// in-lane and then across the four 16-lane groups with two wave64 butterflies.
+// Probabilities are rounded to fp16 only as MFMA operands; the normalisation
+// by the fp32 row sum happens once on the fp32 accumulators.
+#include <math.h>
+
+#include "common.hip.h"
+
+namespace et {
+
+struct MhaArgs {
+    const _Float16 *Q, *K, *V;
+    _Float16 *Z;
+    const _Float16 *mask;  // [S x S] additive or nullptr
+    const int32_t *lens;   // [B] or nullptr
+    int ldq, ldk, ldv, ldz;
+    int S, nh;
+    float scale_log2e;  // scale * log2(e)
+    int causal;
+};
+
+constexpr int kKeyBlock = 128;          // keys staged per iteration
+constexpr int kNKB = kKeyBlock / 16;    // 16-key MFMA blocks per iteration
+constexpr float kLog2e = 1.4426950408889634f;
+
+template <int HD>
+struct MhaLds {
+    static constexpr int ldk = HD + 8;           // halfs per staged K row
+    static constexpr int ldvt = kKeyBlock + 8;   // halfs per staged V^T row
+    static constexpr int k_halfs = kKeyBlock * ldk;
+    static constexpr int vt_halfs = HD * ldvt;
+    static constexpr size_t bytes = (size_t)(k_halfs + vt_halfs) * sizeof(_Float16);
+};
+
+template <int HD>
+__global__ __launch_bounds__(256) void mha_fused_kernel(const MhaArgs a) {
+    using L = MhaLds<HD>;
+    constexpr int KS = HD / 32;  // K=32 MFMA steps over the head dimension
+    constexpr int DB = HD / 16;  // 16-wide output blocks of the head dimension
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    _Float16 *Ks = reinterpret_cast<_Float16 *>(smem_raw);
+    _Float16 *Vt = Ks + L::k_halfs;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int nwave = blockDim.x >> 6;
+    const int r16 = lane & 15;
+    const int g = lane >> 4;
+    const int h = blockIdx.y;
+    const int b = blockIdx.z;
+    const int S = a.S;
+    const size_t row0 = (size_t)b * S;  // first token row of this sequence
+    const int q = (blockIdx.x * nwave + wave) * 16 + r16;  // this lane's query
+    const bool q_ok = q < S;
+    int klimit = S;
+    if (a.lens) klimit = min(S, max(a.lens[b], 0));
+
+    // Q fragments: B operand, lane supplies Q[q][32*ks + 8g .. +7]
+    h8 qf[KS];
+    {
+        const _Float16 *qp = a.Q + (row0 + (q_ok ? q : 0)) * a.ldq + h * HD + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            qf[ks] = *reinterpret_cast<const h8 *>(qp + 32 * ks);
+            if (!q_ok) qf[ks] = h8{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+    }
+
+    f4 o[DB];
+#pragma unroll
+    for (int d = 0; d < DB; d++) o[d] = f4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY;  // running max of this lane's query (log2 domain)
+    float l_part = 0.0f;      // this lane's share of the running row sum
+
+    const int nblocks = (klimit + kKeyBlock - 1) / kKeyBlock;
+    for (int blk = 0; blk < nblocks; blk++) {
+        const int k0 = blk * kKeyBlock;
+        if (blk > 0) __syncthreads();
+        // ---- stage K block: 16-byte vectors, rows beyond S zero-filled
+        {
+            constexpr int vec_per_row = HD / 8;
+            for (int v = threadIdx.x; v < kKeyBlock * vec_per_row; v += blockDim.x) {
+                const int r = v / vec_per_row, c = v - r * vec_per_row;
+                h8 val = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (k0 + r < S)
+                    val = *reinterpret_cast<const h8 *>(a.K + (row0 + k0 + r) * a.ldk + h * HD + c * 8);
+                *reinterpret_cast<h8 *>(Ks + r * L::ldk + c * 8) = val;
+            }
+        }
+        // ---- stage V block transposed: a thread takes 4 keys x 8 dims
+        {
+            constexpr int dgroups = HD / 8;
+            for (int u = threadIdx.x; u < (kKeyBlock / 4) * dgroups; u += blockDim.x) {
+                const int kg = u / dgroups, dg = u - kg * dgroups;
+                h8 rows[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int key = k0 + kg * 4 + i;
+                    rows[i] = h8{0, 0, 0, 0, 0, 0, 0, 0};
+                    if (key < S)
+                        rows[i] = *reinterpret_cast<const h8 *>(a.V + (row0 + key) * a.ldv + h * HD + dg * 8);
+                }
+#pragma unroll
+                for (int d = 0; d < 8; d++) {
+                    h4 col = {rows[0][d], rows[1][d], rows[2][d], rows[3][d]};
+                    *reinterpret_cast<h4 *>(Vt + (dg * 8 + d) * L::ldvt + kg * 4) = col;
+                }
+            }
+        }
+        __syncthreads();
+
+        // ---- scores of 16 queries against the 128 staged keys
+        f4 sc[kNKB];
+#pragma unroll
+        for (int kb = 0; kb < kNKB; kb++) {
+            sc[kb] = f4{0.f, 0.f, 0.f, 0.f};
+            if (k0 + kb * 16 < klimit) {  // wave-uniform: skip fully padded key blocks
+                const _Float16 *kp = Ks + (kb * 16 + r16) * L::ldk + 8 * g;
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++) {
+                    const h8 kf = *reinterpret_cast<const h8 *>(kp + 32 * ks);
+                    sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[ks], sc[kb], 0, 0, 0);
+                }
+            }
+        }
+
+        // ---- scale, mask, block max
+        float m_blk = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < kNKB; kb++) {
+            const int key0 = k0 + kb * 16 + 4 * g;
+            float mk[4] = {0.f, 0.f, 0.f, 0.f};
+            if (a.mask && q_ok && key0 < S) {
+                const h4 mv = *reinterpret_cast<const h4 *>(a.mask + (size_t)q * S + key0);
+#pragma unroll
+                for (int j = 0; j < 4; j++) mk[j] = (float)mv[j] * kLog2e;
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int key = key0 + j;
+                float s = sc[kb][j] * a.scale_log2e + mk[j];
+                if (key >= klimit || (a.causal && key > q)) s = -INFINITY;
+                sc[kb][j] = s;
+                m_blk = fmaxf(m_blk, s);
+            }
+        }
+        m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 16, kWave));
+        m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, kWave));
+
+        const float m_new = fmaxf(m_run, m_blk);
+        // all keys so far masked: keep everything at zero without inf - inf
+        const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+        const float alpha = exp2f(m_run - m_use);  // m_run = -inf gives 0
+        m_run = m_new;
+        l_part *= alpha;
+#pragma unroll
+        for (int d = 0; d < DB; d++) o[d] *= alpha;
+
+        // ---- probabilities (fp32 sum, fp16 operands) and O^T += V^T P^T
+#pragma unroll
+        for (int s2 = 0; s2 < kNKB / 2; s2++) {
+            if (k0 + s2 * 32 >= klimit) continue;  // both key blocks fully padded
+            h8 pf;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float p0 = exp2f(sc[2 * s2][j] - m_use);
+                const float p1 = exp2f(sc[2 * s2 + 1][j] - m_use);
+                const _Float16 h0 = (_Float16)p0, h1 = (_Float16)p1;
+                // the row sum uses the values that enter the MFMA
+                l_part += (float)h0 + (float)h1;
+                pf[j] = h0;
+                pf[4 + j] = h1;
+            }
+#pragma unroll
+            for (int d = 0; d < DB; d++) {
+                const _Float16 *vp = Vt + (d * 16 + r16) * L::ldvt + s2 * 32 + 4 * g;
+                const h4 v0 = *reinterpret_cast<const h4 *>(vp);
+                const h4 v1 = *reinterpret_cast<const h4 *>(vp + 16);
+                const h8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[d], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- normalise and store: lane holds dims 16d + 4g..4g+3 of query r16
+    float l = l_part;
+    l += __shfl_xor(l, 16, kWave);
+    l += __shfl_xor(l, 32, kWave);
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    if (q_ok) {
+        _Float16 *zp = a.Z + (row0 + q) * a.ldz + h * HD + 4 * g;
+#pragma unroll
+        for (int d = 0; d < DB; d++) {
+            h4 out;
+#pragma unroll
+            for (int j = 0; j < 4; j++) out[j] = (_Float16)(o[d][j] * inv);
+            *reinterpret_cast<h4 *>(zp + 16 * d) = out;
+        }
+    }
+}
+
+template <int HD>
+static int launch_mha(const MhaArgs &args, int B, hipStream_t stream) {
+    auto kernel = mha_fused_kernel<HD>;
+    constexpr size_t lds = MhaLds<HD>::bytes;
+    if (lds > 64 * 1024) {
+        static bool raised = false;
+        if (!raised) {
+            ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+            raised = true;
+        }
+    }
+    // 4 waves = 64 query rows per workgroup; 2 waves when that leaves a
+    // half-empty strip (S = 32, 96, ...).
+    const int qblocks = args.S / 16;
+    const int nwave = (qblocks % 4 == 0) ? 4 : (qblocks % 2 == 0 ? 2 : 1);
+    const dim3 grid((qblocks + nwave - 1) / nwave, args.nh, B);
+    kernel<<<grid, nwave * 64, lds, stream>>>(args);
+    return check_launch("mha_fused_kernel");
+}
+
+}  // namespace et
+
+using namespace et;
+
+extern "C" {
+
+int et_mha_fused_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V, int ldq, int ldk, int ldv,
+                     et_f16 *Z, int ldz, const et_f16 *mask, const int32_t *lens, int B, int S,
+                     int nh, int hd, float scale, int flags, et_stream stream) {
+    ET_REQUIRE(Q && K && V && Z, ET_ERR_INVALID_ARG, "et_mha_fused_f16: NULL pointer");
+    ET_REQUIRE(B >= 0 && S > 0 && nh > 0 && hd > 0, ET_ERR_INVALID_ARG,
+               "et_mha_fused_f16: B=%d S=%d nh=%d hd=%d", B, S, nh, hd);
+    ET_REQUIRE((flags & ~ET_MHA_CAUSAL) == 0, ET_ERR_INVALID_ARG, "et_mha_fused_f16: flags=%d",
+               flags);
+    ET_REQUIRE(S % 16 == 0, ET_ERR_UNSUPPORTED, "et_mha_fused_f16: S=%d must be a multiple of 16",
+               S);
+    ET_REQUIRE(hd == 32 || hd == 64 || hd == 128, ET_ERR_UNSUPPORTED,
+               "et_mha_fused_f16: head dim %d not in {32, 64, 128}", hd);
+    const int width = nh * hd;
+    ET_REQUIRE(ldq >= width && ldk >= width && ldv >= width && ldz >= width, ET_ERR_INVALID_ARG,
+               "et_mha_fused_f16: row strides (%d %d %d %d) smaller than nh*hd=%d", ldq, ldk, ldv,
+               ldz, width);
+    ET_REQUIRE(ldq % 8 == 0 && ldk % 8 == 0 && ldv % 8 == 0 && ldz % 4 == 0, ET_ERR_UNSUPPORTED,
+               "et_mha_fused_f16: row strides must keep 16-byte alignment");
+    ET_REQUIRE(((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) |
+                 reinterpret_cast<uintptr_t>(V)) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(Z) & 7) == 0,
+               ET_ERR_UNSUPPORTED, "et_mha_fused_f16: operands must be 16-byte aligned");
+    ET_REQUIRE(B <= 65535 && nh <= 65535, ET_ERR_UNSUPPORTED, "et_mha_fused_f16: grid too large");
+    if (B == 0) return ET_OK;
+    MhaArgs args;
+    args.Q = reinterpret_cast<const _Float16 *>(Q);
+    args.K = reinterpret_cast<const _Float16 *>(K);
+    args.V = reinterpret_cast<const _Float16 *>(V);
+    args.Z = reinterpret_cast<_Float16 *>(Z);
+    args.mask = reinterpret_cast<const _Float16 *>(mask);
+    args.lens = lens;
+    args.ldq = ldq;
+    args.ldk = ldk;
+    args.ldv = ldv;
+    args.ldz = ldz;
+    args.S = S;
+    args.nh = nh;
+    args.scale_log2e = scale * kLog2e;
+    args.causal = (flags & ET_MHA_CAUSAL) ? 1 : 0;
+    switch (hd) {
+        case 32: return launch_mha<32>(args, B, as_stream(stream));
+        case 64: return launch_mha<64>(args, B, as_stream(stream));
+        default: return launch_mha<128>(args, B, as_stream(stream));
+    }
+}
+
+}  // extern "C"

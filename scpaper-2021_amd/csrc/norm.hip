@@ -1,0 +1,165 @@
+// SkipLayerNorm / LayerNorm for gfx950: one wavefront owns one row, the row
+// stays in registers between the statistics and the normalisation, so HBM sees
+// each input once and the output once.  Statistics are fp32 (mean, then the
+// centred second moment), wave64 butterfly reductions, no LDS.
+#include "common.hip.h"
+
+namespace et {
+
+constexpr int kRowsPerBlock = 4;  // 4 waves of 64 lanes
+
+__device__ __forceinline__ void unpack4(uint2 raw, float (&f)[4]) {
+    const h2 lo = __builtin_bit_cast(h2, raw.x);
+    const h2 hi = __builtin_bit_cast(h2, raw.y);
+    f[0] = (float)lo[0];
+    f[1] = (float)lo[1];
+    f[2] = (float)hi[0];
+    f[3] = (float)hi[1];
+}
+
+__device__ __forceinline__ uint2 pack4(const float (&f)[4]) {
+    h2 lo, hi;
+    lo[0] = (_Float16)f[0];
+    lo[1] = (_Float16)f[1];
+    hi[0] = (_Float16)f[2];
+    hi[1] = (_Float16)f[3];
+    uint2 raw;
+    raw.x = __builtin_bit_cast(uint32_t, lo);
+    raw.y = __builtin_bit_cast(uint32_t, hi);
+    return raw;
+}
+
+// NIT = number of 4-element chunks each lane owns: chunk c = lane + 64*i.
+template <int NIT, bool SKIP>
+__global__ __launch_bounds__(kWave *kRowsPerBlock) void layernorm_rows_kernel(
+    _Float16 *__restrict__ out, const _Float16 *__restrict__ src,
+    const _Float16 *__restrict__ skip, const _Float16 *__restrict__ gamma,
+    const _Float16 *__restrict__ beta, int rows, int H, float eps) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int row = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int chunks = H >> 2;
+    const uint2 *s = reinterpret_cast<const uint2 *>(src + (size_t)row * H);
+    const uint2 *k = SKIP ? reinterpret_cast<const uint2 *>(skip + (size_t)row * H) : nullptr;
+
+    float x[NIT][4];
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NIT; i++) {
+        const int c = lane + kWave * i;
+        if (c < chunks) {
+            unpack4(s[c], x[i]);
+            if (SKIP) {
+                float y[4];
+                unpack4(k[c], y);
+#pragma unroll
+                for (int j = 0; j < 4; j++) x[i][j] += y[j];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) sum += x[i][j];
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) x[i][j] = 0.0f;
+        }
+    }
+    const float inv_h = 1.0f / (float)H;
+    const float mean = wave_sum(sum) * inv_h;
+    float sq = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NIT; i++) {
+        const int c = lane + kWave * i;
+        if (c < chunks) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float d = x[i][j] - mean;
+                sq += d * d;
+            }
+        }
+    }
+    const float rstd = rsqrtf(wave_sum(sq) * inv_h + eps);
+
+    const uint2 *g = reinterpret_cast<const uint2 *>(gamma);
+    const uint2 *b = reinterpret_cast<const uint2 *>(beta);
+    uint2 *o = reinterpret_cast<uint2 *>(out + (size_t)row * H);
+#pragma unroll
+    for (int i = 0; i < NIT; i++) {
+        const int c = lane + kWave * i;
+        if (c < chunks) {
+            float gg[4], bb[4], y[4];
+            unpack4(g[c], gg);
+            unpack4(b[c], bb);
+#pragma unroll
+            for (int j = 0; j < 4; j++) y[j] = (x[i][j] - mean) * rstd * gg[j] + bb[j];
+            o[c] = pack4(y);
+        }
+    }
+}
+
+template <bool SKIP>
+static int launch_layernorm(_Float16 *out, const _Float16 *src, const _Float16 *skip,
+                            const _Float16 *gamma, const _Float16 *beta, int rows, int H,
+                            float eps, hipStream_t stream) {
+    const int chunks = H / 4;
+    const int nit = (chunks + kWave - 1) / kWave;
+    const dim3 grid((rows + kRowsPerBlock - 1) / kRowsPerBlock), block(kWave * kRowsPerBlock);
+#define ET_LN_CASE(N)                                                                   \
+    case N:                                                                             \
+        layernorm_rows_kernel<N, SKIP><<<grid, block, 0, stream>>>(out, src, skip, gamma, \
+                                                                   beta, rows, H, eps);  \
+        break;
+    switch (nit) {
+        ET_LN_CASE(1) ET_LN_CASE(2) ET_LN_CASE(3) ET_LN_CASE(4)
+        ET_LN_CASE(5) ET_LN_CASE(6) ET_LN_CASE(7) ET_LN_CASE(8)
+        default:
+            if (nit <= 16) {
+                layernorm_rows_kernel<16, SKIP><<<grid, block, 0, stream>>>(out, src, skip, gamma,
+                                                                            beta, rows, H, eps);
+            } else {
+                layernorm_rows_kernel<32, SKIP><<<grid, block, 0, stream>>>(out, src, skip, gamma,
+                                                                            beta, rows, H, eps);
+            }
+    }
+#undef ET_LN_CASE
+    return check_launch("layernorm_rows_kernel");
+}
+
+static int check_ln_args(const char *fn, const void *out, const void *src, const void *gamma,
+                         const void *beta, int rows, int H) {
+    ET_REQUIRE(out && src && gamma && beta, ET_ERR_INVALID_ARG, "%s: NULL pointer", fn);
+    ET_REQUIRE(rows >= 0 && H > 0, ET_ERR_INVALID_ARG, "%s: rows=%d H=%d", fn, rows, H);
+    ET_REQUIRE(H % 4 == 0 && H <= 8192, ET_ERR_UNSUPPORTED,
+               "%s: H=%d must be a multiple of 4 and at most 8192", fn, H);
+    return ET_OK;
+}
+
+}  // namespace et
+
+using namespace et;
+
+extern "C" {
+
+int et_skip_layernorm_f16(et_f16 *out, const et_f16 *src, const et_f16 *skip,
+                          const et_f16 *gamma, const et_f16 *beta, int rows, int H, float eps,
+                          et_stream stream) {
+    int s = check_ln_args("et_skip_layernorm_f16", out, src, gamma, beta, rows, H);
+    if (s != ET_OK) return s;
+    ET_REQUIRE(skip != nullptr, ET_ERR_INVALID_ARG, "et_skip_layernorm_f16: skip is NULL");
+    if (rows == 0) return ET_OK;
+    return launch_layernorm<true>(
+        reinterpret_cast<_Float16 *>(out), reinterpret_cast<const _Float16 *>(src),
+        reinterpret_cast<const _Float16 *>(skip), reinterpret_cast<const _Float16 *>(gamma),
+        reinterpret_cast<const _Float16 *>(beta), rows, H, eps, as_stream(stream));
+}
+
+int et_layernorm_f16(et_f16 *out, const et_f16 *src, const et_f16 *gamma, const et_f16 *beta,
+                     int rows, int H, float eps, et_stream stream) {
+    int s = check_ln_args("et_layernorm_f16", out, src, gamma, beta, rows, H);
+    if (s != ET_OK) return s;
+    if (rows == 0) return ET_OK;
+    return launch_layernorm<false>(
+        reinterpret_cast<_Float16 *>(out), reinterpret_cast<const _Float16 *>(src), nullptr,
+        reinterpret_cast<const _Float16 *>(gamma), reinterpret_cast<const _Float16 *>(beta), rows,
+        H, eps, as_stream(stream));
+}
+
+}  // extern "C"

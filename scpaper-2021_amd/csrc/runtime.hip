@@ -1,0 +1,241 @@
+// Device buffers, streams, events, fills and fp32<->fp16 conversion behind the
+// C ABI, plus the status/error plumbing shared by every entry point.
+#include <stdarg.h>
+#include <string.h>
+
+#include "common.hip.h"
+
+namespace et {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+}
+
+int fail(int status, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return status;
+}
+
+int check_hip(hipError_t e, const char *what) {
+    if (e == hipSuccess) return ET_OK;
+    int status = ET_ERR_LAUNCH;
+    if (e == hipErrorOutOfMemory || e == hipErrorMemoryAllocation) status = ET_ERR_ALLOC;
+    if (e == hipErrorNoDevice || e == hipErrorInvalidDevice) status = ET_ERR_NO_DEVICE;
+    return fail(status, "%s: %s", what, hipGetErrorString(e));
+}
+
+int check_launch(const char *kernel) { return check_hip(hipGetLastError(), kernel); }
+
+template <typename T>
+__global__ void fill_kernel(T *dst, size_t n, T value) {
+    size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) dst[i] = value;
+}
+
+__global__ void f32_to_f16_kernel(_Float16 *dst, const float *src, size_t n) {
+    size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) dst[i] = (_Float16)src[i];  // v_cvt_f16_f32: round-to-nearest-even
+}
+
+__global__ void f16_to_f32_kernel(float *dst, const _Float16 *src, size_t n) {
+    size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += step) dst[i] = (float)src[i];
+}
+
+static inline unsigned grid_for(size_t n, unsigned block) {
+    size_t g = (n + block - 1) / block;
+    const size_t cap = 256u * 16u;
+    return (unsigned)(g < 1 ? 1 : (g > cap ? cap : g));
+}
+
+}  // namespace et
+
+using namespace et;
+
+extern "C" {
+
+const char *et_status_string(int status) {
+    switch (status) {
+        case ET_OK: return "ok";
+        case ET_ERR_INVALID_ARG: return "invalid argument";
+        case ET_ERR_UNSUPPORTED: return "unsupported shape";
+        case ET_ERR_ALLOC: return "allocation failed";
+        case ET_ERR_LAUNCH: return "HIP launch or copy failed";
+        case ET_ERR_IO: return "file error";
+        case ET_ERR_NO_DEVICE: return "no usable device";
+        default: return "unknown status";
+    }
+}
+
+const char *et_last_error(void) { return g_err; }
+
+int et_device_info(char *name, int cap, int *num_cu, int *lds_bytes) {
+    int dev = 0;
+    ET_HIP(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    ET_HIP(hipGetDeviceProperties(&prop, dev));
+    if (name && cap > 0) {
+        snprintf(name, (size_t)cap, "%s (%s)", prop.name, prop.gcnArchName);
+    }
+    if (num_cu) *num_cu = prop.multiProcessorCount;
+    if (lds_bytes) *lds_bytes = (int)prop.sharedMemPerBlock;
+    return ET_OK;
+}
+
+int et_malloc(void **ptr, size_t bytes) {
+    ET_REQUIRE(ptr != nullptr, ET_ERR_INVALID_ARG, "et_malloc: ptr is NULL");
+    *ptr = nullptr;
+    if (bytes == 0) bytes = 16;  // a valid, distinct pointer even for empty buffers
+    void *p = nullptr;
+    ET_HIP(hipMalloc(&p, bytes));
+    int s = check_hip(hipMemset(p, 0, bytes), "hipMemset");
+    if (s != ET_OK) {
+        (void)hipFree(p);
+        return s;
+    }
+    *ptr = p;
+    return ET_OK;
+}
+
+int et_free(void *ptr) {
+    if (!ptr) return ET_OK;
+    ET_HIP(hipFree(ptr));
+    return ET_OK;
+}
+
+int et_memset(void *ptr, int byte, size_t bytes, et_stream stream) {
+    ET_REQUIRE(ptr != nullptr || bytes == 0, ET_ERR_INVALID_ARG, "et_memset: ptr is NULL");
+    if (bytes == 0) return ET_OK;
+    // A fill kernel rather than hipMemsetAsync, so that a caller may record
+    // this call into a HIP graph.
+    const uint32_t b = (uint32_t)(byte & 0xff);
+    if ((reinterpret_cast<uintptr_t>(ptr) | bytes) % 4 == 0) {
+        fill_kernel<uint32_t><<<grid_for(bytes / 4, 256), 256, 0, as_stream(stream)>>>(
+            static_cast<uint32_t *>(ptr), bytes / 4, b * 0x01010101u);
+    } else {
+        fill_kernel<uint8_t><<<grid_for(bytes, 256), 256, 0, as_stream(stream)>>>(
+            static_cast<uint8_t *>(ptr), bytes, (uint8_t)b);
+    }
+    return check_launch("fill_kernel<bytes>");
+}
+
+int et_memcpy_h2d(void *dst, const void *src_host, size_t bytes) {
+    ET_REQUIRE((dst && src_host) || bytes == 0, ET_ERR_INVALID_ARG, "et_memcpy_h2d: NULL pointer");
+    if (bytes == 0) return ET_OK;
+    ET_HIP(hipMemcpy(dst, src_host, bytes, hipMemcpyHostToDevice));
+    return ET_OK;
+}
+
+int et_memcpy_d2h(void *dst_host, const void *src, size_t bytes) {
+    ET_REQUIRE((dst_host && src) || bytes == 0, ET_ERR_INVALID_ARG, "et_memcpy_d2h: NULL pointer");
+    if (bytes == 0) return ET_OK;
+    ET_HIP(hipMemcpy(dst_host, src, bytes, hipMemcpyDeviceToHost));
+    return ET_OK;
+}
+
+int et_memcpy_d2d(void *dst, const void *src, size_t bytes, et_stream stream) {
+    ET_REQUIRE((dst && src) || bytes == 0, ET_ERR_INVALID_ARG, "et_memcpy_d2d: NULL pointer");
+    if (bytes == 0) return ET_OK;
+    ET_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, as_stream(stream)));
+    return ET_OK;
+}
+
+int et_fill_f16(et_f16 *dst, size_t n, et_f16 value, et_stream stream) {
+    ET_REQUIRE(dst != nullptr || n == 0, ET_ERR_INVALID_ARG, "et_fill_f16: dst is NULL");
+    if (n == 0) return ET_OK;
+    fill_kernel<uint16_t><<<grid_for(n, 256), 256, 0, as_stream(stream)>>>(dst, n, value);
+    return check_launch("fill_kernel<u16>");
+}
+
+int et_fill_i32(int32_t *dst, size_t n, int32_t value, et_stream stream) {
+    ET_REQUIRE(dst != nullptr || n == 0, ET_ERR_INVALID_ARG, "et_fill_i32: dst is NULL");
+    if (n == 0) return ET_OK;
+    fill_kernel<int32_t><<<grid_for(n, 256), 256, 0, as_stream(stream)>>>(dst, n, value);
+    return check_launch("fill_kernel<i32>");
+}
+
+int et_f32_to_f16(et_f16 *dst, const float *src, size_t n, et_stream stream) {
+    ET_REQUIRE((dst && src) || n == 0, ET_ERR_INVALID_ARG, "et_f32_to_f16: NULL pointer");
+    if (n == 0) return ET_OK;
+    f32_to_f16_kernel<<<grid_for(n, 256), 256, 0, as_stream(stream)>>>(
+        reinterpret_cast<_Float16 *>(dst), src, n);
+    return check_launch("f32_to_f16_kernel");
+}
+
+int et_f16_to_f32(float *dst, const et_f16 *src, size_t n, et_stream stream) {
+    ET_REQUIRE((dst && src) || n == 0, ET_ERR_INVALID_ARG, "et_f16_to_f32: NULL pointer");
+    if (n == 0) return ET_OK;
+    f16_to_f32_kernel<<<grid_for(n, 256), 256, 0, as_stream(stream)>>>(
+        dst, reinterpret_cast<const _Float16 *>(src), n);
+    return check_launch("f16_to_f32_kernel");
+}
+
+int et_stream_create(et_stream *stream) {
+    ET_REQUIRE(stream != nullptr, ET_ERR_INVALID_ARG, "et_stream_create: stream is NULL");
+    hipStream_t s;
+    ET_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream = s;
+    return ET_OK;
+}
+
+int et_stream_destroy(et_stream stream) {
+    if (!stream) return ET_OK;
+    ET_HIP(hipStreamDestroy(as_stream(stream)));
+    return ET_OK;
+}
+
+int et_stream_sync(et_stream stream) {
+    ET_HIP(hipStreamSynchronize(as_stream(stream)));
+    return ET_OK;
+}
+
+int et_device_sync(void) {
+    ET_HIP(hipDeviceSynchronize());
+    return ET_OK;
+}
+
+int et_event_create(et_event *ev) {
+    ET_REQUIRE(ev != nullptr, ET_ERR_INVALID_ARG, "et_event_create: ev is NULL");
+    hipEvent_t e;
+    ET_HIP(hipEventCreate(&e));
+    *ev = e;
+    return ET_OK;
+}
+
+int et_event_destroy(et_event ev) {
+    if (!ev) return ET_OK;
+    ET_HIP(hipEventDestroy(reinterpret_cast<hipEvent_t>(ev)));
+    return ET_OK;
+}
+
+int et_event_record(et_event ev, et_stream stream) {
+    ET_REQUIRE(ev != nullptr, ET_ERR_INVALID_ARG, "et_event_record: ev is NULL");
+    ET_HIP(hipEventRecord(reinterpret_cast<hipEvent_t>(ev), as_stream(stream)));
+    return ET_OK;
+}
+
+int et_event_sync(et_event ev) {
+    ET_REQUIRE(ev != nullptr, ET_ERR_INVALID_ARG, "et_event_sync: ev is NULL");
+    ET_HIP(hipEventSynchronize(reinterpret_cast<hipEvent_t>(ev)));
+    return ET_OK;
+}
+
+int et_event_elapsed_ms(float *ms, et_event start, et_event stop) {
+    ET_REQUIRE(ms && start && stop, ET_ERR_INVALID_ARG, "et_event_elapsed_ms: NULL argument");
+    ET_HIP(hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start),
+                               reinterpret_cast<hipEvent_t>(stop)));
+    return ET_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,173 @@
+"""Shared helpers of the GPU parity tests, the smoke test and the bench:
+seeded synthetic weights, upload/download, and oracle comparison."""
+from __future__ import annotations
+
+import math
+import sys
+from pathlib import Path
+
+import numpy as np
+import torch
+
+ROOT = Path(__file__).resolve().parent.parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+from oracle import formats as F  # noqa: E402
+from oracle import layers as L  # noqa: E402
+
+
+def rng(seed: int) -> torch.Generator:
+    g = torch.Generator()
+    g.manual_seed(seed)
+    return g
+
+
+def randn(shape, seed, std=1.0, dtype=np.float16) -> np.ndarray:
+    return (torch.randn(*shape, generator=rng(seed)) * std).numpy().astype(dtype)
+
+
+def f32(a: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(np.asarray(a, dtype=np.float32))
+
+
+def max_abs(a, b) -> float:
+    return float(np.max(np.abs(np.asarray(a, np.float32) - np.asarray(b, np.float32)))) if np.size(a) else 0.0
+
+
+class BsrWeight:
+    """Seeded tile-sparse weight: pattern from the format oracle, values N(0, std)."""
+
+    def __init__(self, out, inp, sparsity, seed, std=0.02, bias_std=0.0, dead_block_rows=(),
+                 dead_block_cols=()):
+        self.out, self.inp = out, inp
+        if dead_block_rows or dead_block_cols:
+            self.row_ptr, self.col_idx = dead_aware_pattern(out, inp, sparsity, seed, dead_block_rows,
+                                                            dead_block_cols)
+        else:
+            self.row_ptr, self.col_idx = F.gen_tile_pattern(out, inp, sparsity, seed)
+        n = len(self.col_idx)
+        self.tiles = randn((n, 256), seed + 1, std)
+        self.bias = randn((out,), seed + 2, bias_std) if bias_std else np.zeros(out, np.float16)
+        self.dense = F.bsr16_to_dense(self.row_ptr, self.col_idx, self.tiles, inp)  # fp16 values
+
+    def upload(self, et):
+        self.d_row_ptr = et.DeviceBuffer.from_numpy(self.row_ptr)
+        self.d_col_idx = et.DeviceBuffer.from_numpy(self.col_idx if len(self.col_idx) else np.zeros(1, np.int32))
+        self.d_tiles = et.DeviceBuffer.from_numpy(self.tiles if len(self.tiles) else np.zeros((1, 256), np.float16))
+        self.d_bias = et.DeviceBuffer.from_numpy(self.bias)
+        return self
+
+    def forward(self, et, dX, dY, T, act=0, stream=None):
+        et.linear_bsr16(self.d_row_ptr, self.d_col_idx, self.d_tiles, self.d_bias, dX, dY, T,
+                        self.inp, self.out, act, stream)
+
+
+def dead_aware_pattern(out, inp, sparsity, seed, dead_block_rows, dead_block_cols):
+    """Tile pattern with whole block-rows / block-columns removed (attention-aware
+    pruning of V rows and the matching O columns); the surviving-tile count stays
+    int(total*(1-sparsity)), chosen among the live positions in permuted order."""
+    br, bc = out // 16, inp // 16
+    total = br * bc
+    ntile = F.tile_count(out, inp, sparsity)
+    perm = F.permutation(total, seed)
+    ys, xs = perm // bc, perm % bc
+    live = ~np.isin(ys, list(dead_block_rows)) & ~np.isin(xs, list(dead_block_cols))
+    kept = perm[live][:ntile]
+    ys, xs = kept // bc, kept % bc
+    row_ptr = np.zeros(br + 1, np.int32)
+    cols = []
+    for r in range(br):
+        c = xs[ys == r]
+        cols.append(c)
+        row_ptr[r + 1] = row_ptr[r] + len(c)
+    col_idx = np.concatenate(cols).astype(np.int32) if cols else np.zeros(0, np.int32)
+    return row_ptr, col_idx
+
+
+class LayerWeights:
+    """One encoder layer: BSR Wqkv [3H,H], Wo [H,H], W1 [FF,H], W2 [H,FF] + LN params."""
+
+    def __init__(self, H, nh, dimFF, sparsity, seed, attention_aware=0.0, bias_std=0.02):
+        hd = H // nh
+        dead_v, dead_o = (), ()
+        if attention_aware > 0:
+            # per head, the last `attention_aware` share of the V rows (16-row groups) is dead
+            per_head_blocks = hd // 16
+            ndead = int(per_head_blocks * attention_aware)
+            dead_feat_blocks = [h * per_head_blocks + (per_head_blocks - 1 - i)
+                                for h in range(nh) for i in range(ndead)]
+            dead_v = tuple(2 * (H // 16) + b for b in dead_feat_blocks)  # V rows of Wqkv
+            dead_o = tuple(dead_feat_blocks)                             # matching O input columns
+        self.qkv = BsrWeight(3 * H, H, sparsity, seed * 100 + 1, bias_std=bias_std, dead_block_rows=dead_v)
+        if dead_v:
+            # a dead V feature has no weights and no bias
+            for b in dead_v:
+                self.qkv.bias[16 * b:16 * b + 16] = 0
+        self.o = BsrWeight(H, H, sparsity, seed * 100 + 11, bias_std=bias_std, dead_block_cols=dead_o)
+        self.l1 = BsrWeight(dimFF, H, sparsity, seed * 100 + 21, bias_std=bias_std)
+        self.l2 = BsrWeight(H, dimFF, sparsity, seed * 100 + 31, bias_std=bias_std)
+        self.g1 = (1.0 + randn((H,), seed * 100 + 41, 0.1, np.float32)).astype(np.float16)
+        self.be1 = randn((H,), seed * 100 + 42, 0.1)
+        self.g2 = (1.0 + randn((H,), seed * 100 + 43, 0.1, np.float32)).astype(np.float16)
+        self.be2 = randn((H,), seed * 100 + 44, 0.1)
+        self.H, self.nh, self.dimFF = H, nh, dimFF
+
+    def oracle_params(self) -> L.LayerParams:
+        return L.LayerParams(f32(self.qkv.dense), f32(self.qkv.bias), f32(self.o.dense), f32(self.o.bias),
+                             f32(self.l1.dense), f32(self.l1.bias), f32(self.l2.dense), f32(self.l2.bias),
+                             f32(self.g1), f32(self.be1), f32(self.g2), f32(self.be2))
+
+    def upload(self, et):
+        for w in (self.qkv, self.o, self.l1, self.l2):
+            w.upload(et)
+        self.d_g1, self.d_be1 = et.DeviceBuffer.from_numpy(self.g1), et.DeviceBuffer.from_numpy(self.be1)
+        self.d_g2, self.d_be2 = et.DeviceBuffer.from_numpy(self.g2), et.DeviceBuffer.from_numpy(self.be2)
+        return self
+
+
+class LayerScratch:
+    def __init__(self, et, T, H, dimFF):
+        E = et.DeviceBuffer.empty
+        self.qkv = E((T, 3 * H), np.float16)
+        self.z = E((T, H), np.float16)
+        self.attn = E((T, H), np.float16)
+        self.ln1 = E((T, H), np.float16)
+        self.ff = E((T, dimFF), np.float16)
+        self.ff2 = E((T, H), np.float16)
+
+
+def layer_forward_abi(et, w: LayerWeights, sc: LayerScratch, dX, dOut, B, S, d_lens=None, act=2,
+                      eps=1e-5, flags=0, d_mask=None, stream=None):
+    """One encoder layer through the kernel-level C ABI (the launch sequence the
+    C++ Encoder class issues)."""
+    H, nh = w.H, w.nh
+    hd = H // nh
+    T = B * S
+    w.qkv.forward(et, dX, sc.qkv, T, 0, stream)
+    q, k, v = sc.qkv.ptr, sc.qkv.offset(2 * H), sc.qkv.offset(4 * H)
+    et.mha_fused(q, k, v, 3 * H, 3 * H, 3 * H, sc.z, H, d_mask, d_lens, B, S, nh, hd,
+                 1.0 / math.sqrt(hd), flags, stream)
+    w.o.forward(et, sc.z, sc.attn, T, 0, stream)
+    et.skip_layernorm(sc.ln1, sc.attn, dX, w.d_g1, w.d_be1, T, H, eps, stream)
+    w.l1.forward(et, sc.ln1, sc.ff, T, act, stream)
+    w.l2.forward(et, sc.ff, sc.ff2, T, 0, stream)
+    et.skip_layernorm(dOut, sc.ff2, sc.ln1, w.d_g2, w.d_be2, T, H, eps, stream)
+
+
+def run_layer_case(et, H, nh, dimFF, S, B, sparsity, seed, lens=None, nlayers=1, attention_aware=0.0):
+    """Runs nlayers encoder layers on the GPU and returns the max-abs error
+    against the fp16-storage oracle."""
+    T = B * S
+    layers = [LayerWeights(H, nh, dimFF, sparsity, seed + i, attention_aware).upload(et) for i in range(nlayers)]
+    x = randn((T, H), seed + 1000, 1.0)
+    sc = LayerScratch(et, T, H, dimFF)
+    bufs = [et.DeviceBuffer.from_numpy(x), et.DeviceBuffer.empty((T, H), np.float16)]
+    d_lens = et.DeviceBuffer.from_numpy(np.asarray(lens, np.int32)) if lens is not None else None
+    for i, w in enumerate(layers):
+        layer_forward_abi(et, w, sc, bufs[i % 2], bufs[(i + 1) % 2], B, S, d_lens)
+    got = bufs[nlayers % 2].numpy(np.float16, (T, H))
+    cfg = L.LayerConfig(nh=nh, B=B, act="gelu", lens=None if lens is None else torch.as_tensor(lens),
+                        store=torch.float16)
+    want = L.encoder_stack(f32(x), [w.oracle_params() for w in layers], cfg).numpy()
+    return max_abs(got, want)

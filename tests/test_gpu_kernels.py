@@ -1,0 +1,320 @@
+"""GPU parity of the kernel-level C ABI against the CPU oracle (same seeded
+inputs).  fp16 path: max-abs <= 2e-2 is the bar the engine is built to; the
+per-kernel tests below hold tighter bounds where the arithmetic allows."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import formats as F
+from oracle import layers as L
+from tests import harness as Hn
+
+pytestmark = pytest.mark.gpu
+
+TOL_F16 = 2e-2
+
+
+def up(et, a):
+    return et.DeviceBuffer.from_numpy(a)
+
+
+# ---------------------------------------------------------------- runtime ----
+
+def test_device_is_gfx950(et):
+    info = et.device_info()
+    print(info)
+    assert "gfx950" in info["name"]
+    assert info["num_cu"] >= 1
+
+
+def test_fill_convert_roundtrip(et):
+    n = 100003
+    src = Hn.randn((n,), 3, 3.0, np.float32)
+    d_src = up(et, src)
+    d_h = et.DeviceBuffer.empty((n,), np.float16)
+    et.check(et.lib().et_f32_to_f16(d_h.ptr, d_src.ptr, n, None))
+    got = d_h.numpy()
+    assert np.array_equal(got.view(np.uint16), src.astype(np.float16).view(np.uint16))  # RN-even, bit exact
+    d_f = et.DeviceBuffer.empty((n,), np.float32)
+    et.check(et.lib().et_f16_to_f32(d_f.ptr, d_h.ptr, n, None))
+    assert np.array_equal(d_f.numpy(), got.astype(np.float32))
+    et.check(et.lib().et_fill_f16(d_h.ptr, n, int(np.float16(0.2).view(np.uint16)), None))
+    assert np.all(d_h.numpy() == np.float16(0.2))
+    et.check(et.lib().et_memset(d_h.ptr, 0, n * 2, None))
+    assert np.all(d_h.numpy().view(np.uint16) == 0)
+    fresh = et.DeviceBuffer.empty((4096,), np.float16)  # et_malloc zero-fills (CUDA_ptr(size))
+    assert np.all(fresh.numpy().view(np.uint16) == 0)
+
+
+# ---------------------------------------------------------------- norms ------
+
+@pytest.mark.parametrize("rows,H", [(1024, 768), (2048, 1024), (128, 800), (7, 64), (33, 2048), (5, 4100)])
+def test_skip_layernorm(et, rows, H):
+    src, skip = Hn.randn((rows, H), 1), Hn.randn((rows, H), 2)
+    gamma = (1 + Hn.randn((H,), 3, 0.1, np.float32)).astype(np.float16)
+    beta = Hn.randn((H,), 4, 0.1)
+    d_out = et.DeviceBuffer.empty((rows, H), np.float16)
+    et.skip_layernorm(d_out, up(et, src), up(et, skip), up(et, gamma), up(et, beta), rows, H, 1e-5)
+    want = L.skip_layernorm(Hn.f32(src), Hn.f32(skip), Hn.f32(gamma), Hn.f32(beta), 1e-5, torch.float16)
+    # one fp16 rounding of an O(4) value: half an ulp = 2e-3
+    assert Hn.max_abs(d_out.numpy(), want.numpy()) <= 4e-3
+
+
+@pytest.mark.parametrize("rows,H", [(1024, 768), (16, 1024), (3, 800)])
+def test_layernorm(et, rows, H):
+    src = Hn.randn((rows, H), 5, 2.0)
+    gamma = (1 + Hn.randn((H,), 6, 0.1, np.float32)).astype(np.float16)
+    beta = Hn.randn((H,), 7, 0.1)
+    d_out = et.DeviceBuffer.empty((rows, H), np.float16)
+    et.layernorm(d_out, up(et, src), up(et, gamma), up(et, beta), rows, H, 1e-5)
+    want = L.layernorm(Hn.f32(src), Hn.f32(gamma), Hn.f32(beta), 1e-5, torch.float16)
+    assert Hn.max_abs(d_out.numpy(), want.numpy()) <= 4e-3
+
+
+def test_layernorm_rejects_bad_shape(et):
+    d = et.DeviceBuffer.empty((16, 16), np.float16)
+    st = et.lib().et_layernorm_f16(d.ptr, d.ptr, d.ptr, d.ptr, 4, 6, 1e-5, None)
+    assert st == et.ET_ERR_UNSUPPORTED
+    st = et.lib().et_skip_layernorm_f16(d.ptr, d.ptr, None, d.ptr, d.ptr, 4, 8, 1e-5, None)
+    assert st == et.ET_ERR_INVALID_ARG
+    assert b"skip" in et.lib().et_last_error()
+
+
+# ---------------------------------------------------------------- elementwise
+
+@pytest.mark.parametrize("n", [1024 * 3072, 1000003, 5])
+def test_gelu_relu(et, n):
+    x = Hn.randn((n,), 8, 2.0)
+    d_x = up(et, x)
+    d_y = et.DeviceBuffer.empty((n,), np.float16)
+    et.check(et.lib().et_gelu_f16(d_y.ptr, d_x.ptr, n, None))
+    want = L.gelu_tanh(Hn.f32(x)).half().numpy()
+    assert Hn.max_abs(d_y.numpy(), want) <= 2e-3
+    et.check(et.lib().et_relu_f16(d_x.ptr, d_x.ptr, n, None))  # in place
+    assert np.array_equal(d_x.numpy(), np.maximum(x, np.float16(0)))
+
+
+@pytest.mark.parametrize("rows,cols", [(128, 768), (33, 50)])
+def test_bias_add(et, rows, cols):
+    x, b = Hn.randn((rows, cols), 9), Hn.randn((cols,), 10)
+    d_x = up(et, x)
+    et.check(et.lib().et_bias_add_f16(d_x.ptr, up(et, b).ptr, rows, cols, None))
+    want = (x.astype(np.float32) + b.astype(np.float32)).astype(np.float16)
+    assert np.array_equal(d_x.numpy().view(np.uint16), want.view(np.uint16))
+
+
+# ---------------------------------------------------------------- BSR linear -
+
+BSR_CASES = [
+    # T, in, out, sparsity, act
+    (2048, 768, 768, 0.8, 0),
+    (2048, 768, 768, 0.9, 0),
+    (2048, 768, 3072, 0.8, 2),
+    (2048, 3072, 768, 0.8, 0),
+    (1024, 768, 2304, 0.8, 0),
+    (128, 800, 208, 0.5, 1),     # the example model's FFN shape (example/main.cu:29)
+    (16, 16, 16, 0.0, 0),
+    (48, 64, 32, 0.3, 2),
+    (2048, 4096, 1024, 0.9, 0),  # BERT-large FFN
+    (64, 6144, 64, 0.5, 0),      # input too wide for an LDS-staged strip
+]
+
+
+@pytest.mark.parametrize("T,inp,out,sp,act", BSR_CASES)
+def test_linear_bsr16(et, T, inp, out, sp, act):
+    w = Hn.BsrWeight(out, inp, sp, seed=11, bias_std=0.1).upload(et)
+    x = Hn.randn((T, inp), 12)
+    d_y = et.DeviceBuffer.empty((T, out), np.float16)
+    w.forward(et, up(et, x), d_y, T, act)
+    want = L.linear(Hn.f32(x), Hn.f32(w.dense), Hn.f32(w.bias), {0: None, 1: "relu", 2: "gelu"}[act],
+                    torch.float16)
+    err = Hn.max_abs(d_y.numpy(), want.numpy())
+    print(f"bsr T={T} in={inp} out={out} sp={sp}: ntile={len(w.col_idx)} max-abs={err:.2e}")
+    # |y| stays below ~4 here: one fp16 rounding (<= 2e-3) plus accumulation-order noise
+    assert err <= 4e-3
+
+
+def test_linear_bsr16_closed_form_all_ones(et):
+    """All-ones input and all-ones tiles: Y[t][o] = 16 * tiles_in_block_row(o/16) + bias
+    (the only closed form the reference's driver offers, Linear/test/test_tile.cu:56-75)."""
+    T, inp, out = 64, 256, 128
+    row_ptr, col_idx = F.gen_tile_pattern(out, inp, 0.6, seed=5)
+    tiles = np.ones((len(col_idx), 256), np.float16)
+    bias = np.full(out, 0.5, np.float16)
+    x = np.ones((T, inp), np.float16)
+    d_y = et.DeviceBuffer.empty((T, out), np.float16)
+    et.linear_bsr16(up(et, row_ptr), up(et, col_idx), up(et, tiles), up(et, bias), up(et, x), d_y, T, inp, out)
+    per_row = np.diff(row_ptr)
+    want = np.repeat(16.0 * per_row + 0.5, 16)[None, :].repeat(T, 0)
+    assert np.array_equal(d_y.numpy().astype(np.float32), want.astype(np.float32))
+
+
+def test_linear_bsr16_empty_rows_and_no_bias(et):
+    T, inp, out = 32, 64, 64
+    row_ptr = np.array([0, 0, 2, 2, 3], np.int32)  # block-rows 0 and 2 hold no tile
+    col_idx = np.array([3, 0, 1], np.int32)
+    tiles = Hn.randn((3, 256), 21, 0.5)
+    x = Hn.randn((T, inp), 22)
+    d_y = et.DeviceBuffer.empty((T, out), np.float16)
+    et.check(et.lib().et_fill_f16(d_y.ptr, T * out, 0x7E00, None))  # NaN: every element must be written
+    et.linear_bsr16(up(et, row_ptr), up(et, col_idx), up(et, tiles), None, up(et, x), d_y, T, inp, out)
+    W = F.bsr16_to_dense(row_ptr, col_idx, tiles, inp)
+    want = L.linear(Hn.f32(x), Hn.f32(W), None, None, torch.float16).numpy()
+    got = d_y.numpy()
+    assert np.all(got[:, :16] == 0) and np.all(got[:, 32:48] == 0)
+    assert Hn.max_abs(got, want) <= 4e-3
+
+
+def test_linear_bsr16_tile_order_is_free(et):
+    """Permuting the tiles inside each block-row (with their column ids) leaves Y unchanged
+    up to accumulation order."""
+    T, inp, out = 64, 256, 64
+    w = Hn.BsrWeight(out, inp, 0.5, seed=31)
+    col2, tiles2 = w.col_idx.copy(), w.tiles.copy()
+    for r in range(out // 16):
+        lo, hi = w.row_ptr[r], w.row_ptr[r + 1]
+        col2[lo:hi] = w.col_idx[lo:hi][::-1]
+        tiles2[lo:hi] = w.tiles[lo:hi][::-1]
+    x = Hn.randn((T, inp), 32)
+    d_x = up(et, x)
+    ys = []
+    for c, t in ((w.col_idx, w.tiles), (col2, tiles2)):
+        d_y = et.DeviceBuffer.empty((T, out), np.float16)
+        et.linear_bsr16(up(et, w.row_ptr), up(et, c), up(et, t), None, d_x, d_y, T, inp, out)
+        ys.append(d_y.numpy())
+    assert Hn.max_abs(ys[0], ys[1]) <= 1e-3
+
+
+def test_linear_bsr16_rejects_bad_args(et):
+    d = et.DeviceBuffer.empty((64, 64), np.float16)
+    f = et.lib().et_linear_bsr16_f16
+    assert f(d.ptr, d.ptr, d.ptr, None, d.ptr, d.ptr, 20, 64, 64, 0, None) == et.ET_ERR_UNSUPPORTED
+    assert f(None, d.ptr, d.ptr, None, d.ptr, d.ptr, 16, 64, 64, 0, None) == et.ET_ERR_INVALID_ARG
+    assert f(d.ptr, d.ptr, d.ptr, None, d.ptr, d.ptr, 16, 64, 64, 9, None) == et.ET_ERR_INVALID_ARG
+    assert f(d.ptr, d.ptr, d.ptr, None, d.ptr, d.ptr, 0, 64, 64, 0, None) == et.ET_OK  # empty batch
+
+
+@pytest.mark.parametrize("mt,stage,threads,rpw", [(1, 1, 256, 4), (2, 1, 128, 3), (4, 1, 512, 8),
+                                                  (4, 0, 256, 5), (1, 0, 64, 1), (2, 0, 512, 48)])
+def test_linear_bsr16_every_geometry(et, mt, stage, threads, rpw):
+    """Each launch geometry of the kernel gives the same result, including a token count that
+    is not a multiple of the strip."""
+    T, inp, out = 80, 768, 768
+    w = Hn.BsrWeight(out, inp, 0.8, seed=41, bias_std=0.1).upload(et)
+    x = Hn.randn((T, inp), 42)
+    d_y = et.DeviceBuffer.empty((T, out), np.float16)
+    et.check(et.lib().et_linear_bsr16_f16_geom(w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, w.d_bias.ptr,
+                                               up(et, x).ptr, d_y.ptr, T, inp, out, 2, mt, stage, threads, rpw,
+                                               None))
+    want = L.linear(Hn.f32(x), Hn.f32(w.dense), Hn.f32(w.bias), "gelu", torch.float16)
+    assert Hn.max_abs(d_y.numpy(), want.numpy()) <= 4e-3
+
+
+# ---------------------------------------------------------------- attention --
+
+def run_mha(et, B, S, nh, hd, seed, lens=None, causal=False, mask=None, single_buffer=False):
+    H = nh * hd
+    T = B * S
+    if single_buffer:
+        qkv = Hn.randn((T, 3 * H), seed, 1.0)
+        d_qkv = up(et, qkv)
+        q, k, v = qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:]
+        pq, pk, pv, ld = d_qkv.ptr, d_qkv.offset(2 * H), d_qkv.offset(4 * H), 3 * H
+        keep = [d_qkv]
+    else:
+        q, k, v = Hn.randn((T, H), seed), Hn.randn((T, H), seed + 1), Hn.randn((T, H), seed + 2)
+        keep = [up(et, q), up(et, k), up(et, v)]
+        pq, pk, pv, ld = keep[0].ptr, keep[1].ptr, keep[2].ptr, H
+    d_z = et.DeviceBuffer.empty((T, H), np.float16)
+    et.check(et.lib().et_fill_f16(d_z.ptr, T * H, 0x7E00, None))
+    d_lens = up(et, np.asarray(lens, np.int32)) if lens is not None else None
+    d_mask = up(et, mask.astype(np.float16)) if mask is not None else None
+    et.mha_fused(pq, pk, pv, ld, ld, ld, d_z, H, d_mask, d_lens, B, S, nh, hd, 1.0 / math.sqrt(hd),
+                 et.MHA_CAUSAL if causal else 0)
+    want = L.mha(Hn.f32(q), Hn.f32(k), Hn.f32(v), nh, B, mask=None if mask is None else Hn.f32(mask),
+                 lens=lens, causal=causal, store=torch.float16)
+    return d_z.numpy(), want.numpy()
+
+
+@pytest.mark.parametrize("B", [1, 4, 16])
+def test_mha_block_config(et, B):
+    """Attention core of the BERT-base block: S128, 12 heads x 64, right padding U{64..128}."""
+    lens = torch.randint(64, 129, (B,), generator=Hn.rng(100 + B)).numpy()
+    got, want = run_mha(et, B, 128, 12, 64, seed=50, lens=lens, single_buffer=True)
+    err = Hn.max_abs(got, want)
+    print(f"mha B={B} lens={lens.tolist()} max-abs={err:.2e}")
+    assert err <= 2e-3
+
+
+@pytest.mark.parametrize("B,S,nh,hd,causal", [(1, 128, 12, 64, True), (2, 512, 16, 64, False),
+                                              (1, 384, 12, 64, False), (3, 32, 4, 32, False),
+                                              (2, 48, 2, 128, True), (1, 16, 1, 64, False),
+                                              (2, 272, 4, 64, True)])
+def test_mha_shapes(et, B, S, nh, hd, causal):
+    got, want = run_mha(et, B, S, nh, hd, seed=60, causal=causal)
+    assert Hn.max_abs(got, want) <= 2e-3
+
+
+def test_mha_additive_mask_and_lens(et):
+    B, S, nh, hd = 2, 128, 4, 64
+    mask = Hn.randn((S, S), 70, 1.0, np.float32)
+    mask[torch.rand(S, S, generator=Hn.rng(71)).numpy() < 0.3] = -np.inf
+    mask[np.arange(S), np.arange(S)] = 0.0  # every query keeps at least itself ...
+    mask[:, 0] = 0.0                        # ... and key 0, which survives any padding
+    lens = np.array([128, 77])
+    got, want = run_mha(et, B, S, nh, hd, seed=72, lens=lens, mask=mask)
+    assert Hn.max_abs(got, want) <= 2e-3
+
+
+def test_mha_padding_properties(et):
+    """Padded keys get exactly zero weight: changing K/V rows beyond lens changes nothing,
+    and each sequence of a batch equals the same sequence run alone."""
+    B, S, nh, hd = 3, 128, 12, 64
+    H = nh * hd
+    lens = np.array([64, 100, 128], np.int32)
+    q, k, v = Hn.randn((B * S, H), 80), Hn.randn((B * S, H), 81), Hn.randn((B * S, H), 82)
+    k2, v2 = k.copy(), v.copy()
+    for b in range(B):
+        k2[b * S + lens[b]:(b + 1) * S] = np.float16(50.0)
+        v2[b * S + lens[b]:(b + 1) * S] = np.float16(-1000.0)
+
+    def run(qq, kk, vv, BB, ll):
+        d_z = et.DeviceBuffer.empty((BB * S, H), np.float16)
+        et.mha_fused(up(et, qq), up(et, kk), up(et, vv), H, H, H, d_z, H, None, up(et, ll), BB, S, nh, hd,
+                     0.125)
+        return d_z.numpy()
+
+    base = run(q, k, v, B, lens)
+    assert np.array_equal(base, run(q, k2, v2, B, lens))
+    for b in range(B):
+        sl = slice(b * S, (b + 1) * S)
+        alone = run(q[sl], k[sl], v[sl], 1, lens[b:b + 1])
+        assert np.array_equal(base[sl], alone)
+    assert np.all(np.isfinite(base.astype(np.float32)))
+
+
+def test_mha_zero_length_sequence_gives_zeros(et):
+    B, S, nh, hd = 2, 32, 2, 64
+    got, _ = run_mha(et, B, S, nh, hd, seed=90, lens=np.array([0, 32]))
+    assert np.all(got[:S] == 0)
+
+
+def test_mha_rejects_bad_args(et):
+    d = et.DeviceBuffer.empty((128, 768), np.float16)
+    f = et.lib().et_mha_fused_f16
+    args = lambda S, hd, ld: (d.ptr, d.ptr, d.ptr, ld, ld, ld, d.ptr, ld, None, None, 1, S, 12, hd, 0.125, 0, None)
+    assert f(*args(120, 64, 768)) == et.ET_ERR_UNSUPPORTED   # S % 16
+    assert f(*args(128, 48, 768)) == et.ET_ERR_UNSUPPORTED   # head dim
+    assert f(*args(128, 64, 512)) == et.ET_ERR_INVALID_ARG   # stride < nh*hd
+    assert f(None, d.ptr, d.ptr, 768, 768, 768, d.ptr, 768, None, None, 1, 128, 12, 64, 0.125, 0, None) == et.ET_ERR_INVALID_ARG
+
+
+# ---------------------------------------------------------------- layer ------
+
+@pytest.mark.parametrize("B,lens", [(1, None), (2, [100, 128])])
+def test_encoder_layer_via_kernels(et, B, lens):
+    err = Hn.run_layer_case(et, H=768, nh=12, dimFF=3072, S=128, B=B, sparsity=0.8, seed=3, lens=lens)
+    print(f"layer B={B} max-abs={err:.2e}")
+    assert err <= TOL_F16
