@@ -1,0 +1,277 @@
+// Multi-head self-attention block — the reference's Attention<cfg>
+// (Attention/Attention.h:10-266): Q/K/V projections, fused attention, output
+// projection, with the same configuration tags and constructor signatures.
+//
+// Differences from the reference, all deliberate:
+//  * every on-the-fly tag runs the one fused gfx950 kernel (scores, mask,
+//    softmax and P*V in registers/LDS, fp32 accumulation, 1/sqrt(hd) scale);
+//    the tags stay distinct types so that callers keep compiling;
+//  * a batch of sequences is supported: `batch` sequences of model->seq_len rows,
+//    optional per-sequence key lengths (right padding);
+//  * the mask is a property the caller sets (none by default, causal, or an
+//    additive [S x S] matrix) instead of the hard-wired causal mask of
+//    Attention/Attention.h:96-104;
+//  * all launches go to ONE stream passed to forward(), nothing joins on the host
+//    (the reference fans Q/K/V out to three streams and blocks on them,
+//    Attention/Attention.h:122-127), so a forward can be captured into a HIP graph.
+#pragma once
+#include <cmath>
+#include <memory>
+#include <type_traits>
+#include <vector>
+
+#include "Linear.h"
+#include "Model.h"
+
+using ptr_t = et::DeviceBuffer<half>;
+
+template <typename _WQ_t, typename _WK_t, typename _WV_t, typename _WO_t, typename _attn_t,
+          bool _isSingleKernel = false, bool _isPara = true,
+          typename = typename std::enable_if<!(_isSingleKernel && _isPara)>::type>
+struct Attention_config {
+    using WQ_t = _WQ_t;
+    using WK_t = _WK_t;
+    using WV_t = _WV_t;
+    using WO_t = _WO_t;
+    using attn_t = _attn_t;
+    static constexpr bool isPara = _isPara;  // kept for source compatibility; one stream is used
+    static constexpr bool isSingleKernel = _isSingleKernel;
+    using W_t = typename std::conditional<_isSingleKernel, _WQ_t, void>::type;
+};
+
+// attention kernel tags (Attention/Attention.h:26-33)
+struct OTF_attn {};
+struct Norm_attn {};
+struct Prune_attn {};
+struct OTF_attn_full {};
+struct OTF_attn_tile {};
+struct OTF_attn_sharedQK {};
+struct OTF_attn_full_mixed {};
+struct OTF_attn_Ofused {};
+
+namespace et {
+
+// What a fused attention call needs beyond Q, K, V: sequences, mask, stream.
+struct AttnRun {
+    int batch = 1;
+    const int *lens = nullptr;   // device int32[batch] or nullptr
+    const half *mask = nullptr;  // device additive [S x S] or nullptr
+    bool causal = false;
+    float scale = 0.0f;          // 0 = 1/sqrt(head_dim)
+    stream_t stream = nullptr;
+};
+
+inline void fused_mha(const half *q, const half *k, const half *v, int ldq, int ldk, int ldv, half *z,
+                      int ldz, const Model_t &m, const AttnRun &run) {
+    const int hd = m.kdim / m.nhead;
+    require(m.vdim == m.kdim, "fused attention: vdim must equal kdim");
+    const float scale = run.scale != 0.0f ? run.scale : 1.0f / std::sqrt((float)hd);
+    etChk(et_mha_fused_f16(f16(q), f16(k), f16(v), ldq, ldk, ldv, f16(z), ldz, f16(run.mask), run.lens,
+                           run.batch, m.seq_len, m.nhead, hd, scale, run.causal ? ET_MHA_CAUSAL : 0,
+                           run.stream));
+}
+
+}  // namespace et
+
+// Free-function form (Attention/Attention.h:35-45,144-181).  mat_qk is unused by
+// the fused kernel (scores never reach memory) and may be null.
+template <typename _attn_type>
+void Multihead_atttion(ptr_t *mat_q, ptr_t *mat_k, ptr_t *mat_v, ptr_t *mat_qk, const ptr_t *mask,
+                       ptr_t *mat_z, std::shared_ptr<Model_t> model, et::AttnRun run = et::AttnRun()) {
+    static_assert(!std::is_same<_attn_type, Prune_attn>::value, "Prune_attn takes a col_mat V");
+    (void)mat_qk;
+    if (mask && !run.mask) run.mask = mask->get();
+    if constexpr (std::is_same<_attn_type, Norm_attn>::value) {
+        // Unfused baseline: scores through memory (Attention/Attention.cu:8-36).
+        et::require(mat_qk != nullptr, "Norm_attn needs the mat_qk workspace");
+        const int hd = model->kdim / model->nhead;
+        const float scale = run.scale != 0.0f ? run.scale : 1.0f / std::sqrt((float)hd);
+        etChk(et_mha_unfused_f16(et::f16(mat_q->get()), et::f16(mat_k->get()), et::f16(mat_v->get()),
+                                 model->kdim, model->kdim, model->vdim, et::f16(mat_z->get()), model->vdim,
+                                 et::f16(mat_qk->get()), et::f16(run.mask), run.lens, run.batch,
+                                 model->seq_len, model->nhead, hd, scale, run.causal ? ET_MHA_CAUSAL : 0,
+                                 run.stream));
+        return;
+    }
+    et::fused_mha(mat_q->get(), mat_k->get(), mat_v->get(), model->kdim, model->kdim, model->vdim,
+                  mat_z->get(), model->vdim, *model, run);
+}
+
+// Attention-aware form: V is compact [S x nnz] with col_id / head_ptr metadata
+// (Attention/Attention.cu:54-78).  Pruned columns of Z are written as zero.
+template <typename _attn_type>
+void Multihead_atttion(ptr_t *mat_q, ptr_t *mat_k, col_mat *mat_v, ptr_t *mat_qk, const ptr_t *mask,
+                       ptr_t *mat_z, std::shared_ptr<Model_t> model, et::AttnRun run = et::AttnRun()) {
+    static_assert(std::is_same<_attn_type, Prune_attn>::value, "a col_mat V belongs to Prune_attn");
+    (void)mat_qk;
+    if (mask && !run.mask) run.mask = mask->get();
+    et::require(mat_v->head_ptr != nullptr, "Prune_attn: col_mat::set_metadata was not called");
+    const int hd = model->kdim / model->nhead;
+    const float scale = run.scale != 0.0f ? run.scale : 1.0f / std::sqrt((float)hd);
+    etChk(et_mha_compactv_f16(et::f16(mat_q->get()), et::f16(mat_k->get()), et::f16(mat_v->cols->get()),
+                              model->kdim, model->kdim, mat_v->ldm, mat_v->col_id->get(),
+                              mat_v->head_ptr->get(), mat_v->nnz_col, et::f16(mat_z->get()), model->vdim,
+                              et::f16(run.mask), run.lens, run.batch, model->seq_len, model->nhead, hd,
+                              model->vdim / model->nhead, scale, run.causal ? ET_MHA_CAUSAL : 0, run.stream));
+}
+
+// Attention followed by the tile-sparse output projection
+// (Attention/kernel_fuseO.h:6-9, Attention/kernel_fuseO.cu:254-290).  The
+// reference joins the two with a grid-wide barrier inside one cooperative
+// launch; here they are two back-to-back launches on one stream, which orders
+// them without occupying the device with a spinning grid.
+inline void Multihead_atttion_fuseO(half *mat_q, half *mat_k, half *mat_v, const half *mask, half *mat_z,
+                                    const int *row_ptr, const int *row_offset, const half *data,
+                                    const half *bias, std::shared_ptr<Model_t> model, half *out,
+                                    et::AttnRun run = et::AttnRun()) {
+    if (mask && !run.mask) run.mask = mask;
+    et::fused_mha(mat_q, mat_k, mat_v, model->kdim, model->kdim, model->vdim, mat_z, model->vdim, *model, run);
+    etChk(et_linear_bsr16_f16(row_ptr, row_offset, et::f16(data), et::f16(bias), et::f16(mat_z), et::f16(out),
+                              run.batch * model->seq_len, model->vdim, model->emdim, ET_ACT_NONE, run.stream));
+}
+
+template <typename T> struct __matv_helper { using type = ptr_t; };
+template <> struct __matv_helper<Prune_attn> { using type = col_mat; };
+
+namespace et {
+
+// Mask / padding state shared by both Attention forms and FusedAttention.
+class AttnState {
+  public:
+    AttnState(std::shared_ptr<Model_t> m, int batch) : model_(std::move(m)), batch_(batch) {
+        require(batch >= 1, "Attention: batch must be at least 1");
+        require(model_->nhead > 0 && model_->kdim % model_->nhead == 0, "Attention: kdim % nhead != 0");
+    }
+    // additive [S x S] mask from host memory (the reference's layout); nullptr removes it
+    void set_mask(const half *host_mask) {
+        if (!host_mask) { mask_.reset(); return; }
+        const std::size_t n = (std::size_t)model_->seq_len * model_->seq_len;
+        mask_ = std::make_unique<ptr_t>(host_mask, n);
+    }
+    void set_causal(bool on) { causal_ = on; }
+    // right padding: keys >= lens[b] of sequence b are ignored; nullptr removes it
+    void set_lens(const int *host_lens) {
+        if (!host_lens) { lens_.reset(); return; }
+        lens_ = std::make_unique<DeviceBuffer<int>>(host_lens, (std::size_t)batch_);
+    }
+    int batch() const { return batch_; }
+    int rows() const { return batch_ * model_->seq_len; }
+    AttnRun run(stream_t stream) const {
+        AttnRun r;
+        r.batch = batch_;
+        r.lens = lens_ ? lens_->get() : nullptr;
+        r.mask = mask_ ? mask_->get() : nullptr;
+        r.causal = causal_;
+        r.stream = stream;
+        return r;
+    }
+
+  protected:
+    std::shared_ptr<Model_t> model_;
+    int batch_;
+    bool causal_ = false;
+    std::unique_ptr<ptr_t> mask_;
+    std::unique_ptr<DeviceBuffer<int>> lens_;
+};
+
+}  // namespace et
+
+template <typename _config, typename = void> class Attention {};
+
+// separate Q, K, V projections — Attention/Attention.h:57-142
+template <typename _config>
+class Attention<_config, std::enable_if_t<!_config::isSingleKernel>> : public et::AttnState {
+    using config = _config;
+    using linearQ_t = Linear<typename config::WQ_t>;
+    using linearK_t = Linear<typename config::WK_t>;
+    using linearV_t = Linear<typename config::WV_t>;
+    using linearO_t = Linear<typename config::WO_t>;
+    using mat_v_t = typename __matv_helper<typename config::attn_t>::type;
+    static constexpr bool kPruned = std::is_same<typename config::attn_t, Prune_attn>::value;
+
+    std::unique_ptr<linearQ_t> linearQ;
+    std::unique_ptr<linearK_t> linearK;
+    std::unique_ptr<linearV_t> linearV;
+    std::unique_ptr<linearO_t> linearO;
+    std::unique_ptr<ptr_t> mat_k, mat_q, mat_qk, mat_z;
+    std::unique_ptr<mat_v_t> mat_v;
+    std::shared_ptr<Model_t> model;
+
+  public:
+    Attention(std::unique_ptr<linearQ_t> _linearQ, std::unique_ptr<linearK_t> _linearK,
+              std::unique_ptr<linearV_t> _linearV, std::unique_ptr<linearO_t> _linearO,
+              std::shared_ptr<Model_t> _model, int batch = 1)
+        : et::AttnState(_model, batch), linearQ(std::move(_linearQ)), linearK(std::move(_linearK)),
+          linearV(std::move(_linearV)), linearO(std::move(_linearO)), model(_model) {
+        static_assert(std::is_same<typename config::W_t, void>::value, "separate-QKV form");
+        const std::size_t T = (std::size_t)rows();
+        mat_k = std::make_unique<ptr_t>(T * model->kdim);
+        mat_q = std::make_unique<ptr_t>(T * model->kdim);
+        mat_z = std::make_unique<ptr_t>(T * model->vdim);
+        if constexpr (std::is_same<typename config::attn_t, Norm_attn>::value)
+            mat_qk = std::make_unique<ptr_t>(T * model->seq_len * model->nhead);
+        if constexpr (kPruned) {
+            static_assert(std::is_same<typename config::WV_t, row_mat>::value,
+                          "Prune_attn needs a row-pruned V projection");
+            const int nnz = linearV->weight.nnz_row();
+            mat_v = std::make_unique<col_mat>((int)T, model->vdim, nnz);
+            mat_v->set_metadata(*linearV->weight.row_id, nnz, model->nhead, model->vdim);
+        } else {
+            mat_v = std::make_unique<ptr_t>(T * model->vdim);
+        }
+    }
+
+    void forward(half *out, half *query, half *key, half *value, et::stream_t stream = nullptr) {
+        linearQ->forward(mat_q->get(), query, stream);
+        linearK->forward(mat_k->get(), key, stream);
+        linearV->forward(mat_v->get(), value, stream);
+        const et::AttnRun r = run(stream);
+        if constexpr (std::is_same<OTF_attn_Ofused, typename config::attn_t>::value) {
+            static_assert(std::is_same<typename config::WO_t, tile_mat>::value,
+                          "the O-fused form needs a tile-sparse output projection");
+            Multihead_atttion_fuseO(mat_q->get(), mat_k->get(), mat_v->get(), nullptr, mat_z->get(),
+                                    linearO->weight.row_ptr.get(), linearO->weight.row_offset.get(),
+                                    linearO->weight.data.get(), linearO->bias.get(), model, out, r);
+        } else {
+            Multihead_atttion<typename config::attn_t>(mat_q.get(), mat_k.get(), mat_v.get(), mat_qk.get(),
+                                                       nullptr, mat_z.get(), model, r);
+            linearO->forward(out, mat_z->get(), stream);
+        }
+    }
+};
+
+// one projection H -> (2*kdim + vdim), attention over column slices of its output
+// — Attention/Attention.h:204-266, kernel Attention/Attention_single.cu:10-108
+template <typename _config>
+class Attention<_config, std::enable_if_t<_config::isSingleKernel>> : public et::AttnState {
+    using config = _config;
+    using linearQKV_t = Linear<typename config::W_t>;
+    using linearO_t = Linear<typename config::WO_t>;
+
+    std::unique_ptr<linearQKV_t> linearQKV;
+    std::unique_ptr<linearO_t> linearO;
+    std::unique_ptr<ptr_t> mat_qkv, mat_z;
+    std::shared_ptr<Model_t> model;
+
+  public:
+    Attention(std::unique_ptr<linearQKV_t> _linearQKV, std::unique_ptr<linearO_t> _linearO,
+              std::shared_ptr<Model_t> _model, int batch = 1)
+        : et::AttnState(_model, batch), linearQKV(std::move(_linearQKV)), linearO(std::move(_linearO)),
+          model(_model) {
+        static_assert(!std::is_same<typename config::W_t, void>::value, "single-projection form");
+        const std::size_t T = (std::size_t)rows();
+        mat_qkv = std::make_unique<ptr_t>(T * (model->kdim * 2 + model->vdim));
+        mat_z = std::make_unique<ptr_t>(T * model->vdim);
+    }
+
+    void forward(half *out, half *query, half *key, half *value, et::stream_t stream = nullptr) {
+        et::require(query == key && key == value, "single-projection attention is self-attention");
+        linearQKV->forward(mat_qkv->get(), query, stream);
+        const int ldm = model->kdim * 2 + model->vdim;
+        half *Q = mat_qkv->get();
+        half *K = Q + model->kdim;
+        half *V = K + model->kdim;
+        et::fused_mha(Q, K, V, ldm, ldm, ldm, mat_z->get(), model->vdim, *model, run(stream));
+        linearO->forward(out, mat_z->get(), stream);
+    }
+};

@@ -1,0 +1,120 @@
+// Transformer encoder layer (post-LN with skip connections) — the reference's
+// Encoder<cfg> and Encoder_fuse<cfg> (Encoder/Encoder.h:10-139):
+//   a  = attn(src)              y1  = SkipLN1(a, src)
+//   f  = act(linear1(y1))       out = SkipLN2(linear2(f), y1)
+// The activation is applied inside linear1's kernel epilogue (on the fp32
+// accumulator) rather than as a separate pass over [rows x dimFF]; act<>() is
+// still provided for callers that use it stand-alone.  forward() issues six
+// launches on one stream, never blocks the host and writes nothing to stdout.
+#pragma once
+#include <memory>
+#include <type_traits>
+
+#include "Attention.h"
+#include "Fused_attention.h"
+#include "LayerNorm.h"
+#include "Linear.h"
+#include "Model.h"
+#include "SkipLayerNorm.h"
+
+template <typename _attn, typename _l1, typename _l2, typename _act_t> struct Encoder_config {
+    using attn_config = _attn;
+    using linear1_config = _l1;
+    using linear2_config = _l2;
+    using act_t = _act_t;
+};
+
+struct RELU_OP {};
+struct GELU_OP {};
+
+namespace GELU {
+// tanh-form GELU over n values (Encoder/Encoder.cu:41-68)
+inline void computeGelu(et::stream_t stream, int n, const half *input, half *output) {
+    etChk(et_gelu_f16(reinterpret_cast<et_f16 *>(output), reinterpret_cast<const et_f16 *>(input),
+                      (std::size_t)n, stream));
+}
+}  // namespace GELU
+
+namespace et {
+template <typename ACT_OP_t> constexpr int act_code() {
+    return std::is_same<ACT_OP_t, RELU_OP>::value ? ET_ACT_RELU
+           : std::is_same<ACT_OP_t, GELU_OP>::value ? ET_ACT_GELU
+                                                    : ET_ACT_NONE;
+}
+}  // namespace et
+
+// in-place activation (Encoder/Encoder.h:27-37)
+template <typename ACT_OP_t> void act(half *data, int size, et::stream_t stream = nullptr) {
+    if constexpr (std::is_same<ACT_OP_t, RELU_OP>::value) {
+        etChk(et_relu_f16(reinterpret_cast<et_f16 *>(data), reinterpret_cast<const et_f16 *>(data),
+                          (std::size_t)size, stream));
+    } else if constexpr (std::is_same<ACT_OP_t, GELU_OP>::value) {
+        GELU::computeGelu(stream, size, data, data);
+    }
+}
+
+namespace et {
+
+// The layer body shared by Encoder and Encoder_fuse.
+template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_OP_t> class EncoderLayer {
+  protected:
+    std::unique_ptr<attn_t> attn;
+    std::unique_ptr<SkipLayerNorm> LN1, LN2;
+    std::unique_ptr<linear1_t> linear1;
+    std::unique_ptr<linear2_t> linear2;
+    std::shared_ptr<Model_t> model;
+    int rows;
+
+  public:
+    DeviceBuffer<half> temp_linear;  // [rows x dimFF]
+    DeviceBuffer<half> temp_attn;    // [rows x emdim]
+    DeviceBuffer<half> temp_LN;      // [rows x emdim]
+
+    EncoderLayer(std::unique_ptr<attn_t> _attn, std::unique_ptr<SkipLayerNorm> _LN1,
+                 std::unique_ptr<SkipLayerNorm> _LN2, std::unique_ptr<linear1_t> _linear1,
+                 std::unique_ptr<linear2_t> _linear2, std::shared_ptr<Model_t> _model)
+        : attn(std::move(_attn)), LN1(std::move(_LN1)), LN2(std::move(_LN2)), linear1(std::move(_linear1)),
+          linear2(std::move(_linear2)), model(std::move(_model)), rows(attn->rows()),
+          temp_linear((std::size_t)rows * model->dimFF), temp_attn((std::size_t)rows * model->emdim),
+          temp_LN((std::size_t)rows * model->emdim) {
+        require(linear1->size == rows && linear2->size == rows,
+                "Encoder: the Linear layers must be built for batch * seq_len rows");
+    }
+
+    attn_t &attention() { return *attn; }
+    int token_rows() const { return rows; }
+
+    void forward(half *out, half *src, stream_t stream = nullptr) {
+        attn->forward(temp_attn.get(), src, src, src, stream);
+        LN1->forward(temp_LN.get(), temp_attn.get(), src, rows, stream);
+        linear1->forward_act(temp_linear.get(), temp_LN.get(), act_code<ACT_OP_t>(), stream);
+        linear2->forward(temp_attn.get(), temp_linear.get(), stream);
+        LN2->forward(out, temp_attn.get(), temp_LN.get(), rows, stream);
+    }
+};
+
+}  // namespace et
+
+// Encoder/Encoder.h:49-97
+template <typename _config>
+class Encoder : public et::EncoderLayer<Attention<typename _config::attn_config>,
+                                        Linear<typename _config::linear1_config>,
+                                        Linear<typename _config::linear2_config>, typename _config::act_t> {
+    using base = et::EncoderLayer<Attention<typename _config::attn_config>,
+                                  Linear<typename _config::linear1_config>,
+                                  Linear<typename _config::linear2_config>, typename _config::act_t>;
+
+  public:
+    using base::base;
+};
+
+// Encoder with the pre-computed-VO attention (Encoder/Encoder.h:99-139): tile-sparse
+// FFN, GELU.
+template <typename _attn_config>
+class Encoder_fuse
+    : public et::EncoderLayer<FusedAttention<_attn_config>, Linear<tile_mat>, Linear<tile_mat>, GELU_OP> {
+    using base = et::EncoderLayer<FusedAttention<_attn_config>, Linear<tile_mat>, Linear<tile_mat>, GELU_OP>;
+
+  public:
+    using base::base;
+};

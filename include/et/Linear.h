@@ -1,0 +1,207 @@
+// y = x W^T + b for every weight container — the reference's Linear<MAT>
+// (Linear/Linear.h:17-167).  W is the PyTorch [out x in] matrix; x and y are
+// row-major [size x features] device pointers owned by the caller; `size` (the
+// number of token rows, = batch * seq_len) is fixed at construction.  Each
+// forward is ONE kernel launch on the given stream: bias (and, through
+// forward_act, the activation) is applied on the fp32 accumulator in the
+// kernel's epilogue, and the row/column-pruned forms gather/scatter inside the
+// GEMM instead of the reference's extra passes.  Nothing blocks the host.
+#pragma once
+#include <memory>
+#include <utility>
+#include <vector>
+
+#include "CUDA_ptr.hpp"
+#include "mat_type.h"
+
+using base_mat = et::DeviceBuffer<half>;  // dense [out x in] row-major (Linear/Linear.h:9)
+
+namespace et {
+inline const et_f16 *f16(const half *p) { return reinterpret_cast<const et_f16 *>(p); }
+inline et_f16 *f16(half *p) { return reinterpret_cast<et_f16 *>(p); }
+}  // namespace et
+
+template <typename MAT> class Linear;  // only the specialisations below exist
+
+// dense weight — Linear/Linear.h:32-66
+template <> class Linear<base_mat> {
+  public:
+    const int in_size;
+    const int out_size;
+    base_mat weight;
+    et::DeviceBuffer<half> bias;
+    int size;
+
+    Linear(int _in_size, int _out_size, const base_mat &w, const half *b, int _size)
+        : in_size(_in_size), out_size(_out_size), weight(w), bias(b, (std::size_t)_out_size), size(_size) {
+        et::require(w.size == (std::size_t)_in_size * _out_size, "Linear<base_mat>: weight must hold out*in values");
+    }
+    Linear(int _in_size, int _out_size, base_mat &&w, const half *b, int _size)
+        : in_size(_in_size), out_size(_out_size), weight(std::move(w)), bias(b, (std::size_t)_out_size),
+          size(_size) {
+        et::require(weight.size == (std::size_t)_in_size * _out_size, "Linear<base_mat>: weight must hold out*in values");
+    }
+    void forward(half *output, const half *input, et::stream_t stream = nullptr) const {
+        forward_act(output, input, ET_ACT_NONE, stream);
+    }
+    void forward_act(half *output, const half *input, int act, et::stream_t stream = nullptr) const {
+        etChk(et_linear_dense_f16(et::f16(weight.get()), et::f16(bias.get()), et::f16(input), et::f16(output),
+                                  size, in_size, out_size, act, stream));
+    }
+};
+
+// output-feature pruning — Linear/Linear.h:69-86, Linear/SPMM_row.cu:48-95
+template <> class Linear<row_mat> {
+  public:
+    const uint32_t in_size;
+    const uint32_t out_size;
+    row_mat weight;
+    et::DeviceBuffer<half> bias;
+    int size;
+
+    Linear(int _in_size, int _out_size, const row_mat &w, const half *b, int _size)
+        : in_size(_in_size), out_size(_out_size), weight(w), bias(b, (std::size_t)_out_size), size(_size) {}
+    Linear(int _in_size, int _out_size, row_mat &&w, const half *b, int _size)
+        : in_size(_in_size), out_size(_out_size), weight(std::move(w)), bias(b, (std::size_t)_out_size),
+          size(_size) {}
+    // full-width output: pruned features carry their bias alone
+    void forward(half *output, const half *input, et::stream_t stream = nullptr) const {
+        forward_act(output, input, ET_ACT_NONE, stream);
+    }
+    void forward_act(half *output, const half *input, int act, et::stream_t stream = nullptr) const {
+        etChk(et_linear_rowpruned_f16(et::f16(weight.rows->get()), weight.row_id->get(), weight.nnz_row(),
+                                      et::f16(bias.get()), et::f16(input), et::f16(output), size,
+                                      (int)in_size, (int)out_size, act, stream));
+    }
+    // compact output [size x nnz_row] written into a col_mat (the compact V of the
+    // attention-aware path, Linear/SPMM_row.cu:78-95); the bias of each surviving
+    // feature is applied (the reference leaves that line commented out).
+    void forward(col_mat *output, const half *input, et::stream_t stream = nullptr) const {
+        etChk(et_linear_rowpruned_compact_f16(et::f16(weight.rows->get()), weight.row_id->get(),
+                                              weight.nnz_row(), et::f16(bias.get()), et::f16(input),
+                                              et::f16(output->cols->get()), size, (int)in_size, stream));
+    }
+};
+
+// input-feature pruning — Linear/Linear.h:115-131, Linear/SPMM_col.cu:41-69
+template <> class Linear<col_mat> {
+  public:
+    const uint32_t in_size;
+    const uint32_t out_size;
+    col_mat weight;
+    et::DeviceBuffer<half> bias;
+    int size;
+
+    Linear(int _in_size, int _out_size, const col_mat &w, const half *b, int _size)
+        : in_size(_in_size), out_size(_out_size), weight(w), bias(b, (std::size_t)_out_size), size(_size) {}
+    Linear(int _in_size, int _out_size, col_mat &&w, const half *b, int _size)
+        : in_size(_in_size), out_size(_out_size), weight(std::move(w)), bias(b, (std::size_t)_out_size),
+          size(_size) {}
+    void forward(half *output, const half *input, et::stream_t stream = nullptr) const {
+        forward_act(output, input, ET_ACT_NONE, stream);
+    }
+    void forward_act(half *output, const half *input, int act, et::stream_t stream = nullptr) const {
+        etChk(et_linear_colpruned_f16(et::f16(weight.cols->get()), weight.col_id->get(), weight.nnz_col,
+                                      et::f16(bias.get()), et::f16(input), et::f16(output), size,
+                                      (int)in_size, (int)out_size, act, stream));
+    }
+};
+
+// 16x16 tile pruning — Linear/Linear.h:133-151, Linear/SPMM_tile.cu:312-324
+template <> class Linear<tile_mat> {
+  public:
+    const uint32_t in_size;
+    const uint32_t out_size;
+    const int size;
+    tile_mat weight;
+    et::DeviceBuffer<half> bias;
+
+    Linear(int _in_size, int _out_size, const tile_mat &w, const half *b, int _size)
+        : in_size(_in_size), out_size(_out_size), size(_size), weight(w), bias(b, (std::size_t)_out_size) {
+        check();
+    }
+    Linear(int _in_size, int _out_size, const tile_mat &w, et::DeviceBuffer<half> &b, int _size)
+        : in_size(_in_size), out_size(_out_size), size(_size), weight(w), bias(b) {
+        check();
+    }
+    Linear(int _in_size, int _out_size, tile_mat &&w, const half *b, int _size)
+        : in_size(_in_size), out_size(_out_size), size(_size), weight(std::move(w)),
+          bias(b, (std::size_t)_out_size) {
+        check();
+    }
+    Linear(Linear<tile_mat> &&other) = default;
+
+    void forward(half *output, const half *const input, et::stream_t stream = nullptr) {
+        forward_act(output, input, ET_ACT_NONE, stream);
+    }
+    void forward_act(half *output, const half *input, int act, et::stream_t stream = nullptr) {
+        etChk(et_linear_bsr16_f16(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
+                                  et::f16(bias.get()), et::f16(input), et::f16(output), size, (int)in_size,
+                                  (int)out_size, act, stream));
+    }
+
+  private:
+    void check() const {
+        et::require(weight.blk_row_num * 16 == (int)out_size && weight.blk_col_num * 16 == (int)in_size,
+                    "Linear<tile_mat>: weight shape does not match in/out sizes");
+        et::require(bias.size == out_size, "Linear<tile_mat>: bias must hold out_size values");
+    }
+};
+
+// unstructured CSR — Linear/Linear.h:88-112, Linear/cusp.cu:23-82
+template <> class Linear<csr_mat> {
+  public:
+    const uint32_t in_size;
+    const uint32_t out_size;
+    const int size;
+    std::unique_ptr<et::DeviceBuffer<int>> indptr;
+    std::unique_ptr<et::DeviceBuffer<int>> indices;
+    std::unique_ptr<et::DeviceBuffer<half>> data;
+    et::DeviceBuffer<half> bias;
+
+    Linear(int _in_size, int _out_size, const csr_mat &w, const half *b, int _size)
+        : in_size(_in_size), out_size(_out_size), size(_size), bias(b, (std::size_t)_out_size) {
+        et::require(w.nrow == _out_size && w.ncol == _in_size, "Linear<csr_mat>: weight shape mismatch");
+        std::vector<half> h(w.data.size());
+        for (std::size_t i = 0; i < h.size(); i++) h[i] = static_cast<half>(w.data[i]);
+        indptr = std::make_unique<et::DeviceBuffer<int>>(w.indptr);
+        indices = std::make_unique<et::DeviceBuffer<int>>(w.indices);
+        data = std::make_unique<et::DeviceBuffer<half>>(h);
+    }
+    Linear(Linear<csr_mat> &&other) = default;
+    void forward(half *output, const half *input, et::stream_t stream = nullptr) {
+        forward_act(output, input, ET_ACT_NONE, stream);
+    }
+    void forward_act(half *output, const half *input, int act, et::stream_t stream = nullptr) {
+        etChk(et_linear_csr_f16(indptr->get(), indices->get(), et::f16(data->get()), et::f16(bias.get()),
+                                et::f16(input), et::f16(output), size, (int)in_size, (int)out_size, act,
+                                stream));
+    }
+};
+
+// 1x16 vector pruning — Linear/Linear.h:153-167 (the reference's kernel is a stub,
+// Linear/SPMM1x16.cu:35-124; this one computes y = x W^T + b)
+template <> class Linear<mat1x16> {
+  public:
+    const uint32_t in_size;
+    const uint32_t out_size;
+    const int size;
+    mat1x16 weight;
+    et::DeviceBuffer<half> bias;
+
+    Linear(int _in_size, int _out_size, const mat1x16 &w, const half *b, int _size)
+        : in_size(_in_size), out_size(_out_size), size(_size), weight(w), bias(b, (std::size_t)_out_size) {}
+    Linear(int _in_size, int _out_size, mat1x16 &&w, const half *b, int _size)
+        : in_size(_in_size), out_size(_out_size), size(_size), weight(std::move(w)),
+          bias(b, (std::size_t)_out_size) {}
+    void forward(half *output, const half *input, et::stream_t stream = nullptr) {
+        forward_act(output, input, ET_ACT_NONE, stream);
+    }
+    void forward_act(half *output, const half *input, int act, et::stream_t stream = nullptr) {
+        etChk(et_linear_vec1x16_f16(weight.tile_idx.get(), weight.row_idx.get(), et::f16(weight.data.get()),
+                                    et::f16(bias.get()), et::f16(input), et::f16(output), size,
+                                    (int)in_size, (int)out_size, act, stream));
+    }
+};
+
+#include "gen_linear.hpp"

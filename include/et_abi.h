@@ -28,6 +28,7 @@ extern "C" {
 typedef uint16_t et_f16;  /* IEEE binary16 bit pattern */
 typedef void *et_stream;  /* hipStream_t; NULL = the null stream */
 typedef void *et_event;   /* hipEvent_t */
+typedef void *et_graph;   /* an instantiated HIP graph (hipGraphExec_t) */
 
 enum et_status {
     ET_OK = 0,
@@ -48,6 +49,7 @@ enum et_mha_flags {
 
 const char *et_status_string(int status);
 const char *et_last_error(void);
+void et_set_last_error(const char *message); /* for layers built on this ABI */
 /* library / device identification: fills name (<= cap bytes, NUL terminated),
  * compute-unit count and LDS bytes per workgroup of the current device. */
 int et_device_info(char *name, int cap, int *num_cu, int *lds_bytes);
@@ -77,6 +79,18 @@ int et_event_destroy(et_event ev);
 int et_event_record(et_event ev, et_stream stream);
 int et_event_sync(et_event ev);
 int et_event_elapsed_ms(float *ms, et_event start, et_event stop);
+
+/* HIP-graph capture of a launch sequence: everything issued on `stream` between
+ * begin and end is recorded instead of executed; et_graph_launch replays it with
+ * one submission.  This is how the N-layer caller loop of the reference drivers
+ * (test/Table2/template.hpp:46-48, example/main.cu:175-177) is issued without
+ * per-kernel launch latency.  `stream` must come from et_stream_create.  The
+ * entry points of this library allocate nothing and never synchronise, so any
+ * sequence of them may be captured (run it once eagerly first). */
+int et_graph_begin_capture(et_stream stream);
+int et_graph_end_capture(et_stream stream, et_graph *graph);
+int et_graph_launch(et_graph graph, et_stream stream);
+int et_graph_destroy(et_graph graph);
 
 /* ------------------------------------------------------------------------
  * Linear layers: Y[T x out] = act(X[T x in] * W^T + bias).
@@ -147,6 +161,29 @@ int et_linear_colpruned_f16(const et_f16 *cols, const int32_t *col_id,
                             et_f16 *Y, int T, int in, int out, int act,
                             et_stream stream);
 
+/* 1x16 vector-sparse weight (mat1x16): for row-set r (16 output features) and
+ * part p (16 input features) the surviving 1x16 vectors are idx in
+ * [tile_idx[r*(in/16+1)+p], tile_idx[r*(in/16+1)+p+1]); row_idx[idx] % 16 is
+ * the row inside the set and data[16*idx .. 16*idx+15] the weights.
+ * Completes Linear<mat1x16> (Linear/Linear.h:153-167), whose reference kernel
+ * (Linear/SPMM1x16.cu:35-124) is never launched and stores nothing. */
+int et_linear_vec1x16_f16(const int32_t *tile_idx, const int32_t *row_idx,
+                          const et_f16 *data, const et_f16 *bias,
+                          const et_f16 *X, et_f16 *Y, int T, int in, int out,
+                          int act, et_stream stream);
+
+/* Unstructured CSR weight over [out x in] (indices need not be sorted inside a
+ * row).  T may be any size; out % 4 == 0.  Replaces Linear<csr_mat>::forward
+ * (Linear/cusp.cu:23-82, cusparseSpMM + bias map); no workspace is allocated. */
+int et_linear_csr_f16(const int32_t *indptr, const int32_t *indices,
+                      const et_f16 *data, const et_f16 *bias, const et_f16 *X,
+                      et_f16 *Y, int T, int in, int out, int act,
+                      et_stream stream);
+
+/* C[r][c] = bias[c] (0 when bias is NULL) for a dense [rows x cols] matrix. */
+int et_fill_rows_bias_f16(et_f16 *C, const et_f16 *bias, int rows, int cols,
+                          et_stream stream);
+
 /* ------------------------------------------------------------------------
  * Fused multi-head self-attention (scores never leave the chip).
  *
@@ -168,6 +205,61 @@ int et_mha_fused_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V,
                      int ldq, int ldk, int ldv, et_f16 *Z, int ldz,
                      const et_f16 *mask, const int32_t *lens, int B, int S,
                      int nh, int hd, float scale, int flags, et_stream stream);
+
+/* Attention-aware pruning: W_V is row-pruned, so V arrives compact,
+ * Vc[T x nnz_col] (row stride ldvc), holding only the surviving V columns.
+ * v_col_id[nnz_col] (ascending) are their full-width positions and
+ * v_head_ptr[nh+1] splits them by head.  P*V runs over the surviving columns
+ * only; Z is written full width [T x nh*vhd] with zeros in pruned columns.
+ * Completes Multihead_atttion<Prune_attn> (Attention/Attention.cu:54-78), whose
+ * reference kernel never stores Z (Attention/kernels.cu:453-458). */
+int et_mha_compactv_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *Vc,
+                        int ldq, int ldk, int ldvc, const int32_t *v_col_id,
+                        const int32_t *v_head_ptr, int nnz_col, et_f16 *Z,
+                        int ldz, const et_f16 *mask, const int32_t *lens, int B,
+                        int S, int nh, int hd, int vhd, float scale, int flags,
+                        et_stream stream);
+
+/* Softmax probabilities written to memory: P[b*S + q][h*S + key] (row stride
+ * nh*S), the layout of the reference's __kernel_fused_attention_NOTF
+ * (Fused_attention/Fused_attention.cu:118-206).  S <= 512. */
+int et_mha_probs_f16(const et_f16 *Q, const et_f16 *K, int ldq, int ldk,
+                     et_f16 *P, const et_f16 *mask, const int32_t *lens, int B,
+                     int S, int nh, int hd, float scale, int flags,
+                     et_stream stream);
+
+/* Unfused baseline: probabilities through the workspace P[T x nh*S], then a
+ * batched P*V GEMM per (sequence, head).  Replaces Multihead_atttion<Norm_attn>
+ * (Attention/Attention.cu:8-36: batched GEMM, mask map, softmax kernel, GEMM). */
+int et_mha_unfused_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V,
+                       int ldq, int ldk, int ldv, et_f16 *Z, int ldz, et_f16 *P,
+                       const et_f16 *mask, const int32_t *lens, int B, int S,
+                       int nh, int hd, float scale, int flags,
+                       et_stream stream);
+
+/* Pre-multiplied value/output projection: VO[b][h] (S x N) = X[b] (S x H) *
+ * W[h] (H x N) + bias[h]; W is [nh][H][N] row-major, bias [nh][N] (may be
+ * NULL), VO is [B][nh][S][N].  Replaces Linear_VO::forward and
+ * Linear_VO_prune::forward (Fused_attention/Linear_VO.h:39-58,79-95:
+ * cublasHgemmStridedBatched + add_bias_VO). */
+int et_linear_vo_f16(const et_f16 *W, const et_f16 *bias, const et_f16 *X,
+                     et_f16 *VO, int B, int S, int H, int N, int nh,
+                     et_stream stream);
+
+/* E.T. attention over the pre-multiplied VO: out[b] = sum_h P_h[b] VO[b][h] +
+ * bias_o, with P = softmax(scale * Q_h K_h^T + mask) written to the workspace
+ * P[T x nh*S] on the way.  N is the width of VO; when col_scatter != NULL the N
+ * result columns go to columns col_scatter[n] of out (row stride out_width) and
+ * the other columns of out receive bias_o alone.  Replaces
+ * Fused_Multihead_attention<NOTF_fused_attn> / <OTF_fused_attn> and
+ * Fused_prune_Multihead_attention (Fused_attention/Fused_attention.cu:207-308)
+ * plus the bias map of FusedAttention::forward (Fused_attention.h:109-115). */
+int et_mha_vo_f16(const et_f16 *Q, const et_f16 *K, int ldq, int ldk,
+                  const et_f16 *VO, et_f16 *P, et_f16 *out,
+                  const et_f16 *bias_o, const int32_t *col_scatter,
+                  const et_f16 *mask, const int32_t *lens, int B, int S, int nh,
+                  int hd, int N, int out_width, float scale, int flags,
+                  et_stream stream);
 
 /* ------------------------------------------------------------------------
  * Normalisation and element-wise operators.
@@ -195,6 +287,116 @@ int et_relu_f16(et_f16 *out, const et_f16 *in, size_t n, et_stream stream);
  * bias lambdas (Linear/Linear.h:57-63, Fused_attention/Fused_attention.h:109-115). */
 int et_bias_add_f16(et_f16 *data, const et_f16 *bias, int rows, int cols,
                     et_stream stream);
+
+/* ------------------------------------------------------------------------
+ * Encoder stack: nlayer post-LN encoder layers, layer i feeding layer i+1,
+ *   a = Attn(x); y1 = SkipLN1(a, x); f = L2(act(L1(y1))); out = SkipLN2(f, y1)
+ * assembled from host weights and run as ONE HIP-graph replay per forward.
+ * This is the C form of the reference's model assembly and inference loop
+ * (example/main.cu:24-182: Weights -> tile_mat -> Linear -> Attention ->
+ * SkipLayerNorm -> Encoder, then model[i]->forward chained) over
+ * Encoder<cfg>::forward (Encoder/Encoder.h:81-96) with the single-projection
+ * attention (Attention/Attention.h:246-265).  The handle owns its weights and
+ * scratch; forward takes caller-owned device buffers of batch*seq_len rows.
+ * One handle serves one host thread at a time.
+ * ------------------------------------------------------------------------ */
+typedef struct et_model_s *et_model;
+
+typedef struct et_model_desc {
+    int kdim, vdim, seq_len, nhead, dimFF, emdim, nlayer; /* Model_t (Model.h:2-10) */
+    int batch;     /* sequences per forward; activations have batch*seq_len rows */
+    int act;       /* ET_ACT_RELU or ET_ACT_GELU (Encoder_config::act_t)          */
+    float eps;     /* LayerNorm epsilon; <= 0 selects 1e-5                        */
+    int causal;    /* != 0: causal mask (the reference's hard-wired one)          */
+    int use_graph; /* != 0: replay a captured HIP graph; 0: launch kernel by kernel */
+} et_model_desc;
+
+/* which matrix of a layer */
+enum et_weight { ET_W_QKV = 0, ET_W_O = 1, ET_W_FF1 = 2, ET_W_FF2 = 3 };
+
+int et_model_create(const et_model_desc *desc, et_model *out);
+/* 16x16 BSR weight in the exporter's layout (example/npy2pt.py:75-119): host
+ * row_ptr[out/16+1], column[ntile], data[ntile][256], bias[out] (NULL = 0).
+ * fp32 values are rounded to fp16 (nearest-even); the _f16 form takes fp16 bits. */
+int et_model_set_bsr16(et_model m, int layer, int which, const int32_t *row_ptr,
+                       const int32_t *column, const float *data, int ntile,
+                       const float *bias);
+int et_model_set_bsr16_f16(et_model m, int layer, int which, const int32_t *row_ptr,
+                           const int32_t *column, const et_f16 *data, int ntile,
+                           const et_f16 *bias);
+/* dense [out x in] weight (Linear<base_mat>); a layer is all-BSR or all-dense */
+int et_model_set_dense(et_model m, int layer, int which, const float *W,
+                       const float *bias);
+int et_model_set_dense_f16(et_model m, int layer, int which, const et_f16 *W,
+                           const et_f16 *bias);
+/* SkipLayerNorm which = 0 (after attention) or 1 (after the FFN): host gamma, beta[emdim] */
+int et_model_set_norm(et_model m, int layer, int which, const float *gamma,
+                      const float *beta);
+int et_model_set_norm_f16(et_model m, int layer, int which, const et_f16 *gamma,
+                          const et_f16 *beta);
+/* right padding: host lens[batch], keys >= lens[b] are ignored; NULL removes it */
+int et_model_set_lens(et_model m, const int32_t *lens_host);
+/* additive [seq_len x seq_len] mask from host memory; NULL removes it */
+int et_model_set_mask(et_model m, const et_f16 *mask_host);
+/* uploads the weights and builds the layer objects; weights are fixed afterwards */
+int et_model_finalize(et_model m);
+/* builds a finalized model from weights.txt + .npz archives (example/weights.hpp:32-47) */
+int et_model_load(const char *weights_txt, const char *dir,
+                  const et_model_desc *desc, et_model *out);
+/* out, in: device [batch*seq_len x emdim].  Asynchronous; stream NULL = the
+ * model's own stream (wait with et_model_sync).  in and out may not alias. */
+int et_model_forward(et_model m, et_f16 *out, const et_f16 *in, et_stream stream);
+/* one layer, launched kernel by kernel (Encoder<cfg>::forward) */
+int et_model_forward_layer(et_model m, int layer, et_f16 *out, const et_f16 *in,
+                           et_stream stream);
+int et_model_sync(et_model m);
+int et_model_destroy(et_model m);
+
+/* ------------------------------------------------------------------------
+ * Host-side construction of the sparse weight structures (integer work on
+ * host pointers, usable without a GPU).  Outputs are caller-allocated; a
+ * function that produces a data-dependent number of entries reports it through
+ * its last argument and accepts NULL for the variable-length outputs on a
+ * sizing call.  Random structure is seeded: ids are taken in ascending order
+ * of their SplitMix64 key, which stands in for the reference's
+ * std::random_shuffle.
+ * ------------------------------------------------------------------------ */
+
+/* out[0..n) = the seeded permutation of 0..n-1. */
+int et_fmt_permutation(int64_t n, uint64_t seed, int64_t *out);
+/* int(total * (1.0 - (double)sparsity)) — mat_type/tile_mat/tile_mat.cu:12.
+ * Returns the count itself (not a status). */
+int et_fmt_kept_count(int64_t total, float sparsity);
+/* tile_mat::gen_sparse_mat structure (mat_type/tile_mat/tile_mat.cu:7-40):
+ * row_ptr[nrow/16+1], row_offset[kept_count(total tiles)] in permuted order. */
+int et_fmt_tile_pattern(int nrow, int ncol, float sparsity, uint64_t seed,
+                        int32_t *row_ptr, int32_t *row_offset, int *ntile);
+/* Exporter gen_csr (example/npy2pt.py:75-109): tiles of W[nrow x ncol] with a
+ * non-zero element, block-rows in order, columns ascending; data[ntile][256]. */
+int et_fmt_dense_to_bsr16(const float *W, int nrow, int ncol, int32_t *row_ptr,
+                          int32_t *column, float *data, int *ntile);
+/* row_mat::gen_sparse_mat ids (mat_type/row_mat/row_mat.cu:14-25), ascending. */
+int et_fmt_row_ids(int nrow, float sparsity, uint64_t seed, int32_t *ids, int *count);
+/* col_mat::gen_sparse_mat ids (mat_type/col_mat/col_mat.cu:22-32), permuted order. */
+int et_fmt_col_ids(int ncol, float sparsity, uint64_t seed, int32_t *ids, int *count);
+/* col_mat::set_metadata (mat_type/col_mat/col_mat.cu:34-58): out[nhead+1]. */
+int et_fmt_head_ptr(const int32_t *col_id, int nnz_col, int nhead, int full_dim,
+                    int32_t *out);
+/* mat1x16 (mat_type/mat1x16/mat1x16.h:5-22) in the layout its kernel reads
+ * (Linear/SPMM1x16.cu:52-74): tile_idx[(nrow/16)*(ncol/16+1)] global offsets,
+ * row_idx[ntile], data[pad16(ntile)][16]. */
+int et_fmt_dense_to_1x16(const float *W, int nrow, int ncol, int32_t *tile_idx,
+                         int32_t *row_idx, float *data, int *ntile);
+int et_fmt_1x16_pattern(int nrow, int ncol, float sparsity, uint64_t seed,
+                        int32_t *tile_idx, int32_t *row_idx, int *ntile);
+/* csr_mat (mat_type/csr_mat/csr_mat.h:11-42, generator csr_mat.cpp:25-67). */
+int et_fmt_dense_to_csr(const float *W, int nrow, int ncol, int32_t *indptr,
+                        int32_t *indices, float *data, int *nnz);
+int et_fmt_csr_pattern(int nrow, int ncol, float sparsity, uint64_t seed,
+                       int32_t *indptr, int32_t *indices, int *nnz);
+/* .csr file reader (mat_type/csr_mat/csr_mat.h:19-35). */
+int et_fmt_csr_read(const char *path, int *nrow, int *ncol, int *nnz,
+                    int32_t *indptr, int32_t *indices, float *data);
 
 #ifdef __cplusplus
 }

@@ -71,7 +71,54 @@ _SIGNATURES = {
     "et_gelu_f16": (_vp, _vp, _sz, _vp),
     "et_relu_f16": (_vp, _vp, _sz, _vp),
     "et_bias_add_f16": (_vp, _vp, _i, _i, _vp),
+    "et_fill_rows_bias_f16": (_vp, _vp, _i, _i, _vp),
+    "et_linear_vec1x16_f16": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_linear_csr_f16": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_mha_compactv_f16": (_vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i,
+                            _f, _i, _vp),
+    "et_mha_probs_f16": (_vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp),
+    "et_mha_unfused_f16": (_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp),
+    "et_linear_vo_f16": (_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp),
+    "et_mha_vo_f16": (_vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp),
+    "et_graph_begin_capture": (_vp,),
+    "et_graph_end_capture": (_vp, C.POINTER(_vp)),
+    "et_graph_launch": (_vp, _vp),
+    "et_graph_destroy": (_vp,),
+    "et_model_create": (_vp, C.POINTER(_vp)),
+    "et_model_set_bsr16": (_vp, _i, _i, _vp, _vp, _vp, _i, _vp),
+    "et_model_set_bsr16_f16": (_vp, _i, _i, _vp, _vp, _vp, _i, _vp),
+    "et_model_set_dense": (_vp, _i, _i, _vp, _vp),
+    "et_model_set_dense_f16": (_vp, _i, _i, _vp, _vp),
+    "et_model_set_norm": (_vp, _i, _i, _vp, _vp),
+    "et_model_set_norm_f16": (_vp, _i, _i, _vp, _vp),
+    "et_model_set_lens": (_vp, _vp),
+    "et_model_set_mask": (_vp, _vp),
+    "et_model_finalize": (_vp,),
+    "et_model_load": (C.c_char_p, C.c_char_p, _vp, C.POINTER(_vp)),
+    "et_model_forward": (_vp, _vp, _vp, _vp),
+    "et_model_forward_layer": (_vp, _i, _vp, _vp, _vp),
+    "et_model_sync": (_vp,),
+    "et_model_destroy": (_vp,),
+    "et_fmt_permutation": (C.c_int64, C.c_uint64, _vp),
+    "et_fmt_kept_count": (C.c_int64, _f),
+    "et_fmt_tile_pattern": (_i, _i, _f, C.c_uint64, _vp, _vp, C.POINTER(_i)),
+    "et_fmt_dense_to_bsr16": (_vp, _i, _i, _vp, _vp, _vp, C.POINTER(_i)),
+    "et_fmt_row_ids": (_i, _f, C.c_uint64, _vp, C.POINTER(_i)),
+    "et_fmt_col_ids": (_i, _f, C.c_uint64, _vp, C.POINTER(_i)),
+    "et_fmt_head_ptr": (_vp, _i, _i, _i, _vp),
+    "et_fmt_dense_to_1x16": (_vp, _i, _i, _vp, _vp, _vp, C.POINTER(_i)),
+    "et_fmt_1x16_pattern": (_i, _i, _f, C.c_uint64, _vp, _vp, C.POINTER(_i)),
+    "et_fmt_dense_to_csr": (_vp, _i, _i, _vp, _vp, _vp, C.POINTER(_i)),
+    "et_fmt_csr_pattern": (_i, _i, _f, C.c_uint64, _vp, _vp, C.POINTER(_i)),
+    "et_fmt_csr_read": (C.c_char_p, C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), _vp, _vp, _vp),
 }
+
+W_QKV, W_O, W_FF1, W_FF2 = 0, 1, 2, 3
+
+
+class ModelDesc(C.Structure):
+    _fields_ = [("kdim", _i), ("vdim", _i), ("seq_len", _i), ("nhead", _i), ("dimFF", _i), ("emdim", _i),
+                ("nlayer", _i), ("batch", _i), ("act", _i), ("eps", _f), ("causal", _i), ("use_graph", _i)]
 _RESTYPES = {"et_status_string": C.c_char_p, "et_last_error": C.c_char_p}
 
 _lib = None
@@ -241,3 +288,88 @@ def skip_layernorm(out, src, skip, gamma, beta, rows, H, eps=1e-5, stream=None):
 
 def layernorm(out, src, gamma, beta, rows, H, eps=1e-5, stream=None):
     check(lib().et_layernorm_f16(_ptr(out), _ptr(src), _ptr(gamma), _ptr(beta), rows, H, eps, stream))
+
+
+# ---------------------------------------------------------------------------
+# Encoder stack handle (et_model_*)
+# ---------------------------------------------------------------------------
+
+def _np_ptr(a):
+    return None if a is None else a.ctypes.data
+
+
+class Model:
+    """Encoder stack assembled from host weights; forward replays one HIP graph."""
+
+    def __init__(self, H, nh, dimFF, S, nlayer, batch=1, act=ACT_GELU, eps=1e-5, causal=False, use_graph=True,
+                 handle=None):
+        self.desc = ModelDesc(H, H, S, nh, dimFF, H, nlayer, batch, act, eps, int(causal), int(use_graph))
+        self.rows, self.H = batch * S, H
+        if handle is None:
+            h = _vp()
+            check(lib().et_model_create(C.byref(self.desc), C.byref(h)))
+            handle = h.value
+        self.handle = handle
+
+    @classmethod
+    def load(cls, weights_txt, directory, H, nh, dimFF, S, nlayer, **kw):
+        self = cls.__new__(cls)
+        Model.__init__(self, H, nh, dimFF, S, nlayer, handle=0, **kw)
+        h = _vp()
+        check(lib().et_model_load(str(weights_txt).encode(), str(directory).encode(), C.byref(self.desc),
+                                  C.byref(h)))
+        self.handle = h.value
+        return self
+
+    def set_bsr16(self, layer, which, row_ptr, column, data, bias):
+        row_ptr = np.ascontiguousarray(row_ptr, np.int32)
+        column = np.ascontiguousarray(column, np.int32)
+        data = np.ascontiguousarray(data)
+        bias = None if bias is None else np.ascontiguousarray(bias, data.dtype)
+        fn = lib().et_model_set_bsr16_f16 if data.dtype == np.float16 else lib().et_model_set_bsr16
+        assert data.dtype in (np.float16, np.float32)
+        check(fn(self.handle, layer, which, _np_ptr(row_ptr), _np_ptr(column), _np_ptr(data), len(column),
+                 _np_ptr(bias)))
+
+    def set_dense(self, layer, which, W, bias):
+        W = np.ascontiguousarray(W)
+        bias = None if bias is None else np.ascontiguousarray(bias, W.dtype)
+        fn = lib().et_model_set_dense_f16 if W.dtype == np.float16 else lib().et_model_set_dense
+        check(fn(self.handle, layer, which, _np_ptr(W), _np_ptr(bias)))
+
+    def set_norm(self, layer, which, gamma, beta):
+        gamma = np.ascontiguousarray(gamma)
+        beta = np.ascontiguousarray(beta, gamma.dtype)
+        fn = lib().et_model_set_norm_f16 if gamma.dtype == np.float16 else lib().et_model_set_norm
+        check(fn(self.handle, layer, which, _np_ptr(gamma), _np_ptr(beta)))
+
+    def set_lens(self, lens):
+        lens = None if lens is None else np.ascontiguousarray(lens, np.int32)
+        check(lib().et_model_set_lens(self.handle, _np_ptr(lens)))
+
+    def set_mask(self, mask):
+        mask = None if mask is None else np.ascontiguousarray(mask, np.float16)
+        check(lib().et_model_set_mask(self.handle, _np_ptr(mask)))
+
+    def finalize(self):
+        check(lib().et_model_finalize(self.handle))
+
+    def forward(self, out, inp, stream=None):
+        check(lib().et_model_forward(self.handle, _ptr(out), _ptr(inp), stream))
+
+    def forward_layer(self, layer, out, inp, stream=None):
+        check(lib().et_model_forward_layer(self.handle, layer, _ptr(out), _ptr(inp), stream))
+
+    def sync(self):
+        check(lib().et_model_sync(self.handle))
+
+    def destroy(self):
+        if self.handle:
+            lib().et_model_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass

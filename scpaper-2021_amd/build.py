@@ -40,6 +40,8 @@ def _compile(src: Path) -> Path:
     cmd = [HIPCC, *COMMON]
     if src.suffix == ".hip":
         cmd += DEVICE
+    else:
+        cmd += ["-x", "c++"]  # host-only translation unit: no device pass
     cmd += ["-c", str(src), "-o", str(obj)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     # hipcc's host pass does not know the packed-fp32 feature name; that
@@ -62,7 +64,7 @@ def build_all(jobs: int | None = None, verbose: bool = True) -> Path:
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
         objs = list(pool.map(_compile, srcs))
     tmp = LIB.with_suffix(".so.tmp")
-    cmd = [HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", *map(str, objs), "-o", str(tmp)]
+    cmd = [HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", *map(str, objs), "-lz", "-o", str(tmp)]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed: {' '.join(cmd)}\n{res.stderr}")

@@ -33,6 +33,11 @@ struct MhaArgs {
     int S, nh;
     float scale_log2e;  // scale * log2(e)
     int causal;
+    // compact-V form only: V is [rows x nnz] holding the surviving V columns;
+    // head h owns compact columns [v_head_ptr[h], v_head_ptr[h+1]), which stand
+    // for the full-width columns v_col_id[.] (all inside head h's slice of Z).
+    const int32_t *v_col_id;
+    const int32_t *v_head_ptr;
 };
 
 constexpr int kKeyBlock = 128;          // keys staged per iteration
@@ -48,7 +53,7 @@ struct MhaLds {
     static constexpr size_t bytes = (size_t)(k_halfs + vt_halfs) * sizeof(_Float16);
 };
 
-template <int HD>
+template <int HD, bool COMPACT>
 __global__ __launch_bounds__(256) void mha_fused_kernel(const MhaArgs a) {
     using L = MhaLds<HD>;
     constexpr int KS = HD / 32;  // K=32 MFMA steps over the head dimension
@@ -70,6 +75,12 @@ __global__ __launch_bounds__(256) void mha_fused_kernel(const MhaArgs a) {
     const bool q_ok = q < S;
     int klimit = S;
     if (a.lens) klimit = min(S, max(a.lens[b], 0));
+    // compact-V: this head's surviving V columns
+    int vc0 = 0, vlive = HD;
+    if (COMPACT) {
+        vc0 = a.v_head_ptr[h];
+        vlive = min(a.v_head_ptr[h + 1] - vc0, HD);
+    }
 
     // Q fragments: B operand, lane supplies Q[q][32*ks + 8g .. +7]
     h8 qf[KS];
@@ -113,8 +124,17 @@ __global__ __launch_bounds__(256) void mha_fused_kernel(const MhaArgs a) {
                 for (int i = 0; i < 4; i++) {
                     const int key = k0 + kg * 4 + i;
                     rows[i] = h8{0, 0, 0, 0, 0, 0, 0, 0};
-                    if (key < S)
+                    if (COMPACT) {
+                        // compact columns start at an arbitrary element: scalar loads
+                        if (key < S) {
+                            const _Float16 *vp = a.V + (row0 + key) * a.ldv + vc0 + dg * 8;
+#pragma unroll
+                            for (int d = 0; d < 8; d++)
+                                if (dg * 8 + d < vlive) rows[i][d] = vp[d];
+                        }
+                    } else if (key < S) {
                         rows[i] = *reinterpret_cast<const h8 *>(a.V + (row0 + key) * a.ldv + h * HD + dg * 8);
+                    }
                 }
 #pragma unroll
                 for (int d = 0; d < 8; d++) {
@@ -189,6 +209,7 @@ __global__ __launch_bounds__(256) void mha_fused_kernel(const MhaArgs a) {
             }
 #pragma unroll
             for (int d = 0; d < DB; d++) {
+                if (COMPACT && d * 16 >= vlive) continue;  // no surviving column in this block
                 const _Float16 *vp = Vt + (d * 16 + r16) * L::ldvt + s2 * 32 + 4 * g;
                 const h4 v0 = *reinterpret_cast<const h4 *>(vp);
                 const h4 v1 = *reinterpret_cast<const h4 *>(vp + 16);
@@ -203,7 +224,7 @@ __global__ __launch_bounds__(256) void mha_fused_kernel(const MhaArgs a) {
     l += __shfl_xor(l, 16, kWave);
     l += __shfl_xor(l, 32, kWave);
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    if (q_ok) {
+    if (q_ok && !COMPACT) {
         _Float16 *zp = a.Z + (row0 + q) * a.ldz + h * HD + 4 * g;
 #pragma unroll
         for (int d = 0; d < DB; d++) {
@@ -213,11 +234,33 @@ __global__ __launch_bounds__(256) void mha_fused_kernel(const MhaArgs a) {
             *reinterpret_cast<h4 *>(zp + 16 * d) = out;
         }
     }
+    if (COMPACT) {
+        // Full-width Z: pruned columns of this head's slice are zero, surviving
+        // ones are scattered to v_col_id.  The zero fill is made visible before
+        // the scatter so that the scatter wins wherever both touch an element.
+        _Float16 *zrow = a.Z + (row0 + (q_ok ? q : 0)) * a.ldz;
+        if (q_ok) {
+            const h4 z4 = {0, 0, 0, 0};
+#pragma unroll
+            for (int d = 0; d < DB; d++) *reinterpret_cast<h4 *>(zrow + h * HD + 16 * d + 4 * g) = z4;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        if (q_ok) {
+#pragma unroll
+            for (int d = 0; d < DB; d++) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int dc = d * 16 + 4 * g + j;
+                    if (dc < vlive) zrow[a.v_col_id[vc0 + dc]] = (_Float16)(o[d][j] * inv);
+                }
+            }
+        }
+    }
 }
 
-template <int HD>
+template <int HD, bool COMPACT>
 static int launch_mha(const MhaArgs &args, int B, hipStream_t stream) {
-    auto kernel = mha_fused_kernel<HD>;
+    auto kernel = mha_fused_kernel<HD, COMPACT>;
     constexpr size_t lds = MhaLds<HD>::bytes;
     if (lds > 64 * 1024) {
         static bool raised = false;
@@ -281,10 +324,56 @@ int et_mha_fused_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V, int ldq,
     args.nh = nh;
     args.scale_log2e = scale * kLog2e;
     args.causal = (flags & ET_MHA_CAUSAL) ? 1 : 0;
+    args.v_col_id = nullptr;
+    args.v_head_ptr = nullptr;
     switch (hd) {
-        case 32: return launch_mha<32>(args, B, as_stream(stream));
-        case 64: return launch_mha<64>(args, B, as_stream(stream));
-        default: return launch_mha<128>(args, B, as_stream(stream));
+        case 32: return launch_mha<32, false>(args, B, as_stream(stream));
+        case 64: return launch_mha<64, false>(args, B, as_stream(stream));
+        default: return launch_mha<128, false>(args, B, as_stream(stream));
+    }
+}
+
+int et_mha_compactv_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *Vc, int ldq, int ldk, int ldvc,
+                        const int32_t *v_col_id, const int32_t *v_head_ptr, int nnz_col, et_f16 *Z,
+                        int ldz, const et_f16 *mask, const int32_t *lens, int B, int S, int nh, int hd,
+                        int vhd, float scale, int flags, et_stream stream) {
+    ET_REQUIRE(Q && K && Vc && Z && v_col_id && v_head_ptr, ET_ERR_INVALID_ARG,
+               "et_mha_compactv_f16: NULL pointer");
+    ET_REQUIRE(B >= 0 && S > 0 && nh > 0 && hd > 0 && nnz_col >= 0, ET_ERR_INVALID_ARG,
+               "et_mha_compactv_f16: B=%d S=%d nh=%d hd=%d nnz_col=%d", B, S, nh, hd, nnz_col);
+    ET_REQUIRE((flags & ~ET_MHA_CAUSAL) == 0, ET_ERR_INVALID_ARG, "et_mha_compactv_f16: flags=%d", flags);
+    ET_REQUIRE(S % 16 == 0, ET_ERR_UNSUPPORTED, "et_mha_compactv_f16: S=%d must be a multiple of 16", S);
+    ET_REQUIRE(hd == 32 || hd == 64 || hd == 128, ET_ERR_UNSUPPORTED,
+               "et_mha_compactv_f16: head dim %d not in {32, 64, 128}", hd);
+    ET_REQUIRE(vhd == hd, ET_ERR_UNSUPPORTED,
+               "et_mha_compactv_f16: V head width %d must equal the Q/K head width %d", vhd, hd);
+    ET_REQUIRE(ldq >= nh * hd && ldk >= nh * hd && ldz >= nh * vhd && ldvc >= nnz_col, ET_ERR_INVALID_ARG,
+               "et_mha_compactv_f16: row strides too small");
+    ET_REQUIRE(ldq % 8 == 0 && ldk % 8 == 0 && ldz % 4 == 0, ET_ERR_UNSUPPORTED,
+               "et_mha_compactv_f16: row strides must keep 16-byte alignment");
+    ET_REQUIRE(B <= 65535 && nh <= 65535, ET_ERR_UNSUPPORTED, "et_mha_compactv_f16: grid too large");
+    if (B == 0) return ET_OK;
+    MhaArgs args;
+    args.Q = reinterpret_cast<const _Float16 *>(Q);
+    args.K = reinterpret_cast<const _Float16 *>(K);
+    args.V = reinterpret_cast<const _Float16 *>(Vc);
+    args.Z = reinterpret_cast<_Float16 *>(Z);
+    args.mask = reinterpret_cast<const _Float16 *>(mask);
+    args.lens = lens;
+    args.ldq = ldq;
+    args.ldk = ldk;
+    args.ldv = ldvc;
+    args.ldz = ldz;
+    args.S = S;
+    args.nh = nh;
+    args.scale_log2e = scale * kLog2e;
+    args.causal = (flags & ET_MHA_CAUSAL) ? 1 : 0;
+    args.v_col_id = v_col_id;
+    args.v_head_ptr = v_head_ptr;
+    switch (hd) {
+        case 32: return launch_mha<32, true>(args, B, as_stream(stream));
+        case 64: return launch_mha<64, true>(args, B, as_stream(stream));
+        default: return launch_mha<128, true>(args, B, as_stream(stream));
     }
 }
 

@@ -1,0 +1,341 @@
+// Dense fp16 GEMM with fp32 accumulation for gfx950, and the Linear layers
+// built on it (dense, row-pruned, column-pruned weights).
+//
+//   C[M x N] = A[M x K] * B^T   (B stored [N x K]: both operands K-contiguous,
+//                                the natural MFMA feed)        trans_b = 1
+//   C[M x N] = A[M x K] * B     (B stored [K x N]; the tile is transposed on
+//                                its way into LDS)             trans_b = 0
+//
+// A workgroup of 4 waves (2 x 2) computes a (32*TM) x (32*TN) tile of C; each
+// wave owns TM x TN accumulators of 16x16.  K is walked in steps of 64 through
+// one LDS stage per operand (row stride padded by 16 bytes); the next stage is
+// prefetched into registers while v_mfma_f32_16x16x32_f16 consumes the current
+// one.  The MFMA A operand is fed from the B matrix and vice versa, so a lane
+// ends with four consecutive columns of one row of C and stores 8 bytes.
+//
+// Optional fusions, all in the prologue/epilogue of the same kernel:
+//   a_gather : column k of A is read from X[:, a_gather[k]]   (col_mat Linear:
+//              replaces the reference's separate gather pass, Linear/SPMM_col.cu:8-23)
+//   c_scatter: column n of the result is written to C[:, c_scatter[n]]
+//              (row_mat Linear: replaces the scatter pass, Linear/SPMM_row.cu:14-30)
+//   bias/act : y = act(acc + bias[column]) on the fp32 accumulator.
+#include "gemm.hip.h"
+
+namespace et {
+
+constexpr int kBK = 64;
+constexpr int kLdT = kBK + 8;  // halfs per LDS tile row
+
+template <int TM, int TN, bool TRANS_B, bool GATHER>
+__global__ __launch_bounds__(256) void gemm_f16_kernel(const GemmArgs g) {
+    constexpr int BM = 32 * TM, BN = 32 * TN;
+    constexpr int VA = BM * (kBK / 8) / 256;  // 16-byte vectors of the A stage per thread
+    constexpr int VB = BN * (kBK / 8) / 256;
+    __shared__ __align__(16) _Float16 As[BM * kLdT];
+    __shared__ __align__(16) _Float16 Bs[BN * kLdT];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int r16 = lane & 15, grp = lane >> 4;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const long long zo = blockIdx.z / g.batch_inner, zi = blockIdx.z % g.batch_inner;
+    const _Float16 *A = g.A + zo * g.sAo + zi * g.sAi;
+    const _Float16 *B = g.B + zo * g.sBo + zi * g.sBi;
+    _Float16 *Cm = g.C + zo * g.sCo + zi * g.sCi;
+    const _Float16 *bias = g.bias ? g.bias + zo * g.sBias_o + zi * g.sBias_i : nullptr;
+    const h8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    f4 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = f4{0.f, 0.f, 0.f, 0.f};
+
+    h8 ra[VA], rb[VB];
+
+    auto load_stage = [&](int k0) {
+#pragma unroll
+        for (int v = 0; v < VA; v++) {
+            const int idx = tid + v * 256;
+            const int r = idx >> 3, c = idx & 7;  // kBK/8 = 8 vectors per row
+            const int m = m0 + r, k = k0 + c * 8;
+            h8 val = zero8;
+            if (m < g.M && k < g.K) {
+                if (GATHER) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) val[e] = A[(size_t)m * g.lda + g.a_gather[k + e]];
+                } else {
+                    val = *reinterpret_cast<const h8 *>(A + (size_t)m * g.lda + k);
+                }
+            }
+            ra[v] = val;
+        }
+#pragma unroll
+        for (int v = 0; v < VB; v++) {
+            const int idx = tid + v * 256;
+            h8 val = zero8;
+            if (TRANS_B) {
+                const int r = idx >> 3, c = idx & 7;
+                const int n = n0 + r, k = k0 + c * 8;
+                if (n < g.N && k < g.K) val = *reinterpret_cast<const h8 *>(B + (size_t)n * g.ldb + k);
+            } else {
+                // B is [K x N]: vector = 8 consecutive n of one k
+                constexpr int vec_per_k = BN / 8;
+                const int kk = idx / vec_per_k, c = idx - kk * vec_per_k;
+                const int k = k0 + kk, n = n0 + c * 8;
+                if (k < g.K && n < g.N) val = *reinterpret_cast<const h8 *>(B + (size_t)k * g.ldb + n);
+            }
+            rb[v] = val;
+        }
+    };
+    auto store_stage = [&]() {
+#pragma unroll
+        for (int v = 0; v < VA; v++) {
+            const int idx = tid + v * 256;
+            const int r = idx >> 3, c = idx & 7;
+            *reinterpret_cast<h8 *>(As + r * kLdT + c * 8) = ra[v];
+        }
+#pragma unroll
+        for (int v = 0; v < VB; v++) {
+            const int idx = tid + v * 256;
+            if (TRANS_B) {
+                const int r = idx >> 3, c = idx & 7;
+                *reinterpret_cast<h8 *>(Bs + r * kLdT + c * 8) = rb[v];
+            } else {
+                constexpr int vec_per_k = BN / 8;
+                const int kk = idx / vec_per_k, c = idx - kk * vec_per_k;
+#pragma unroll
+                for (int e = 0; e < 8; e++) Bs[(c * 8 + e) * kLdT + kk] = rb[v][e];
+            }
+        }
+    };
+
+    load_stage(0);
+    for (int k0 = 0; k0 < g.K; k0 += kBK) {
+        __syncthreads();  // previous stage fully consumed
+        store_stage();
+        __syncthreads();
+        if (k0 + kBK < g.K) load_stage(k0 + kBK);
+#pragma unroll
+        for (int ks = 0; ks < kBK / 32; ks++) {
+            h8 fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+                fa[i] = *reinterpret_cast<const h8 *>(As + ((wm * TM + i) * 16 + r16) * kLdT + ks * 32 + grp * 8);
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                fb[j] = *reinterpret_cast<const h8 *>(Bs + ((wn * TN + j) * 16 + r16) * kLdT + ks * 32 + grp * 8);
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+        }
+    }
+
+    // epilogue: lane holds C[m = r16 of block i][n = 4*grp .. +3 of block j]
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int m = m0 + (wm * TM + i) * 16 + r16;
+        if (m >= g.M) continue;
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int n = n0 + (wn * TN + j) * 16 + grp * 4;
+            if (n >= g.N) continue;
+            if (g.c_scatter) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int col = g.c_scatter[n + e];
+                    float y = acc[i][j][e];
+                    if (bias) y += (float)bias[col];
+                    Cm[(size_t)m * g.ldc + col] = (_Float16)apply_act(y, g.act);
+                }
+            } else {
+                h4 o;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float y = acc[i][j][e];
+                    if (bias) y += (float)bias[g.bias_idx ? g.bias_idx[n + e] : n + e];
+                    o[e] = (_Float16)apply_act(y, g.act);
+                }
+                *reinterpret_cast<h4 *>(Cm + (size_t)m * g.ldc + n) = o;
+            }
+        }
+    }
+}
+
+// C[r][c] = act(bias[c]) for the columns a row-pruned weight does not produce.
+__global__ __launch_bounds__(256) void bias_rows_kernel(_Float16 *__restrict__ C,
+                                                        const _Float16 *__restrict__ bias, int rows,
+                                                        int cols, int ldc, int act) {
+    const size_t total = (size_t)rows * cols;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (size_t e = blockIdx.x * (size_t)blockDim.x + threadIdx.x; e < total; e += step) {
+        const int r = (int)(e / cols), c = (int)(e - (size_t)r * cols);
+        const float b = bias ? (float)bias[c] : 0.0f;
+        C[(size_t)r * ldc + c] = (_Float16)apply_act(b, act);
+    }
+}
+
+template <int TM, int TN>
+static int launch_gemm_tile(const GemmArgs &g, int batch, bool trans_b, hipStream_t stream) {
+    const dim3 grid((g.N + 32 * TN - 1) / (32 * TN), (g.M + 32 * TM - 1) / (32 * TM), batch);
+    const bool gather = g.a_gather != nullptr;
+    if (trans_b) {
+        if (gather) gemm_f16_kernel<TM, TN, true, true><<<grid, 256, 0, stream>>>(g);
+        else gemm_f16_kernel<TM, TN, true, false><<<grid, 256, 0, stream>>>(g);
+    } else {
+        if (gather) gemm_f16_kernel<TM, TN, false, true><<<grid, 256, 0, stream>>>(g);
+        else gemm_f16_kernel<TM, TN, false, false><<<grid, 256, 0, stream>>>(g);
+    }
+    return check_launch("gemm_f16_kernel");
+}
+
+// 128x128 tiles once they still give a few hundred workgroups, 64x64 otherwise.
+int launch_gemm(const GemmArgs &g, int batch, bool trans_b, hipStream_t stream) {
+    const long long big = (long long)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
+    if (big >= 512) return launch_gemm_tile<4, 4>(g, batch, trans_b, stream);
+    return launch_gemm_tile<2, 2>(g, batch, trans_b, stream);
+}
+
+static int check_gemm_shape(const char *fn, int M, int N, int K) {
+    ET_REQUIRE(M >= 0 && N > 0 && K > 0, ET_ERR_INVALID_ARG, "%s: M=%d N=%d K=%d", fn, M, N, K);
+    ET_REQUIRE(M % 16 == 0 && N % 16 == 0 && K % 16 == 0, ET_ERR_UNSUPPORTED,
+               "%s: M=%d N=%d K=%d must be multiples of 16", fn, M, N, K);
+    return ET_OK;
+}
+
+static inline const _Float16 *H(const et_f16 *p) { return reinterpret_cast<const _Float16 *>(p); }
+static inline _Float16 *H(et_f16 *p) { return reinterpret_cast<_Float16 *>(p); }
+
+}  // namespace et
+
+using namespace et;
+
+extern "C" {
+
+int et_gemm_f16(const et_f16 *A, const et_f16 *B, et_f16 *C, int M, int N, int K, int lda, int ldb,
+                int ldc, int trans_b, int batch, long long strideA, long long strideB,
+                long long strideC, et_stream stream) {
+    ET_REQUIRE(A && B && C, ET_ERR_INVALID_ARG, "et_gemm_f16: NULL pointer");
+    int s = check_gemm_shape("et_gemm_f16", M, N, K);
+    if (s != ET_OK) return s;
+    ET_REQUIRE(batch >= 1 && batch <= 65535, ET_ERR_INVALID_ARG, "et_gemm_f16: batch=%d", batch);
+    ET_REQUIRE(lda >= K && ldc >= N && ldb >= (trans_b ? K : N), ET_ERR_INVALID_ARG,
+               "et_gemm_f16: leading dimensions (%d %d %d) too small", lda, ldb, ldc);
+    ET_REQUIRE(lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 && strideA % 8 == 0 && strideB % 8 == 0 &&
+                   strideC % 4 == 0,
+               ET_ERR_UNSUPPORTED, "et_gemm_f16: strides must keep 16-byte operand alignment");
+    ET_REQUIRE(((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(C) & 7) == 0,
+               ET_ERR_UNSUPPORTED, "et_gemm_f16: operands must be 16-byte aligned");
+    if (M == 0) return ET_OK;
+    GemmArgs g = gemm_args(H(A), H(B), H(C), M, N, K, lda, ldb, ldc);
+    g.sAo = strideA;
+    g.sBo = strideB;
+    g.sCo = strideC;
+    return launch_gemm(g, batch, trans_b != 0, as_stream(stream));
+}
+
+int et_linear_dense_f16(const et_f16 *W, const et_f16 *bias, const et_f16 *X, et_f16 *Y, int T,
+                        int in, int out, int act, et_stream stream) {
+    ET_REQUIRE(W && X && Y, ET_ERR_INVALID_ARG, "et_linear_dense_f16: NULL pointer");
+    ET_REQUIRE(act >= ET_ACT_NONE && act <= ET_ACT_GELU, ET_ERR_INVALID_ARG,
+               "et_linear_dense_f16: act=%d", act);
+    int s = check_gemm_shape("et_linear_dense_f16", T, out, in);
+    if (s != ET_OK) return s;
+    if (T == 0) return ET_OK;
+    GemmArgs g = gemm_args(H(X), H(W), H(Y), T, out, in, in, in, out);
+    g.bias = H(bias);
+    g.act = act;
+    return launch_gemm(g, 1, true, as_stream(stream));
+}
+
+int et_linear_rowpruned_f16(const et_f16 *rows, const int32_t *row_id, int nnz_row,
+                            const et_f16 *bias, const et_f16 *X, et_f16 *Y, int T, int in, int out,
+                            int act, et_stream stream) {
+    ET_REQUIRE(rows && row_id && X && Y, ET_ERR_INVALID_ARG, "et_linear_rowpruned_f16: NULL pointer");
+    ET_REQUIRE(act >= ET_ACT_NONE && act <= ET_ACT_GELU, ET_ERR_INVALID_ARG,
+               "et_linear_rowpruned_f16: act=%d", act);
+    ET_REQUIRE(nnz_row >= 0 && nnz_row <= out, ET_ERR_INVALID_ARG,
+               "et_linear_rowpruned_f16: nnz_row=%d out=%d", nnz_row, out);
+    int s = check_gemm_shape("et_linear_rowpruned_f16", T, out, in);
+    if (s != ET_OK) return s;
+    ET_REQUIRE(nnz_row % 16 == 0, ET_ERR_UNSUPPORTED,
+               "et_linear_rowpruned_f16: nnz_row=%d must be a multiple of 16", nnz_row);
+    if (T == 0) return ET_OK;
+    hipStream_t st = as_stream(stream);
+    if (nnz_row < out) {
+        // pruned features carry the bias alone; live ones are overwritten below
+        const size_t total = (size_t)T * out;
+        size_t blocks = (total + 255) / 256;
+        if (blocks > 2048) blocks = 2048;
+        bias_rows_kernel<<<(unsigned)blocks, 256, 0, st>>>(H(Y), H(bias), T, out, out, act);
+        s = check_launch("bias_rows_kernel");
+        if (s != ET_OK) return s;
+    }
+    if (nnz_row == 0) return ET_OK;
+    GemmArgs g = gemm_args(H(X), H(rows), H(Y), T, nnz_row, in, in, in, out);
+    g.bias = H(bias);
+    g.c_scatter = row_id;
+    g.act = act;
+    return launch_gemm(g, 1, true, st);
+}
+
+int et_linear_rowpruned_compact_f16(const et_f16 *rows, const int32_t *row_id, int nnz_row,
+                                    const et_f16 *bias, const et_f16 *X, et_f16 *Yc, int T, int in,
+                                    et_stream stream) {
+    ET_REQUIRE(rows && X && Yc, ET_ERR_INVALID_ARG, "et_linear_rowpruned_compact_f16: NULL pointer");
+    ET_REQUIRE(bias == nullptr || row_id != nullptr, ET_ERR_INVALID_ARG,
+               "et_linear_rowpruned_compact_f16: bias needs row_id");
+    int s = check_gemm_shape("et_linear_rowpruned_compact_f16", T, nnz_row, in);
+    if (s != ET_OK) return s;
+    if (T == 0) return ET_OK;
+    // Compact output: column j holds feature row_id[j]; its bias is bias[row_id[j]].
+    GemmArgs g = gemm_args(H(X), H(rows), H(Yc), T, nnz_row, in, in, in, nnz_row);
+    g.bias = H(bias);
+    g.bias_idx = bias ? row_id : nullptr;
+    return launch_gemm(g, 1, true, as_stream(stream));
+}
+
+int et_fill_rows_bias_f16(et_f16 *C, const et_f16 *bias, int rows, int cols, et_stream stream) {
+    ET_REQUIRE(C != nullptr, ET_ERR_INVALID_ARG, "et_fill_rows_bias_f16: C is NULL");
+    ET_REQUIRE(rows >= 0 && cols > 0, ET_ERR_INVALID_ARG, "et_fill_rows_bias_f16: rows=%d cols=%d", rows, cols);
+    if (rows == 0) return ET_OK;
+    const size_t total = (size_t)rows * cols;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 2048) blocks = 2048;
+    bias_rows_kernel<<<(unsigned)blocks, 256, 0, as_stream(stream)>>>(H(C), H(bias), rows, cols, cols, ET_ACT_NONE);
+    return check_launch("bias_rows_kernel");
+}
+
+int et_linear_colpruned_f16(const et_f16 *cols, const int32_t *col_id, int nnz_col,
+                            const et_f16 *bias, const et_f16 *X, et_f16 *Y, int T, int in, int out,
+                            int act, et_stream stream) {
+    ET_REQUIRE(cols && col_id && X && Y, ET_ERR_INVALID_ARG, "et_linear_colpruned_f16: NULL pointer");
+    ET_REQUIRE(act >= ET_ACT_NONE && act <= ET_ACT_GELU, ET_ERR_INVALID_ARG,
+               "et_linear_colpruned_f16: act=%d", act);
+    ET_REQUIRE(nnz_col >= 0 && nnz_col <= in, ET_ERR_INVALID_ARG,
+               "et_linear_colpruned_f16: nnz_col=%d in=%d", nnz_col, in);
+    ET_REQUIRE(in > 0 && T % 16 == 0 && out % 16 == 0 && nnz_col % 16 == 0 && T >= 0 && out > 0,
+               ET_ERR_UNSUPPORTED,
+               "et_linear_colpruned_f16: T=%d out=%d nnz_col=%d must be multiples of 16", T, out,
+               nnz_col);
+    if (T == 0) return ET_OK;
+    hipStream_t st = as_stream(stream);
+    if (nnz_col == 0) {
+        const size_t total = (size_t)T * out;
+        size_t blocks = (total + 255) / 256;
+        if (blocks > 2048) blocks = 2048;
+        bias_rows_kernel<<<(unsigned)blocks, 256, 0, st>>>(H(Y), H(bias), T, out, out, act);
+        return check_launch("bias_rows_kernel");
+    }
+    GemmArgs g = gemm_args(H(X), H(cols), H(Y), T, out, nnz_col, in, nnz_col, out);
+    g.bias = H(bias);
+    g.a_gather = col_id;
+    g.act = act;
+    return launch_gemm(g, 1, true, st);
+}
+
+}  // extern "C"

@@ -80,6 +80,8 @@ const char *et_status_string(int status) {
 
 const char *et_last_error(void) { return g_err; }
 
+void et_set_last_error(const char *message) { set_error("%s", message ? message : ""); }
+
 int et_device_info(char *name, int cap, int *num_cu, int *lds_bytes) {
     int dev = 0;
     ET_HIP(hipGetDevice(&dev));
@@ -202,6 +204,39 @@ int et_stream_sync(et_stream stream) {
 
 int et_device_sync(void) {
     ET_HIP(hipDeviceSynchronize());
+    return ET_OK;
+}
+
+int et_graph_begin_capture(et_stream stream) {
+    ET_REQUIRE(stream != nullptr, ET_ERR_INVALID_ARG,
+               "et_graph_begin_capture: capture needs a stream from et_stream_create");
+    ET_HIP(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeRelaxed));
+    return ET_OK;
+}
+
+int et_graph_end_capture(et_stream stream, et_graph *graph) {
+    ET_REQUIRE(stream != nullptr && graph != nullptr, ET_ERR_INVALID_ARG,
+               "et_graph_end_capture: NULL argument");
+    *graph = nullptr;
+    hipGraph_t g = nullptr;
+    ET_HIP(hipStreamEndCapture(as_stream(stream), &g));
+    hipGraphExec_t exec = nullptr;
+    int s = check_hip(hipGraphInstantiate(&exec, g, nullptr, nullptr, 0), "hipGraphInstantiate");
+    (void)hipGraphDestroy(g);
+    if (s != ET_OK) return s;
+    *graph = exec;
+    return ET_OK;
+}
+
+int et_graph_launch(et_graph graph, et_stream stream) {
+    ET_REQUIRE(graph != nullptr, ET_ERR_INVALID_ARG, "et_graph_launch: graph is NULL");
+    ET_HIP(hipGraphLaunch(reinterpret_cast<hipGraphExec_t>(graph), as_stream(stream)));
+    return ET_OK;
+}
+
+int et_graph_destroy(et_graph graph) {
+    if (!graph) return ET_OK;
+    ET_HIP(hipGraphExecDestroy(reinterpret_cast<hipGraphExec_t>(graph)));
     return ET_OK;
 }
 

@@ -171,3 +171,25 @@ def run_layer_case(et, H, nh, dimFF, S, B, sparsity, seed, lens=None, nlayers=1,
                         store=torch.float16)
     want = L.encoder_stack(f32(x), [w.oracle_params() for w in layers], cfg).numpy()
     return max_abs(got, want)
+
+
+def build_model(et, layers, S, B, act=2, lens=None, use_graph=True, causal=False, eps=1e-5):
+    """Encoder stack through et_model_* from a list of LayerWeights (exact fp16 bits)."""
+    w0 = layers[0]
+    m = et.Model(w0.H, w0.nh, w0.dimFF, S, len(layers), batch=B, act=act, eps=eps, causal=causal,
+                 use_graph=use_graph)
+    for i, w in enumerate(layers):
+        for which, bw in ((et.W_QKV, w.qkv), (et.W_O, w.o), (et.W_FF1, w.l1), (et.W_FF2, w.l2)):
+            m.set_bsr16(i, which, bw.row_ptr, bw.col_idx, bw.tiles, bw.bias)
+        m.set_norm(i, 0, w.g1, w.be1)
+        m.set_norm(i, 1, w.g2, w.be2)
+    if lens is not None:
+        m.set_lens(lens)
+    m.finalize()
+    return m
+
+
+def oracle_stack(x, layers, B, lens=None, act="gelu", causal=False, eps=1e-5, store=torch.float16):
+    cfg = L.LayerConfig(nh=layers[0].nh, B=B, act=act, eps=eps, causal=causal,
+                        lens=None if lens is None else torch.as_tensor(np.asarray(lens)), store=store)
+    return L.encoder_stack(f32(x), [w.oracle_params() for w in layers], cfg).numpy()
