@@ -16,7 +16,10 @@ from pathlib import Path
 import numpy as np
 
 PKG_DIR = Path(__file__).resolve().parent
-LIB_PATH = PKG_DIR / "lib" / "libet_hip.so"
+import os as _os
+
+# ET_LIB_PATH selects another build of the same library (kernel tuning experiments).
+LIB_PATH = Path(_os.environ.get("ET_LIB_PATH") or (PKG_DIR / "lib" / "libet_hip.so"))
 
 ET_OK = 0
 ET_ERR_INVALID_ARG = -1

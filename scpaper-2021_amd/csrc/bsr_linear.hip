@@ -1,19 +1,30 @@
 // Y[T x out] = act(X[T x in] * W^T + bias), W stored as 16x16 tiles (BSR over
 // the [out x in] matrix, tile rows = output features) — gfx950 MFMA kernel.
 //
-// One workgroup owns a strip of MT*16 token rows and a contiguous group of
-// block-rows of W.  The token strip of X is staged once in LDS (row stride
-// padded by 16 bytes, so the 16 rows a fragment read touches fall in distinct
-// banks) and every wave walks the tiles of its block-rows two at a time:
-// v_mfma_f32_16x16x32_f16 contracts 32 values, i.e. tile t (k 0..15) and tile
-// t+1 (k 16..31) of the same block-row in one instruction.  The reference tile
-// layout [tile][out 16][in 16] is exactly the MFMA A-operand feed: lane
-// (r = lane%16, g = lane/16) reads 8 consecutive halfs of row r of tile
-// t + g/2 at offset 8*(g%2), so a tile pair is one contiguous 1 KiB wave load.
-// The B operand is the matching 16-token x 16-feature block of X.  The
-// accumulator of lane (r, g) is C[feature 4g..4g+3][token r]: four consecutive
-// output features of one token, stored as one 8-byte write after bias and
-// activation in fp32.
+// Work split.  One workgroup owns a strip of MT*16 token rows and a contiguous
+// group of block-rows of W; its waves take those block-rows round-robin.  The
+// strip of X is staged once in LDS (row stride padded by 16 bytes: the 16 rows
+// a fragment read touches fall in distinct banks).  Workgroups are numbered so
+// that all groups of one strip run on the same XCD (private L2).
+//
+// Matrix-core feed.  v_mfma_f32_16x16x32_f16 contracts 32 values, i.e. tile t
+// (k 0..15) and tile t+1 (k 16..31) of one block-row in a single instruction —
+// a "slot".  The reference tile layout [tile][out 16][in 16] is exactly the
+// MFMA A-operand feed: lane (r = lane%16, g = lane/16) reads 8 consecutive
+// halfs of row r of tile t + g/2 at offset 8*(g%2), so a slot is one contiguous
+// 1 KiB wave load.  The B operand is the matching 16-token x 16-feature block
+// of X from LDS.  The accumulator of lane (r, g) is C[feature 4g..4g+3][token r]:
+// four consecutive output features of one token, stored as one 8-byte write
+// after bias and activation in fp32.
+//
+// Latency and issue rate.  A global load costs on the order of a microsecond and
+// a lone wave issues one vector instruction every few cycles, so the kernel keeps
+// the per-slot instruction count minimal (one weight load and one index load with
+// immediate offsets from per-row base pointers, one LDS read and one MFMA per
+// 16-token block) and keeps loads in flight across rows: the row pointers of all
+// rows of a wave are fetched with one load, and the weights, indices and bias of
+// the next row group (up to kSlots slots) are requested before the current one is
+// multiplied.  Several workgroups per compute unit cover the rest.
 //
 // Tile order inside a block-row is free (the sum commutes), as in the
 // reference kernel (Linear/SPMM_tile.cu:277-283).
@@ -33,36 +44,181 @@ struct BsrArgs {
     int act;
 };
 
-constexpr int kLdsPad = 8;  // halfs
+constexpr int kXcds = 8;      // accelerator dies, each with a private L2
+constexpr int kLdsPad = 8;    // halfs
+constexpr int kSlots = 8;     // slots per row group held in registers (two groups resident)
+constexpr int kStageU = 8;    // 16-byte strip vectors a thread keeps in flight
+constexpr int kMaxWaveRows = 64;  // block-rows one wave can own (one lane each)
 
-template <int MT, bool STAGE>
+template <int ACT> __device__ __forceinline__ float act_fixed(float x) {
+    if (ACT == ET_ACT_RELU) return x > 0.0f ? x : 0.0f;
+    if (ACT == ET_ACT_GELU) return gelu_tanh(x);
+    return x;
+}
+
+__device__ __forceinline__ int lane_read(int v, int lane) {
+    return __builtin_amdgcn_readlane(v, lane);
+}
+
+// ACT is a template parameter: the epilogue carries no run-time branch and each
+// fused activation is a separately named kernel in a profile.
+template <int MT, bool STAGE, int ACT>
 __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     extern __shared__ __align__(16) unsigned char smem_raw[];
     _Float16 *xs = reinterpret_cast<_Float16 *>(smem_raw);
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nwave = blockDim.x >> 6;
+    const int nthr = blockDim.x;
     const int r16 = lane & 15;
     const int g = lane >> 4;
-    const int sel = g >> 1;         // which tile of the pair this lane feeds
+    const int sel = g >> 1;         // which tile of the slot this lane feeds
     const int koff = (g & 1) << 3;  // offset of its 8 k-values inside the tile
-    const int tok0 = blockIdx.y * (MT * 16);
+    // Workgroup id -> (token strip, block-row group), XCD-aware.  Workgroups are
+    // handed to the 8 XCDs round-robin by linear id and each XCD has its own L2, so
+    // strip s is pinned to XCD s % 8 and the groups of one strip follow each other on
+    // that XCD: a strip of X is fetched into one L2 only and reused there.
     const int nbr = a.out >> 4;
-    const int rb_begin = blockIdx.x * a.rows_per_wg;
+    const int ngroups = (nbr + a.rows_per_wg - 1) / a.rows_per_wg;
+    const int nstrips = (a.T + MT * 16 - 1) / (MT * 16);
+    const int xcd = blockIdx.x % kXcds, k_in_xcd = blockIdx.x / kXcds;
+    const int strip = xcd + kXcds * (k_in_xcd / ngroups);
+    const int group = k_in_xcd % ngroups;
+    if (strip >= nstrips) return;  // padding of the last round of strips (whole workgroup)
+    const int tok0 = strip * (MT * 16);
+    const int rb_begin = group * a.rows_per_wg;
     const int rb_end = min(rb_begin + a.rows_per_wg, nbr);
     const int lds_ld = a.in + kLdsPad;
+    const h8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
+    // ---- row pointers of this wave's block-rows: rows rb_begin + wave + nwave*i,
+    // lane i holds [lo, hi) of row i (first in the load queue: loads return in
+    // issue order and everything below depends on these few bytes)
+    const int nrw = max(0, (rb_end - rb_begin - wave + nwave - 1) / nwave);
+    int rp_lo = 0, rp_hi = 0;
+    if (lane < nrw) {
+        const int rb = rb_begin + wave + nwave * lane;
+        rp_lo = a.row_ptr[rb];
+        rp_hi = a.row_ptr[rb + 1];
+    }
+
+    // ---- strip copy, first batch: loads only.  X[tok0 .. tok0+MT*16) is one
+    // contiguous block of global memory; only the LDS side has padded rows.
+    const int vec_per_row = a.in >> 3;
+    const int rows_here = min(MT * 16, a.T - tok0);
+    const int total_vec = STAGE ? rows_here * vec_per_row : 0;
+    const h8 *src = reinterpret_cast<const h8 *>(a.X + (size_t)tok0 * a.in);
+    h8 sv[kStageU];
     if (STAGE) {
-        const int vec_per_row = a.in >> 3;
-        const int total = MT * 16 * vec_per_row;
-        for (int v = threadIdx.x; v < total; v += blockDim.x) {
-            const int r = v / vec_per_row;
-            const int c = v - r * vec_per_row;
-            const int tok = tok0 + r;
-            h8 val = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (tok < a.T) val = *reinterpret_cast<const h8 *>(a.X + (size_t)tok * a.in + c * 8);
-            *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) = val;
+#pragma unroll
+        for (int u = 0; u < kStageU; u++) {
+            const int idx = threadIdx.x + u * nthr;
+            if (idx < total_vec) sv[u] = src[idx];
+        }
+    }
+
+    // ---- row-group stream of this wave.  An item is up to kSlots slots of one
+    // block-row; (it_row, it_part) is the next item to request.
+    h8 w[2][kSlots];
+    int col[2][kSlots];
+    h4 bias_v[2];
+    int g_row[2], g_nsl[2];  // resident items: wave row index (-1 = none), slots in the item
+    bool g_last[2];          // item ends its block-row
+    int it_row = 0, it_part = 0;
+    // skip rows without tiles (they are written at the end)
+    auto skip_empty = [&]() {
+        while (it_row < nrw && lane_read(rp_hi, it_row) == lane_read(rp_lo, it_row)) it_row++;
+    };
+    skip_empty();
+    auto issue_item = [&](int buf) {
+        if (it_row >= nrw) {
+            g_row[buf] = -1;
+            return;
+        }
+        const int t0 = lane_read(rp_lo, it_row), t1 = lane_read(rp_hi, it_row);
+        const int nsl_row = (t1 - t0 + 1) >> 1;
+        const int first_slot = it_part * kSlots;
+        const int nsl = min(kSlots, nsl_row - first_slot);
+        const bool last = first_slot + nsl == nsl_row;
+        const bool odd_tail = last && ((t1 - t0) & 1);  // the last slot holds one tile only
+        g_row[buf] = it_row;
+        g_nsl[buf] = nsl;
+        g_last[buf] = last;
+        const int tf = t0 + 2 * first_slot;  // first tile of the item
+        // per-lane base pointers; slot p adds an immediate p*1024 B / p*8 B
+        const _Float16 *wp = a.tiles + (size_t)(tf + sel) * 256 + r16 * 16 + koff;
+        const int32_t *cp = a.col_idx + tf + sel;
+#pragma unroll
+        for (int p = 0; p < kSlots; p++) {
+            if (p < nsl) {
+                if (odd_tail && p == nsl - 1) {
+                    // lanes of the missing second tile: zero weights, index of the first tile
+                    w[buf][p] = zero8;
+                    if (sel == 0) w[buf][p] = *reinterpret_cast<const h8 *>(wp + p * 512);
+                    col[buf][p] = a.col_idx[tf + 2 * p];
+                } else {
+                    w[buf][p] = *reinterpret_cast<const h8 *>(wp + p * 512);
+                    col[buf][p] = cp[2 * p];
+                }
+            } else if (p & 1) {
+                w[buf][p] = zero8;  // partner of the last slot inside a two-slot step
+                col[buf][p] = 0;
+            }
+        }
+        if (last) {  // the item that finishes the row carries its bias
+            bias_v[buf] = h4{0, 0, 0, 0};
+            if (a.bias)
+                bias_v[buf] = *reinterpret_cast<const h4 *>(a.bias + (rb_begin + wave + nwave * it_row) * 16 + g * 4);
+        }
+        if (last) {
+            it_row++;
+            it_part = 0;
+            skip_empty();
+        } else {
+            it_part++;
+        }
+    };
+    issue_item(0);
+    issue_item(1);
+
+    // ---- strip copy: write the first batch, then the rest
+    if (STAGE) {
+        const int dr = nthr / vec_per_row, dc = nthr - dr * vec_per_row;  // (row, col) step of +nthr
+        int r = threadIdx.x / vec_per_row, c = threadIdx.x - r * vec_per_row;
+#pragma unroll
+        for (int u = 0; u < kStageU; u++) {
+            const int idx = threadIdx.x + u * nthr;
+            if (idx < total_vec) *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) = sv[u];
+            r += dr;
+            c += dc;
+            if (c >= vec_per_row) {
+                c -= vec_per_row;
+                r++;
+            }
+        }
+        for (int base = threadIdx.x + kStageU * nthr; base < total_vec; base += nthr * kStageU) {
+#pragma unroll
+            for (int u = 0; u < kStageU; u++) {
+                const int idx = base + u * nthr;
+                if (idx < total_vec) sv[u] = src[idx];
+            }
+#pragma unroll
+            for (int u = 0; u < kStageU; u++) {
+                const int idx = base + u * nthr;
+                if (idx < total_vec) *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) = sv[u];
+                r += dr;
+                c += dc;
+                if (c >= vec_per_row) {
+                    c -= vec_per_row;
+                    r++;
+                }
+            }
+        }
+        // rows beyond T (a partial last strip) read as zero
+        for (int idx = total_vec + threadIdx.x; idx < MT * 16 * vec_per_row; idx += nthr) {
+            const int rr = idx / vec_per_row, cc = idx - rr * vec_per_row;
+            *reinterpret_cast<h8 *>(xs + rr * lds_ld + cc * 8) = zero8;
         }
         __syncthreads();
     }
@@ -80,69 +236,62 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
             xrow[m] = a.X + (size_t)(tok_ok[m] ? tok : 0) * a.in + koff;
         }
     }
-    const h8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
-    for (int rb = rb_begin + wave; rb < rb_end; rb += nwave) {
-        f4 acc[MT];
+    // ---- multiply
+    f4 acc[MT];
 #pragma unroll
-        for (int m = 0; m < MT; m++) acc[m] = f4{0.f, 0.f, 0.f, 0.f};
+    for (int m = 0; m < MT; m++) acc[m] = f4{0.f, 0.f, 0.f, 0.f};
 
-        const int t_begin = a.row_ptr[rb];
-        const int t_end = a.row_ptr[rb + 1];
-        const _Float16 *wbase = a.tiles + r16 * 16 + koff;
-
-        // Software pipeline: operands of pair p+1 are in flight while pair p
-        // is multiplied.
-        int ti = t_begin + sel;
-        bool ok = ti < t_end;
-        h8 w_cur = zero8, x_cur[MT];
-        {
-            const int col = ok ? a.col_idx[ti] : 0;
-            if (ok) w_cur = *reinterpret_cast<const h8 *>(wbase + (size_t)ti * 256);
-#pragma unroll
-            for (int m = 0; m < MT; m++) {
-                x_cur[m] = *reinterpret_cast<const h8 *>(xrow[m] + col * 16);
-                if (!ok || (!STAGE && !tok_ok[m])) x_cur[m] = zero8;
-            }
-        }
-        for (int t = t_begin; t < t_end; t += 2) {
-            const int tn = ti + 2;
-            const bool okn = tn < t_end;
-            h8 w_nxt = zero8, x_nxt[MT];
-            {
-                const int coln = okn ? a.col_idx[tn] : 0;
-                if (okn) w_nxt = *reinterpret_cast<const h8 *>(wbase + (size_t)tn * 256);
-#pragma unroll
-                for (int m = 0; m < MT; m++) {
-                    x_nxt[m] = *reinterpret_cast<const h8 *>(xrow[m] + coln * 16);
-                    if (!okn || (!STAGE && !tok_ok[m])) x_nxt[m] = zero8;
-                }
-            }
-#pragma unroll
-            for (int m = 0; m < MT; m++)
-                acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w_cur, x_cur[m], acc[m], 0, 0, 0);
-            w_cur = w_nxt;
-#pragma unroll
-            for (int m = 0; m < MT; m++) x_cur[m] = x_nxt[m];
-            ti = tn;
-        }
-
-        // epilogue: lane holds features 16*rb + 4g .. +3 of token r16
-        const int f0 = rb * 16 + g * 4;
-        float b[4] = {0.f, 0.f, 0.f, 0.f};
-        if (a.bias) {
-            const h4 bv = *reinterpret_cast<const h4 *>(a.bias + f0);
-#pragma unroll
-            for (int j = 0; j < 4; j++) b[j] = (float)bv[j];
-        }
+    // bias + activation + store of one finished block-row, then clear
+    auto flush = [&](int wave_row, h4 bv) {
+        const int f0 = (rb_begin + wave + nwave * wave_row) * 16 + g * 4;
 #pragma unroll
         for (int m = 0; m < MT; m++) {
-            if (!tok_ok[m]) continue;
-            h4 o;
+            if (tok_ok[m]) {
+                h4 o;
 #pragma unroll
-            for (int j = 0; j < 4; j++) o[j] = (_Float16)apply_act(acc[m][j] + b[j], a.act);
-            const int tok = tok0 + m * 16 + r16;
-            *reinterpret_cast<h4 *>(a.Y + (size_t)tok * a.out + f0) = o;
+                for (int j = 0; j < 4; j++) o[j] = (_Float16)act_fixed<ACT>(acc[m][j] + (float)bv[j]);
+                const int tok = tok0 + m * 16 + r16;
+                *reinterpret_cast<h4 *>(a.Y + (size_t)tok * a.out + f0) = o;
+            }
+            acc[m] = f4{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+
+    while (g_row[0] >= 0) {
+#pragma unroll
+        for (int buf = 0; buf < 2; buf++) {
+            if (g_row[buf] >= 0) {
+                const int nsl = g_nsl[buf];
+#pragma unroll
+                for (int p0 = 0; p0 < kSlots; p0 += 2) {
+                    if (p0 < nsl) {  // wave-uniform; slot p0+1 is real or zero-weighted
+                        h8 x[2][MT];
+#pragma unroll
+                        for (int q = 0; q < 2; q++)
+#pragma unroll
+                            for (int m = 0; m < MT; m++) {
+                                x[q][m] = *reinterpret_cast<const h8 *>(xrow[m] + col[buf][p0 + q] * 16);
+                                if (!STAGE && !tok_ok[m]) x[q][m] = zero8;
+                            }
+#pragma unroll
+                        for (int q = 0; q < 2; q++)
+#pragma unroll
+                            for (int m = 0; m < MT; m++)
+                                acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[buf][p0 + q], x[q][m], acc[m], 0, 0, 0);
+                    }
+                }
+                if (g_last[buf]) flush(g_row[buf], bias_v[buf]);
+                issue_item(buf);  // request the item after next into the buffer just drained
+            }
+        }
+    }
+    // block-rows without any tile still produce act(bias)
+    for (int r = 0; r < nrw; r++) {
+        if (lane_read(rp_hi, r) == lane_read(rp_lo, r)) {
+            h4 bv = {0, 0, 0, 0};
+            if (a.bias) bv = *reinterpret_cast<const h4 *>(a.bias + (rb_begin + wave + nwave * r) * 16 + g * 4);
+            flush(r, bv);
         }
     }
 }
@@ -155,37 +304,60 @@ struct BsrPlan {
     size_t lds;
 };
 
-// Launch geometry.  The strip is staged in LDS whenever MT*16 rows of X fit
-// in the 160 KiB a workgroup may hold; the block-row group is sized so that
-// the grid is a few workgroups per compute unit.
-static BsrPlan plan_bsr(int T, int in, int out) {
-    BsrPlan p;
-    const size_t lds_cap = 160 * 1024;
-    const size_t row_bytes = (size_t)(in + kLdsPad) * sizeof(_Float16);
-    p.stage = true;
-    if (T >= 64 && 64 * row_bytes <= lds_cap / 2) p.mt = 4;
-    else if (T >= 32 && 32 * row_bytes <= lds_cap / 2) p.mt = 2;
-    else if (16 * row_bytes <= lds_cap) p.mt = 1;
-    else { p.mt = 4; p.stage = false; }
-    p.lds = p.stage ? (size_t)p.mt * 16 * row_bytes : 0;
-    p.threads = 256;
-    const int nbr = out / 16;
-    const int strips = (T + p.mt * 16 - 1) / (p.mt * 16);
-    const int nwave = p.threads / 64;
-    // aim for about 1024 workgroups, at least one block-row per wave
-    int groups = (1024 + strips - 1) / strips;
-    if (groups < 1) groups = 1;
-    int rpw = (nbr + groups - 1) / groups;
-    rpw = ((rpw + nwave - 1) / nwave) * nwave;
-    if (rpw > nbr) rpw = nbr;
-    if (rpw < 1) rpw = 1;
-    p.rows_per_wg = rpw;
-    return p;
+// LDS of one workgroup: the padded strip (when staged).
+static size_t bsr_lds_bytes(int mt, bool stage, int in, int rows_per_wg) {
+    (void)rows_per_wg;
+    return stage ? (size_t)mt * 16 * (in + kLdsPad) * sizeof(_Float16) : 0;
 }
 
-template <int MT, bool STAGE>
-static int launch_bsr(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
-    auto kernel = bsr16_linear_kernel<MT, STAGE>;
+// Launch geometry.  The strip is staged in LDS whenever it fits next to a second
+// workgroup (half of the 160 KiB of a compute unit), else alone, else X is read
+// from global memory.  Measured on MI355X the kernel is fastest with about one
+// workgroup of 8 waves per compute unit (~200-256 workgroups): fewer, larger
+// workgroups re-read less of X and W through the L2.  Small problems that cannot
+// fill the device that way fall back to narrower strips and smaller workgroups.
+static BsrPlan plan_bsr(int T, int in, int out) {
+    const size_t lds_cap = 160 * 1024;
+    const size_t row_bytes = (size_t)(in + kLdsPad) * sizeof(_Float16);
+    const int nbr = out / 16;
+    int mt_fit = 0;  // widest strip that can be staged
+    if (32 * row_bytes <= lds_cap / 2) mt_fit = 2;
+    else if (16 * row_bytes <= lds_cap) mt_fit = 1;
+    struct Cand { int mt, threads; };
+    Cand cands[6];
+    int nc = 0;
+    if (mt_fit == 2 && T >= 32) { cands[nc++] = {2, 512}; cands[nc++] = {2, 256}; }
+    if (mt_fit >= 1) { cands[nc++] = {1, 512}; cands[nc++] = {1, 256}; cands[nc++] = {1, 128}; }
+    if (mt_fit == 0) { cands[nc++] = {2, 256}; }
+    BsrPlan best{};
+    int best_wgs = -1;
+    for (int i = 0; i < nc; i++) {
+        BsrPlan p;
+        p.mt = cands[i].mt;
+        p.stage = mt_fit != 0;
+        p.threads = cands[i].threads;
+        const int nwave = p.threads / 64;
+        const int strips = (T + p.mt * 16 - 1) / (p.mt * 16);
+        const int groups = strips >= 256 ? 1 : 256 / strips;
+        int rpw = (nbr + groups - 1) / groups;
+        rpw = ((rpw + nwave - 1) / nwave) * nwave;
+        if (rpw > nbr) rpw = nbr;
+        if (rpw > kMaxWaveRows * nwave) rpw = kMaxWaveRows * nwave;
+        p.rows_per_wg = rpw;
+        p.lds = bsr_lds_bytes(p.mt, p.stage, in, rpw);
+        const int wgs = strips * ((nbr + rpw - 1) / rpw);
+        if (wgs > best_wgs) {
+            best = p;
+            best_wgs = wgs;
+        }
+        if (wgs >= 160) break;  // enough to occupy the device: prefer the earlier candidate
+    }
+    return best;
+}
+
+template <int MT, bool STAGE, int ACT>
+static int launch_bsr_act(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
+    auto kernel = bsr16_linear_kernel<MT, STAGE, ACT>;
     if (p.lds > 64 * 1024) {
         static bool raised = false;  // per instantiation
         if (!raised) {
@@ -195,10 +367,21 @@ static int launch_bsr(const BsrArgs &args, const BsrPlan &p, hipStream_t stream)
         }
     }
     const int nbr = args.out / 16;
-    const dim3 grid((nbr + p.rows_per_wg - 1) / p.rows_per_wg,
-                    (args.T + MT * 16 - 1) / (MT * 16));
+    const int ngroups = (nbr + p.rows_per_wg - 1) / p.rows_per_wg;
+    const int nstrips = (args.T + MT * 16 - 1) / (MT * 16);
+    const int strip_rounds = (nstrips + kXcds - 1) / kXcds;
+    const dim3 grid((unsigned)(strip_rounds * kXcds * ngroups));
     kernel<<<grid, p.threads, p.lds, stream>>>(args);
     return check_launch("bsr16_linear_kernel");
+}
+
+template <int MT, bool STAGE>
+static int launch_bsr(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
+    switch (args.act) {
+        case ET_ACT_RELU: return launch_bsr_act<MT, STAGE, ET_ACT_RELU>(args, p, stream);
+        case ET_ACT_GELU: return launch_bsr_act<MT, STAGE, ET_ACT_GELU>(args, p, stream);
+        default: return launch_bsr_act<MT, STAGE, ET_ACT_NONE>(args, p, stream);
+    }
 }
 
 static int dispatch_bsr(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
@@ -276,7 +459,9 @@ int et_linear_bsr16_f16_geom(const int32_t *row_ptr, const int32_t *col_idx, con
     p.stage = stage != 0;
     p.threads = threads;
     p.rows_per_wg = rows_per_wg;
-    p.lds = p.stage ? (size_t)mt * 16 * (in + kLdsPad) * sizeof(_Float16) : 0;
+    p.lds = bsr_lds_bytes(mt, p.stage, in, rows_per_wg);
+    ET_REQUIRE(rows_per_wg <= kMaxWaveRows * (threads / 64), ET_ERR_UNSUPPORTED,
+               "et_linear_bsr16_f16_geom: at most %d block-rows per wave", kMaxWaveRows);
     ET_REQUIRE(p.lds <= 160 * 1024, ET_ERR_UNSUPPORTED,
                "et_linear_bsr16_f16_geom: strip of %d rows x %d does not fit LDS", mt * 16, in);
     BsrArgs args{row_ptr,
