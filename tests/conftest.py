@@ -21,3 +21,16 @@ def et():
     pkg = entry.load_package()
     pkg.lib()
     return pkg
+
+
+@pytest.fixture(autouse=True)
+def _release_device_buffers():
+    """Frees the buffers tests/harness.up() kept alive, after the device has drained."""
+    yield
+    from tests import harness
+
+    if harness.KEEP:
+        import __graft_entry__ as entry
+
+        entry.load_package().sync()
+        harness.KEEP.clear()

@@ -17,6 +17,18 @@ from oracle import formats as F  # noqa: E402
 from oracle import layers as L  # noqa: E402
 
 
+# Device buffers created through up() stay alive until the test that made them ends
+# (tests/conftest.py clears the list): a kernel launch is asynchronous, so a temporary
+# whose raw pointer was passed to the C ABI must not be freed when the expression ends.
+KEEP: list = []
+
+
+def up(et, a):
+    buf = et.DeviceBuffer.from_numpy(a)
+    KEEP.append(buf)
+    return buf
+
+
 def rng(seed: int) -> torch.Generator:
     g = torch.Generator()
     g.manual_seed(seed)

@@ -1,0 +1,57 @@
+"""The native library loads without a GPU and exports every symbol include/et_abi.h declares."""
+import ctypes
+import re
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def declared_symbols():
+    text = (ROOT / "include" / "et_abi.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)  # comments cite names that are not declarations
+    return sorted(set(re.findall(r"\b(et_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_surface():
+    names = declared_symbols()
+    for must in ("et_linear_bsr16_f16", "et_mha_fused_f16", "et_skip_layernorm_f16", "et_model_forward",
+                 "et_linear_dense_f16", "et_linear_rowpruned_f16", "et_linear_colpruned_f16",
+                 "et_linear_vec1x16_f16", "et_linear_csr_f16", "et_mha_compactv_f16", "et_mha_vo_f16",
+                 "et_fmt_dense_to_bsr16", "et_graph_launch"):
+        assert must in names
+    assert len(names) >= 70
+
+
+def test_library_exports_every_declared_symbol(et):
+    lib = et.lib()
+    missing = [n for n in declared_symbols() if not hasattr(lib, n)]
+    assert missing == []
+
+
+def test_binding_has_argtypes_for_every_declared_symbol(et):
+    untyped = [n for n in declared_symbols()
+               if n not in et._SIGNATURES and n not in ("et_status_string", "et_last_error", "et_set_last_error")]
+    assert untyped == []
+
+
+def test_status_strings_and_error_channel(et):
+    lib = et.lib()
+    assert lib.et_status_string(0) == b"ok"
+    assert b"unsupported" in lib.et_status_string(et.ET_ERR_UNSUPPORTED)
+    lib.et_set_last_error.argtypes = [ctypes.c_char_p]
+    lib.et_set_last_error(b"probe message")
+    assert lib.et_last_error() == b"probe message"
+    # a host-side entry point fails with a status and a message, never aborts
+    n = ctypes.c_int()
+    st = lib.et_fmt_tile_pattern(30, 64, 0.5, 1, None, None, ctypes.byref(n))
+    assert st == et.ET_ERR_INVALID_ARG and b"multiples of 16" in lib.et_last_error()
+
+
+def test_no_product_file_imports_the_oracle():
+    """The oracle is test infrastructure: nothing under the package or include/ may use it."""
+    offenders = []
+    for path in list((ROOT / "scpaper-2021_amd").rglob("*")) + list((ROOT / "include").rglob("*")):
+        if path.is_file() and path.suffix in (".py", ".h", ".hpp", ".hip", ".cpp") and "build" not in path.parts:
+            if re.search(r"^\s*(from|import)\s+oracle\b|oracle/", path.read_text(), flags=re.M):
+                offenders.append(str(path))
+    assert offenders == []

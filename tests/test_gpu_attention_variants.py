@@ -1,0 +1,117 @@
+"""GPU parity of the attention forms whose operands differ from the plain fused kernel:
+probabilities in memory, the unfused baseline, the pre-computed-VO attention (dense and
+column-pruned) and the attention-aware compact-V form."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import formats as F
+from oracle import layers as L
+from tests import harness as Hn
+
+pytestmark = pytest.mark.gpu
+
+
+up = Hn.up
+
+
+@pytest.mark.parametrize("B,S,nh,hd,causal", [(2, 128, 12, 64, False), (1, 512, 4, 64, True), (3, 48, 2, 32, False)])
+def test_probs_and_unfused(et, B, S, nh, hd, causal):
+    H, T = nh * hd, B * S
+    q, k, v = Hn.randn((T, H), 1), Hn.randn((T, H), 2), Hn.randn((T, H), 3)
+    lens = np.array([S, S // 2 + 1, S - 5][:B], np.int32)
+    d_p = et.DeviceBuffer.empty((T, nh * S), np.float16)
+    d_z = et.DeviceBuffer.empty((T, H), np.float16)
+    flags = et.MHA_CAUSAL if causal else 0
+    scale = 1 / math.sqrt(hd)
+    et.check(et.lib().et_mha_unfused_f16(up(et, q).ptr, up(et, k).ptr, up(et, v).ptr, H, H, H, d_z.ptr, H, d_p.ptr, None,
+                                         up(et, lens).ptr, B, S, nh, hd, scale, flags, None))
+    z, P = L.mha(Hn.f32(q), Hn.f32(k), Hn.f32(v), nh, B, lens=lens, causal=causal, return_probs=True)
+    got_p = d_p.numpy().astype(np.float32).reshape(B, S, nh, S).transpose(0, 2, 1, 3)  # [b][h][q][key]
+    assert Hn.max_abs(got_p, P.numpy()) <= 1e-3
+    assert abs(got_p.sum(-1) - 1).max() <= 4e-3
+    for b in range(B):
+        assert np.all(got_p[b, :, :, lens[b]:] == 0)
+    assert Hn.max_abs(d_z.numpy(), z.numpy()) <= 4e-3
+
+
+def vo_case(seed, H, nh, N_keep=None):
+    g = Hn.rng(seed)
+    rn = lambda *s: (torch.randn(*s, generator=g) * 0.05)
+    Wq, Wk, Wv, Wo = rn(H, H), rn(H, H), rn(H, H), rn(H, H)
+    bq, bk, bv, bo = rn(H), rn(H), rn(H), rn(H)
+    hd = H // nh
+    Wvo = torch.stack([Wv[h * hd:(h + 1) * hd].T @ Wo[:, h * hd:(h + 1) * hd].T for h in range(nh)])  # [nh][H][H]
+    bvo = torch.stack([bv[h * hd:(h + 1) * hd] @ Wo[:, h * hd:(h + 1) * hd].T for h in range(nh)])
+    h16 = lambda t: t.numpy().astype(np.float16)
+    return dict(Wq=h16(Wq), Wk=h16(Wk), bq=h16(bq), bk=h16(bk), Wvo=h16(Wvo), bvo=h16(bvo), bo=h16(bo))
+
+
+@pytest.mark.parametrize("B,S,H,nh,pruned", [(1, 128, 768, 12, False), (2, 64, 256, 4, False), (2, 64, 256, 4, True)])
+def test_vo_attention(et, B, S, H, nh, pruned):
+    """Linear_VO + probabilities + one GEMM per sequence == the oracle's sum_h P_h VO_h + b_O."""
+    T, hd = B * S, H // nh
+    c = vo_case(7, H, nh)
+    x = Hn.randn((T, H), 8)
+    lens = np.array([S, S - 9][:B], np.int32)
+    Wvo, bvo = c["Wvo"], c["bvo"]
+    col_id = None
+    if pruned:
+        col_id = np.sort(F.gen_col_ids(H, 0.5, seed=9)).astype(np.int32)
+        Wvo, bvo = np.ascontiguousarray(Wvo[:, :, col_id]), np.ascontiguousarray(bvo[:, col_id])
+    N = Wvo.shape[2]
+    # Q, K projections through the dense Linear kernel
+    d_q, d_k = et.DeviceBuffer.empty((T, H), np.float16), et.DeviceBuffer.empty((T, H), np.float16)
+    d_x = up(et, x)
+    et.linear_dense(up(et, c["Wq"]), up(et, c["bq"]), d_x, d_q, T, H, H)
+    et.linear_dense(up(et, c["Wk"]), up(et, c["bk"]), d_x, d_k, T, H, H)
+    d_vo = et.DeviceBuffer.empty((B, nh, S, N), np.float16)
+    et.check(et.lib().et_linear_vo_f16(up(et, Wvo).ptr, up(et, bvo).ptr, d_x.ptr, d_vo.ptr, B, S, H, N, nh, None))
+    want_vo = (x.astype(np.float32).reshape(B, 1, S, H) @ Wvo.astype(np.float32)[None] +
+               bvo.astype(np.float32)[None, :, None, :]).astype(np.float16)
+    assert Hn.max_abs(d_vo.numpy(), want_vo) <= 4e-3
+    d_p = et.DeviceBuffer.empty((T, nh * S), np.float16)
+    d_out = et.DeviceBuffer.empty((T, H), np.float16)
+    et.check(et.lib().et_fill_f16(d_out.ptr, T * H, 0x7E00, None))
+    et.check(et.lib().et_mha_vo_f16(d_q.ptr, d_k.ptr, H, H, d_vo.ptr, d_p.ptr, d_out.ptr, up(et, c["bo"]).ptr,
+                                    None if col_id is None else up(et, col_id).ptr, None, up(et, lens).ptr, B, S, nh, hd,
+                                    N, H, 1 / math.sqrt(hd), 0, None))
+    Wvo_full, bvo_full = c["Wvo"].astype(np.float32), c["bvo"].astype(np.float32)
+    if pruned:  # pruned columns of W_VO are zero; their outputs carry b_O alone
+        m = np.zeros(H, bool); m[col_id] = True
+        Wvo_full, bvo_full = Wvo_full * m, bvo_full * m
+    want = L.fused_vo_attention(Hn.f32(x), Hn.f32(x), Hn.f32(x), Hn.f32(c["Wq"]), Hn.f32(c["bq"]), Hn.f32(c["Wk"]),
+                                Hn.f32(c["bk"]), torch.from_numpy(Wvo_full), torch.from_numpy(bvo_full), Hn.f32(c["bo"]),
+                                nh, B, lens=lens, store=torch.float16).numpy()
+    got = d_out.numpy()
+    assert Hn.max_abs(got, want) <= 6e-3
+    if pruned:
+        dead = np.setdiff1d(np.arange(H), col_id)
+        assert np.array_equal(got[:, dead], np.broadcast_to(c["bo"][dead], (T, len(dead))))
+
+
+@pytest.mark.parametrize("B,S,nh,hd,keep", [(2, 128, 12, 64, 0.75), (1, 48, 4, 32, 0.5), (1, 272, 2, 64, 0.25)])
+def test_compact_v_attention(et, B, S, nh, hd, keep):
+    """Attention-aware pruning: V arrives compact with col_id / head_ptr; Z is full width with
+    zeros in pruned columns and equals dense attention over V with the pruned columns zeroed."""
+    H, T = nh * hd, B * S
+    q, k = Hn.randn((T, H), 30), Hn.randn((T, H), 31)
+    col_id = F.gen_row_ids(H, 1 - keep, seed=32)  # surviving V columns, ascending (row ids of W_V)
+    hp = F.head_ptr(col_id, len(col_id), nh, H)
+    assert hp[-1] == len(col_id)
+    vc = Hn.randn((T, len(col_id)), 33)
+    lens = np.array([S, S - 7][:B], np.int32)
+    d_z = et.DeviceBuffer.empty((T, H), np.float16)
+    et.check(et.lib().et_fill_f16(d_z.ptr, T * H, 0x7E00, None))
+    et.check(et.lib().et_mha_compactv_f16(up(et, q).ptr, up(et, k).ptr, up(et, vc).ptr, H, H, len(col_id),
+                                          up(et, col_id).ptr, up(et, hp).ptr, len(col_id), d_z.ptr, H, None,
+                                          up(et, lens).ptr, B, S, nh, hd, hd, 1 / math.sqrt(hd), 0, None))
+    v_full = np.zeros((T, H), np.float16)
+    v_full[:, col_id] = vc
+    want = L.mha(Hn.f32(q), Hn.f32(k), Hn.f32(v_full), nh, B, lens=lens, store=torch.float16).numpy()
+    got = d_z.numpy()
+    assert Hn.max_abs(got, want) <= 2e-3
+    dead = np.setdiff1d(np.arange(H), col_id)
+    assert np.all(got[:, dead] == 0)

@@ -16,8 +16,7 @@ pytestmark = pytest.mark.gpu
 TOL_F16 = 2e-2
 
 
-def up(et, a):
-    return et.DeviceBuffer.from_numpy(a)
+up = Hn.up
 
 
 # ---------------------------------------------------------------- runtime ----
