@@ -35,6 +35,9 @@ struct Array {
 using npz_t = std::map<std::string, Array>;  // keyed by array name (without ".npy")
 
 Array parse_npy(const char *buf, std::size_t len, const std::string &what);
+// writes a little-endian C-order .npy (version 1.0); descr e.g. "<f4", "<i4", "<f2"
+void npy_save(const std::string &path, const void *data, const std::string &descr, std::size_t word_size,
+              const std::vector<std::size_t> &shape);
 Array npy_load(const std::string &path);
 npz_t npz_load(const std::string &path);
 

@@ -71,7 +71,26 @@ def build_all(jobs: int | None = None, verbose: bool = True) -> Path:
     os.replace(tmp, LIB)
     if verbose:
         print(f"built {LIB} from {len(srcs)} sources")
+    build_programs(verbose)
     return LIB
+
+
+# C++ programs written against the class layer (include/et/*.h) and linked with the library.
+PROGRAMS = {ROOT / "tests" / "cpp" / "class_layer_cases.cpp": ROOT / "tests" / "cpp" / "bin" / "class_layer_cases"}
+
+
+def build_programs(verbose: bool = True) -> None:
+    for src, exe in PROGRAMS.items():
+        if not src.exists():
+            continue
+        exe.parent.mkdir(exist_ok=True)
+        cmd = [HIPCC, *COMMON, "-x", "c++", str(src), "-L", str(LIBDIR), "-let_hip",
+               f"-Wl,-rpath,{LIBDIR}", "-Wl,-rpath,$ORIGIN/../../../scpaper-2021_amd/lib", "-o", str(exe)]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        if res.returncode != 0:
+            raise RuntimeError(f"program build failed: {' '.join(cmd)}\n{res.stderr}")
+        if verbose:
+            print(f"built {exe}")
 
 
 if __name__ == "__main__":

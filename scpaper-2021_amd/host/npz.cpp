@@ -109,6 +109,28 @@ Array parse_npy(const char *buf, std::size_t len, const std::string &what) {
     return a;
 }
 
+void npy_save(const std::string &path, const void *data, const std::string &descr, std::size_t word_size,
+              const std::vector<std::size_t> &shape) {
+    std::string dict = "{'descr': '" + descr + "', 'fortran_order': False, 'shape': (";
+    std::size_t n = 1;
+    for (std::size_t i = 0; i < shape.size(); i++) {
+        dict += std::to_string(shape[i]) + (shape.size() == 1 || i + 1 < shape.size() ? "," : "");
+        if (i + 1 < shape.size()) dict += " ";
+        n *= shape[i];
+    }
+    dict += "), }";
+    while ((10 + dict.size() + 1) % 64 != 0) dict += ' ';
+    dict += '\n';
+    std::ofstream f(path, std::ios::binary);
+    if (!f) throw Error(ET_ERR_IO, "cannot create " + path);
+    const unsigned char head[10] = {0x93, 'N', 'U', 'M', 'P', 'Y', 1, 0, (unsigned char)(dict.size() & 0xff),
+                                    (unsigned char)(dict.size() >> 8)};
+    f.write(reinterpret_cast<const char *>(head), 10);
+    f.write(dict.data(), (std::streamsize)dict.size());
+    f.write(static_cast<const char *>(data), (std::streamsize)(n * word_size));
+    if (!f) throw Error(ET_ERR_IO, "cannot write " + path);
+}
+
 Array npy_load(const std::string &path) {
     const std::vector<char> buf = read_file(path);
     return parse_npy(buf.data(), buf.size(), path);

@@ -1,0 +1,272 @@
+// Drives the C++ class layer (include/et/*.h) the way the reference's own
+// programs do, and writes the results as .npy files for the pytest side to
+// compare with the CPU oracle.  Usage:  class_layer_cases <case> <dir>
+//   example       two ReLU encoder layers + a decoder Linear loaded from weights.txt/.npz,
+//                 the model assembly of the reference example (example/main.cu:24-182)
+//   prune_attn    Attention<tile, tile, row_mat, tile, Prune_attn> (attention-aware pruning)
+//   fused_attn    FusedAttention<NOTF_fused_attn> with the W_VO built by et::build_vo_weight
+//   fused_prune   FusedAttention<NOTF_fused_prune_attn> over a column-pruned W_VO
+//   factories     the gen_* test factories: closed forms of the reference drivers
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <iostream>
+#include <string>
+
+#include "et/Encoder.h"
+#include "et/weights.hpp"
+#include "et/wtime.h"
+
+using et::npy::npy_load;
+using et::npy::npy_save;
+
+static std::vector<half> load_half(const std::string &path) {
+    auto a = npy_load(path);
+    return vec_F2H(a.as_vector<float>());
+}
+static void save_half(const std::string &path, const et::DeviceBuffer<half> &buf, std::size_t rows, std::size_t cols) {
+    std::vector<half> h = buf.to_host();
+    std::vector<float> f(h.size());
+    for (std::size_t i = 0; i < h.size(); i++) f[i] = static_cast<float>(h[i]);
+    npy_save(path, f.data(), "<f4", 4, {rows, cols});
+}
+static std::vector<int> load_int(const std::string &path) { return npy_load(path).as_vector<int>(); }
+static std::vector<int> read_meta(const std::string &dir) { return load_int(dir + "/meta.npy"); }
+
+static tile_mat tile_from(Weights &w, const std::string &name, int in) {
+    return tile_mat(w.load_mat<int>("row_ptr", name), w.load_mat<int>("column", name),
+                    vec_F2H(w.load_mat<float>("data", name)), in / 16);
+}
+
+// ---- example/main.cu ------------------------------------------------------------
+static int run_example(const std::string &dir) {
+    using mat_t = tile_mat;
+    using attn_config = Attention_config<mat_t, mat_t, mat_t, mat_t, OTF_attn_full, true, false>;
+    using encoder_config = Encoder_config<attn_config, mat_t, mat_t, RELU_OP>;
+    const auto meta = read_meta(dir);  // kdim vdim seq nhead dimFF emdim nlayer batch decoder_width
+    auto para = std::make_shared<Model_t>(Model_t{meta[0], meta[1], meta[2], meta[3], meta[4], meta[5], meta[6]});
+    const int batch = meta[7], text = meta[8];
+    const int rows = batch * para->seq_len;
+    Weights weights(dir + "/weights.txt", dir + "/");
+    std::vector<std::unique_ptr<Encoder<encoder_config>>> model((std::size_t)para->nlayer);
+    for (int l = 0; l < para->nlayer; l++) {
+        const std::string pre = "transformer_encoder.layers." + std::to_string(l) + ".";
+        const auto QKVname = pre + "self_attn.in_proj_.npz";
+        et::DeviceBuffer<half> BQKV(vec_F2H(weights.load_mat<float>("B", QKVname)));
+        auto LQKV = std::make_unique<Linear<mat_t>>(para->emdim, para->kdim * 3, tile_from(weights, QKVname, para->emdim),
+                                                    BQKV, rows);
+        const auto Oname = pre + "self_attn.out_proj..npz";
+        et::DeviceBuffer<half> BO(vec_F2H(weights.load_mat<float>("B", Oname)));
+        auto LO = std::make_unique<Linear<mat_t>>(para->vdim, para->emdim, tile_from(weights, Oname, para->vdim), BO, rows);
+        auto attn = std::make_unique<Attention<attn_config>>(std::move(LQKV), std::move(LO), para, batch);
+        const auto LN1name = pre + "norm1..npz", LN2name = pre + "norm2..npz";
+        auto LN1 = std::make_unique<SkipLayerNorm>(vec_F2H(weights.load_mat<float>("W", LN1name)).data(),
+                                                   vec_F2H(weights.load_mat<float>("B", LN1name)).data(), para->emdim);
+        auto LN2 = std::make_unique<SkipLayerNorm>(vec_F2H(weights.load_mat<float>("W", LN2name)).data(),
+                                                   vec_F2H(weights.load_mat<float>("B", LN2name)).data(), para->emdim);
+        const auto L1name = pre + "linear1..npz", L2name = pre + "linear2..npz";
+        et::DeviceBuffer<half> BL1(vec_F2H(weights.load_mat<float>("B", L1name)));
+        auto L1 = std::make_unique<Linear<mat_t>>(para->emdim, para->dimFF, tile_from(weights, L1name, para->emdim), BL1, rows);
+        et::DeviceBuffer<half> BL2(vec_F2H(weights.load_mat<float>("B", L2name)));
+        auto L2 = std::make_unique<Linear<mat_t>>(para->dimFF, para->emdim, tile_from(weights, L2name, para->dimFF), BL2, rows);
+        model[(std::size_t)l] = std::make_unique<Encoder<encoder_config>>(std::move(attn), std::move(LN1), std::move(LN2),
+                                                                          std::move(L1), std::move(L2), para);
+    }
+    const auto Dname = std::string("decoder..npz");
+    et::DeviceBuffer<half> BD(vec_F2H(weights.load_mat<float>("B", Dname)));
+    auto LD = std::make_unique<Linear<mat_t>>(para->emdim, text, tile_from(weights, Dname, para->emdim), BD, rows);
+
+    et::DeviceBuffer<half> IN(load_half(dir + "/input.npy"));
+    et::DeviceBuffer<half> A((std::size_t)rows * para->emdim), B((std::size_t)rows * para->emdim);
+    et::DeviceBuffer<half> OUT((std::size_t)rows * text);
+    half *src = IN.get();
+    for (int l = 0; l < para->nlayer; l++) {
+        half *dst = (l % 2 == 0) ? A.get() : B.get();
+        model[(std::size_t)l]->forward(dst, src);
+        src = dst;
+    }
+    LD->forward(OUT.get(), src);
+    etChk(et_device_sync());
+    save_half(dir + "/out.npy", OUT, (std::size_t)rows, (std::size_t)text);
+    save_half(dir + "/hidden.npy", (para->nlayer % 2 == 1) ? A : B, (std::size_t)rows, (std::size_t)para->emdim);
+    // the reference's timing protocol on the same objects (lib/wtime.h:22-35)
+    const double us = wtime_new(
+        20, [&]() { model[0]->forward(A.get(), IN.get()); }, []() { etChk(et_device_sync()); });
+    std::printf("encoder layer forward: %.1f us\n", us);
+    return 0;
+}
+
+// ---- attention-aware pruning (test/Table2/template.hpp:56-97) -------------------
+static int run_prune_attn(const std::string &dir) {
+    using attn_config = Attention_config<tile_mat, tile_mat, row_mat, tile_mat, Prune_attn, false, true>;
+    const auto meta = read_meta(dir);  // H seq nhead batch
+    const int H = meta[0], S = meta[1], nh = meta[2], batch = meta[3], rows = batch * S;
+    auto para = std::make_shared<Model_t>(Model_t{H, H, S, nh, 4 * H, H, 1});
+    auto dense_tile_linear = [&](const std::string &tag) {
+        auto W = npy_load(dir + "/W" + tag + ".npy").as_vector<float>();
+        auto b = load_half(dir + "/b" + tag + ".npy");
+        return std::make_unique<Linear<tile_mat>>(H, H, tile_mat::from_dense(W.data(), H, H), b.data(), rows);
+    };
+    auto LQ = dense_tile_linear("q"), LK = dense_tile_linear("k"), LO = dense_tile_linear("o");
+    auto row_id = load_int(dir + "/v_row_id.npy");
+    auto v_rows = load_half(dir + "/v_rows.npy");
+    auto bv = load_half(dir + "/bv.npy");
+    row_mat WV(et::DeviceBuffer<int>(row_id), et::DeviceBuffer<half>(v_rows), H, H);
+    auto LV = std::make_unique<Linear<row_mat>>(H, H, std::move(WV), bv.data(), rows);
+    Attention<attn_config> attn(std::move(LQ), std::move(LK), std::move(LV), std::move(LO), para, batch);
+    auto lens = load_int(dir + "/lens.npy");
+    attn.set_lens(lens.data());
+    et::DeviceBuffer<half> X(load_half(dir + "/input.npy")), OUT((std::size_t)rows * H);
+    attn.forward(OUT.get(), X.get(), X.get(), X.get());
+    etChk(et_device_sync());
+    save_half(dir + "/out.npy", OUT, (std::size_t)rows, (std::size_t)H);
+    return 0;
+}
+
+// ---- pre-computed VO attention (Fused_attention/test/testfused.cu:17-97) --------
+template <typename tag> static int run_fused(const std::string &dir) {
+    using attn_config = Attention_config<base_mat, base_mat, base_mat, base_mat, tag, false, true>;
+    const auto meta = read_meta(dir);  // H seq nhead batch
+    const int H = meta[0], S = meta[1], nh = meta[2], batch = meta[3], rows = batch * S;
+    auto para = std::make_shared<Model_t>(Model_t{H, H, S, nh, 4 * H, H, 1});
+    auto dense_linear = [&](const std::string &tag2) {
+        auto W = load_half(dir + "/W" + tag2 + ".npy");
+        auto b = load_half(dir + "/b" + tag2 + ".npy");
+        return std::make_unique<Linear<base_mat>>(H, H, base_mat(W), b.data(), rows);
+    };
+    auto LQ = dense_linear("q"), LK = dense_linear("k");
+    auto Wv = npy_load(dir + "/Wv.npy").as_vector<float>(), bv = npy_load(dir + "/bv.npy").as_vector<float>();
+    auto Wo = npy_load(dir + "/Wo.npy").as_vector<float>();
+    std::vector<float> Wvo, bvo;
+    et::build_vo_weight(Wv.data(), bv.data(), Wo.data(), H, H, H, nh, Wvo, bvo);
+    et::DeviceBuffer<half> biasO(load_half(dir + "/bo.npy"));
+    et::DeviceBuffer<half> X(load_half(dir + "/input.npy")), OUT((std::size_t)rows * H);
+    auto lens = load_int(dir + "/lens.npy");
+    if constexpr (std::is_same<tag, NOTF_fused_prune_attn>::value) {
+        auto col_id = load_int(dir + "/vo_col_id.npy");
+        const std::size_t N = col_id.size();
+        std::vector<half> Wc((std::size_t)nh * H * N), bc((std::size_t)nh * N);
+        for (int h = 0; h < nh; h++) {
+            for (int i = 0; i < H; i++)
+                for (std::size_t j = 0; j < N; j++)
+                    Wc[((std::size_t)h * H + i) * N + j] = static_cast<half>(Wvo[((std::size_t)h * H + i) * H + col_id[j]]);
+            for (std::size_t j = 0; j < N; j++) bc[(std::size_t)h * N + j] = static_cast<half>(bvo[(std::size_t)h * H + col_id[j]]);
+        }
+        col_mat W(et::DeviceBuffer<int>(col_id), et::DeviceBuffer<half>(Wc), nh * H, H, (int)N);
+        auto LVO = std::make_unique<Linear_VO_prune>(W, et::DeviceBuffer<half>(bc), para);
+        FusedAttention<attn_config> attn(std::move(LQ), std::move(LK), std::move(LVO), biasO, para, batch);
+        attn.set_lens(lens.data());
+        attn.forward(OUT.get(), X.get(), X.get(), X.get());
+    } else {
+        auto LVO = std::make_unique<Linear_VO>(et::DeviceBuffer<half>(vec_F2H(Wvo)), et::DeviceBuffer<half>(vec_F2H(bvo)), para);
+        FusedAttention<attn_config> attn(std::move(LQ), std::move(LK), std::move(LVO), biasO, para, batch);
+        attn.set_lens(lens.data());
+        attn.forward(OUT.get(), X.get(), X.get(), X.get());
+    }
+    etChk(et_device_sync());
+    save_half(dir + "/out.npy", OUT, (std::size_t)rows, (std::size_t)H);
+    // the offline W_VO builder's result, for the test to check against numpy
+    npy_save(dir + "/Wvo.npy", Wvo.data(), "<f4", 4, {(std::size_t)nh, (std::size_t)H, (std::size_t)H});
+    npy_save(dir + "/bvo.npy", bvo.data(), "<f4", 4, {(std::size_t)nh, (std::size_t)H});
+    return 0;
+}
+
+// ---- gen_* factories: closed forms of the reference drivers ---------------------
+static float first_value(const et::DeviceBuffer<half> &b, std::size_t i = 0) { return static_cast<float>(b.to_host()[i]); }
+
+static int run_factories(const std::string &dir) {
+    std::vector<float> out;
+    const int T = 64;
+    et::DeviceBuffer<half> X1024((std::size_t)T * 1024, half_one), Y((std::size_t)T * 1024);
+    // dense ones: in_size * 1 + 0.5 (Linear/test/test_cublas.cu:12-19), at a width fp16 holds exactly
+    et::DeviceBuffer<half> X256((std::size_t)T * 256, half_one);
+    gen_dense_linear<base_mat>(128, 256, T)->forward(Y.get(), X256.get());
+    out.push_back(first_value(Y, 5));                                   // 256.5
+    gen_dense_linear<tile_mat>(128, 256, T)->forward(Y.get(), X256.get());
+    out.push_back(first_value(Y, 5));                                   // 256.5
+    // tile-sparse ones: 16 * tiles_in_block_row + 0.5 (Linear/test/test_tile.cu:56-75)
+    {
+        auto lin = gen_sparse_linear<tile_mat>(128, 256, T, 0.5f);
+        lin->forward(Y.get(), X256.get());
+        auto rp = lin->weight.row_ptr.to_host();
+        out.push_back(first_value(Y, 0));
+        out.push_back(16.0f * (float)(rp[1] - rp[0]) + 0.5f);          // expected for block-row 0
+        out.push_back((float)lin->weight.num_blk);                     // 64 of 128 tiles
+    }
+    gen_dense_linear<row_mat>(128, 256, T)->forward(Y.get(), X256.get());
+    out.push_back(first_value(Y, 7));                                   // 256.5
+    {
+        auto lin = gen_sparse_linear<row_mat>(128, 256, T, 0.5f);      // 64 live rows: x.w + b, others b alone
+        lin->forward(Y.get(), X256.get());
+        auto ids = lin->weight.row_id->to_host();
+        auto y = Y.to_host();
+        out.push_back(static_cast<float>(y[(std::size_t)ids[0]]));       // 256.5
+        int dead = 0;
+        while (std::find(ids.begin(), ids.end(), dead) != ids.end()) dead++;
+        out.push_back(static_cast<float>(y[(std::size_t)dead]));         // 0.5
+        out.push_back((float)ids.size());                                // 64
+    }
+    {
+        auto lin = gen_sparse_linear<col_mat>(128, 256, T, 0.5f);      // 128 live inputs, weights 0.5
+        lin->forward(Y.get(), X256.get());
+        out.push_back(first_value(Y, 3));                               // 128 * 0.5 + 0.5 = 64.5
+    }
+    gen_dense_linear<csr_mat>(128, 256, T)->forward(Y.get(), X256.get());
+    out.push_back(first_value(Y, 9));                                   // 256.5
+    gen_dense_linear<mat1x16>(128, 256, T)->forward(Y.get(), X256.get());
+    out.push_back(first_value(Y, 11));                                  // 256.5
+    // Linear_VO with weight 0.2, bias 0.2, input ones over 1024 features: 0.2*1024 + 0.2 = 205.0
+    // (Fused_attention/test/testVO.cu:10-16; the fp16 result is 205.0 exactly)
+    {
+        auto para = std::make_shared<Model_t>(Model_t{1024, 1024, 64, 16, 4096, 1024, 1});
+        const half p2 = static_cast<half>(0.2f);
+        Linear_VO vo(et::DeviceBuffer<half>((std::size_t)16 * 1024 * 1024, p2), et::DeviceBuffer<half>((std::size_t)16 * 1024, p2), para);
+        et::DeviceBuffer<half> VO((std::size_t)16 * 64 * 1024);
+        vo.forward(VO.get(), X1024.get());
+        etChk(et_device_sync());
+        out.push_back(first_value(VO, 12345));
+    }
+    // SkipLayerNorm test instance: gamma = beta = 0.2; a constant row normalises to beta
+    {
+        auto ln = gen_skLN(768);
+        et::DeviceBuffer<half> A((std::size_t)T * 768, static_cast<half>(0.7f)), B((std::size_t)T * 768, static_cast<half>(0.1f)),
+            O((std::size_t)T * 768);
+        ln->forward(O.get(), A.get(), B.get(), T);
+        out.push_back(first_value(O, 100));                             // 0.2
+    }
+    // DeviceBuffer value semantics: deep copy, move, clear, set
+    {
+        et::DeviceBuffer<half> a(8, static_cast<half>(3.0f));
+        et::DeviceBuffer<half> b(a);
+        a.set(static_cast<half>(4.0f));
+        out.push_back(first_value(b));                                  // 3 (deep copy)
+        et::DeviceBuffer<half> c(std::move(a));
+        out.push_back(first_value(c));                                  // 4
+        c.clear();
+        out.push_back(first_value(c));                                  // 0
+        out.push_back((float)(a.get() == nullptr));                     // 1: moved-from
+    }
+    etChk(et_device_sync());
+    npy_save(dir + "/factories.npy", out.data(), "<f4", 4, {out.size()});
+    return 0;
+}
+
+int main(int argc, char **argv) {
+    if (argc < 3) {
+        std::fprintf(stderr, "usage: %s <case> <dir>\n", argv[0]);
+        return 2;
+    }
+    const std::string which = argv[1], dir = argv[2];
+    try {
+        if (which == "example") return run_example(dir);
+        if (which == "prune_attn") return run_prune_attn(dir);
+        if (which == "fused_attn") return run_fused<NOTF_fused_attn>(dir);
+        if (which == "fused_prune") return run_fused<NOTF_fused_prune_attn>(dir);
+        if (which == "factories") return run_factories(dir);
+        std::fprintf(stderr, "unknown case %s\n", which.c_str());
+        return 2;
+    } catch (const et::Error &e) {
+        std::fprintf(stderr, "et::Error %d: %s\n", e.status(), e.what());
+        return 1;
+    }
+}

@@ -1,0 +1,138 @@
+"""The C++ class layer used directly, as a caller written against the reference's headers would
+(tests/cpp/class_layer_cases.cpp): example-style model assembly from weights.txt + .npz, the
+attention-aware Prune_attn form, FusedAttention (dense and column-pruned W_VO) and the gen_*
+factories.  The program writes .npy files; the CPU oracle is the judge."""
+import subprocess
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import formats as F
+from oracle import layers as L
+from tests import harness as Hn
+
+pytestmark = pytest.mark.gpu
+
+EXE = Path(__file__).resolve().parent / "cpp" / "bin" / "class_layer_cases"
+
+
+def run_case(case, d):
+    assert EXE.exists(), f"{EXE} is missing: build it with `python scpaper-2021_amd/build.py`"
+    res = subprocess.run([str(EXE), case, str(d)], capture_output=True, text=True, timeout=120)
+    print(res.stdout, res.stderr)
+    assert res.returncode == 0, res.stderr
+    return res
+
+
+def test_example_model_from_npz(tmp_path):
+    """Two ReLU encoder layers + decoder, the reference example's shape family (emdim 800 is not a
+    multiple of the head size the kernels take, so 768 / 4 heads x 192 is not used either): H 512,
+    4 heads x 128, FFN 208, decoder 1024 wide, batch 2 x seq 64."""
+    H, nh, FF, S, B, TEXT, NL = 512, 4, 208, 64, 2, 1024, 2
+    layers = [Hn.LayerWeights(H, nh, FF, 0.6, seed=70 + i) for i in range(NL)]
+    dec = Hn.BsrWeight(TEXT, H, 0.7, seed=90, bias_std=0.02)
+    names = []
+    for i, w in enumerate(layers):
+        pre = f"transformer_encoder.layers.{i}."
+        for nm, bw in (("self_attn.in_proj_", w.qkv), ("self_attn.out_proj.", w.o), ("linear1.", w.l1), ("linear2.", w.l2)):
+            F.save_weight_npz(str(tmp_path / (pre + nm)), bw.dense.astype(np.float32), bw.bias.astype(np.float32))
+            names.append(pre + nm + ".npz")
+        for nm, (g, b) in (("norm1.", (w.g1, w.be1)), ("norm2.", (w.g2, w.be2))):
+            F.save_weight_npz(str(tmp_path / (pre + nm)), g.astype(np.float32), b.astype(np.float32))
+            names.append(pre + nm + ".npz")
+    F.save_weight_npz(str(tmp_path / "decoder."), dec.dense.astype(np.float32), dec.bias.astype(np.float32))
+    names.append("decoder..npz")
+    (tmp_path / "weights.txt").write_text("\n".join(names) + "\n")
+    x = Hn.randn((B * S, H), 91)
+    np.save(tmp_path / "input.npy", x.astype(np.float32))
+    np.save(tmp_path / "meta.npy", np.array([H, H, S, nh, FF, H, NL, B, TEXT], np.int32))
+    res = run_case("example", tmp_path)
+    assert "encoder layer forward" in res.stdout
+    hidden = Hn.oracle_stack(x, layers, B, act="relu")
+    want = L.linear(torch.from_numpy(hidden), Hn.f32(dec.dense), Hn.f32(dec.bias), None, torch.float16).numpy()
+    assert Hn.max_abs(np.load(tmp_path / "hidden.npy"), hidden) <= 2e-2
+    assert Hn.max_abs(np.load(tmp_path / "out.npy"), want) <= 2e-2
+
+
+def attention_inputs(tmp_path, H, nh, S, B, seed):
+    g = Hn.rng(seed)
+    rn = lambda *s: (torch.randn(*s, generator=g) * 0.05).numpy().astype(np.float16)
+    W = {k: rn(H, H) for k in "qkvo"}
+    b = {k: rn(H) for k in "qkvo"}
+    x = Hn.randn((B * S, H), seed + 1)
+    lens = np.array([S, S - 11][:B], np.int32)
+    for k in "qkvo":
+        np.save(tmp_path / f"W{k}.npy", W[k].astype(np.float32))
+        np.save(tmp_path / f"b{k}.npy", b[k].astype(np.float32))
+    np.save(tmp_path / "input.npy", x.astype(np.float32))
+    np.save(tmp_path / "lens.npy", lens)
+    np.save(tmp_path / "meta.npy", np.array([H, S, nh, B], np.int32))
+    return W, b, x, lens
+
+
+def test_prune_attn_class(tmp_path):
+    """Attention<tile, tile, row_mat, tile, Prune_attn>: W_V row-pruned, V kept compact, P*V over
+    the surviving columns, Z full width — equals standard attention with the pruned W_V rows (and
+    their bias) zero."""
+    H, nh, S, B = 256, 4, 64, 2
+    W, b, x, lens = attention_inputs(tmp_path, H, nh, S, B, 110)
+    row_id = F.gen_row_ids(H, 0.25, seed=5)  # 192 of 256 V features survive
+    np.save(tmp_path / "v_row_id.npy", row_id)
+    np.save(tmp_path / "v_rows.npy", W["v"][row_id].astype(np.float32))
+    run_case("prune_attn", tmp_path)
+    Wv = np.zeros_like(W["v"]); Wv[row_id] = W["v"][row_id]
+    bv = np.zeros_like(b["v"]); bv[row_id] = b["v"][row_id]
+    st = torch.float16
+    q = L.linear(Hn.f32(x), Hn.f32(W["q"]), Hn.f32(b["q"]), store=st)
+    k = L.linear(Hn.f32(x), Hn.f32(W["k"]), Hn.f32(b["k"]), store=st)
+    v = L.linear(Hn.f32(x), Hn.f32(Wv), Hn.f32(bv), store=st)
+    z = L.mha(q, k, v, nh, B, lens=lens, store=st)
+    want = L.linear(z, Hn.f32(W["o"]), Hn.f32(b["o"]), store=st).numpy()
+    assert Hn.max_abs(np.load(tmp_path / "out.npy"), want) <= 6e-3
+
+
+@pytest.mark.parametrize("case", ["fused_attn", "fused_prune"])
+def test_fused_attention_class(tmp_path, case):
+    """FusedAttention with W_VO built by et::build_vo_weight equals standard attention followed by
+    the output projection (the E.T. identity); the pruned form keeps half of the W_VO columns."""
+    H, nh, S, B = 256, 4, 64, 2
+    W, b, x, lens = attention_inputs(tmp_path, H, nh, S, B, 120)
+    hd = H // nh
+    col_id = np.sort(F.gen_col_ids(H, 0.5, seed=6)).astype(np.int32)
+    np.save(tmp_path / "vo_col_id.npy", col_id)
+    run_case(case, tmp_path)
+    f = lambda a: a.astype(np.float32)
+    Wvo = np.stack([f(W["v"])[h * hd:(h + 1) * hd].T @ f(W["o"])[:, h * hd:(h + 1) * hd].T for h in range(nh)])
+    bvo = np.stack([f(b["v"])[h * hd:(h + 1) * hd] @ f(W["o"])[:, h * hd:(h + 1) * hd].T for h in range(nh)])
+    assert Hn.max_abs(np.load(tmp_path / "Wvo.npy"), Wvo) <= 1e-5  # the offline builder
+    assert Hn.max_abs(np.load(tmp_path / "bvo.npy"), bvo) <= 1e-5
+    st = torch.float16
+    if case == "fused_prune":
+        m = np.zeros(H, bool); m[col_id] = True
+        Wvo, bvo = Wvo * m, bvo * m
+    Wvo16, bvo16 = torch.from_numpy(Wvo).half().float(), torch.from_numpy(bvo).half().float()
+    want = L.fused_vo_attention(Hn.f32(x), Hn.f32(x), Hn.f32(x), Hn.f32(W["q"]), Hn.f32(b["q"]), Hn.f32(W["k"]),
+                                Hn.f32(b["k"]), Wvo16, bvo16, Hn.f32(b["o"]), nh, B, lens=lens, store=st).numpy()
+    got = np.load(tmp_path / "out.npy")
+    assert Hn.max_abs(got, want) <= 6e-3
+    if case == "fused_attn":  # and the identity with plain attention + output projection
+        q = L.linear(Hn.f32(x), Hn.f32(W["q"]), Hn.f32(b["q"]), store=st)
+        k = L.linear(Hn.f32(x), Hn.f32(W["k"]), Hn.f32(b["k"]), store=st)
+        v = L.linear(Hn.f32(x), Hn.f32(W["v"]), Hn.f32(b["v"]))
+        std = L.linear(L.mha(q, k, v, nh, B, lens=lens), Hn.f32(W["o"]), Hn.f32(b["o"])).numpy()
+        assert Hn.max_abs(got, std) <= 2e-2
+
+
+def test_factories_closed_forms(tmp_path):
+    run_case("factories", tmp_path)
+    v = np.load(tmp_path / "factories.npy").tolist()
+    dense_b, dense_t, sp_got, sp_want, sp_ntile, row_dense, row_live, row_dead, row_n, col_v, csr_v, v16, vo, ln, *db = v
+    assert dense_b == 256.5 and dense_t == 256.5
+    assert sp_got == sp_want and sp_ntile == 64
+    assert row_dense == 256.5 and row_live == 256.5 and row_dead == 0.5 and row_n == 64
+    assert col_v == 64.5 and csr_v == 256.5 and v16 == 256.5
+    assert vo == 205.0  # the reference driver's expected value (Fused_attention/test/testVO.cu:10-16)
+    assert abs(ln - 0.2) < 1e-3
+    assert db == [3.0, 4.0, 0.0, 1.0]
