@@ -32,6 +32,10 @@ SPARSITY = 0.8
 ATTENTION_AWARE = 0.25
 
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak (vendor figure)
+# HBM-side bytes per launch of the FFN up-projection kernel: rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a streaming
+# kernel of known size (profiles/encoder_stack_bert_base_b8_s128_hbm_traffic.txt).
+FFN_UP_TRAFFIC_BYTES = (4622.4 * 1.9992 + 6144.0 * 1.0) * 1024
 
 
 def build_layers(Hn):
@@ -111,6 +115,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--eager", action="store_true", help="launch kernel by kernel instead of replaying a graph")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch a plain streaming kernel of known size (ReLU over 64 MiB in, 64 MiB out) "
+                         "three times, as the reference point for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this engine runs on ONE GPU (every sequence is independent; more GPUs would "
@@ -138,7 +145,7 @@ def main():
     roofline = {"bound": "mfma", "kernel": "bsr16_linear_kernel<2,true,GELU> 3072x768 @80% T=1024",
                 "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 5), "us_per_launch": round(ksec * 1e6, 3),
-                "flop_per_launch": flops, "traffic": None}
+                "flop_per_launch": flops, "traffic": round(FFN_UP_TRAFFIC_BYTES)}
 
     out = {
         "metric": "BERT-base encoder seqs/sec + per-layer latency µs, seq128 fp16 80% tile-sparse",
@@ -152,6 +159,13 @@ def main():
                    "launch": "eager" if args.eager else "hip-graph"},
         "roofline": roofline,
     }
+    if args.calibrate:
+        n = 32 * 1024 * 1024  # fp16 elements: 64 MiB read, 64 MiB written per launch
+        src = et.DeviceBuffer.from_numpy(np.ones(n, np.float16))
+        dst = et.DeviceBuffer.empty((n,), np.float16)
+        for _ in range(3):
+            et.check(et.lib().et_relu_f16(dst.ptr, src.ptr, n, None))
+        et.sync()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(Hn, layers, x)
     print(json.dumps(out))
