@@ -86,8 +86,14 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
 
     void forward(half *out, half *src, stream_t stream = nullptr) {
         attn->forward(temp_attn.get(), src, src, src, stream);
-        LN1->forward(temp_LN.get(), temp_attn.get(), src, rows, stream);
-        linear1->forward_act(temp_linear.get(), temp_LN.get(), act_code<ACT_OP_t>(), stream);
+        if constexpr (std::is_same_v<linear1_t, Linear<tile_mat>>) {
+            // SkipLayerNorm rides in the prologue of the tile-sparse linear1
+            linear1->forward_skipln_act(temp_linear.get(), temp_LN.get(), temp_attn.get(), src, *LN1,
+                                        act_code<ACT_OP_t>(), stream);
+        } else {
+            LN1->forward(temp_LN.get(), temp_attn.get(), src, rows, stream);
+            linear1->forward_act(temp_linear.get(), temp_LN.get(), act_code<ACT_OP_t>(), stream);
+        }
         linear2->forward(temp_attn.get(), temp_linear.get(), stream);
         LN2->forward(out, temp_attn.get(), temp_LN.get(), rows, stream);
     }

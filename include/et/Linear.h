@@ -139,6 +139,19 @@ template <> class Linear<tile_mat> {
                                   et::f16(bias.get()), et::f16(input), et::f16(output), size, (int)in_size,
                                   (int)out_size, act, stream));
     }
+    // ln_out = ln(src + skip); output = act(ln_out * W^T + bias) in one launch: the
+    // SkipLayerNorm -> Linear -> activation sequence of Encoder/Encoder.h:85-89.  LN_t is
+    // SkipLayerNorm (gamma(), beta(), epsilon(), width()).
+    template <typename LN_t>
+    void forward_skipln_act(half *output, half *ln_out, const half *src, const half *skip, const LN_t &ln,
+                            int act, et::stream_t stream = nullptr) {
+        et::require(ln.width() == (int)in_size, "Linear<tile_mat>: LayerNorm width must equal in_size");
+        etChk(et_skipln_linear_bsr16_f16(et::f16(src), et::f16(skip), et::f16(ln.gamma()), et::f16(ln.beta()),
+                                         ln.epsilon(), et::f16(ln_out), weight.row_ptr.get(),
+                                         weight.row_offset.get(), et::f16(weight.data.get()),
+                                         et::f16(bias.get()), et::f16(output), size, (int)in_size,
+                                         (int)out_size, act, stream));
+    }
 
   private:
     void check() const {

@@ -25,6 +25,9 @@ class SkipLayerNorm {
                                     reinterpret_cast<const et_f16 *>(bias.get()), num, size, eps, stream));
     }
     int width() const { return size; }
+    const half *gamma() const { return weight.get(); }
+    const half *beta() const { return bias.get(); }
+    float epsilon() const { return eps; }
 };
 
 // gamma = beta = 0.2, the reference's test instance (SkipLayerNorm/SkipLayerNorm.cu:84-88)

@@ -108,6 +108,21 @@ int et_linear_bsr16_f16(const int32_t *row_ptr, const int32_t *col_idx,
                         const et_f16 *X, et_f16 *Y, int T, int in, int out,
                         int act, et_stream stream);
 
+/* SkipLayerNorm fused into the tile-sparse Linear that consumes it:
+ *   ln_out = LayerNorm(src + skip) * gamma + beta      (written, [T x in])
+ *   Y      = act(ln_out * W^T + bias)
+ * in one kernel: the normalisation happens while the token strip is staged on
+ * chip, so the Linear does not wait for a LayerNorm kernel to drain.  Same values
+ * as et_skip_layernorm_f16 followed by et_linear_bsr16_f16 (which is what runs
+ * when in > 1024).  Replaces LN1->forward + linear1->forward + act<>() of
+ * Encoder<cfg>::forward (Encoder/Encoder.h:85-89). */
+int et_skipln_linear_bsr16_f16(const et_f16 *src, const et_f16 *skip,
+                               const et_f16 *gamma, const et_f16 *beta, float eps,
+                               et_f16 *ln_out, const int32_t *row_ptr,
+                               const int32_t *col_idx, const et_f16 *tiles,
+                               const et_f16 *bias, et_f16 *Y, int T, int in,
+                               int out, int act, et_stream stream);
+
 /* Tuning hook: et_linear_bsr16_f16 with an explicit launch geometry — mt in
  * {1,2,4} 16-token blocks per workgroup strip, stage != 0 keeps the strip of X
  * in LDS, threads per workgroup (multiple of 64, <= 512) and block-rows of W per

@@ -31,6 +31,7 @@ struct MhaArgs {
     const int32_t *lens;   // [B] or nullptr
     int ldq, ldk, ldv, ldz;
     int S, nh;
+    int nbh;            // sequences * heads
     float scale_log2e;  // scale * log2(e)
     int causal;
     // compact-V form only: V is [rows x nnz] holding the surviving V columns;
@@ -40,6 +41,7 @@ struct MhaArgs {
     const int32_t *v_head_ptr;
 };
 
+constexpr int kXcds = 8;                // accelerator dies, each with a private L2
 constexpr int kKeyBlock = 128;          // keys staged per iteration
 constexpr int kNKB = kKeyBlock / 16;    // 16-key MFMA blocks per iteration
 constexpr float kLog2e = 1.4426950408889634f;
@@ -53,8 +55,8 @@ struct MhaLds {
     static constexpr size_t bytes = (size_t)(k_halfs + vt_halfs) * sizeof(_Float16);
 };
 
-template <int HD, bool COMPACT>
-__global__ __launch_bounds__(256) void mha_fused_kernel(const MhaArgs a) {
+template <int HD, bool COMPACT, int NW>
+__global__ __launch_bounds__(64 * NW) void mha_fused_kernel(const MhaArgs a) {
     using L = MhaLds<HD>;
     constexpr int KS = HD / 32;  // K=32 MFMA steps over the head dimension
     constexpr int DB = HD / 16;  // 16-wide output blocks of the head dimension
@@ -64,14 +66,22 @@ __global__ __launch_bounds__(256) void mha_fused_kernel(const MhaArgs a) {
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int nwave = blockDim.x >> 6;
+    constexpr int nwave = NW;
+    constexpr int nthr = 64 * NW;
     const int r16 = lane & 15;
     const int g = lane >> 4;
-    const int h = blockIdx.y;
-    const int b = blockIdx.z;
     const int S = a.S;
+    // Workgroup id -> (sequence*head, query strip), XCD-aware: workgroups go to the 8
+    // XCDs round-robin by id, so the query strips of one (sequence, head) are given ids
+    // that land on the same XCD and share its K and V in that L2.
+    const int qstrips = (S + 16 * nwave - 1) / (16 * nwave);
+    const int xcd = blockIdx.x % kXcds, k_in_xcd = blockIdx.x / kXcds;
+    const int bh = xcd + kXcds * (k_in_xcd / qstrips);
+    if (bh >= a.nbh) return;  // padding of the last round (whole workgroup)
+    const int qstrip = k_in_xcd % qstrips;
+    const int b = bh / a.nh, h = bh - b * a.nh;
     const size_t row0 = (size_t)b * S;  // first token row of this sequence
-    const int q = (blockIdx.x * nwave + wave) * 16 + r16;  // this lane's query
+    const int q = (qstrip * nwave + wave) * 16 + r16;  // this lane's query
     const bool q_ok = q < S;
     int klimit = S;
     if (a.lens) klimit = min(S, max(a.lens[b], 0));
@@ -103,43 +113,62 @@ __global__ __launch_bounds__(256) void mha_fused_kernel(const MhaArgs a) {
     for (int blk = 0; blk < nblocks; blk++) {
         const int k0 = blk * kKeyBlock;
         if (blk > 0) __syncthreads();
-        // ---- stage K block: 16-byte vectors, rows beyond S zero-filled
+        // ---- stage the K block and the transposed V block: every global load of the
+        // block is issued before the first LDS write (one memory round trip)
         {
             constexpr int vec_per_row = HD / 8;
-            for (int v = threadIdx.x; v < kKeyBlock * vec_per_row; v += blockDim.x) {
-                const int r = v / vec_per_row, c = v - r * vec_per_row;
-                h8 val = {0, 0, 0, 0, 0, 0, 0, 0};
-                if (k0 + r < S)
-                    val = *reinterpret_cast<const h8 *>(a.K + (row0 + k0 + r) * a.ldk + h * HD + c * 8);
-                *reinterpret_cast<h8 *>(Ks + r * L::ldk + c * 8) = val;
-            }
-        }
-        // ---- stage V block transposed: a thread takes 4 keys x 8 dims
-        {
+            constexpr int KV = kKeyBlock * vec_per_row / nthr;  // K vectors per thread
             constexpr int dgroups = HD / 8;
-            for (int u = threadIdx.x; u < (kKeyBlock / 4) * dgroups; u += blockDim.x) {
+            constexpr int v_units = (kKeyBlock / 4) * dgroups;  // V units of 4 keys x 8 dims
+            constexpr int VU = (v_units + nthr - 1) / nthr;       // ... per thread
+            static_assert(KV >= 1 && kKeyBlock * vec_per_row % nthr == 0, "K block must split evenly");
+            h8 kreg[KV];
+            h8 vreg[VU][4];
+#pragma unroll
+            for (int i = 0; i < KV; i++) {
+                const int v = threadIdx.x + i * nthr;
+                const int r = v / vec_per_row, c = v - r * vec_per_row;
+                kreg[i] = h8{0, 0, 0, 0, 0, 0, 0, 0};
+                if (k0 + r < S)
+                    kreg[i] = *reinterpret_cast<const h8 *>(a.K + (row0 + k0 + r) * a.ldk + h * HD + c * 8);
+            }
+#pragma unroll
+            for (int j = 0; j < VU; j++) {
+                const int u = threadIdx.x + j * nthr;
                 const int kg = u / dgroups, dg = u - kg * dgroups;
-                h8 rows[4];
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    const int key = k0 + kg * 4 + i;
-                    rows[i] = h8{0, 0, 0, 0, 0, 0, 0, 0};
+                    const int key = (u < v_units) ? k0 + kg * 4 + i : S;  // surplus threads load nothing
+                    vreg[j][i] = h8{0, 0, 0, 0, 0, 0, 0, 0};
                     if (COMPACT) {
                         // compact columns start at an arbitrary element: scalar loads
                         if (key < S) {
                             const _Float16 *vp = a.V + (row0 + key) * a.ldv + vc0 + dg * 8;
 #pragma unroll
                             for (int d = 0; d < 8; d++)
-                                if (dg * 8 + d < vlive) rows[i][d] = vp[d];
+                                if (dg * 8 + d < vlive) vreg[j][i][d] = vp[d];
                         }
                     } else if (key < S) {
-                        rows[i] = *reinterpret_cast<const h8 *>(a.V + (row0 + key) * a.ldv + h * HD + dg * 8);
+                        vreg[j][i] = *reinterpret_cast<const h8 *>(a.V + (row0 + key) * a.ldv + h * HD + dg * 8);
                     }
                 }
+            }
 #pragma unroll
-                for (int d = 0; d < 8; d++) {
-                    h4 col = {rows[0][d], rows[1][d], rows[2][d], rows[3][d]};
-                    *reinterpret_cast<h4 *>(Vt + (dg * 8 + d) * L::ldvt + kg * 4) = col;
+            for (int i = 0; i < KV; i++) {
+                const int v = threadIdx.x + i * nthr;
+                const int r = v / vec_per_row, c = v - r * vec_per_row;
+                *reinterpret_cast<h8 *>(Ks + r * L::ldk + c * 8) = kreg[i];
+            }
+#pragma unroll
+            for (int j = 0; j < VU; j++) {
+                const int u = threadIdx.x + j * nthr;
+                const int kg = u / dgroups, dg = u - kg * dgroups;
+                if (u < v_units) {
+#pragma unroll
+                    for (int d = 0; d < 8; d++) {
+                        h4 col = {vreg[j][0][d], vreg[j][1][d], vreg[j][2][d], vreg[j][3][d]};
+                        *reinterpret_cast<h4 *>(Vt + (dg * 8 + d) * L::ldvt + kg * 4) = col;
+                    }
                 }
             }
         }
@@ -258,9 +287,9 @@ __global__ __launch_bounds__(256) void mha_fused_kernel(const MhaArgs a) {
     }
 }
 
-template <int HD, bool COMPACT>
-static int launch_mha(const MhaArgs &args, int B, hipStream_t stream) {
-    auto kernel = mha_fused_kernel<HD, COMPACT>;
+template <int HD, bool COMPACT, int NW>
+static int launch_mha_nw(const MhaArgs &args, hipStream_t stream) {
+    auto kernel = mha_fused_kernel<HD, COMPACT, NW>;
     constexpr size_t lds = MhaLds<HD>::bytes;
     if (lds > 64 * 1024) {
         static bool raised = false;
@@ -270,13 +299,21 @@ static int launch_mha(const MhaArgs &args, int B, hipStream_t stream) {
             raised = true;
         }
     }
-    // 4 waves = 64 query rows per workgroup; 2 waves when that leaves a
-    // half-empty strip (S = 32, 96, ...).
-    const int qblocks = args.S / 16;
-    const int nwave = (qblocks % 4 == 0) ? 4 : (qblocks % 2 == 0 ? 2 : 1);
-    const dim3 grid((qblocks + nwave - 1) / nwave, args.nh, B);
-    kernel<<<grid, nwave * 64, lds, stream>>>(args);
+    const int qstrips = (args.S + 16 * NW - 1) / (16 * NW);
+    const int rounds = (args.nbh + kXcds - 1) / kXcds;
+    kernel<<<dim3((unsigned)(rounds * kXcds * qstrips)), 64 * NW, lds, stream>>>(args);
     return check_launch("mha_fused_kernel");
+}
+
+// 4 waves = 64 query rows per workgroup; 2 or 1 waves when that would leave a
+// half-empty strip (S = 32, 96, 16, ...).
+template <int HD, bool COMPACT>
+static int launch_mha(const MhaArgs &args, int B, hipStream_t stream) {
+    (void)B;
+    const int qblocks = args.S / 16;
+    if (qblocks % 4 == 0) return launch_mha_nw<HD, COMPACT, 4>(args, stream);
+    if (qblocks % 2 == 0) return launch_mha_nw<HD, COMPACT, 2>(args, stream);
+    return launch_mha_nw<HD, COMPACT, 1>(args, stream);
 }
 
 }  // namespace et
@@ -307,7 +344,7 @@ int et_mha_fused_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V, int ldq,
                  reinterpret_cast<uintptr_t>(V)) & 15) == 0 &&
                    (reinterpret_cast<uintptr_t>(Z) & 7) == 0,
                ET_ERR_UNSUPPORTED, "et_mha_fused_f16: operands must be 16-byte aligned");
-    ET_REQUIRE(B <= 65535 && nh <= 65535, ET_ERR_UNSUPPORTED, "et_mha_fused_f16: grid too large");
+    ET_REQUIRE((long long)B * nh * (S / 16) < (1LL << 30), ET_ERR_UNSUPPORTED, "et_mha_fused_f16: grid too large");
     if (B == 0) return ET_OK;
     MhaArgs args;
     args.Q = reinterpret_cast<const _Float16 *>(Q);
@@ -322,6 +359,7 @@ int et_mha_fused_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V, int ldq,
     args.ldz = ldz;
     args.S = S;
     args.nh = nh;
+    args.nbh = B * nh;
     args.scale_log2e = scale * kLog2e;
     args.causal = (flags & ET_MHA_CAUSAL) ? 1 : 0;
     args.v_col_id = nullptr;
@@ -351,7 +389,7 @@ int et_mha_compactv_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *Vc, int 
                "et_mha_compactv_f16: row strides too small");
     ET_REQUIRE(ldq % 8 == 0 && ldk % 8 == 0 && ldz % 4 == 0, ET_ERR_UNSUPPORTED,
                "et_mha_compactv_f16: row strides must keep 16-byte alignment");
-    ET_REQUIRE(B <= 65535 && nh <= 65535, ET_ERR_UNSUPPORTED, "et_mha_compactv_f16: grid too large");
+    ET_REQUIRE((long long)B * nh * (S / 16) < (1LL << 30), ET_ERR_UNSUPPORTED, "et_mha_compactv_f16: grid too large");
     if (B == 0) return ET_OK;
     MhaArgs args;
     args.Q = reinterpret_cast<const _Float16 *>(Q);
@@ -366,6 +404,7 @@ int et_mha_compactv_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *Vc, int 
     args.ldz = ldz;
     args.S = S;
     args.nh = nh;
+    args.nbh = B * nh;
     args.scale_log2e = scale * kLog2e;
     args.causal = (flags & ET_MHA_CAUSAL) ? 1 : 0;
     args.v_col_id = v_col_id;

@@ -42,6 +42,11 @@ struct BsrArgs {
     int T, in, out;
     int rows_per_wg;  // block-rows of W per workgroup
     int act;
+    // fused SkipLayerNorm prologue (LN kernels only): X = LN(ln_src + ln_skip)*gamma + beta is
+    // formed while the strip is staged; the workgroups of block-row group 0 also write it to ln_out
+    const _Float16 *ln_src, *ln_skip, *ln_gamma, *ln_beta;
+    _Float16 *ln_out;
+    float ln_eps;
 };
 
 constexpr int kXcds = 8;      // accelerator dies, each with a private L2
@@ -62,8 +67,9 @@ __device__ __forceinline__ int lane_read(int v, int lane) {
 
 // ACT is a template parameter: the epilogue carries no run-time branch and each
 // fused activation is a separately named kernel in a profile.
-template <int MT, bool STAGE, int ACT>
+template <int MT, bool STAGE, int ACT, int LN = 0>
 __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
+    static_assert(!LN || STAGE, "the fused LayerNorm prologue writes the strip to LDS");
     extern __shared__ __align__(16) unsigned char smem_raw[];
     _Float16 *xs = reinterpret_cast<_Float16 *>(smem_raw);
 
@@ -110,11 +116,40 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     const int total_vec = STAGE ? rows_here * vec_per_row : 0;
     const h8 *src = reinterpret_cast<const h8 *>(a.X + (size_t)tok0 * a.in);
     h8 sv[kStageU];
-    if (STAGE) {
+    if (STAGE && !LN) {
 #pragma unroll
         for (int u = 0; u < kStageU; u++) {
             const int idx = threadIdx.x + u * nthr;
             if (idx < total_vec) sv[u] = src[idx];
+        }
+    }
+    // Fused SkipLayerNorm: a wave normalises rows wave, wave+nwave, ... of the strip
+    // (at most kLnRows of them); all their loads are issued here, one round trip.
+    constexpr int kLnRows = LN ? MT * 16 / 8 : 1;        // rows per wave: LN kernels run 8 waves
+    constexpr int kLnNit = LN ? LN : 1;                  // 4-element chunks per lane (LN = ceil(in / 256))
+    uint2 ln_s[kLnRows][kLnNit], ln_k[kLnRows][kLnNit], ln_g[kLnNit], ln_b[kLnNit];
+    const int ln_chunks = a.in >> 2;
+    if (LN) {
+        // unconditional loads (indices past the row or the strip are clamped and the values
+        // selected away later): loads under a branch get a basic block of their own, where
+        // the compiler waits for each in turn instead of once for all
+#pragma unroll
+        for (int i = 0; i < kLnNit; i++) {
+            const int c = min(lane + 64 * i, ln_chunks - 1);
+            ln_g[i] = reinterpret_cast<const uint2 *>(a.ln_gamma)[c];
+            ln_b[i] = reinterpret_cast<const uint2 *>(a.ln_beta)[c];
+        }
+#pragma unroll
+        for (int rr = 0; rr < kLnRows; rr++) {
+            const int r = min(wave + 8 * rr, rows_here - 1);
+            const uint2 *ps = reinterpret_cast<const uint2 *>(a.ln_src + (size_t)(tok0 + r) * a.in);
+            const uint2 *pk = reinterpret_cast<const uint2 *>(a.ln_skip + (size_t)(tok0 + r) * a.in);
+#pragma unroll
+            for (int i = 0; i < kLnNit; i++) {
+                const int c = min(lane + 64 * i, ln_chunks - 1);
+                ln_s[rr][i] = ps[c];
+                ln_k[rr][i] = pk[c];
+            }
         }
     }
 
@@ -182,8 +217,66 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     issue_item(0);
     issue_item(1);
 
+    // ---- fused SkipLayerNorm: statistics in fp32 per row (wave64 butterflies), the
+    // normalised row goes to LDS as fp16 — the value a separate LayerNorm kernel would
+    // have stored — and, from block-row group 0, to ln_out
+    if (LN) {
+        auto unpack = [](uint2 raw, float (&f)[4]) {
+            const h2 lo = __builtin_bit_cast(h2, raw.x), hi = __builtin_bit_cast(h2, raw.y);
+            f[0] = (float)lo[0]; f[1] = (float)lo[1]; f[2] = (float)hi[0]; f[3] = (float)hi[1];
+        };
+        const float inv_h = 1.0f / (float)a.in;
+#pragma unroll
+        for (int rr = 0; rr < kLnRows; rr++) {
+            const int r = wave + 8 * rr;  // 8 waves: always inside the strip
+            const bool row_ok = r < rows_here;
+            float x[kLnNit][4];
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < kLnNit; i++) {
+                const bool ok = lane + 64 * i < ln_chunks;
+                float y[4];
+                unpack(ln_s[rr][i], x[i]);
+                unpack(ln_k[rr][i], y);
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    x[i][j] = ok ? x[i][j] + y[j] : 0.0f;
+                    sum += x[i][j];
+                }
+            }
+            const float mean = wave_sum(sum) * inv_h;
+            float sq = 0.0f;
+#pragma unroll
+            for (int i = 0; i < kLnNit; i++) {
+                const bool ok = lane + 64 * i < ln_chunks;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float d = ok ? x[i][j] - mean : 0.0f;
+                    sq += d * d;
+                }
+            }
+            const float rstd = rsqrtf(wave_sum(sq) * inv_h + a.ln_eps);
+#pragma unroll
+            for (int i = 0; i < kLnNit; i++) {
+                const int c = lane + 64 * i;
+                float gg[4], bb[4];
+                unpack(ln_g[i], gg);
+                unpack(ln_b[i], bb);
+                h4 o;
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    o[j] = row_ok ? (_Float16)((x[i][j] - mean) * rstd * gg[j] + bb[j]) : (_Float16)0;
+                if (c < ln_chunks) {
+                    *reinterpret_cast<h4 *>(xs + r * lds_ld + c * 4) = o;  // rows past T stay zero
+                    if (group == 0 && row_ok)
+                        *reinterpret_cast<h4 *>(a.ln_out + (size_t)(tok0 + r) * a.in + c * 4) = o;
+                }
+            }
+        }
+        __syncthreads();
+    }
     // ---- strip copy: write the first batch, then the rest
-    if (STAGE) {
+    if (STAGE && !LN) {
         const int dr = nthr / vec_per_row, dc = nthr - dr * vec_per_row;  // (row, col) step of +nthr
         int r = threadIdx.x / vec_per_row, c = threadIdx.x - r * vec_per_row;
 #pragma unroll
@@ -355,9 +448,30 @@ static BsrPlan plan_bsr(int T, int in, int out) {
     return best;
 }
 
-template <int MT, bool STAGE, int ACT>
+// Geometry of the kernels with the fused SkipLayerNorm prologue: 8 waves, staged strip.
+static BsrPlan plan_bsr_ln(int T, int in, int out) {
+    const size_t lds_cap = 160 * 1024;
+    const size_t row_bytes = (size_t)(in + kLdsPad) * sizeof(_Float16);
+    const int nbr = out / 16;
+    BsrPlan p{};
+    p.stage = 16 * row_bytes <= lds_cap;
+    p.mt = (T >= 32 && 32 * row_bytes <= lds_cap / 2) ? 2 : 1;
+    p.threads = 512;
+    const int nwave = 8;
+    const int strips = (T + p.mt * 16 - 1) / (p.mt * 16);
+    const int groups = strips >= 256 ? 1 : 256 / strips;
+    int rpw = (nbr + groups - 1) / groups;
+    rpw = ((rpw + nwave - 1) / nwave) * nwave;
+    if (rpw > nbr) rpw = nbr;
+    if (rpw > kMaxWaveRows * nwave) rpw = kMaxWaveRows * nwave;
+    p.rows_per_wg = rpw;
+    p.lds = bsr_lds_bytes(p.mt, p.stage, in, rpw);
+    return p;
+}
+
+template <int MT, bool STAGE, int ACT, int LN = 0>
 static int launch_bsr_act(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
-    auto kernel = bsr16_linear_kernel<MT, STAGE, ACT>;
+    auto kernel = bsr16_linear_kernel<MT, STAGE, ACT, LN>;
     if (p.lds > 64 * 1024) {
         static bool raised = false;  // per instantiation
         if (!raised) {
@@ -382,6 +496,28 @@ static int launch_bsr(const BsrArgs &args, const BsrPlan &p, hipStream_t stream)
         case ET_ACT_GELU: return launch_bsr_act<MT, STAGE, ET_ACT_GELU>(args, p, stream);
         default: return launch_bsr_act<MT, STAGE, ET_ACT_NONE>(args, p, stream);
     }
+}
+
+// fused SkipLayerNorm prologue: staged strips of 16 or 32 rows, 8 waves, in <= 1024
+template <int MT, int NIT>
+static int dispatch_bsr_ln_act(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
+    switch (args.act) {
+        case ET_ACT_RELU: return launch_bsr_act<MT, true, ET_ACT_RELU, NIT>(args, p, stream);
+        case ET_ACT_GELU: return launch_bsr_act<MT, true, ET_ACT_GELU, NIT>(args, p, stream);
+        default: return launch_bsr_act<MT, true, ET_ACT_NONE, NIT>(args, p, stream);
+    }
+}
+template <int MT>
+static int dispatch_bsr_ln_mt(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
+    switch ((args.in + 255) / 256) {  // 4-element chunks per lane
+        case 1: return dispatch_bsr_ln_act<MT, 1>(args, p, stream);
+        case 2: return dispatch_bsr_ln_act<MT, 2>(args, p, stream);
+        case 3: return dispatch_bsr_ln_act<MT, 3>(args, p, stream);
+        default: return dispatch_bsr_ln_act<MT, 4>(args, p, stream);
+    }
+}
+static int dispatch_bsr_ln(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
+    return p.mt == 2 ? dispatch_bsr_ln_mt<2>(args, p, stream) : dispatch_bsr_ln_mt<1>(args, p, stream);
 }
 
 static int dispatch_bsr(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
@@ -434,10 +570,49 @@ int et_linear_bsr16_f16(const int32_t *row_ptr, const int32_t *col_idx, const et
                  in,
                  out,
                  0,
-                 act};
+                 act,
+                 nullptr, nullptr, nullptr, nullptr, nullptr, 0.0f};
     BsrPlan p = plan_bsr(T, in, out);
     args.rows_per_wg = p.rows_per_wg;
     return dispatch_bsr(args, p, as_stream(stream));
+}
+
+int et_skipln_linear_bsr16_f16(const et_f16 *src, const et_f16 *skip, const et_f16 *gamma,
+                               const et_f16 *beta, float eps, et_f16 *ln_out, const int32_t *row_ptr,
+                               const int32_t *col_idx, const et_f16 *tiles, const et_f16 *bias, et_f16 *Y,
+                               int T, int in, int out, int act, et_stream stream) {
+    ET_REQUIRE(src && skip && gamma && beta && ln_out, ET_ERR_INVALID_ARG,
+               "et_skipln_linear_bsr16_f16: NULL pointer");
+    int s = bsr_check(row_ptr, col_idx, tiles, ln_out, Y, T, in, out, act);
+    if (s != ET_OK) return s;
+    if (T == 0) return ET_OK;
+    // the fused prologue keeps a row in registers as 4 chunks of 4 values per lane and needs a
+    // staged strip; otherwise the two operators run back to back
+    // (and must not normalise in place: every block-row group of a strip reads src and skip)
+    BsrPlan p = plan_bsr_ln(T, in, out);
+    if (in > 1024 || !p.stage || ln_out == src || ln_out == skip) {
+        s = et_skip_layernorm_f16(ln_out, src, skip, gamma, beta, T, in, eps, stream);
+        if (s != ET_OK) return s;
+        return et_linear_bsr16_f16(row_ptr, col_idx, tiles, bias, ln_out, Y, T, in, out, act, stream);
+    }
+    BsrArgs args{row_ptr,
+                 col_idx,
+                 reinterpret_cast<const _Float16 *>(tiles),
+                 reinterpret_cast<const _Float16 *>(bias),
+                 nullptr,
+                 reinterpret_cast<_Float16 *>(Y),
+                 T,
+                 in,
+                 out,
+                 p.rows_per_wg,
+                 act,
+                 reinterpret_cast<const _Float16 *>(src),
+                 reinterpret_cast<const _Float16 *>(skip),
+                 reinterpret_cast<const _Float16 *>(gamma),
+                 reinterpret_cast<const _Float16 *>(beta),
+                 reinterpret_cast<_Float16 *>(ln_out),
+                 eps};
+    return dispatch_bsr_ln(args, p, as_stream(stream));
 }
 
 // Tuning hook: same computation with an explicit launch geometry.  mt in
@@ -474,7 +649,8 @@ int et_linear_bsr16_f16_geom(const int32_t *row_ptr, const int32_t *col_idx, con
                  in,
                  out,
                  rows_per_wg,
-                 act};
+                 act,
+                 nullptr, nullptr, nullptr, nullptr, nullptr, 0.0f};
     return dispatch_bsr(args, p, as_stream(stream));
 }
 

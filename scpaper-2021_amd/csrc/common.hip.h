@@ -39,16 +39,35 @@ inline hipStream_t as_stream(et_stream s) { return reinterpret_cast<hipStream_t>
 int check_launch(const char *kernel);
 
 // ---- wave64 reductions ----------------------------------------------------
-// Butterfly over the 64 lanes of a wavefront: every lane ends with the total.
+// Every lane ends with the total.  All 64 lanes must be active.  The 16 lanes of a
+// DPP row are folded with cross-lane VALU operands (quad swaps, then row rotations
+// by 4 and 8), which never touch the LDS crossbar; the four row totals are then read
+// through scalar registers, in a fixed order, so the result is the same in every lane.
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+    const int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false);
+    return __builtin_bit_cast(float, r);
+}
+constexpr int kDppQuadXor1 = 0xB1;  // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;  // quad_perm:[2,3,0,1]
+constexpr int kDppRowRor4 = 0x124;  // row_ror:4
+constexpr int kDppRowRor8 = 0x128;  // row_ror:8
+
+__device__ __forceinline__ float lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
-    return v;
+    v += dpp_move<kDppQuadXor1>(v);
+    v += dpp_move<kDppQuadXor2>(v);
+    v += dpp_move<kDppRowRor4>(v);
+    v += dpp_move<kDppRowRor8>(v);
+    return (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
-    return v;
+    v = fmaxf(v, dpp_move<kDppQuadXor1>(v));
+    v = fmaxf(v, dpp_move<kDppQuadXor2>(v));
+    v = fmaxf(v, dpp_move<kDppRowRor4>(v));
+    v = fmaxf(v, dpp_move<kDppRowRor8>(v));
+    return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)), fmaxf(lane_value(v, 32), lane_value(v, 48)));
 }
 
 // tanh-form GELU, x*(0.5 + 0.5*tanh(x*(0.035677408*x^2 + 0.7978845608)))

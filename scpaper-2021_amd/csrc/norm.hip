@@ -42,24 +42,40 @@ __global__ __launch_bounds__(kWave *kRowsPerBlock) void layernorm_rows_kernel(
     const uint2 *s = reinterpret_cast<const uint2 *>(src + (size_t)row * H);
     const uint2 *k = SKIP ? reinterpret_cast<const uint2 *>(skip + (size_t)row * H) : nullptr;
 
+    // Every load of the row is issued before the first use, so src, skip, gamma and beta
+    // arrive in one round trip.  The loads are unconditional (a chunk index past the row is
+    // clamped onto the last chunk and its value ignored): loads under a branch end up in a
+    // basic block of their own, where the compiler waits for each of them in turn.
+    const uint2 *g = reinterpret_cast<const uint2 *>(gamma);
+    const uint2 *b = reinterpret_cast<const uint2 *>(beta);
+    uint2 rs[NIT], rk[NIT], rg[NIT], rb[NIT];
+#pragma unroll
+    for (int i = 0; i < NIT; i++) {
+        const int c = min(lane + kWave * i, chunks - 1);
+        rs[i] = s[c];
+        if (SKIP) rk[i] = k[c];
+        rg[i] = g[c];
+        rb[i] = b[c];
+    }
+
+    // values past the row are selected away, not branched around: a branch would give the
+    // compiler a block to sink the loads into
     float x[NIT][4];
     float sum = 0.0f;
 #pragma unroll
     for (int i = 0; i < NIT; i++) {
-        const int c = lane + kWave * i;
-        if (c < chunks) {
-            unpack4(s[c], x[i]);
-            if (SKIP) {
-                float y[4];
-                unpack4(k[c], y);
+        const bool ok = lane + kWave * i < chunks;
+        unpack4(rs[i], x[i]);
+        if (SKIP) {
+            float y[4];
+            unpack4(rk[i], y);
 #pragma unroll
-                for (int j = 0; j < 4; j++) x[i][j] += y[j];
-            }
+            for (int j = 0; j < 4; j++) x[i][j] += y[j];
+        }
 #pragma unroll
-            for (int j = 0; j < 4; j++) sum += x[i][j];
-        } else {
-#pragma unroll
-            for (int j = 0; j < 4; j++) x[i][j] = 0.0f;
+        for (int j = 0; j < 4; j++) {
+            x[i][j] = ok ? x[i][j] : 0.0f;
+            sum += x[i][j];
         }
     }
     const float inv_h = 1.0f / (float)H;
@@ -67,27 +83,23 @@ __global__ __launch_bounds__(kWave *kRowsPerBlock) void layernorm_rows_kernel(
     float sq = 0.0f;
 #pragma unroll
     for (int i = 0; i < NIT; i++) {
-        const int c = lane + kWave * i;
-        if (c < chunks) {
+        const bool ok = lane + kWave * i < chunks;
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const float d = x[i][j] - mean;
-                sq += d * d;
-            }
+        for (int j = 0; j < 4; j++) {
+            const float d = ok ? x[i][j] - mean : 0.0f;
+            sq += d * d;
         }
     }
     const float rstd = rsqrtf(wave_sum(sq) * inv_h + eps);
 
-    const uint2 *g = reinterpret_cast<const uint2 *>(gamma);
-    const uint2 *b = reinterpret_cast<const uint2 *>(beta);
     uint2 *o = reinterpret_cast<uint2 *>(out + (size_t)row * H);
 #pragma unroll
     for (int i = 0; i < NIT; i++) {
         const int c = lane + kWave * i;
         if (c < chunks) {
             float gg[4], bb[4], y[4];
-            unpack4(g[c], gg);
-            unpack4(b[c], bb);
+            unpack4(rg[i], gg);
+            unpack4(rb[i], bb);
 #pragma unroll
             for (int j = 0; j < 4; j++) y[j] = (x[i][j] - mean) * rstd * gg[j] + bb[j];
             o[c] = pack4(y);

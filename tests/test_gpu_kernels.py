@@ -195,6 +195,61 @@ def test_linear_bsr16_rejects_bad_args(et):
     assert f(d.ptr, d.ptr, d.ptr, None, d.ptr, d.ptr, 0, 64, 64, 0, None) == et.ET_OK  # empty batch
 
 
+@pytest.mark.parametrize("T,inp,out,sp,act", [(1024, 768, 3072, 0.8, 2), (1008, 768, 3072, 0.8, 2),
+                                               (48, 256, 512, 0.5, 1), (16, 1024, 256, 0.9, 0),
+                                               (64, 2048, 256, 0.9, 0), (128, 72 * 4, 160, 0.6, 2)])
+def test_skipln_linear_bsr16(et, T, inp, out, sp, act):
+    """SkipLayerNorm fused into the tile-sparse Linear: same values as the two operators
+    launched one after the other (in > 1024 takes that route inside the call)."""
+    if inp % 16:
+        pytest.skip("feature width must be a multiple of 16")
+    w = Hn.BsrWeight(out, inp, sp, seed=21, bias_std=0.05).upload(et)
+    src, skip = Hn.randn((T, inp), 22), Hn.randn((T, inp), 23)
+    gamma = (1 + Hn.randn((inp,), 24, 0.1, np.float32)).astype(np.float16)
+    beta = Hn.randn((inp,), 25, 0.1)
+    d_src, d_skip, d_g, d_b = up(et, src), up(et, skip), up(et, gamma), up(et, beta)
+    d_ln = et.DeviceBuffer.empty((T, inp), np.float16)
+    d_y = et.DeviceBuffer.empty((T, out), np.float16)
+    et.check(et.lib().et_skipln_linear_bsr16_f16(d_src.ptr, d_skip.ptr, d_g.ptr, d_b.ptr, 1e-5, d_ln.ptr,
+                                                 w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, w.d_bias.ptr,
+                                                 d_y.ptr, T, inp, out, act, None))
+    et.sync()
+    # the two separate operators
+    d_ln2 = et.DeviceBuffer.empty((T, inp), np.float16)
+    d_y2 = et.DeviceBuffer.empty((T, out), np.float16)
+    et.skip_layernorm(d_ln2, d_src, d_skip, d_g, d_b, T, inp, 1e-5)
+    w.forward(et, d_ln2, d_y2, T, act)
+    et.sync()
+    ln, ln2 = d_ln.numpy(), d_ln2.numpy()
+    # the normalised rows may differ by one fp16 rounding where fp32 contraction differs
+    assert Hn.max_abs(ln, ln2) <= 4e-3
+    want_ln = L.skip_layernorm(Hn.f32(src), Hn.f32(skip), Hn.f32(gamma), Hn.f32(beta), 1e-5, torch.float16)
+    assert Hn.max_abs(ln, want_ln.numpy()) <= 4e-3
+    # the Linear consumes exactly the rows it wrote: oracle on ln_out
+    want = L.linear(Hn.f32(ln), Hn.f32(w.dense), Hn.f32(w.bias), {0: None, 1: "relu", 2: "gelu"}[act],
+                    torch.float16)
+    assert Hn.max_abs(d_y.numpy(), want.numpy()) <= 5e-3
+    assert Hn.max_abs(d_y.numpy(), d_y2.numpy()) <= 2e-2
+
+
+def test_skipln_linear_bsr16_in_place_falls_back(et):
+    """ln_out aliasing src is legal: the call then runs the two operators back to back."""
+    T, inp, out = 64, 256, 256
+    w = Hn.BsrWeight(out, inp, 0.5, seed=31, bias_std=0.05).upload(et)
+    src, skip = Hn.randn((T, inp), 32), Hn.randn((T, inp), 33)
+    gamma, beta = np.ones(inp, np.float16), np.zeros(inp, np.float16)
+    d_src, d_skip, d_g, d_b = up(et, src), up(et, skip), up(et, gamma), up(et, beta)
+    d_y = et.DeviceBuffer.empty((T, out), np.float16)
+    et.check(et.lib().et_skipln_linear_bsr16_f16(d_src.ptr, d_skip.ptr, d_g.ptr, d_b.ptr, 1e-5, d_src.ptr,
+                                                 w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, w.d_bias.ptr,
+                                                 d_y.ptr, T, inp, out, 0, None))
+    et.sync()
+    want_ln = L.skip_layernorm(Hn.f32(src), Hn.f32(skip), Hn.f32(gamma), Hn.f32(beta), 1e-5, torch.float16)
+    assert Hn.max_abs(d_src.numpy(), want_ln.numpy()) <= 4e-3
+    want = L.linear(Hn.f32(d_src.numpy()), Hn.f32(w.dense), Hn.f32(w.bias), None, torch.float16)
+    assert Hn.max_abs(d_y.numpy(), want.numpy()) <= 5e-3
+
+
 @pytest.mark.parametrize("mt,stage,threads,rpw", [(1, 1, 256, 4), (2, 1, 128, 3), (4, 1, 512, 8),
                                                   (4, 0, 256, 5), (1, 0, 64, 1), (2, 0, 512, 48)])
 def test_linear_bsr16_every_geometry(et, mt, stage, threads, rpw):
