@@ -91,19 +91,29 @@ template <> class Linear<col_mat> {
     col_mat weight;
     et::DeviceBuffer<half> bias;
     int size;
+    mutable et::DeviceBuffer<half> gathered;  // [size x nnz_col] compact activations (the workspace of Linear/Linear.h:124)
 
     Linear(int _in_size, int _out_size, const col_mat &w, const half *b, int _size)
-        : in_size(_in_size), out_size(_out_size), weight(w), bias(b, (std::size_t)_out_size), size(_size) {}
+        : in_size(_in_size), out_size(_out_size), weight(w), bias(b, (std::size_t)_out_size), size(_size),
+          gathered((std::size_t)_size * weight.nnz_col) {}
     Linear(int _in_size, int _out_size, col_mat &&w, const half *b, int _size)
         : in_size(_in_size), out_size(_out_size), weight(std::move(w)), bias(b, (std::size_t)_out_size),
-          size(_size) {}
+          size(_size), gathered((std::size_t)_size * weight.nnz_col) {}
     void forward(half *output, const half *input, et::stream_t stream = nullptr) const {
         forward_act(output, input, ET_ACT_NONE, stream);
     }
+    // gather the surviving input features once, then one dense GEMM with the bias and the
+    // activation in its epilogue
     void forward_act(half *output, const half *input, int act, et::stream_t stream = nullptr) const {
-        etChk(et_linear_colpruned_f16(et::f16(weight.cols->get()), weight.col_id->get(), weight.nnz_col,
-                                      et::f16(bias.get()), et::f16(input), et::f16(output), size,
-                                      (int)in_size, (int)out_size, act, stream));
+        if (weight.nnz_col == 0 || size == 0) {
+            etChk(et_linear_colpruned_f16(et::f16(weight.cols->get()), weight.col_id->get(), weight.nnz_col,
+                                          et::f16(bias.get()), et::f16(input), et::f16(output), size,
+                                          (int)in_size, (int)out_size, act, stream));
+            return;
+        }
+        etChk(et_linear_colpruned_ws_f16(et::f16(weight.cols->get()), weight.col_id->get(), weight.nnz_col,
+                                         et::f16(bias.get()), et::f16(input), et::f16(output),
+                                         et::f16(gathered.get()), size, (int)in_size, (int)out_size, act, stream));
     }
 };
 

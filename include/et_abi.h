@@ -176,6 +176,21 @@ int et_linear_colpruned_f16(const et_f16 *cols, const int32_t *col_id,
                             et_f16 *Y, int T, int in, int out, int act,
                             et_stream stream);
 
+/* dst[T x nnz_col] = X[:, col_id]: the gather pass of the column-pruned Linear
+ * (Linear/SPMM_col.cu:25-39).  nnz_col % 8 == 0; dst and col_id 16-byte aligned. */
+int et_gather_cols_f16(et_f16 *dst, const et_f16 *X, const int32_t *col_id, int T,
+                       int in, int nnz_col, et_stream stream);
+
+/* et_linear_colpruned_f16 through a caller-owned workspace [T x nnz_col]: gather
+ * once, then a dense GEMM over the compact activations — the reference's own
+ * sequence (Linear/SPMM_col.cu:57-69).  The workspace-free call gathers inside
+ * the GEMM, once per output-column block, and is the slower of the two whenever
+ * out spans more than one block. */
+int et_linear_colpruned_ws_f16(const et_f16 *cols, const int32_t *col_id,
+                               int nnz_col, const et_f16 *bias, const et_f16 *X,
+                               et_f16 *Y, et_f16 *workspace, int T, int in,
+                               int out, int act, et_stream stream);
+
 /* 1x16 vector-sparse weight (mat1x16): for row-set r (16 output features) and
  * part p (16 input features) the surviving 1x16 vectors are idx in
  * [tile_idx[r*(in/16+1)+p], tile_idx[r*(in/16+1)+p+1]); row_idx[idx] % 16 is

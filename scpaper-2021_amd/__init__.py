@@ -64,6 +64,8 @@ _SIGNATURES = {
     "et_linear_bsr16_f16": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_linear_bsr16_f16_geom": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp),
     "et_skipln_linear_bsr16_f16": (_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_gather_cols_f16": (_vp, _vp, _vp, _i, _i, _i, _vp),
+    "et_linear_colpruned_ws_f16": (_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_linear_dense_f16": (_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_gemm_f16": (_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _ll, _ll, _ll, _vp),
     "et_linear_rowpruned_f16": (_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp),

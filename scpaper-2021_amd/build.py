@@ -76,7 +76,8 @@ def build_all(jobs: int | None = None, verbose: bool = True) -> Path:
 
 
 # C++ programs written against the class layer (include/et/*.h) and linked with the library.
-PROGRAMS = {ROOT / "tests" / "cpp" / "class_layer_cases.cpp": ROOT / "tests" / "cpp" / "bin" / "class_layer_cases"}
+PROGRAMS = {ROOT / "tests" / "cpp" / "class_layer_cases.cpp": ROOT / "tests" / "cpp" / "bin" / "class_layer_cases",
+            PKG / "programs" / "et_sweeps.cpp": PKG / "bin" / "et_sweeps"}
 
 
 def build_programs(verbose: bool = True) -> None:
@@ -84,8 +85,9 @@ def build_programs(verbose: bool = True) -> None:
         if not src.exists():
             continue
         exe.parent.mkdir(exist_ok=True)
+        rel = os.path.relpath(LIBDIR, exe.parent)  # the tree may be copied elsewhere: rpath relative to the program
         cmd = [HIPCC, *COMMON, "-x", "c++", str(src), "-L", str(LIBDIR), "-let_hip",
-               f"-Wl,-rpath,{LIBDIR}", "-Wl,-rpath,$ORIGIN/../../../scpaper-2021_amd/lib", "-o", str(exe)]
+               f"-Wl,-rpath,{LIBDIR}", f"-Wl,-rpath,$ORIGIN/{rel}", "-o", str(exe)]
         res = subprocess.run(cmd, capture_output=True, text=True)
         if res.returncode != 0:
             raise RuntimeError(f"program build failed: {' '.join(cmd)}\n{res.stderr}")

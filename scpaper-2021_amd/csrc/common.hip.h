@@ -73,10 +73,13 @@ __device__ __forceinline__ float wave_max(float v) {
 // tanh-form GELU, x*(0.5 + 0.5*tanh(x*(0.035677408*x^2 + 0.7978845608)))
 // (the form the reference evaluates, Encoder/Encoder.cu:25-37).
 __device__ __forceinline__ float gelu_tanh(float x) {
-    const float u = x * (0.035677408136f * x * x + 0.7978845608028654f);
-    // tanh(u) = 1 - 2/(exp(2u)+1); exp overflow to +inf gives 1, underflow gives -1.
-    const float t = 1.0f - 2.0f / (__expf(2.0f * u) + 1.0f);
-    return x * (0.5f + 0.5f * t);
+    // 0.5 + 0.5*tanh(u) = 1 - 1/(exp(2u) + 1), and exp(2u) = exp2(x*(c1*x^2 + c0)) with
+    // 2*log2(e) folded into the polynomial: one exp2, one reciprocal, four multiply-adds.
+    // exp2 overflow to +inf gives x, underflow to 0 gives 0.
+    constexpr float k2log2e = 2.8853900817779268f;
+    constexpr float c1 = 0.035677408136f * k2log2e, c0 = 0.7978845608028654f * k2log2e;
+    const float e = __builtin_amdgcn_exp2f(x * (c1 * x * x + c0));
+    return x - x * __builtin_amdgcn_rcpf(e + 1.0f);
 }
 
 __device__ __forceinline__ float apply_act(float x, int act) {

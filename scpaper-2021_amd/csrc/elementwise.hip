@@ -20,7 +20,21 @@ __global__ __launch_bounds__(256) void unary_kernel(_Float16 *__restrict__ out,
     const bool aligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
     size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
     if (aligned) {
-        for (size_t v = i; v < nvec; v += step) {
+        // four 16-byte loads in flight per lane before the first use
+        constexpr int kU = 4;
+        size_t v = i;
+        for (; v + (kU - 1) * step < nvec; v += kU * step) {
+            h8 x[kU];
+#pragma unroll
+            for (int u = 0; u < kU; u++) x[u] = reinterpret_cast<const h8 *>(in)[v + u * step];
+#pragma unroll
+            for (int u = 0; u < kU; u++) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) x[u][j] = (_Float16)unary<OP>((float)x[u][j]);
+                reinterpret_cast<h8 *>(out)[v + u * step] = x[u];
+            }
+        }
+        for (; v < nvec; v += step) {
             h8 x = reinterpret_cast<const h8 *>(in)[v];
 #pragma unroll
             for (int j = 0; j < 8; j++) x[j] = (_Float16)unary<OP>((float)x[j]);

@@ -209,6 +209,29 @@ static int check_gemm_shape(const char *fn, int M, int N, int K) {
 static inline const _Float16 *H(const et_f16 *p) { return reinterpret_cast<const _Float16 *>(p); }
 static inline _Float16 *H(et_f16 *p) { return reinterpret_cast<_Float16 *>(p); }
 
+// Column gather: dst[t][j] = X[t][col_id[j]], 8 gathered columns per lane (two 16-byte
+// index loads, eight 2-byte reads inside one row of X, one 16-byte store) — the
+// gather pass of the column-pruned Linear (Linear/SPMM_col.cu:25-39).
+__global__ __launch_bounds__(256) void gather_cols_kernel(_Float16 *__restrict__ dst,
+                                                          const _Float16 *__restrict__ X,
+                                                          const int32_t *__restrict__ col_id, int T,
+                                                          int in, int nnz) {
+    const int per_row = nnz >> 3;
+    const size_t total = (size_t)T * per_row;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (size_t v = blockIdx.x * (size_t)blockDim.x + threadIdx.x; v < total; v += step) {
+        const size_t t = v / per_row;
+        const int c = (int)(v - t * per_row) * 8;
+        const int4 i0 = *reinterpret_cast<const int4 *>(col_id + c);
+        const int4 i1 = *reinterpret_cast<const int4 *>(col_id + c + 4);
+        const _Float16 *row = X + t * (size_t)in;
+        h8 o;
+        o[0] = row[i0.x]; o[1] = row[i0.y]; o[2] = row[i0.z]; o[3] = row[i0.w];
+        o[4] = row[i1.x]; o[5] = row[i1.y]; o[6] = row[i1.z]; o[7] = row[i1.w];
+        *reinterpret_cast<h8 *>(dst + t * (size_t)nnz + c) = o;
+    }
+}
+
 }  // namespace et
 
 using namespace et;
@@ -336,6 +359,37 @@ int et_linear_colpruned_f16(const et_f16 *cols, const int32_t *col_id, int nnz_c
     g.a_gather = col_id;
     g.act = act;
     return launch_gemm(g, 1, true, st);
+}
+
+int et_gather_cols_f16(et_f16 *dst, const et_f16 *X, const int32_t *col_id, int T, int in, int nnz_col,
+                       et_stream stream) {
+    ET_REQUIRE(dst && X && col_id, ET_ERR_INVALID_ARG, "et_gather_cols_f16: NULL pointer");
+    ET_REQUIRE(T >= 0 && in > 0 && nnz_col >= 0, ET_ERR_INVALID_ARG, "et_gather_cols_f16: T=%d in=%d nnz_col=%d", T,
+               in, nnz_col);
+    ET_REQUIRE(nnz_col % 8 == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0 &&
+                   (reinterpret_cast<uintptr_t>(col_id) & 15) == 0,
+               ET_ERR_UNSUPPORTED, "et_gather_cols_f16: nnz_col=%d must be a multiple of 8, dst and col_id 16-byte aligned",
+               nnz_col);
+    const size_t total = (size_t)T * (nnz_col / 8);
+    if (total == 0) return ET_OK;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    gather_cols_kernel<<<(unsigned)blocks, 256, 0, as_stream(stream)>>>(H(dst), H(X), col_id, T, in, nnz_col);
+    return check_launch("gather_cols_kernel");
+}
+
+int et_linear_colpruned_ws_f16(const et_f16 *cols, const int32_t *col_id, int nnz_col, const et_f16 *bias,
+                               const et_f16 *X, et_f16 *Y, et_f16 *workspace, int T, int in, int out, int act,
+                               et_stream stream) {
+    ET_REQUIRE(workspace != nullptr, ET_ERR_INVALID_ARG, "et_linear_colpruned_ws_f16: workspace is NULL");
+    if (nnz_col == 0 || T == 0)  // nothing to gather: bias and activation alone
+        return et_linear_colpruned_f16(cols, col_id, nnz_col, bias, X, Y, T, in, out, act, stream);
+    ET_REQUIRE(cols && col_id && X && Y, ET_ERR_INVALID_ARG, "et_linear_colpruned_ws_f16: NULL pointer");
+    ET_REQUIRE(nnz_col > 0 && nnz_col <= in, ET_ERR_INVALID_ARG, "et_linear_colpruned_ws_f16: nnz_col=%d in=%d",
+               nnz_col, in);
+    int s = et_gather_cols_f16(workspace, X, col_id, T, in, nnz_col, stream);
+    if (s != ET_OK) return s;
+    return et_linear_dense_f16(cols, bias, workspace, Y, T, nnz_col, out, act, stream);
 }
 
 }  // extern "C"

@@ -1,0 +1,216 @@
+#!/usr/bin/env python3
+"""Per-kernel throughput against the roofline that bounds it, through the C ABI.
+
+    python scpaper-2021_amd/kernel_bench.py [--set configs|scale|all] [--json FILE]
+
+`configs` are the shapes of the benchmark configurations (attention block at batch
+1/4/16, the tile/row/column-pruned Linears at 2048 token rows, the BERT-large-shaped
+layer); `scale` are shapes large enough that launch latency no longer matters, which
+is where a kernel's fraction of the machine peak means something.  Every kernel is
+recorded N times into one HIP graph and the graph is replayed between two HIP events
+on its stream, so the figure is device time per launch.
+
+Work counted is ALGORITHMIC: 2*256*ntile*T flops for a tile-sparse Linear,
+2*T*in*out for a dense one, 4*S*S*hd*nh*B for the attention core, and the bytes a
+normalisation or activation must move (inputs read once, output written once).
+Peaks: 2500 TFLOP/s dense fp16 matrix rate, 8 TB/s HBM (vendor figures, MI355X).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import sys
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent.parent
+sys.path.insert(0, str(ROOT))
+
+import __graft_entry__ as entry  # noqa: E402
+
+MFMA_PEAK_TFLOPS = 2500.0
+HBM_PEAK_TBS = 8.0
+
+
+class Bench:
+    def __init__(self):
+        self.et = entry.load_package()
+        self.lib = self.et.lib()
+        self.stream = C.c_void_p()
+        self.et.check(self.lib.et_stream_create(C.byref(self.stream)))
+        self.rng = np.random.default_rng(0)
+        self.rows = []
+
+    def rnd(self, shape, std=1.0):
+        return (self.rng.standard_normal(shape, dtype=np.float32) * std).astype(np.float16)
+
+    def dev(self, a):
+        return self.et.DeviceBuffer.from_numpy(a)
+
+    def empty(self, shape):
+        return self.et.DeviceBuffer.empty(shape, np.float16)
+
+    def time_us(self, fn, launches, replays=3):
+        et, lib, s = self.et, self.lib, self.stream
+        fn()
+        et.check(lib.et_stream_sync(s))
+        et.check(lib.et_graph_begin_capture(s))
+        for _ in range(launches):
+            fn()
+        g = C.c_void_p()
+        et.check(lib.et_graph_end_capture(s, C.byref(g)))
+        et.check(lib.et_graph_launch(g, s))
+        et.check(lib.et_stream_sync(s))
+        with et.Timer(s) as t:
+            for _ in range(replays):
+                et.check(lib.et_graph_launch(g, s))
+        et.check(lib.et_graph_destroy(g))
+        return t.ms * 1e3 / (launches * replays)
+
+    def record(self, kernel, shape, us, work, bound):
+        if bound == "mfma":
+            achieved, peak, unit = work / us / 1e6, MFMA_PEAK_TFLOPS, "TFLOP/s"
+        else:
+            achieved, peak, unit = work / us / 1e6, HBM_PEAK_TBS, "TB/s"
+        row = {"kernel": kernel, "shape": shape, "us": round(us, 2), "bound": bound,
+               "achieved": round(achieved, 2), "peak": peak, "unit": unit, "frac": round(achieved / peak, 4)}
+        self.rows.append(row)
+        print(f"{kernel:<22} {shape:<44} {us:10.1f} us  {achieved:8.2f} {unit:<8} {100 * achieved / peak:5.1f} % of {bound} peak",
+              flush=True)
+
+    # ---- kernels -------------------------------------------------------------------
+    def layernorm(self, rows, H, launches):
+        et = self.et
+        a, b, o = self.dev(self.rnd((rows, H))), self.dev(self.rnd((rows, H))), self.empty((rows, H))
+        g = self.dev(np.ones(H, np.float16))
+        us = self.time_us(lambda: et.skip_layernorm(o, a, b, g, g, rows, H, 1e-5, self.stream), launches)
+        self.record("skip_layernorm", f"{rows} x {H}", us, 3 * rows * H * 2 + 4 * H, "hbm")
+        us = self.time_us(lambda: et.layernorm(o, a, g, g, rows, H, 1e-5, self.stream), launches)
+        self.record("layernorm", f"{rows} x {H}", us, 2 * rows * H * 2 + 4 * H, "hbm")
+
+    def gelu(self, n, launches):
+        a, o = self.dev(self.rnd((n,))), self.empty((n,))
+        us = self.time_us(lambda: self.et.check(self.lib.et_gelu_f16(o.ptr, a.ptr, n, self.stream)), launches)
+        self.record("gelu", f"{n} values", us, 2 * n * 2, "hbm")
+
+    def mha(self, B, S, nh, hd, launches, lens=None):
+        et = self.et
+        H = nh * hd
+        qkv, z = self.dev(self.rnd((B * S, 3 * H))), self.empty((B * S, H))
+        d_lens = self.dev(np.asarray(lens, np.int32)) if lens is not None else None
+        us = self.time_us(lambda: et.mha_fused(qkv.ptr, qkv.offset(2 * H), qkv.offset(4 * H), 3 * H, 3 * H, 3 * H,
+                                               z, H, None, d_lens, B, S, nh, hd, hd ** -0.5, 0, self.stream), launches)
+        pairs = B * S * S if lens is None else int(sum(int(n) * int(n) for n in lens))
+        tag = "" if lens is None else " padded"
+        self.record("mha_fused", f"B{B} S{S} nh{nh} hd{hd}{tag}", us, 4 * pairs * hd * nh, "mfma")
+
+    def dense(self, T, n_in, n_out, launches):
+        et = self.et
+        W, x, y = self.dev(self.rnd((n_out, n_in), 0.02)), self.dev(self.rnd((T, n_in))), self.empty((T, n_out))
+        us = self.time_us(lambda: et.linear_dense(W, None, x, y, T, n_in, n_out, 0, self.stream), launches)
+        self.record("linear_dense", f"T{T} in{n_in} out{n_out}", us, 2 * T * n_in * n_out, "mfma")
+
+    def tile_pattern(self, n_out, n_in, sparsity, seed):
+        """Seeded random tile structure from the library's own generator."""
+        total = (n_out // 16) * (n_in // 16)
+        row_ptr = np.zeros(n_out // 16 + 1, np.int32)
+        col = np.zeros(max(total, 1), np.int32)
+        ntile = C.c_int()
+        self.et.check(self.lib.et_fmt_tile_pattern(n_out, n_in, sparsity, seed, row_ptr.ctypes.data, col.ctypes.data,
+                                                   C.byref(ntile)))
+        return row_ptr, col[:max(ntile.value, 1)].copy(), ntile.value
+
+    def ids(self, fn, n, sparsity, seed):
+        out = np.zeros(n + 16, np.int32)
+        count = C.c_int()
+        self.et.check(fn(n, sparsity, seed, out.ctypes.data, C.byref(count)))
+        return out[:count.value].copy()
+
+    def bsr(self, T, n_in, n_out, sparsity, launches):
+        et = self.et
+        row_ptr, col, ntile = self.tile_pattern(n_out, n_in, sparsity, 5)
+        d_rp, d_col = self.dev(row_ptr), self.dev(col)
+        tiles = self.dev(self.rnd((max(ntile, 1), 256), 0.02))
+        bias = self.dev(np.zeros(n_out, np.float16))
+        x, y = self.dev(self.rnd((T, n_in))), self.empty((T, n_out))
+        us = self.time_us(lambda: et.linear_bsr16(d_rp, d_col, tiles, bias, x, y, T, n_in, n_out, 0, self.stream),
+                          launches)
+        self.record("linear_bsr16", f"T{T} in{n_in} out{n_out} sparsity {sparsity}", us, 2 * 256 * ntile * T, "mfma")
+
+    def rowcol(self, T, n_in, n_out, sparsity, launches):
+        et, lib = self.et, self.lib
+        row_id = self.ids(lib.et_fmt_row_ids, n_out, sparsity, 7)
+        rows = self.dev(self.rnd((len(row_id), n_in), 0.02))
+        d_ids = self.dev(np.asarray(row_id, np.int32))
+        bias = self.dev(np.zeros(n_out, np.float16))
+        x, y = self.dev(self.rnd((T, n_in))), self.empty((T, n_out))
+        us = self.time_us(lambda: et.check(lib.et_linear_rowpruned_f16(rows.ptr, d_ids.ptr, len(row_id), bias.ptr,
+                                                                      x.ptr, y.ptr, T, n_in, n_out, 0, self.stream)),
+                          launches)
+        self.record("linear_rowpruned", f"T{T} in{n_in} out{n_out} sparsity {sparsity}", us,
+                    2 * T * n_in * len(row_id), "mfma")
+        col_id = self.ids(lib.et_fmt_col_ids, n_in, sparsity, 8)
+        cols = self.dev(self.rnd((n_out, len(col_id)), 0.02))
+        d_cid = self.dev(np.asarray(col_id, np.int32))
+        ws = self.empty((T, len(col_id)))  # gather once, then a dense GEMM over the compact activations
+        us = self.time_us(lambda: et.check(lib.et_linear_colpruned_ws_f16(cols.ptr, d_cid.ptr, len(col_id), bias.ptr,
+                                                                         x.ptr, y.ptr, ws.ptr, T, n_in, n_out, 0,
+                                                                         self.stream)), launches)
+        self.record("linear_colpruned", f"T{T} in{n_in} out{n_out} sparsity {sparsity}", us,
+                    2 * T * len(col_id) * n_out, "mfma")
+
+
+def run_configs(b: Bench):
+    rng = np.random.default_rng(1)
+    for B in (1, 4, 16):  # attention block, right padding with lengths in [64, 128]
+        b.mha(B, 128, 12, 64, 50)
+        b.mha(B, 128, 12, 64, 50, lens=rng.integers(64, 129, B))
+    for n_in, n_out in ((768, 768), (768, 3072), (3072, 768)):  # pruned Linears at 2048 token rows
+        for sp in (0.8, 0.9):
+            b.bsr(2048, n_in, n_out, sp, 50)
+        b.rowcol(2048, n_in, n_out, 0.5, 20)
+        b.dense(2048, n_in, n_out, 20)
+    b.layernorm(1024, 768, 50)   # the 12-layer workload's SkipLayerNorm
+    b.layernorm(2048, 1024, 50)  # BERT-large-shaped layer
+    b.mha(4, 512, 16, 64, 20)
+    b.mha(4, 512, 16, 64, 20, lens=rng.integers(256, 513, 4))
+    for n_in, n_out in ((1024, 1024), (1024, 3072), (1024, 4096), (4096, 1024)):
+        b.bsr(2048, n_in, n_out, 0.9, 50)
+
+
+def run_scale(b: Bench):
+    b.layernorm(65536, 768, 10)
+    b.layernorm(131072, 1024, 10)
+    b.gelu(128 * 1024 * 1024, 10)
+    b.mha(64, 512, 16, 64, 10)
+    b.mha(16, 2048, 16, 64, 5)
+    b.mha(16, 2048, 8, 128, 5)
+    b.dense(8192, 4096, 4096, 5)
+    b.dense(16384, 8192, 8192, 3)
+    b.bsr(16384, 768, 3072, 0.8, 10)
+    b.bsr(16384, 3072, 768, 0.8, 10)
+    b.bsr(16384, 4096, 4096, 0.5, 3)
+    b.rowcol(16384, 4096, 4096, 0.5, 3)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--set", choices=("configs", "scale", "all"), default="all")
+    ap.add_argument("--json", default=None, help="also write the rows as JSON to this file")
+    args = ap.parse_args()
+    b = Bench()
+    print(json.dumps(b.et.device_info()))
+    if args.set in ("configs", "all"):
+        print("# shapes of the benchmark configurations")
+        run_configs(b)
+    if args.set in ("scale", "all"):
+        print("# shapes where launch latency no longer matters")
+        run_scale(b)
+    if args.json:
+        Path(args.json).write_text(json.dumps(b.rows, indent=1))
+
+
+if __name__ == "__main__":
+    main()

@@ -102,6 +102,13 @@ def test_linear_colpruned(et, T, inp, out, sp, act):
     # same result as the masked dense weight
     Wd = F.col_mat_to_dense(cols, col_id, inp)
     assert Hn.max_abs(want, L.linear(Hn.f32(x), Hn.f32(Wd), Hn.f32(b), ACT[act], torch.float16).numpy()) <= 2e-3
+    # the workspace form: the gather is bit-exact, the Linear agrees with the oracle
+    d_ws = et.DeviceBuffer.empty((T, len(col_id)), np.float16)
+    d_y2 = et.DeviceBuffer.empty((T, out), np.float16)
+    et.check(et.lib().et_linear_colpruned_ws_f16(up(et, cols).ptr, up(et, col_id).ptr, len(col_id), up(et, b).ptr,
+                                                 up(et, x).ptr, d_y2.ptr, d_ws.ptr, T, inp, out, act, None))
+    assert np.array_equal(d_ws.numpy(), x[:, col_id])
+    assert Hn.max_abs(d_y2.numpy(), want) <= 4e-3
 
 
 @pytest.mark.parametrize("T,inp,out,sp,act", [(2048, 768, 768, 0.8, 0), (128, 768, 3072, 0.5, 2), (16, 32, 16, 0.0, 0),
