@@ -319,6 +319,31 @@ int et_bias_add_f16(et_f16 *data, const et_f16 *bias, int rows, int cols,
                     et_stream stream);
 
 /* ------------------------------------------------------------------------
+ * binary32 twins.  Same contracts as the _f16 functions of the same name with
+ * every pointer a float pointer; values are stored, multiplied and accumulated
+ * in binary32 (MFMA 16x16x4 f32 in the Linear).  They are the verification
+ * path for dense fp32 models — an encoder layer built from them agrees with a
+ * CPU fp32 forward to max-abs 1e-4 — and have no counterpart in the reference,
+ * whose kernels are binary16 only (Linear/Linear.h:9, lib/mma.hpp:6-13).
+ * et_linear_dense_f32: in % 16 == 0, out % 4 == 0, any T.
+ * et_mha_fused_f32: S % 16 == 0, hd in {32, 64, 128}, 16*S floats of scores
+ * must fit on chip (S <= 2048); mask is a float [S x S] matrix.
+ * ------------------------------------------------------------------------ */
+int et_linear_dense_f32(const float *W, const float *bias, const float *X, float *Y,
+                        int T, int in, int out, int act, et_stream stream);
+int et_mha_fused_f32(const float *Q, const float *K, const float *V, int ldq, int ldk,
+                     int ldv, float *Z, int ldz, const float *mask,
+                     const int32_t *lens, int B, int S, int nh, int hd, float scale,
+                     int flags, et_stream stream);
+int et_skip_layernorm_f32(float *out, const float *src, const float *skip,
+                          const float *gamma, const float *beta, int rows, int H,
+                          float eps, et_stream stream);
+int et_layernorm_f32(float *out, const float *src, const float *gamma,
+                     const float *beta, int rows, int H, float eps, et_stream stream);
+int et_gelu_f32(float *out, const float *in, size_t n, et_stream stream);
+int et_relu_f32(float *out, const float *in, size_t n, et_stream stream);
+
+/* ------------------------------------------------------------------------
  * Encoder stack: nlayer post-LN encoder layers, layer i feeding layer i+1,
  *   a = Attn(x); y1 = SkipLN1(a, x); f = L2(act(L1(y1))); out = SkipLN2(f, y1)
  * assembled from host weights and run as ONE HIP-graph replay per forward.

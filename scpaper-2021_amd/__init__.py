@@ -64,6 +64,12 @@ _SIGNATURES = {
     "et_linear_bsr16_f16": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_linear_bsr16_f16_geom": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp),
     "et_skipln_linear_bsr16_f16": (_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_linear_dense_f32": (_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_mha_fused_f32": (_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp),
+    "et_skip_layernorm_f32": (_vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp),
+    "et_layernorm_f32": (_vp, _vp, _vp, _vp, _i, _i, _f, _vp),
+    "et_gelu_f32": (_vp, _vp, _sz, _vp),
+    "et_relu_f32": (_vp, _vp, _sz, _vp),
     "et_gather_cols_f16": (_vp, _vp, _vp, _i, _i, _i, _vp),
     "et_linear_colpruned_ws_f16": (_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_linear_dense_f16": (_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),

@@ -1,0 +1,281 @@
+// fp32 twins of the dense Linear and the fused attention: every value is stored,
+// multiplied and accumulated in binary32 (MFMA 16x16x4 f32 for the Linear, vector
+// FMA for the attention core), so an encoder layer built from them agrees with a
+// CPU fp32 forward to ~1e-5.  This is the verification path for dense fp32 models
+// (the reference is fp16-only, Linear/Linear.h:9); the production path is fp16.
+#include "common.hip.h"
+
+namespace et {
+
+// ---- dense Linear ---------------------------------------------------------------
+// Y[T x out] = act(X[T x in] * W^T + b), W [out x in] row-major.  One workgroup of
+// 4 waves computes a 64-token x 64-feature block; wave (wr, wc) owns tokens
+// 32*wr.. and features 32*wc.. as 2x2 MFMA tiles.  The MFMA A operand is W and the B
+// operand is X, so a lane ends with 4 consecutive output features of one token
+// (one 16-byte store).
+constexpr int kF32Tile = 64;
+constexpr int kF32K = 16;       // k-values staged per step
+constexpr int kF32Ld = kF32K + 1;  // LDS row stride in floats (odd: conflict-free column reads)
+
+template <int ACT>
+__global__ __launch_bounds__(256) void linear_dense_f32_kernel(const float *__restrict__ W,
+                                                               const float *__restrict__ bias,
+                                                               const float *__restrict__ X,
+                                                               float *__restrict__ Y, int T, int in,
+                                                               int out) {
+    __shared__ float xs[kF32Tile * kF32Ld];
+    __shared__ float ws[kF32Tile * kF32Ld];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wr = wave >> 1, wc = wave & 1;
+    const int tok0 = blockIdx.y * kF32Tile, f0 = blockIdx.x * kF32Tile;
+    const int r16 = lane & 15, kq = lane >> 4;
+
+    // staging: thread -> (row 0..63, 4 consecutive k)
+    const int srow = threadIdx.x >> 2, sk = (threadIdx.x & 3) << 2;
+    const bool x_ok = tok0 + srow < T, w_ok = f0 + srow < out;
+    const float *xp = X + (size_t)(tok0 + (x_ok ? srow : 0)) * in + sk;
+    const float *wp = W + (size_t)(f0 + (w_ok ? srow : 0)) * in + sk;
+
+    f4 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) acc[i][j] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    for (int k0 = 0; k0 < in; k0 += kF32K) {
+        float4 xv = *reinterpret_cast<const float4 *>(xp + k0);
+        float4 wv = *reinterpret_cast<const float4 *>(wp + k0);
+        if (!x_ok) xv = float4{0.0f, 0.0f, 0.0f, 0.0f};
+        if (!w_ok) wv = float4{0.0f, 0.0f, 0.0f, 0.0f};
+        __syncthreads();  // the previous step's reads are done
+        float *xd = xs + srow * kF32Ld + sk, *wd = ws + srow * kF32Ld + sk;
+        xd[0] = xv.x; xd[1] = xv.y; xd[2] = xv.z; xd[3] = xv.w;
+        wd[0] = wv.x; wd[1] = wv.y; wd[2] = wv.z; wd[3] = wv.w;
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < kF32K; kk += 4) {
+            float a[2], b[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                a[i] = ws[(wc * 32 + i * 16 + r16) * kF32Ld + kk + kq];  // A[m = feature][k]
+                b[i] = xs[(wr * 32 + i * 16 + r16) * kF32Ld + kk + kq];  // B[k][n = token]
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j], b[i], acc[i][j], 0, 0, 0);
+        }
+    }
+    // acc[i][j]: token tok0 + 32*wr + 16*i + r16, features f0 + 32*wc + 16*j + 4*kq .. +3
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int t = tok0 + wr * 32 + i * 16 + r16;
+        if (t >= T) continue;
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int f = f0 + wc * 32 + j * 16 + kq * 4;
+            if (f >= out) continue;  // out % 4 == 0: a group of 4 is inside or outside
+            float4 o;
+            float *po = reinterpret_cast<float *>(&o);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float v = acc[i][j][e] + (bias ? bias[f + e] : 0.0f);
+                if (ACT == ET_ACT_RELU) v = v > 0.0f ? v : 0.0f;
+                if (ACT == ET_ACT_GELU) v = gelu_tanh(v);
+                po[e] = v;
+            }
+            *reinterpret_cast<float4 *>(Y + (size_t)t * out + f) = o;
+        }
+    }
+}
+
+// ---- fused attention ------------------------------------------------------------
+// One workgroup = 16 queries of one head of one sequence.  The 16 x S strip of scores
+// lives in LDS as fp32; K and V pass through LDS in blocks of 64 keys.  Thread
+// (q = tid/16, c = tid%16) owns scores of keys c, c+16, .. of query q and output
+// features c, c+16, .. of query q.
+constexpr int kAttQ = 16;
+constexpr int kAttKeys = 64;
+
+struct MhaF32Args {
+    const float *Q, *K, *V;
+    float *Z;
+    const float *mask;
+    const int32_t *lens;
+    int ldq, ldk, ldv, ldz;
+    int B, S, nh, hd;
+    float scale;
+    int causal;
+};
+
+template <int HD>
+__global__ __launch_bounds__(256) void mha_fused_f32_kernel(const MhaF32Args a) {
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    float *qs = reinterpret_cast<float *>(smem_raw);  // [16][HD]
+    float *kv = qs + kAttQ * HD;                       // [64][HD + 1]
+    float *sc = kv + kAttKeys * (HD + 1);              // [16][S]
+    const int q0 = blockIdx.x * kAttQ, h = blockIdx.y, b = blockIdx.z;
+    const int q = threadIdx.x >> 4, c = threadIdx.x & 15;
+    const int len = a.lens ? min(max(a.lens[b], 0), a.S) : a.S;
+    const size_t row0 = (size_t)b * a.S;
+    constexpr int kF = HD / 16;  // output features per thread
+
+    float *zrow = a.Z + (row0 + q0 + q) * a.ldz + h * HD;
+    if (len == 0) {  // a sequence without keys: zeros
+#pragma unroll
+        for (int i = 0; i < kF; i++) zrow[c + 16 * i] = 0.0f;
+        return;
+    }
+    for (int i = threadIdx.x; i < kAttQ * HD; i += 256) {
+        const int r = i / HD, d = i - r * HD;
+        qs[i] = a.Q[(row0 + q0 + r) * a.ldq + h * HD + d] * a.scale;
+    }
+    // keys this block of queries can see
+    int kend = len;
+    if (a.causal) kend = min(kend, q0 + kAttQ);
+    const float ninf = -__builtin_inff();
+
+    // ---- scores
+    for (int kb = 0; kb < kend; kb += kAttKeys) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < kAttKeys * HD; i += 256) {
+            const int r = i / HD, d = i - r * HD;
+            kv[r * (HD + 1) + d] = kb + r < kend ? a.K[(row0 + kb + r) * a.ldk + h * HD + d] : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < kAttKeys / 16; i++) {
+            const int kl = c + 16 * i, key = kb + kl;
+            if (key >= kend) continue;
+            float s = 0.0f;
+#pragma unroll 8
+            for (int d = 0; d < HD; d++) s += qs[q * HD + d] * kv[kl * (HD + 1) + d];
+            if (a.mask) s += a.mask[(size_t)(q0 + q) * a.S + key];
+            if (a.causal && key > q0 + q) s = ninf;
+            sc[q * a.S + key] = s;
+        }
+    }
+    __syncthreads();
+    // ---- softmax over keys [0, kend) of row q: 16 threads per row
+    float m = ninf;
+    for (int k = c; k < kend; k += 16) m = fmaxf(m, sc[q * a.S + k]);
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 16));
+    float l = 0.0f;
+    for (int k = c; k < kend; k += 16) {
+        const float p = m == ninf ? 0.0f : __expf(sc[q * a.S + k] - m);
+        sc[q * a.S + k] = p;
+        l += p;
+    }
+#pragma unroll
+    for (int off = 8; off >= 1; off >>= 1) l += __shfl_xor(l, off, 16);
+
+    // ---- Z = P V
+    float acc[kF];
+#pragma unroll
+    for (int i = 0; i < kF; i++) acc[i] = 0.0f;
+    for (int kb = 0; kb < kend; kb += kAttKeys) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < kAttKeys * HD; i += 256) {
+            const int r = i / HD, d = i - r * HD;
+            kv[r * (HD + 1) + d] = kb + r < kend ? a.V[(row0 + kb + r) * a.ldv + h * HD + d] : 0.0f;
+        }
+        __syncthreads();
+        const int nk = min(kAttKeys, kend - kb);
+        for (int k = 0; k < nk; k++) {
+            const float p = sc[q * a.S + kb + k];
+#pragma unroll
+            for (int i = 0; i < kF; i++) acc[i] += p * kv[k * (HD + 1) + c + 16 * i];
+        }
+    }
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+#pragma unroll
+    for (int i = 0; i < kF; i++) zrow[c + 16 * i] = acc[i] * inv;
+}
+
+template <int OP>
+__global__ __launch_bounds__(256) void unary_f32_kernel(float *__restrict__ out, const float *__restrict__ in,
+                                                        size_t n) {
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += step) {
+        const float x = in[i];
+        out[i] = OP == 0 ? gelu_tanh(x) : (x > 0.0f ? x : 0.0f);
+    }
+}
+
+}  // namespace et
+
+using namespace et;
+
+extern "C" {
+
+int et_linear_dense_f32(const float *W, const float *bias, const float *X, float *Y, int T, int in, int out,
+                        int act, et_stream stream) {
+    ET_REQUIRE(W && X && Y, ET_ERR_INVALID_ARG, "et_linear_dense_f32: NULL pointer");
+    ET_REQUIRE(T >= 0 && in > 0 && out > 0, ET_ERR_INVALID_ARG, "et_linear_dense_f32: T=%d in=%d out=%d", T, in, out);
+    ET_REQUIRE(act >= ET_ACT_NONE && act <= ET_ACT_GELU, ET_ERR_INVALID_ARG, "et_linear_dense_f32: act=%d", act);
+    ET_REQUIRE(in % 16 == 0 && out % 4 == 0, ET_ERR_UNSUPPORTED,
+               "et_linear_dense_f32: in=%d must be a multiple of 16, out=%d of 4", in, out);
+    ET_REQUIRE(((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(Y)) & 15) == 0,
+               ET_ERR_UNSUPPORTED, "et_linear_dense_f32: W, X and Y must be 16-byte aligned");
+    if (T == 0) return ET_OK;
+    const dim3 grid((out + kF32Tile - 1) / kF32Tile, (T + kF32Tile - 1) / kF32Tile);
+    hipStream_t st = as_stream(stream);
+    switch (act) {
+        case ET_ACT_RELU: linear_dense_f32_kernel<ET_ACT_RELU><<<grid, 256, 0, st>>>(W, bias, X, Y, T, in, out); break;
+        case ET_ACT_GELU: linear_dense_f32_kernel<ET_ACT_GELU><<<grid, 256, 0, st>>>(W, bias, X, Y, T, in, out); break;
+        default: linear_dense_f32_kernel<ET_ACT_NONE><<<grid, 256, 0, st>>>(W, bias, X, Y, T, in, out); break;
+    }
+    return check_launch("linear_dense_f32_kernel");
+}
+
+int et_mha_fused_f32(const float *Q, const float *K, const float *V, int ldq, int ldk, int ldv, float *Z, int ldz,
+                     const float *mask, const int32_t *lens, int B, int S, int nh, int hd, float scale, int flags,
+                     et_stream stream) {
+    ET_REQUIRE(Q && K && V && Z, ET_ERR_INVALID_ARG, "et_mha_fused_f32: NULL pointer");
+    ET_REQUIRE(B >= 0 && S > 0 && nh > 0, ET_ERR_INVALID_ARG, "et_mha_fused_f32: B=%d S=%d nh=%d", B, S, nh);
+    ET_REQUIRE((flags & ~ET_MHA_CAUSAL) == 0, ET_ERR_INVALID_ARG, "et_mha_fused_f32: flags=%d", flags);
+    ET_REQUIRE(S % 16 == 0 && (hd == 32 || hd == 64 || hd == 128), ET_ERR_UNSUPPORTED,
+               "et_mha_fused_f32: S=%d must be a multiple of 16, hd=%d one of 32, 64, 128", S, hd);
+    const int width = nh * hd;
+    ET_REQUIRE(ldq >= width && ldk >= width && ldv >= width && ldz >= width, ET_ERR_INVALID_ARG,
+               "et_mha_fused_f32: row strides must cover nh*hd=%d", width);
+    const size_t lds = sizeof(float) * ((size_t)kAttQ * hd + (size_t)kAttKeys * (hd + 1) + (size_t)kAttQ * S);
+    ET_REQUIRE(lds <= 160 * 1024, ET_ERR_UNSUPPORTED, "et_mha_fused_f32: S=%d does not fit the on-chip score strip", S);
+    if (B == 0) return ET_OK;
+    MhaF32Args a{Q, K, V, Z, mask, lens, ldq, ldk, ldv, ldz, B, S, nh, hd, scale, (flags & ET_MHA_CAUSAL) ? 1 : 0};
+    const dim3 grid(S / kAttQ, nh, B);
+    hipStream_t st = as_stream(stream);
+#define ET_MHA32(HD)                                                                                         \
+    {                                                                                                        \
+        auto kern = mha_fused_f32_kernel<HD>;                                                                \
+        if (lds > 64 * 1024)                                                                                 \
+            ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                                 \
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));               \
+        kern<<<grid, 256, lds, st>>>(a);                                                                     \
+    }
+    if (hd == 32) ET_MHA32(32) else if (hd == 64) ET_MHA32(64) else ET_MHA32(128)
+#undef ET_MHA32
+    return check_launch("mha_fused_f32_kernel");
+}
+
+int et_gelu_f32(float *out, const float *in, size_t n, et_stream stream) {
+    ET_REQUIRE((out && in) || n == 0, ET_ERR_INVALID_ARG, "et_gelu_f32: NULL pointer");
+    if (n == 0) return ET_OK;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    unary_f32_kernel<0><<<(unsigned)blocks, 256, 0, as_stream(stream)>>>(out, in, n);
+    return check_launch("unary_f32_kernel<gelu>");
+}
+
+int et_relu_f32(float *out, const float *in, size_t n, et_stream stream) {
+    ET_REQUIRE((out && in) || n == 0, ET_ERR_INVALID_ARG, "et_relu_f32: NULL pointer");
+    if (n == 0) return ET_OK;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    unary_f32_kernel<1><<<(unsigned)blocks, 256, 0, as_stream(stream)>>>(out, in, n);
+    return check_launch("unary_f32_kernel<relu>");
+}
+
+}  // extern "C"

@@ -29,26 +29,42 @@ __device__ __forceinline__ uint2 pack4(const float (&f)[4]) {
     return raw;
 }
 
+// binary32 rows: a chunk is one float4
+__device__ __forceinline__ void unpack4(float4 raw, float (&f)[4]) {
+    f[0] = raw.x;
+    f[1] = raw.y;
+    f[2] = raw.z;
+    f[3] = raw.w;
+}
+template <typename RAW> __device__ __forceinline__ RAW pack4_as(const float (&f)[4]);
+template <> __device__ __forceinline__ uint2 pack4_as<uint2>(const float (&f)[4]) { return pack4(f); }
+template <> __device__ __forceinline__ float4 pack4_as<float4>(const float (&f)[4]) {
+    return float4{f[0], f[1], f[2], f[3]};
+}
+template <typename T> struct Chunk4;  // storage type of 4 consecutive elements
+template <> struct Chunk4<_Float16> { using raw = uint2; };
+template <> struct Chunk4<float> { using raw = float4; };
+
 // NIT = number of 4-element chunks each lane owns: chunk c = lane + 64*i.
-template <int NIT, bool SKIP>
+template <typename T, int NIT, bool SKIP>
 __global__ __launch_bounds__(kWave *kRowsPerBlock) void layernorm_rows_kernel(
-    _Float16 *__restrict__ out, const _Float16 *__restrict__ src,
-    const _Float16 *__restrict__ skip, const _Float16 *__restrict__ gamma,
-    const _Float16 *__restrict__ beta, int rows, int H, float eps) {
+    T *__restrict__ out, const T *__restrict__ src, const T *__restrict__ skip,
+    const T *__restrict__ gamma, const T *__restrict__ beta, int rows, int H, float eps) {
+    using raw_t = typename Chunk4<T>::raw;
     const int lane = threadIdx.x & (kWave - 1);
     const int row = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
     if (row >= rows) return;
     const int chunks = H >> 2;
-    const uint2 *s = reinterpret_cast<const uint2 *>(src + (size_t)row * H);
-    const uint2 *k = SKIP ? reinterpret_cast<const uint2 *>(skip + (size_t)row * H) : nullptr;
+    const raw_t *s = reinterpret_cast<const raw_t *>(src + (size_t)row * H);
+    const raw_t *k = SKIP ? reinterpret_cast<const raw_t *>(skip + (size_t)row * H) : nullptr;
 
     // Every load of the row is issued before the first use, so src, skip, gamma and beta
     // arrive in one round trip.  The loads are unconditional (a chunk index past the row is
     // clamped onto the last chunk and its value ignored): loads under a branch end up in a
     // basic block of their own, where the compiler waits for each of them in turn.
-    const uint2 *g = reinterpret_cast<const uint2 *>(gamma);
-    const uint2 *b = reinterpret_cast<const uint2 *>(beta);
-    uint2 rs[NIT], rk[NIT], rg[NIT], rb[NIT];
+    const raw_t *g = reinterpret_cast<const raw_t *>(gamma);
+    const raw_t *b = reinterpret_cast<const raw_t *>(beta);
+    raw_t rs[NIT], rk[NIT], rg[NIT], rb[NIT];
 #pragma unroll
     for (int i = 0; i < NIT; i++) {
         const int c = min(lane + kWave * i, chunks - 1);
@@ -92,7 +108,7 @@ __global__ __launch_bounds__(kWave *kRowsPerBlock) void layernorm_rows_kernel(
     }
     const float rstd = rsqrtf(wave_sum(sq) * inv_h + eps);
 
-    uint2 *o = reinterpret_cast<uint2 *>(out + (size_t)row * H);
+    raw_t *o = reinterpret_cast<raw_t *>(out + (size_t)row * H);
 #pragma unroll
     for (int i = 0; i < NIT; i++) {
         const int c = lane + kWave * i;
@@ -102,21 +118,20 @@ __global__ __launch_bounds__(kWave *kRowsPerBlock) void layernorm_rows_kernel(
             unpack4(rb[i], bb);
 #pragma unroll
             for (int j = 0; j < 4; j++) y[j] = (x[i][j] - mean) * rstd * gg[j] + bb[j];
-            o[c] = pack4(y);
+            o[c] = pack4_as<raw_t>(y);
         }
     }
 }
 
-template <bool SKIP>
-static int launch_layernorm(_Float16 *out, const _Float16 *src, const _Float16 *skip,
-                            const _Float16 *gamma, const _Float16 *beta, int rows, int H,
-                            float eps, hipStream_t stream) {
+template <bool SKIP, typename T>
+static int launch_layernorm(T *out, const T *src, const T *skip, const T *gamma, const T *beta, int rows,
+                            int H, float eps, hipStream_t stream) {
     const int chunks = H / 4;
     const int nit = (chunks + kWave - 1) / kWave;
     const dim3 grid((rows + kRowsPerBlock - 1) / kRowsPerBlock), block(kWave * kRowsPerBlock);
 #define ET_LN_CASE(N)                                                                   \
     case N:                                                                             \
-        layernorm_rows_kernel<N, SKIP><<<grid, block, 0, stream>>>(out, src, skip, gamma, \
+        layernorm_rows_kernel<T, N, SKIP><<<grid, block, 0, stream>>>(out, src, skip, gamma, \
                                                                    beta, rows, H, eps);  \
         break;
     switch (nit) {
@@ -124,10 +139,10 @@ static int launch_layernorm(_Float16 *out, const _Float16 *src, const _Float16 *
         ET_LN_CASE(5) ET_LN_CASE(6) ET_LN_CASE(7) ET_LN_CASE(8)
         default:
             if (nit <= 16) {
-                layernorm_rows_kernel<16, SKIP><<<grid, block, 0, stream>>>(out, src, skip, gamma,
+                layernorm_rows_kernel<T, 16, SKIP><<<grid, block, 0, stream>>>(out, src, skip, gamma,
                                                                             beta, rows, H, eps);
             } else {
-                layernorm_rows_kernel<32, SKIP><<<grid, block, 0, stream>>>(out, src, skip, gamma,
+                layernorm_rows_kernel<T, 32, SKIP><<<grid, block, 0, stream>>>(out, src, skip, gamma,
                                                                             beta, rows, H, eps);
             }
     }
@@ -168,10 +183,27 @@ int et_layernorm_f16(et_f16 *out, const et_f16 *src, const et_f16 *gamma, const 
     int s = check_ln_args("et_layernorm_f16", out, src, gamma, beta, rows, H);
     if (s != ET_OK) return s;
     if (rows == 0) return ET_OK;
-    return launch_layernorm<false>(
+    return launch_layernorm<false, _Float16>(
         reinterpret_cast<_Float16 *>(out), reinterpret_cast<const _Float16 *>(src), nullptr,
         reinterpret_cast<const _Float16 *>(gamma), reinterpret_cast<const _Float16 *>(beta), rows,
         H, eps, as_stream(stream));
+}
+
+int et_skip_layernorm_f32(float *out, const float *src, const float *skip, const float *gamma,
+                          const float *beta, int rows, int H, float eps, et_stream stream) {
+    int s = check_ln_args("et_skip_layernorm_f32", out, src, gamma, beta, rows, H);
+    if (s != ET_OK) return s;
+    ET_REQUIRE(skip != nullptr, ET_ERR_INVALID_ARG, "et_skip_layernorm_f32: skip is NULL");
+    if (rows == 0) return ET_OK;
+    return launch_layernorm<true>(out, src, skip, gamma, beta, rows, H, eps, as_stream(stream));
+}
+
+int et_layernorm_f32(float *out, const float *src, const float *gamma, const float *beta, int rows, int H,
+                     float eps, et_stream stream) {
+    int s = check_ln_args("et_layernorm_f32", out, src, gamma, beta, rows, H);
+    if (s != ET_OK) return s;
+    if (rows == 0) return ET_OK;
+    return launch_layernorm<false, float>(out, src, nullptr, gamma, beta, rows, H, eps, as_stream(stream));
 }
 
 }  // extern "C"

@@ -1,0 +1,157 @@
+"""binary32 twins on the GPU against the CPU oracle, and the dense fp32 encoder layer of the
+first benchmark configuration (one BERT-base layer, batch 1, seq 128) composed from them,
+to the fp32-path tolerance max-abs 1e-4."""
+import importlib.util
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import layers as L
+from tests import harness as Hn
+
+pytestmark = pytest.mark.gpu
+up = Hn.up
+GOLDEN = Path(__file__).parent / "golden"
+TOL_F32 = 1e-4
+ACT = {0: None, 1: "relu", 2: "gelu"}
+
+
+def randf(shape, seed, std=1.0):
+    return (torch.randn(*shape, generator=Hn.rng(seed)) * std).numpy().astype(np.float32)
+
+
+@pytest.mark.parametrize("T,inp,out,act", [(128, 768, 2304, 0), (128, 768, 3072, 2), (128, 3072, 768, 0),
+                                           (100, 48, 20, 1), (1, 16, 4, 0), (77, 160, 132, 2)])
+def test_linear_dense_f32(et, T, inp, out, act):
+    W, b, x = randf((out, inp), 1, 0.05), randf((out,), 2, 0.1), randf((T, inp), 3)
+    d_y = et.DeviceBuffer.empty((T, out), np.float32)
+    et.check(et.lib().et_linear_dense_f32(up(et, W).ptr, up(et, b).ptr, up(et, x).ptr, d_y.ptr, T, inp, out, act, None))
+    want = torch.from_numpy(x.astype(np.float64) @ W.astype(np.float64).T + b)  # binary64 reference
+    want = L.ACTS[ACT[act]](want).numpy()
+    # fp32 accumulation of `inp` products, |y| up to ~10: error ~ sqrt(inp) * 6e-8 * |y|
+    assert Hn.max_abs(d_y.numpy(), want) <= 5e-5
+
+
+def test_linear_dense_f32_no_bias_and_bad_args(et):
+    W, x = randf((32, 32), 4), randf((16, 32), 5)
+    d_y = et.DeviceBuffer.empty((16, 32), np.float32)
+    et.check(et.lib().et_linear_dense_f32(up(et, W).ptr, None, up(et, x).ptr, d_y.ptr, 16, 32, 32, 0, None))
+    assert Hn.max_abs(d_y.numpy(), x @ W.T) <= 1e-5
+    assert et.lib().et_linear_dense_f32(up(et, W).ptr, None, up(et, x).ptr, d_y.ptr, 16, 24, 32, 0, None) \
+        == et.ET_ERR_UNSUPPORTED
+    assert et.lib().et_linear_dense_f32(None, None, up(et, x).ptr, d_y.ptr, 16, 32, 32, 0, None) == et.ET_ERR_INVALID_ARG
+
+
+@pytest.mark.parametrize("B,S,nh,hd,causal,lens,mask", [
+    (1, 128, 12, 64, False, None, False), (3, 128, 12, 64, False, [128, 64, 97], False),
+    (2, 64, 4, 32, True, None, False), (2, 48, 2, 128, False, [0, 48], True), (1, 512, 2, 64, True, [300], False)])
+def test_mha_fused_f32(et, B, S, nh, hd, causal, lens, mask):
+    H = nh * hd
+    qkv = randf((B * S, 3 * H), 6)
+    d_qkv = up(et, qkv)
+    d_z = et.DeviceBuffer.empty((B * S, H), np.float32)
+    m = randf((S, S), 7) if mask else None
+    if mask:
+        m[:, 5] = -np.inf
+    d_m = up(et, m) if mask else None
+    d_l = up(et, np.asarray(lens, np.int32)) if lens is not None else None
+    et.check(et.lib().et_mha_fused_f32(d_qkv.ptr, d_qkv.offset(4 * H), d_qkv.offset(8 * H), 3 * H, 3 * H, 3 * H,
+                                       d_z.ptr, H, d_m.ptr if mask else None, d_l.ptr if lens is not None else None,
+                                       B, S, nh, hd, hd ** -0.5, et.MHA_CAUSAL if causal else 0, None))
+    t = torch.from_numpy(qkv)
+    want = L.mha(t[:, :H], t[:, H:2 * H], t[:, 2 * H:], nh, B, mask=torch.from_numpy(m) if mask else None,
+                 lens=lens, causal=causal)
+    assert Hn.max_abs(d_z.numpy(), want.numpy()) <= 1e-5
+
+
+@pytest.mark.parametrize("rows,H", [(128, 768), (33, 1024), (5, 4100), (7, 64)])
+def test_layernorm_f32(et, rows, H):
+    src, skip = randf((rows, H), 8, 2.0), randf((rows, H), 9)
+    gamma, beta = 1 + randf((H,), 10, 0.1), randf((H,), 11, 0.1)
+    d_out = et.DeviceBuffer.empty((rows, H), np.float32)
+    et.check(et.lib().et_skip_layernorm_f32(d_out.ptr, up(et, src).ptr, up(et, skip).ptr, up(et, gamma).ptr,
+                                            up(et, beta).ptr, rows, H, 1e-5, None))
+    want = torch.nn.functional.layer_norm(torch.from_numpy(src + skip).double(), (H,), torch.from_numpy(gamma).double(),
+                                          torch.from_numpy(beta).double(), 1e-5).float().numpy()
+    assert Hn.max_abs(d_out.numpy(), want) <= 1e-5
+    et.check(et.lib().et_layernorm_f32(d_out.ptr, up(et, src).ptr, up(et, gamma).ptr, up(et, beta).ptr, rows, H,
+                                       1e-5, None))
+    want = torch.nn.functional.layer_norm(torch.from_numpy(src).double(), (H,), torch.from_numpy(gamma).double(),
+                                          torch.from_numpy(beta).double(), 1e-5).float().numpy()
+    assert Hn.max_abs(d_out.numpy(), want) <= 1e-5
+
+
+def test_gelu_relu_f32(et):
+    x = randf((100003,), 12, 3.0)
+    d_o = et.DeviceBuffer.empty(x.shape, np.float32)
+    et.check(et.lib().et_gelu_f32(d_o.ptr, up(et, x).ptr, x.size, None))
+    want = torch.nn.functional.gelu(torch.from_numpy(x).double(), approximate="tanh").float().numpy()
+    assert Hn.max_abs(d_o.numpy(), want) <= 2e-6
+    et.check(et.lib().et_relu_f32(d_o.ptr, up(et, x).ptr, x.size, None))
+    assert np.array_equal(d_o.numpy(), np.maximum(x, 0))
+
+
+def f32_layer(et, x, p, nh, B, act=2, lens=None):
+    """One post-LN encoder layer from the binary32 entry points (weights: dict of numpy fp32)."""
+    lib = et.lib()
+    T, H = x.shape
+    FF = p["W1"].shape[0]
+    S = T // B
+    f = lambda shape: et.DeviceBuffer.empty(shape, np.float32)
+    d = {k: up(et, np.ascontiguousarray(v, dtype=np.float32)) for k, v in p.items()}
+    d_x, qkv, z, a, y1, ff, f2, out = up(et, x), f((T, 3 * H)), f((T, H)), f((T, H)), f((T, H)), f((T, FF)), \
+        f((T, H)), f((T, H))
+    d_l = up(et, np.asarray(lens, np.int32)) if lens is not None else None
+    et.check(lib.et_linear_dense_f32(d["Wqkv"].ptr, d["bqkv"].ptr, d_x.ptr, qkv.ptr, T, H, 3 * H, 0, None))
+    et.check(lib.et_mha_fused_f32(qkv.ptr, qkv.offset(4 * H), qkv.offset(8 * H), 3 * H, 3 * H, 3 * H, z.ptr, H, None,
+                                  d_l.ptr if d_l else None, B, S, nh, H // nh, (H // nh) ** -0.5, 0, None))
+    et.check(lib.et_linear_dense_f32(d["Wo"].ptr, d["bo"].ptr, z.ptr, a.ptr, T, H, H, 0, None))
+    et.check(lib.et_skip_layernorm_f32(y1.ptr, a.ptr, d_x.ptr, d["g1"].ptr, d["be1"].ptr, T, H, 1e-5, None))
+    et.check(lib.et_linear_dense_f32(d["W1"].ptr, d["b1"].ptr, y1.ptr, ff.ptr, T, H, FF, act, None))
+    et.check(lib.et_linear_dense_f32(d["W2"].ptr, d["b2"].ptr, ff.ptr, f2.ptr, T, FF, H, 0, None))
+    et.check(lib.et_skip_layernorm_f32(out.ptr, f2.ptr, y1.ptr, d["g2"].ptr, d["be2"].ptr, T, H, 1e-5, None))
+    return out.numpy()
+
+
+def test_dense_fp32_encoder_layer_matches_library_fixture_and_oracle(et):
+    """First benchmark configuration: one dense BERT-base layer, fp32, batch 1, seq 128, N(0, 0.02)
+    weights, zero biases, unit LayerNorm, N(0, 1) input.  Checked against the committed output of
+    torch.nn.TransformerEncoderLayer and against the CPU oracle, both to max-abs 1e-4."""
+    spec = importlib.util.spec_from_file_location("mk", GOLDEN / "make_encoder_layer_c1.py")
+    mk = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mk)
+    sp = mk.seeded_params()
+    H, FF = mk.H, mk.FF
+    z = lambda n: np.zeros(n, np.float32)
+    p = {"Wqkv": sp["Wqkv"].numpy(), "bqkv": z(3 * H), "Wo": sp["Wo"].numpy(), "bo": z(H), "W1": sp["W1"].numpy(),
+         "b1": z(FF), "W2": sp["W2"].numpy(), "b2": z(H), "g1": np.ones(H, np.float32), "be1": z(H),
+         "g2": np.ones(H, np.float32), "be2": z(H)}
+    y = f32_layer(et, sp["x"].numpy(), p, mk.NH, 1)
+    fx = np.load(GOLDEN / "encoder_layer_c1.npz")
+    assert np.max(np.abs(y[:8] - fx["y_head"])) <= TOL_F32
+    assert abs(float(y.astype(np.float64).sum()) - float(fx["y_sum"])) <= 1e-2
+    assert abs(float(np.abs(y.astype(np.float64)).sum()) - float(fx["y_abs_sum"])) <= 1e-1
+    P = L.LayerParams(sp["Wqkv"], torch.zeros(3 * H), sp["Wo"], torch.zeros(H), sp["W1"], torch.zeros(FF), sp["W2"],
+                      torch.zeros(H), torch.ones(H), torch.zeros(H), torch.ones(H), torch.zeros(H))
+    want = L.encoder_layer(sp["x"], P, L.LayerConfig(nh=mk.NH, act="gelu", eps=1e-5)).numpy()
+    err = float(np.max(np.abs(y - want)))
+    print(f"dense fp32 layer max-abs vs oracle: {err:.2e}")
+    assert err <= TOL_F32
+
+
+def test_fp32_layer_with_biases_padding_and_batch(et):
+    H, nh, FF, S, B = 256, 4, 512, 64, 3
+    g = lambda shape, seed, std: randf(shape, seed, std)
+    p = {"Wqkv": g((3 * H, H), 20, 0.05), "bqkv": g((3 * H,), 21, 0.1), "Wo": g((H, H), 22, 0.05), "bo": g((H,), 23, 0.1),
+         "W1": g((FF, H), 24, 0.05), "b1": g((FF,), 25, 0.1), "W2": g((H, FF), 26, 0.05), "b2": g((H,), 27, 0.1),
+         "g1": 1 + g((H,), 28, 0.1), "be1": g((H,), 29, 0.1), "g2": 1 + g((H,), 30, 0.1), "be2": g((H,), 31, 0.1)}
+    x = randf((B * S, H), 32)
+    lens = [64, 16, 33]
+    y = f32_layer(et, x, p, nh, B, act=1, lens=lens)
+    t = {k: torch.from_numpy(v) for k, v in p.items()}
+    P = L.LayerParams(t["Wqkv"], t["bqkv"], t["Wo"], t["bo"], t["W1"], t["b1"], t["W2"], t["b2"], t["g1"], t["be1"],
+                      t["g2"], t["be2"])
+    want = L.encoder_layer(torch.from_numpy(x), P, L.LayerConfig(nh=nh, B=B, act="relu", lens=lens)).numpy()
+    assert Hn.max_abs(y, want) <= TOL_F32
