@@ -7,8 +7,8 @@ seq 128, batch 8, 80 % 16x16 tile sparsity with attention-aware V/O pruning.
 One "step" is one forward of the whole encoder stack over one batch of synthetic
 token embeddings that already sit in HBM (one HIP-graph replay through the C ABI).
 Prints ONE JSON line: sequences/s (value), ms per step, per-layer latency, the
-roofline of the dominant kernel (the tile-sparse FFN up-projection with fused GELU,
-timed with HIP events on its own stream) and the CPU oracle timed on the host cores.
+roofline of the dominant kernel (SkipLayerNorm + tile-sparse FFN up-projection + GELU in
+one launch, timed with HIP events on its own stream) and the CPU oracle timed on the host cores.
 """
 from __future__ import annotations
 
@@ -35,7 +35,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak (vendor figure)
 # HBM-side bytes per launch of the FFN up-projection kernel: rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a streaming
 # kernel of known size (profiles/encoder_stack_bert_base_b8_s128_hbm_traffic.txt).
-FFN_UP_TRAFFIC_BYTES = (4622.4 * 1.9992 + 6144.0 * 1.0) * 1024
+FFN_UP_TRAFFIC_BYTES = (5420.5 * 1.9989 + 7680.0 * 1.0) * 1024
 
 
 def build_layers(Hn):
@@ -57,20 +57,32 @@ def time_stack(et, model, d_out, d_in, steps, warmup):
 
 
 def time_ffn_kernel(et, w, T, launches_per_graph=64, replays=8):
-    """Average duration of the FFN up-projection kernel (tile-sparse Linear + GELU at the
-    workload's shape): `launches_per_graph` launches recorded into one HIP graph, replayed
-    between two HIP events on the same stream, so no host launch latency is in the figure."""
+    """Average duration of the layer's longest kernel at the workload's shape — y1 = SkipLayerNorm(
+    attention output + layer input), then GELU(y1 W1^T + b1) through the tile-sparse W1, one
+    launch: `launches_per_graph` launches recorded into one HIP graph, replayed between two HIP
+    events on the same stream, so no host launch latency is in the figure."""
     import ctypes as C
     lib = et.lib()
     stream = C.c_void_p()
     et.check(lib.et_stream_create(C.byref(stream)))
-    x = et.DeviceBuffer.from_numpy(np.random.default_rng(0).standard_normal((T, H)).astype(np.float16))
+    rng = np.random.default_rng(0)
+    src = et.DeviceBuffer.from_numpy(rng.standard_normal((T, H)).astype(np.float16))
+    skip = et.DeviceBuffer.from_numpy(rng.standard_normal((T, H)).astype(np.float16))
+    gamma = et.DeviceBuffer.from_numpy(np.ones(H, np.float16))
+    beta = et.DeviceBuffer.from_numpy(np.zeros(H, np.float16))
+    y1 = et.DeviceBuffer.empty((T, H), np.float16)
     y = et.DeviceBuffer.empty((T, FF), np.float16)
-    w.forward(et, x, y, T, et.ACT_GELU, stream)  # eager once (one-time kernel setup)
+
+    def launch():
+        et.check(lib.et_skipln_linear_bsr16_f16(src.ptr, skip.ptr, gamma.ptr, beta.ptr, 1e-5, y1.ptr, w.d_row_ptr.ptr,
+                                                w.d_col_idx.ptr, w.d_tiles.ptr, w.d_bias.ptr, y.ptr, T, H, FF,
+                                                et.ACT_GELU, stream))
+
+    launch()  # eager once (one-time kernel setup)
     et.check(lib.et_stream_sync(stream))
     et.check(lib.et_graph_begin_capture(stream))
     for _ in range(launches_per_graph):
-        w.forward(et, x, y, T, et.ACT_GELU, stream)
+        launch()
     graph = C.c_void_p()
     et.check(lib.et_graph_end_capture(stream, C.byref(graph)))
     et.check(lib.et_graph_launch(graph, stream))  # warm
@@ -135,14 +147,14 @@ def main():
 
     sec = time_stack(et, model, d_out, d_in, args.steps, args.warmup)
 
-    # dominant kernel: FFN up-projection, 3072x768 BSR at 80 %, T = 1024, GELU fused
+    # dominant kernel: SkipLayerNorm + FFN up-projection (3072x768 BSR at 80 %, T = 1024) + GELU
     T = B * S
     w1 = layers[0].l1.upload(et)
     ntile = len(layers[0].l1.col_idx)
     flops = 2.0 * 256 * ntile * T  # algorithmic: 2 * 16*16 * surviving tiles * token rows
     ksec = time_ffn_kernel(et, w1, T)
     achieved = flops / ksec / 1e12
-    roofline = {"bound": "mfma", "kernel": "bsr16_linear_kernel<2,true,GELU> 3072x768 @80% T=1024",
+    roofline = {"bound": "mfma", "kernel": "bsr16_linear_kernel<2,true,GELU,LN> SkipLayerNorm + 3072x768 @80% + GELU, T=1024",
                 "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 5), "us_per_launch": round(ksec * 1e6, 3),
                 "flop_per_launch": flops, "traffic": round(FFN_UP_TRAFFIC_BYTES)}
