@@ -20,6 +20,8 @@
 // by the fp32 row sum happens once on the fp32 accumulators.
 #include <math.h>
 
+#include <type_traits>
+
 #include "common.hip.h"
 
 namespace et {
@@ -55,7 +57,9 @@ struct MhaLds {
     static constexpr size_t bytes = (size_t)(k_halfs + vt_halfs) * sizeof(_Float16);
 };
 
-template <int HD, bool COMPACT, int NW>
+// QT = 16-query tiles per wave: with QT = 2 every K and V^T fragment read from LDS feeds
+// two MFMAs and a workgroup covers 32*NW queries per staged key block.
+template <int HD, bool COMPACT, int NW, int QT>
 __global__ __launch_bounds__(64 * NW) void mha_fused_kernel(const MhaArgs a) {
     using L = MhaLds<HD>;
     constexpr int KS = HD / 32;  // K=32 MFMA steps over the head dimension
@@ -68,23 +72,31 @@ __global__ __launch_bounds__(64 * NW) void mha_fused_kernel(const MhaArgs a) {
     const int wave = threadIdx.x >> 6;
     constexpr int nwave = NW;
     constexpr int nthr = 64 * NW;
+    constexpr int kStripQ = 16 * NW * QT;  // queries per workgroup
     const int r16 = lane & 15;
     const int g = lane >> 4;
     const int S = a.S;
     // Workgroup id -> (sequence*head, query strip), XCD-aware: workgroups go to the 8
     // XCDs round-robin by id, so the query strips of one (sequence, head) are given ids
     // that land on the same XCD and share its K and V in that L2.
-    const int qstrips = (S + 16 * nwave - 1) / (16 * nwave);
+    const int qstrips = (S + kStripQ - 1) / kStripQ;
     const int xcd = blockIdx.x % kXcds, k_in_xcd = blockIdx.x / kXcds;
     const int bh = xcd + kXcds * (k_in_xcd / qstrips);
     if (bh >= a.nbh) return;  // padding of the last round (whole workgroup)
     const int qstrip = k_in_xcd % qstrips;
     const int b = bh / a.nh, h = bh - b * a.nh;
     const size_t row0 = (size_t)b * S;  // first token row of this sequence
-    const int q = (qstrip * nwave + wave) * 16 + r16;  // this lane's query
-    const bool q_ok = q < S;
+    int q[QT];       // this lane's queries
+    bool q_ok[QT];
+#pragma unroll
+    for (int t = 0; t < QT; t++) {
+        q[t] = qstrip * kStripQ + (wave * QT + t) * 16 + r16;
+        q_ok[t] = q[t] < S;
+    }
     int klimit = S;
     if (a.lens) klimit = min(S, max(a.lens[b], 0));
+    // under a causal mask no query of this strip sees a key past the strip's last query
+    if (a.causal) klimit = min(klimit, (qstrip + 1) * kStripQ);
     // compact-V: this head's surviving V columns
     int vc0 = 0, vlive = HD;
     if (COMPACT) {
@@ -93,203 +105,284 @@ __global__ __launch_bounds__(64 * NW) void mha_fused_kernel(const MhaArgs a) {
     }
 
     // Q fragments: B operand, lane supplies Q[q][32*ks + 8g .. +7]
-    h8 qf[KS];
-    {
-        const _Float16 *qp = a.Q + (row0 + (q_ok ? q : 0)) * a.ldq + h * HD + 8 * g;
+    h8 qf[QT][KS];
+#pragma unroll
+    for (int t = 0; t < QT; t++) {
+        const _Float16 *qp = a.Q + (row0 + (q_ok[t] ? q[t] : 0)) * a.ldq + h * HD + 8 * g;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
-            qf[ks] = *reinterpret_cast<const h8 *>(qp + 32 * ks);
-            if (!q_ok) qf[ks] = h8{0, 0, 0, 0, 0, 0, 0, 0};
+            qf[t][ks] = *reinterpret_cast<const h8 *>(qp + 32 * ks);
+            if (!q_ok[t]) qf[t][ks] = h8{0, 0, 0, 0, 0, 0, 0, 0};
         }
     }
 
-    f4 o[DB];
+    f4 o[QT][DB];
+    float m_run[QT];   // running max of this lane's query (log2 domain)
+    float l_part[QT];  // this lane's share of the running row sum
 #pragma unroll
-    for (int d = 0; d < DB; d++) o[d] = f4{0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY;  // running max of this lane's query (log2 domain)
-    float l_part = 0.0f;      // this lane's share of the running row sum
+    for (int t = 0; t < QT; t++) {
+#pragma unroll
+        for (int d = 0; d < DB; d++) o[t][d] = f4{0.f, 0.f, 0.f, 0.f};
+        m_run[t] = -INFINITY;
+        l_part[t] = 0.0f;
+    }
 
+    // ---- staging of one block of keys: K rows and V in units of 4 keys x 8 dims, which
+    // go to LDS transposed.  load_block issues every global load of a block (one memory
+    // round trip); store_block writes them to LDS.  The loads of block i+1 are issued
+    // before block i is multiplied.
+    constexpr int vec_per_row = HD / 8;
+    constexpr int KV = kKeyBlock * vec_per_row / nthr;  // K vectors per thread
+    constexpr int dgroups = HD / 8;
+    constexpr int v_units = (kKeyBlock / 4) * dgroups;  // V units of 4 keys x 8 dims
+    constexpr int VU = (v_units + nthr - 1) / nthr;       // ... per thread
+    static_assert(KV >= 1 && kKeyBlock * vec_per_row % nthr == 0, "K block must split evenly");
+    h8 kreg[KV];
+    h8 vreg[VU][4];
+    auto load_block = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < KV; i++) {
+            const int v = threadIdx.x + i * nthr;
+            const int r = v / vec_per_row, c = v - r * vec_per_row;
+            kreg[i] = h8{0, 0, 0, 0, 0, 0, 0, 0};
+            if (k0 + r < S)
+                kreg[i] = *reinterpret_cast<const h8 *>(a.K + (row0 + k0 + r) * a.ldk + h * HD + c * 8);
+        }
+#pragma unroll
+        for (int j = 0; j < VU; j++) {
+            const int u = threadIdx.x + j * nthr;
+            const int kg = u / dgroups, dg = u - kg * dgroups;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int key = (u < v_units) ? k0 + kg * 4 + i : S;  // surplus threads load nothing
+                vreg[j][i] = h8{0, 0, 0, 0, 0, 0, 0, 0};
+                if (COMPACT) {
+                    // compact columns start at an arbitrary element: scalar loads
+                    if (key < S) {
+                        const _Float16 *vp = a.V + (row0 + key) * a.ldv + vc0 + dg * 8;
+#pragma unroll
+                        for (int d = 0; d < 8; d++)
+                            if (dg * 8 + d < vlive) vreg[j][i][d] = vp[d];
+                    }
+                } else if (key < S) {
+                    vreg[j][i] = *reinterpret_cast<const h8 *>(a.V + (row0 + key) * a.ldv + h * HD + dg * 8);
+                }
+            }
+        }
+    };
+    auto store_block = [&]() {
+#pragma unroll
+        for (int i = 0; i < KV; i++) {
+            const int v = threadIdx.x + i * nthr;
+            const int r = v / vec_per_row, c = v - r * vec_per_row;
+            *reinterpret_cast<h8 *>(Ks + r * L::ldk + c * 8) = kreg[i];
+        }
+#pragma unroll
+        for (int j = 0; j < VU; j++) {
+            const int u = threadIdx.x + j * nthr;
+            const int kg = u / dgroups, dg = u - kg * dgroups;
+            if (u < v_units) {
+#pragma unroll
+                for (int d = 0; d < 8; d++) {
+                    h4 col = {vreg[j][0][d], vreg[j][1][d], vreg[j][2][d], vreg[j][3][d]};
+                    *reinterpret_cast<h4 *>(Vt + (dg * 8 + d) * L::ldvt + kg * 4) = col;
+                }
+            }
+        }
+    };
+
+    // Holding the next block's loads in registers through the multiplication costs 32 or more
+    // VGPRs, i.e. one resident wave per SIMD; measured, the third wave hides the load latency
+    // better than the prefetch does, so it is off.
+    constexpr bool kPrefetch = false;
     const int nblocks = (klimit + kKeyBlock - 1) / kKeyBlock;
+    if (kPrefetch && nblocks > 0) load_block(0);
     for (int blk = 0; blk < nblocks; blk++) {
         const int k0 = blk * kKeyBlock;
-        if (blk > 0) __syncthreads();
-        // ---- stage the K block and the transposed V block: every global load of the
-        // block is issued before the first LDS write (one memory round trip)
-        {
-            constexpr int vec_per_row = HD / 8;
-            constexpr int KV = kKeyBlock * vec_per_row / nthr;  // K vectors per thread
-            constexpr int dgroups = HD / 8;
-            constexpr int v_units = (kKeyBlock / 4) * dgroups;  // V units of 4 keys x 8 dims
-            constexpr int VU = (v_units + nthr - 1) / nthr;       // ... per thread
-            static_assert(KV >= 1 && kKeyBlock * vec_per_row % nthr == 0, "K block must split evenly");
-            h8 kreg[KV];
-            h8 vreg[VU][4];
-#pragma unroll
-            for (int i = 0; i < KV; i++) {
-                const int v = threadIdx.x + i * nthr;
-                const int r = v / vec_per_row, c = v - r * vec_per_row;
-                kreg[i] = h8{0, 0, 0, 0, 0, 0, 0, 0};
-                if (k0 + r < S)
-                    kreg[i] = *reinterpret_cast<const h8 *>(a.K + (row0 + k0 + r) * a.ldk + h * HD + c * 8);
-            }
-#pragma unroll
-            for (int j = 0; j < VU; j++) {
-                const int u = threadIdx.x + j * nthr;
-                const int kg = u / dgroups, dg = u - kg * dgroups;
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int key = (u < v_units) ? k0 + kg * 4 + i : S;  // surplus threads load nothing
-                    vreg[j][i] = h8{0, 0, 0, 0, 0, 0, 0, 0};
-                    if (COMPACT) {
-                        // compact columns start at an arbitrary element: scalar loads
-                        if (key < S) {
-                            const _Float16 *vp = a.V + (row0 + key) * a.ldv + vc0 + dg * 8;
-#pragma unroll
-                            for (int d = 0; d < 8; d++)
-                                if (dg * 8 + d < vlive) vreg[j][i][d] = vp[d];
-                        }
-                    } else if (key < S) {
-                        vreg[j][i] = *reinterpret_cast<const h8 *>(a.V + (row0 + key) * a.ldv + h * HD + dg * 8);
-                    }
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < KV; i++) {
-                const int v = threadIdx.x + i * nthr;
-                const int r = v / vec_per_row, c = v - r * vec_per_row;
-                *reinterpret_cast<h8 *>(Ks + r * L::ldk + c * 8) = kreg[i];
-            }
-#pragma unroll
-            for (int j = 0; j < VU; j++) {
-                const int u = threadIdx.x + j * nthr;
-                const int kg = u / dgroups, dg = u - kg * dgroups;
-                if (u < v_units) {
-#pragma unroll
-                    for (int d = 0; d < 8; d++) {
-                        h4 col = {vreg[j][0][d], vreg[j][1][d], vreg[j][2][d], vreg[j][3][d]};
-                        *reinterpret_cast<h4 *>(Vt + (dg * 8 + d) * L::ldvt + kg * 4) = col;
-                    }
-                }
-            }
-        }
+        if (blk > 0) __syncthreads();  // every wave is done with the previous block
+        if (!kPrefetch) load_block(k0);
+        store_block();
         __syncthreads();
+        if (kPrefetch && blk + 1 < nblocks) load_block(k0 + kKeyBlock);
 
-        // ---- scores of 16 queries against the 128 staged keys
-        f4 sc[kNKB];
+        // The multiplication of one staged block.  FAST (wave-uniform) = every key of the
+        // block is live for every query of the workgroup and nothing is added to the scores:
+        // no per-16-key branches (the LDS reads of the whole block can be issued ahead of
+        // the MFMAs) and the softmax costs one max, one multiply-add, one exp2, half a
+        // conversion and half a dot-accumulate per score.
+        auto multiply = [&](auto fast_tag) {
+            constexpr bool FAST = decltype(fast_tag)::value;
+            // ---- scores of the wave's queries against the 128 staged keys
+            f4 sc[QT][kNKB];
 #pragma unroll
-        for (int kb = 0; kb < kNKB; kb++) {
-            sc[kb] = f4{0.f, 0.f, 0.f, 0.f};
-            if (k0 + kb * 16 < klimit) {  // wave-uniform: skip fully padded key blocks
-                const _Float16 *kp = Ks + (kb * 16 + r16) * L::ldk + 8 * g;
+            for (int kb = 0; kb < kNKB; kb++) {
 #pragma unroll
-                for (int ks = 0; ks < KS; ks++) {
-                    const h8 kf = *reinterpret_cast<const h8 *>(kp + 32 * ks);
-                    sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[ks], sc[kb], 0, 0, 0);
+                for (int t = 0; t < QT; t++) sc[t][kb] = f4{0.f, 0.f, 0.f, 0.f};
+                if (FAST || k0 + kb * 16 < klimit) {  // wave-uniform: skip fully padded key blocks
+                    const _Float16 *kp = Ks + (kb * 16 + r16) * L::ldk + 8 * g;
+#pragma unroll
+                    for (int ks = 0; ks < KS; ks++) {
+                        const h8 kf = *reinterpret_cast<const h8 *>(kp + 32 * ks);
+#pragma unroll
+                        for (int t = 0; t < QT; t++)
+                            sc[t][kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[t][ks], sc[t][kb], 0, 0, 0);
+                    }
                 }
             }
-        }
 
-        // ---- scale, mask, block max
-        float m_blk = -INFINITY;
+            // ---- scale, mask, block max, running max (FAST keeps the raw scores: the scale
+            // is positive there, so the max commutes with it, and it is applied inside the
+            // exponent's multiply-add)
+            float m_use[QT];
 #pragma unroll
-        for (int kb = 0; kb < kNKB; kb++) {
-            const int key0 = k0 + kb * 16 + 4 * g;
-            float mk[4] = {0.f, 0.f, 0.f, 0.f};
-            if (a.mask && q_ok && key0 < S) {
-                const h4 mv = *reinterpret_cast<const h4 *>(a.mask + (size_t)q * S + key0);
+            for (int t = 0; t < QT; t++) {
+                float m_blk = -INFINITY;
+                if (FAST) {
 #pragma unroll
-                for (int j = 0; j < 4; j++) mk[j] = (float)mv[j] * kLog2e;
-            }
+                    for (int kb = 0; kb < kNKB; kb++)
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int key = key0 + j;
-                float s = sc[kb][j] * a.scale_log2e + mk[j];
-                if (key >= klimit || (a.causal && key > q)) s = -INFINITY;
-                sc[kb][j] = s;
-                m_blk = fmaxf(m_blk, s);
-            }
-        }
-        m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 16, kWave));
-        m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, kWave));
+                        for (int j = 0; j < 4; j++) m_blk = fmaxf(m_blk, sc[t][kb][j]);
+                    m_blk *= a.scale_log2e;
+                } else {
+#pragma unroll
+                    for (int kb = 0; kb < kNKB; kb++) {
+                        const int key0 = k0 + kb * 16 + 4 * g;
+                        float mk[4] = {0.f, 0.f, 0.f, 0.f};
+                        if (a.mask && q_ok[t] && key0 < S) {
+                            const h4 mv = *reinterpret_cast<const h4 *>(a.mask + (size_t)q[t] * S + key0);
+#pragma unroll
+                            for (int j = 0; j < 4; j++) mk[j] = (float)mv[j] * kLog2e;
+                        }
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const int key = key0 + j;
+                            float sv = sc[t][kb][j] * a.scale_log2e + mk[j];
+                            if (key >= klimit || (a.causal && key > q[t])) sv = -INFINITY;
+                            sc[t][kb][j] = sv;
+                            m_blk = fmaxf(m_blk, sv);
+                        }
+                    }
+                }
+                m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 16, kWave));
+                m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, kWave));
 
-        const float m_new = fmaxf(m_run, m_blk);
-        // all keys so far masked: keep everything at zero without inf - inf
-        const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-        const float alpha = exp2f(m_run - m_use);  // m_run = -inf gives 0
-        m_run = m_new;
-        l_part *= alpha;
+                const float m_new = fmaxf(m_run[t], m_blk);
+                // all keys so far masked: keep everything at zero without inf - inf
+                m_use[t] = (m_new == -INFINITY) ? 0.0f : m_new;
+                const float alpha = __builtin_amdgcn_exp2f(m_run[t] - m_use[t]);  // m_run = -inf gives 0
+                m_run[t] = m_new;
+                // the running max seldom moves after the first blocks: skip the rescaling of
+                // the accumulators when no lane of the wave needs it
+                if (!__all(alpha == 1.0f)) {
+                    l_part[t] *= alpha;
 #pragma unroll
-        for (int d = 0; d < DB; d++) o[d] *= alpha;
+                    for (int d = 0; d < DB; d++) o[t][d] *= alpha;
+                }
+            }
 
-        // ---- probabilities (fp32 sum, fp16 operands) and O^T += V^T P^T
+            // ---- probabilities (fp32 sum, fp16 operands) and O^T += V^T P^T
+            const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
 #pragma unroll
-        for (int s2 = 0; s2 < kNKB / 2; s2++) {
-            if (k0 + s2 * 32 >= klimit) continue;  // both key blocks fully padded
-            h8 pf;
+            for (int s2 = 0; s2 < kNKB / 2; s2++) {
+                if (!FAST && k0 + s2 * 32 >= klimit) continue;  // both key blocks fully padded
+                h8 pf[QT];
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const float p0 = exp2f(sc[2 * s2][j] - m_use);
-                const float p1 = exp2f(sc[2 * s2 + 1][j] - m_use);
-                const _Float16 h0 = (_Float16)p0, h1 = (_Float16)p1;
-                // the row sum uses the values that enter the MFMA
-                l_part += (float)h0 + (float)h1;
-                pf[j] = h0;
-                pf[4 + j] = h1;
+                for (int t = 0; t < QT; t++) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        float e0, e1;
+                        if (FAST) {
+                            e0 = sc[t][2 * s2][j] * a.scale_log2e - m_use[t];
+                            e1 = sc[t][2 * s2 + 1][j] * a.scale_log2e - m_use[t];
+                        } else {
+                            e0 = sc[t][2 * s2][j] - m_use[t];
+                            e1 = sc[t][2 * s2 + 1][j] - m_use[t];
+                        }
+                        // raw v_exp_f32: results below the normal range flush to zero, which
+                        // the conversion to fp16 would do anyway
+                        const h2 hp = {(_Float16)__builtin_amdgcn_exp2f(e0), (_Float16)__builtin_amdgcn_exp2f(e1)};
+                        // the row sum uses the values that enter the MFMA
+                        l_part[t] = __builtin_amdgcn_fdot2(hp, ones, l_part[t], false);
+                        pf[t][j] = hp[0];
+                        pf[t][4 + j] = hp[1];
+                    }
+                }
+#pragma unroll
+                for (int d = 0; d < DB; d++) {
+                    if (COMPACT && d * 16 >= vlive) continue;  // no surviving column in this block
+                    const _Float16 *vp = Vt + (d * 16 + r16) * L::ldvt + s2 * 32 + 4 * g;
+                    const h4 v0 = *reinterpret_cast<const h4 *>(vp);
+                    const h4 v1 = *reinterpret_cast<const h4 *>(vp + 16);
+                    const h8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+#pragma unroll
+                    for (int t = 0; t < QT; t++)
+                        o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[t], o[t][d], 0, 0, 0);
+                }
             }
-#pragma unroll
-            for (int d = 0; d < DB; d++) {
-                if (COMPACT && d * 16 >= vlive) continue;  // no surviving column in this block
-                const _Float16 *vp = Vt + (d * 16 + r16) * L::ldvt + s2 * 32 + 4 * g;
-                const h4 v0 = *reinterpret_cast<const h4 *>(vp);
-                const h4 v1 = *reinterpret_cast<const h4 *>(vp + 16);
-                const h8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-                o[d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[d], 0, 0, 0);
-            }
-        }
+        };
+        const bool fast = k0 + kKeyBlock <= klimit && a.mask == nullptr && a.scale_log2e > 0.0f &&
+                          (!a.causal || k0 + kKeyBlock <= qstrip * kStripQ + 1);
+        if (fast) multiply(std::true_type{});
+        else multiply(std::false_type{});
     }
 
     // ---- normalise and store: lane holds dims 16d + 4g..4g+3 of query r16
-    float l = l_part;
-    l += __shfl_xor(l, 16, kWave);
-    l += __shfl_xor(l, 32, kWave);
-    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-    if (q_ok && !COMPACT) {
-        _Float16 *zp = a.Z + (row0 + q) * a.ldz + h * HD + 4 * g;
+    float inv[QT];
 #pragma unroll
-        for (int d = 0; d < DB; d++) {
-            h4 out;
+    for (int t = 0; t < QT; t++) {
+        float l = l_part[t];
+        l += __shfl_xor(l, 16, kWave);
+        l += __shfl_xor(l, 32, kWave);
+        inv[t] = l > 0.0f ? 1.0f / l : 0.0f;
+    }
+    if (!COMPACT) {
 #pragma unroll
-            for (int j = 0; j < 4; j++) out[j] = (_Float16)(o[d][j] * inv);
-            *reinterpret_cast<h4 *>(zp + 16 * d) = out;
+        for (int t = 0; t < QT; t++) {
+            if (!q_ok[t]) continue;
+            _Float16 *zp = a.Z + (row0 + q[t]) * a.ldz + h * HD + 4 * g;
+#pragma unroll
+            for (int d = 0; d < DB; d++) {
+                h4 out;
+#pragma unroll
+                for (int j = 0; j < 4; j++) out[j] = (_Float16)(o[t][d][j] * inv[t]);
+                *reinterpret_cast<h4 *>(zp + 16 * d) = out;
+            }
         }
     }
     if (COMPACT) {
         // Full-width Z: pruned columns of this head's slice are zero, surviving
         // ones are scattered to v_col_id.  The zero fill is made visible before
         // the scatter so that the scatter wins wherever both touch an element.
-        _Float16 *zrow = a.Z + (row0 + (q_ok ? q : 0)) * a.ldz;
-        if (q_ok) {
-            const h4 z4 = {0, 0, 0, 0};
 #pragma unroll
-            for (int d = 0; d < DB; d++) *reinterpret_cast<h4 *>(zrow + h * HD + 16 * d + 4 * g) = z4;
+        for (int t = 0; t < QT; t++) {
+            if (q_ok[t]) {
+                _Float16 *zrow = a.Z + (row0 + q[t]) * a.ldz;
+                const h4 z4 = {0, 0, 0, 0};
+#pragma unroll
+                for (int d = 0; d < DB; d++) *reinterpret_cast<h4 *>(zrow + h * HD + 16 * d + 4 * g) = z4;
+            }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-        if (q_ok) {
 #pragma unroll
-            for (int d = 0; d < DB; d++) {
+        for (int t = 0; t < QT; t++) {
+            if (q_ok[t]) {
+                _Float16 *zrow = a.Z + (row0 + q[t]) * a.ldz;
 #pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const int dc = d * 16 + 4 * g + j;
-                    if (dc < vlive) zrow[a.v_col_id[vc0 + dc]] = (_Float16)(o[d][j] * inv);
+                for (int d = 0; d < DB; d++) {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const int dc = d * 16 + 4 * g + j;
+                        if (dc < vlive) zrow[a.v_col_id[vc0 + dc]] = (_Float16)(o[t][d][j] * inv[t]);
+                    }
                 }
             }
         }
     }
 }
 
-template <int HD, bool COMPACT, int NW>
+template <int HD, bool COMPACT, int NW, int QT>
 static int launch_mha_nw(const MhaArgs &args, hipStream_t stream) {
-    auto kernel = mha_fused_kernel<HD, COMPACT, NW>;
+    auto kernel = mha_fused_kernel<HD, COMPACT, NW, QT>;
     constexpr size_t lds = MhaLds<HD>::bytes;
     if (lds > 64 * 1024) {
         static bool raised = false;
@@ -299,21 +392,23 @@ static int launch_mha_nw(const MhaArgs &args, hipStream_t stream) {
             raised = true;
         }
     }
-    const int qstrips = (args.S + 16 * NW - 1) / (16 * NW);
+    const int qstrips = (args.S + 16 * NW * QT - 1) / (16 * NW * QT);
     const int rounds = (args.nbh + kXcds - 1) / kXcds;
     kernel<<<dim3((unsigned)(rounds * kXcds * qstrips)), 64 * NW, lds, stream>>>(args);
     return check_launch("mha_fused_kernel");
 }
 
-// 4 waves = 64 query rows per workgroup; 2 or 1 waves when that would leave a
-// half-empty strip (S = 32, 96, 16, ...).
+// 4 waves per workgroup; 2 or 1 waves when that would leave a half-empty strip
+// (S = 32, 96, 16, ...).  One query tile per wave: two tiles (QT = 2) halve the LDS and
+// L2 traffic per flop but need 256 registers, and the lost third resident wave costs
+// more than that saves (measured 13 % slower at S = 512 and S = 2048).
 template <int HD, bool COMPACT>
 static int launch_mha(const MhaArgs &args, int B, hipStream_t stream) {
     (void)B;
     const int qblocks = args.S / 16;
-    if (qblocks % 4 == 0) return launch_mha_nw<HD, COMPACT, 4>(args, stream);
-    if (qblocks % 2 == 0) return launch_mha_nw<HD, COMPACT, 2>(args, stream);
-    return launch_mha_nw<HD, COMPACT, 1>(args, stream);
+    if (qblocks % 4 == 0) return launch_mha_nw<HD, COMPACT, 4, 1>(args, stream);
+    if (qblocks % 2 == 0) return launch_mha_nw<HD, COMPACT, 2, 1>(args, stream);
+    return launch_mha_nw<HD, COMPACT, 1, 1>(args, stream);
 }
 
 }  // namespace et

@@ -417,8 +417,11 @@ static BsrPlan plan_bsr(int T, int in, int out) {
     if (32 * row_bytes <= lds_cap / 2) mt_fit = 2;
     else if (16 * row_bytes <= lds_cap) mt_fit = 1;
     struct Cand { int mt, threads; };
-    Cand cands[6];
+    Cand cands[7];
     int nc = 0;
+    // many token rows: 64-row strips halve the weight traffic per row again (each tile fetch
+    // feeds four MFMAs); they only pay once 64-row strips alone fill the device
+    if (64 * row_bytes <= lds_cap && T >= 64 * 128) cands[nc++] = {4, 512};
     if (mt_fit == 2 && T >= 32) { cands[nc++] = {2, 512}; cands[nc++] = {2, 256}; }
     if (mt_fit >= 1) { cands[nc++] = {1, 512}; cands[nc++] = {1, 256}; cands[nc++] = {1, 128}; }
     if (mt_fit == 0) { cands[nc++] = {2, 256}; }

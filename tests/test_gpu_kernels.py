@@ -118,6 +118,7 @@ BSR_CASES = [
     (48, 64, 32, 0.3, 2),
     (2048, 4096, 1024, 0.9, 0),  # BERT-large FFN
     (64, 6144, 64, 0.5, 0),      # input too wide for an LDS-staged strip
+    (8192, 768, 768, 0.8, 2),    # enough token rows for 64-row strips
 ]
 
 
@@ -305,9 +306,21 @@ def test_mha_block_config(et, B):
 @pytest.mark.parametrize("B,S,nh,hd,causal", [(1, 128, 12, 64, True), (2, 512, 16, 64, False),
                                               (1, 384, 12, 64, False), (3, 32, 4, 32, False),
                                               (2, 48, 2, 128, True), (1, 16, 1, 64, False),
-                                              (2, 272, 4, 64, True)])
+                                              (2, 272, 4, 64, True),
+                                              # many workgroups per (sequence, head), several key blocks each
+                                              (8, 512, 8, 64, False), (8, 512, 8, 64, True), (16, 256, 8, 32, True)])
 def test_mha_shapes(et, B, S, nh, hd, causal):
     got, want = run_mha(et, B, S, nh, hd, seed=60, causal=causal)
+    assert Hn.max_abs(got, want) <= 2e-3
+
+
+def test_mha_many_strips_with_padding(et):
+    """Right padding at S = 256: lengths that end inside a key block, on a block boundary, inside a
+    query strip, and a zero-length sequence (full blocks take the branch-free path, the last
+    block of a padded sequence the masked one)."""
+    B, S, nh, hd = 16, 256, 16, 64
+    lens = [256, 1, 0, 129, 128, 200, 255, 17] * 2
+    got, want = run_mha(et, B, S, nh, hd, seed=61, lens=lens)
     assert Hn.max_abs(got, want) <= 2e-3
 
 
