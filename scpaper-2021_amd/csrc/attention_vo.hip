@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void mha_probs_kernel(const ProbsArgs a) {
         if (kb < nkb) {
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                sc[kb][j] = exp2f(sc[kb][j] - m);
+                sc[kb][j] = __builtin_amdgcn_exp2f(sc[kb][j] - m);  // raw v_exp_f32: tiny results flush to zero
                 l += sc[kb][j];
             }
         }

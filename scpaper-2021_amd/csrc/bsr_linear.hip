@@ -117,11 +117,11 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     const h8 *src = reinterpret_cast<const h8 *>(a.X + (size_t)tok0 * a.in);
     h8 sv[kStageU];
     if (STAGE && !LN) {
+        // unconditional loads, index clamped into the strip: a load under a branch gets a
+        // basic block of its own and the register allocator's copies there make the wave
+        // wait for it on the spot — a full memory round trip before the weight loads go out
 #pragma unroll
-        for (int u = 0; u < kStageU; u++) {
-            const int idx = threadIdx.x + u * nthr;
-            if (idx < total_vec) sv[u] = src[idx];
-        }
+        for (int u = 0; u < kStageU; u++) sv[u] = src[min((int)threadIdx.x + u * nthr, total_vec - 1)];
     }
     // Fused SkipLayerNorm: a wave normalises rows wave, wave+nwave, ... of the strip
     // (at most kLnRows of them); all their loads are issued here, one round trip.
@@ -292,10 +292,7 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
         }
         for (int base = threadIdx.x + kStageU * nthr; base < total_vec; base += nthr * kStageU) {
 #pragma unroll
-            for (int u = 0; u < kStageU; u++) {
-                const int idx = base + u * nthr;
-                if (idx < total_vec) sv[u] = src[idx];
-            }
+            for (int u = 0; u < kStageU; u++) sv[u] = src[min(base + u * nthr, total_vec - 1)];
 #pragma unroll
             for (int u = 0; u < kStageU; u++) {
                 const int idx = base + u * nthr;
