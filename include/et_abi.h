@@ -123,6 +123,40 @@ int et_skipln_linear_bsr16_f16(const et_f16 *src, const et_f16 *skip,
                                const et_f16 *bias, et_f16 *Y, int T, int in,
                                int out, int act, et_stream stream);
 
+/* LayerNorm split between the Linear that produces a row and the Linear that
+ * consumes it, so that no normalisation kernel runs between them:
+ *
+ *   et_linear_bsr16_resid_stats_f16   V = X W^T + bias + resid  (fp16), and per token
+ *       the sum and the sum of squares of the stored values, split over
+ *       *stat_groups block-row groups: stats[stat_groups][T][2] floats (the caller
+ *       provides room for 16 groups).  No atomics: the sums are reproducible.
+ *   et_norm_linear_bsr16_f16          ln_out = (V - mean) * rstd * gamma + beta with
+ *       mean / rstd from those sums (variance E[v^2] - mean^2, fp32), written
+ *       [T x in], and Y = act(ln_out W^T + bias) — one launch.
+ *   et_norm_from_stats_f16            the normalisation alone (last layer of a stack).
+ *
+ * V is rounded to fp16 once, after the residual is added to the fp32 accumulator.
+ * Together they are SkipLayerNorm::forward (SkipLayerNorm/SkipLayerNorm.cu:73-82)
+ * between two Linear<tile_mat>::forward calls, i.e. the LN1/LN2 steps of
+ * Encoder<cfg>::forward (Encoder/Encoder.h:85-92).
+ * et_linear_bsr16_fused_ln_supported returns 1 when both kernels take the shape
+ * (the token strip, its statistics and the affine vectors must fit in LDS). */
+int et_linear_bsr16_fused_ln_supported(int T, int in, int out);
+int et_linear_bsr16_resid_stats_f16(const int32_t *row_ptr, const int32_t *col_idx,
+                                    const et_f16 *tiles, const et_f16 *bias,
+                                    const et_f16 *X, const et_f16 *resid, et_f16 *V,
+                                    float *stats, int *stat_groups, int T, int in,
+                                    int out, et_stream stream);
+int et_norm_linear_bsr16_f16(const et_f16 *V, const float *stats, int stat_groups,
+                             const et_f16 *gamma, const et_f16 *beta, float eps,
+                             et_f16 *ln_out, const int32_t *row_ptr,
+                             const int32_t *col_idx, const et_f16 *tiles,
+                             const et_f16 *bias, et_f16 *Y, int T, int in, int out,
+                             int act, et_stream stream);
+int et_norm_from_stats_f16(et_f16 *out, const et_f16 *V, const float *stats,
+                           int stat_groups, const et_f16 *gamma, const et_f16 *beta,
+                           int rows, int H, float eps, et_stream stream);
+
 /* Tuning hook: et_linear_bsr16_f16 with an explicit launch geometry — mt in
  * {1,2,4} 16-token blocks per workgroup strip, stage != 0 keeps the strip of X
  * in LDS, threads per workgroup (multiple of 64, <= 512) and block-rows of W per

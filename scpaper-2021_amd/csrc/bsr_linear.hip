@@ -47,7 +47,20 @@ struct BsrArgs {
     const _Float16 *ln_src, *ln_skip, *ln_gamma, *ln_beta;
     _Float16 *ln_out;
     float ln_eps;
+    // NORM prologue (kFxNorm): X holds v = (Linear output + residual) of a producer launched
+    // with kFxRes, st_in its per-row partial sums [st_groups][T][2] (sum, sum of squares); the
+    // strip is normalised with them, ln_gamma, ln_beta and ln_eps on its way into LDS and the
+    // workgroups of block-row group 0 write the normalised rows to ln_out.
+    const float *st_in;
+    int st_groups;
+    // RES epilogue (kFxRes): Y = X W^T + bias + resid, and st_out[group][token] = (sum, sum of
+    // squares) of the fp16 values this workgroup wrote for that token.
+    const _Float16 *resid;
+    float *st_out;
 };
+
+constexpr int kFxNorm = 1;
+constexpr int kFxRes = 2;
 
 constexpr int kXcds = 8;      // accelerator dies, each with a private L2
 constexpr int kLdsPad = 8;    // halfs
@@ -67,9 +80,12 @@ __device__ __forceinline__ int lane_read(int v, int lane) {
 
 // ACT is a template parameter: the epilogue carries no run-time branch and each
 // fused activation is a separately named kernel in a profile.
-template <int MT, bool STAGE, int ACT, int LN = 0>
+template <int MT, bool STAGE, int ACT, int LN = 0, int FX = 0>
 __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     static_assert(!LN || STAGE, "the fused LayerNorm prologue writes the strip to LDS");
+    static_assert(!(FX & kFxNorm) || (STAGE && !LN), "the NORM prologue writes the strip to LDS");
+    constexpr bool NORM = (FX & kFxNorm) != 0;
+    constexpr bool RES = (FX & kFxRes) != 0;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     _Float16 *xs = reinterpret_cast<_Float16 *>(smem_raw);
 
@@ -122,6 +138,18 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
         // wait for it on the spot — a full memory round trip before the weight loads go out
 #pragma unroll
         for (int u = 0; u < kStageU; u++) sv[u] = src[min((int)threadIdx.x + u * nthr, total_vec - 1)];
+    }
+    // NORM: per-row (mean, rstd) and the affine vectors go to LDS behind the strip
+    float2 *stat_lds = reinterpret_cast<float2 *>(xs + MT * 16 * lds_ld);
+    _Float16 *gam_lds = reinterpret_cast<_Float16 *>(stat_lds + MT * 16);
+    _Float16 *bet_lds = gam_lds + a.in;
+    if (NORM) {
+        if ((int)threadIdx.x < rows_here)
+            stat_lds[threadIdx.x] = row_stats(a.st_in, a.st_groups, a.T, tok0 + threadIdx.x, a.in, a.ln_eps);
+        for (int c = threadIdx.x; c < vec_per_row; c += nthr) {
+            *reinterpret_cast<h8 *>(gam_lds + c * 8) = reinterpret_cast<const h8 *>(a.ln_gamma)[c];
+            *reinterpret_cast<h8 *>(bet_lds + c * 8) = reinterpret_cast<const h8 *>(a.ln_beta)[c];
+        }
     }
     // Fused SkipLayerNorm: a wave normalises rows wave, wave+nwave, ... of the strip
     // (at most kLnRows of them); all their loads are issued here, one round trip.
@@ -276,13 +304,26 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
         __syncthreads();
     }
     // ---- strip copy: write the first batch, then the rest
+    if (NORM) __syncthreads();  // statistics and affine vectors are in LDS
+    // value written for strip vector (r, c): the loaded one, or its normalisation
+    auto strip_value = [&](h8 v, int r, int c) {
+        if (!NORM) return v;
+        const float2 st = stat_lds[r];
+        const h8 gm = *reinterpret_cast<const h8 *>(gam_lds + c * 8);
+        const h8 bt = *reinterpret_cast<const h8 *>(bet_lds + c * 8);
+        h8 o;
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] = (_Float16)norm_value((float)v[e], st.x, st.y, (float)gm[e], (float)bt[e]);
+        if (group == 0) *reinterpret_cast<h8 *>(a.ln_out + (size_t)(tok0 + r) * a.in + c * 8) = o;
+        return o;
+    };
     if (STAGE && !LN) {
         const int dr = nthr / vec_per_row, dc = nthr - dr * vec_per_row;  // (row, col) step of +nthr
         int r = threadIdx.x / vec_per_row, c = threadIdx.x - r * vec_per_row;
 #pragma unroll
         for (int u = 0; u < kStageU; u++) {
             const int idx = threadIdx.x + u * nthr;
-            if (idx < total_vec) *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) = sv[u];
+            if (idx < total_vec) *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) = strip_value(sv[u], r, c);
             r += dr;
             c += dc;
             if (c >= vec_per_row) {
@@ -296,7 +337,7 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
 #pragma unroll
             for (int u = 0; u < kStageU; u++) {
                 const int idx = base + u * nthr;
-                if (idx < total_vec) *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) = sv[u];
+                if (idx < total_vec) *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) = strip_value(sv[u], r, c);
                 r += dr;
                 c += dc;
                 if (c >= vec_per_row) {
@@ -333,15 +374,29 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     for (int m = 0; m < MT; m++) acc[m] = f4{0.f, 0.f, 0.f, 0.f};
 
     // bias + activation + store of one finished block-row, then clear
+    float st1[MT], st2[MT];  // RES: this lane's sums over the values it wrote, per token block
+#pragma unroll
+    for (int m = 0; m < MT; m++) st1[m] = st2[m] = 0.0f;
     auto flush = [&](int wave_row, h4 bv) {
         const int f0 = (rb_begin + wave + nwave * wave_row) * 16 + g * 4;
 #pragma unroll
         for (int m = 0; m < MT; m++) {
             if (tok_ok[m]) {
-                h4 o;
-#pragma unroll
-                for (int j = 0; j < 4; j++) o[j] = (_Float16)act_fixed<ACT>(acc[m][j] + (float)bv[j]);
                 const int tok = tok0 + m * 16 + r16;
+                h4 o;
+                if (RES) {
+                    const h4 rv = *reinterpret_cast<const h4 *>(a.resid + (size_t)tok * a.out + f0);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        o[j] = (_Float16)(acc[m][j] + (float)bv[j] + (float)rv[j]);
+                        const float w16 = (float)o[j];  // the statistics describe the stored values
+                        st1[m] += w16;
+                        st2[m] = __builtin_fmaf(w16, w16, st2[m]);
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; j++) o[j] = (_Float16)act_fixed<ACT>(acc[m][j] + (float)bv[j]);
+                }
                 *reinterpret_cast<h4 *>(a.Y + (size_t)tok * a.out + f0) = o;
             }
             acc[m] = f4{0.f, 0.f, 0.f, 0.f};
@@ -382,6 +437,34 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
             h4 bv = {0, 0, 0, 0};
             if (a.bias) bv = *reinterpret_cast<const h4 *>(a.bias + (rb_begin + wave + nwave * r) * 16 + g * 4);
             flush(r, bv);
+        }
+    }
+    if (RES) {
+        // per token: the four lanes that share it, then the waves (through LDS, in wave
+        // order), then one float2 per token and block-row group — no atomics, so the sums
+        // and everything normalised with them are reproducible
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            st1[m] += __shfl_xor(st1[m], 16, 64);
+            st1[m] += __shfl_xor(st1[m], 32, 64);
+            st2[m] += __shfl_xor(st2[m], 16, 64);
+            st2[m] += __shfl_xor(st2[m], 32, 64);
+        }
+        __syncthreads();  // every wave is done reading the strip
+        float2 *red = reinterpret_cast<float2 *>(smem_raw);
+        if (g == 0) {
+#pragma unroll
+            for (int m = 0; m < MT; m++) red[wave * (MT * 16) + m * 16 + r16] = float2{st1[m], st2[m]};
+        }
+        __syncthreads();
+        if ((int)threadIdx.x < rows_here) {
+            float s1 = 0.0f, s2 = 0.0f;
+            for (int wv = 0; wv < nwave; wv++) {
+                const float2 pr = red[wv * (MT * 16) + threadIdx.x];
+                s1 += pr.x;
+                s2 += pr.y;
+            }
+            *reinterpret_cast<float2 *>(a.st_out + ((size_t)group * a.T + tok0 + threadIdx.x) * 2) = float2{s1, s2};
         }
     }
 }
@@ -469,9 +552,40 @@ static BsrPlan plan_bsr_ln(int T, int in, int out) {
     return p;
 }
 
-template <int MT, bool STAGE, int ACT, int LN = 0>
+// Geometry of the kernels with the NORM prologue or the RES epilogue: staged strips of 16 or
+// 32 rows; a RES producer splits a row over at most kMaxStatGroups block-row groups.
+// stage == false in the result means the shape is not supported by these kernels.
+static BsrPlan plan_bsr_fx(int T, int in, int out, int fx) {
+    const size_t lds_cap = 160 * 1024;
+    const size_t row_bytes = (size_t)(in + kLdsPad) * sizeof(_Float16);
+    const size_t extra = (fx & kFxNorm) ? (size_t)4 * in : 0;  // gamma and beta
+    const int nbr = out / 16;
+    BsrPlan p{};
+    auto fits = [&](int mt, size_t cap) { return mt * 16 * (row_bytes + sizeof(float2)) + extra <= cap; };
+    p.stage = fits(1, lds_cap);
+    p.mt = (T >= 32 && fits(2, lds_cap / 2)) ? 2 : 1;
+    p.threads = 512;
+    const int nwave = 8;
+    const int strips = (T + p.mt * 16 - 1) / (p.mt * 16);
+    int groups = strips >= 256 ? 1 : 256 / strips;
+    if ((fx & kFxRes) && groups > kMaxStatGroups) groups = kMaxStatGroups;
+    int rpw = (nbr + groups - 1) / groups;
+    rpw = ((rpw + nwave - 1) / nwave) * nwave;
+    if (rpw > nbr) rpw = nbr;
+    if (rpw > kMaxWaveRows * nwave) {
+        rpw = kMaxWaveRows * nwave;
+        if ((fx & kFxRes) && (nbr + rpw - 1) / rpw > kMaxStatGroups) p.stage = false;  // out > 131072
+    }
+    p.rows_per_wg = rpw;
+    p.lds = p.mt * 16 * (row_bytes + sizeof(float2)) + extra;
+    const size_t red = (size_t)nwave * p.mt * 16 * sizeof(float2);
+    if ((fx & kFxRes) && p.lds < red) p.lds = red;
+    return p;
+}
+
+template <int MT, bool STAGE, int ACT, int LN = 0, int FX = 0>
 static int launch_bsr_act(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
-    auto kernel = bsr16_linear_kernel<MT, STAGE, ACT, LN>;
+    auto kernel = bsr16_linear_kernel<MT, STAGE, ACT, LN, FX>;
     if (p.lds > 64 * 1024) {
         static bool raised = false;  // per instantiation
         if (!raised) {
@@ -518,6 +632,22 @@ static int dispatch_bsr_ln_mt(const BsrArgs &args, const BsrPlan &p, hipStream_t
 }
 static int dispatch_bsr_ln(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
     return p.mt == 2 ? dispatch_bsr_ln_mt<2>(args, p, stream) : dispatch_bsr_ln_mt<1>(args, p, stream);
+}
+
+template <int MT, int FX>
+static int dispatch_bsr_fx_act(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
+    switch (args.act) {
+        case ET_ACT_RELU: return launch_bsr_act<MT, true, ET_ACT_RELU, 0, FX>(args, p, stream);
+        case ET_ACT_GELU: return launch_bsr_act<MT, true, ET_ACT_GELU, 0, FX>(args, p, stream);
+        default: return launch_bsr_act<MT, true, ET_ACT_NONE, 0, FX>(args, p, stream);
+    }
+}
+static int dispatch_bsr_norm(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
+    return p.mt == 2 ? dispatch_bsr_fx_act<2, kFxNorm>(args, p, stream) : dispatch_bsr_fx_act<1, kFxNorm>(args, p, stream);
+}
+static int dispatch_bsr_res(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
+    return p.mt == 2 ? launch_bsr_act<2, true, ET_ACT_NONE, 0, kFxRes>(args, p, stream)
+                     : launch_bsr_act<1, true, ET_ACT_NONE, 0, kFxRes>(args, p, stream);
 }
 
 static int dispatch_bsr(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
@@ -571,7 +701,7 @@ int et_linear_bsr16_f16(const int32_t *row_ptr, const int32_t *col_idx, const et
                  out,
                  0,
                  act,
-                 nullptr, nullptr, nullptr, nullptr, nullptr, 0.0f};
+                 nullptr, nullptr, nullptr, nullptr, nullptr, 0.0f, nullptr, 0, nullptr, nullptr};
     BsrPlan p = plan_bsr(T, in, out);
     args.rows_per_wg = p.rows_per_wg;
     return dispatch_bsr(args, p, as_stream(stream));
@@ -611,8 +741,77 @@ int et_skipln_linear_bsr16_f16(const et_f16 *src, const et_f16 *skip, const et_f
                  reinterpret_cast<const _Float16 *>(gamma),
                  reinterpret_cast<const _Float16 *>(beta),
                  reinterpret_cast<_Float16 *>(ln_out),
-                 eps};
+                 eps,
+                 nullptr, 0, nullptr, nullptr};
     return dispatch_bsr_ln(args, p, as_stream(stream));
+}
+
+int et_linear_bsr16_fused_ln_supported(int T, int in, int out) {
+    if (T <= 0 || in <= 0 || out <= 0 || T % 16 || in % 16 || out % 16) return 0;
+    return plan_bsr_fx(T, in, out, kFxNorm).stage && plan_bsr_fx(T, in, out, kFxRes).stage ? 1 : 0;
+}
+
+int et_linear_bsr16_resid_stats_f16(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles,
+                                    const et_f16 *bias, const et_f16 *X, const et_f16 *resid, et_f16 *V,
+                                    float *stats, int *stat_groups, int T, int in, int out, et_stream stream) {
+    ET_REQUIRE(resid && stats && stat_groups, ET_ERR_INVALID_ARG, "et_linear_bsr16_resid_stats_f16: NULL pointer");
+    int s = bsr_check(row_ptr, col_idx, tiles, X, V, T, in, out, ET_ACT_NONE);
+    if (s != ET_OK) return s;
+    BsrPlan p = plan_bsr_fx(T, in, out, kFxRes);
+    ET_REQUIRE(p.stage, ET_ERR_UNSUPPORTED, "et_linear_bsr16_resid_stats_f16: in=%d out=%d outside the staged range", in,
+               out);
+    *stat_groups = (out / 16 + p.rows_per_wg - 1) / p.rows_per_wg;
+    if (T == 0) return ET_OK;
+    BsrArgs args{row_ptr,
+                 col_idx,
+                 reinterpret_cast<const _Float16 *>(tiles),
+                 reinterpret_cast<const _Float16 *>(bias),
+                 reinterpret_cast<const _Float16 *>(X),
+                 reinterpret_cast<_Float16 *>(V),
+                 T,
+                 in,
+                 out,
+                 p.rows_per_wg,
+                 ET_ACT_NONE,
+                 nullptr, nullptr, nullptr, nullptr, nullptr, 0.0f,
+                 nullptr, 0,
+                 reinterpret_cast<const _Float16 *>(resid),
+                 stats};
+    return dispatch_bsr_res(args, p, as_stream(stream));
+}
+
+int et_norm_linear_bsr16_f16(const et_f16 *V, const float *stats, int stat_groups, const et_f16 *gamma,
+                             const et_f16 *beta, float eps, et_f16 *ln_out, const int32_t *row_ptr,
+                             const int32_t *col_idx, const et_f16 *tiles, const et_f16 *bias, et_f16 *Y, int T,
+                             int in, int out, int act, et_stream stream) {
+    ET_REQUIRE(stats && gamma && beta && ln_out, ET_ERR_INVALID_ARG, "et_norm_linear_bsr16_f16: NULL pointer");
+    ET_REQUIRE(stat_groups >= 1 && stat_groups <= kMaxStatGroups, ET_ERR_INVALID_ARG,
+               "et_norm_linear_bsr16_f16: stat_groups=%d must be in [1, %d]", stat_groups, kMaxStatGroups);
+    ET_REQUIRE(ln_out != V, ET_ERR_INVALID_ARG, "et_norm_linear_bsr16_f16: ln_out must not alias V");
+    int s = bsr_check(row_ptr, col_idx, tiles, V, Y, T, in, out, act);
+    if (s != ET_OK) return s;
+    BsrPlan p = plan_bsr_fx(T, in, out, kFxNorm);
+    ET_REQUIRE(p.stage, ET_ERR_UNSUPPORTED, "et_norm_linear_bsr16_f16: in=%d outside the staged range", in);
+    if (T == 0) return ET_OK;
+    BsrArgs args{row_ptr,
+                 col_idx,
+                 reinterpret_cast<const _Float16 *>(tiles),
+                 reinterpret_cast<const _Float16 *>(bias),
+                 reinterpret_cast<const _Float16 *>(V),
+                 reinterpret_cast<_Float16 *>(Y),
+                 T,
+                 in,
+                 out,
+                 p.rows_per_wg,
+                 act,
+                 nullptr, nullptr,
+                 reinterpret_cast<const _Float16 *>(gamma),
+                 reinterpret_cast<const _Float16 *>(beta),
+                 reinterpret_cast<_Float16 *>(ln_out),
+                 eps,
+                 stats, stat_groups,
+                 nullptr, nullptr};
+    return dispatch_bsr_norm(args, p, as_stream(stream));
 }
 
 // Tuning hook: same computation with an explicit launch geometry.  mt in
@@ -650,7 +849,7 @@ int et_linear_bsr16_f16_geom(const int32_t *row_ptr, const int32_t *col_idx, con
                  out,
                  rows_per_wg,
                  act,
-                 nullptr, nullptr, nullptr, nullptr, nullptr, 0.0f};
+                 nullptr, nullptr, nullptr, nullptr, nullptr, 0.0f, nullptr, 0, nullptr, nullptr};
     return dispatch_bsr(args, p, as_stream(stream));
 }
 

@@ -88,4 +88,36 @@ __device__ __forceinline__ float apply_act(float x, int act) {
     return x;
 }
 
+// ---- LayerNorm split between a producer and a consumer kernel ----------------
+// The producer of a row (a Linear with the residual added in its epilogue) emits, per
+// block-row group, the sum and the sum of squares of the values it stored; any consumer
+// normalises with them.
+constexpr int kMaxStatGroups = 16;  // block-row groups a RES producer may split a row over
+
+// mean and reciprocal standard deviation of a row of H values from its partial sums,
+// added in group order (every consumer of the same sums gets the same bits).  All loads are
+// issued before the first addition (index clamped, surplus selected away): a loop with a
+// run-time trip count would wait for each load in turn.
+__device__ __forceinline__ float2 row_stats(const float *st, int groups, int T, int tok, int H, float eps) {
+    float2 p[kMaxStatGroups];
+#pragma unroll
+    for (int gi = 0; gi < kMaxStatGroups; gi++)
+        p[gi] = *reinterpret_cast<const float2 *>(st + ((size_t)min(gi, groups - 1) * T + tok) * 2);
+    float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+    for (int gi = 0; gi < kMaxStatGroups; gi++) {
+        s1 += gi < groups ? p[gi].x : 0.0f;
+        s2 += gi < groups ? p[gi].y : 0.0f;
+    }
+    const float inv_h = 1.0f / (float)H;
+    const float mean = s1 * inv_h;
+    const float var = fmaxf(__builtin_fmaf(-mean, mean, s2 * inv_h), 0.0f);
+    return float2{mean, rsqrtf(var + eps)};
+}
+
+// one normalised value: the same two roundings wherever it is evaluated
+__device__ __forceinline__ float norm_value(float v, float mean, float rstd, float gm, float bt) {
+    return __builtin_fmaf((v - mean) * rstd, gm, bt);
+}
+
 }  // namespace et
