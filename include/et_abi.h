@@ -123,39 +123,48 @@ int et_skipln_linear_bsr16_f16(const et_f16 *src, const et_f16 *skip,
                                const et_f16 *bias, et_f16 *Y, int T, int in,
                                int out, int act, et_stream stream);
 
-/* LayerNorm split between the Linear that produces a row and the Linear that
- * consumes it, so that no normalisation kernel runs between them:
+/* SkipLayerNorm split between the Linear that produces its first input and the
+ * Linear that consumes its output, so that no normalisation kernel runs between
+ * them:
  *
- *   et_linear_bsr16_resid_stats_f16   V = X W^T + bias + resid  (fp16), and per token
- *       the sum and the sum of squares of the stored values, split over
- *       *stat_groups block-row groups: stats[stat_groups][T][2] floats (the caller
- *       provides room for 16 groups).  No atomics: the sums are reproducible.
- *   et_norm_linear_bsr16_f16          ln_out = (V - mean) * rstd * gamma + beta with
- *       mean / rstd from those sums (variance E[v^2] - mean^2, fp32), written
- *       [T x in], and Y = act(ln_out W^T + bias) — one launch.
- *   et_norm_from_stats_f16            the normalisation alone (last layer of a stack).
+ *   et_linear_bsr16_resid_stats_f16   V = X W^T + bias as usual, plus, per token,
+ *       the sum and the sum of squares of (V as stored + resid), split over
+ *       *stat_groups block-row groups: stats[stat_groups][T][2] floats (the
+ *       caller provides room for 16 groups).  No atomics: the sums are reproducible.
+ *   et_norm_linear_bsr16_f16          ln_out = (V + skip - mean) * rstd * gamma + beta
+ *       with mean / rstd from those sums (variance E[v^2] - mean^2, fp32; skip is
+ *       the resid of the producer; the sum is formed in fp32 and never stored),
+ *       written [T x in], and Y = act(ln_out W^T + bias) — one launch.
+ *   et_norm_from_stats_f16            the normalisation alone (last layer of a stack);
+ *       bit-identical to the ln_out of the fused form.
  *
- * V is rounded to fp16 once, after the residual is added to the fp32 accumulator.
  * Together they are SkipLayerNorm::forward (SkipLayerNorm/SkipLayerNorm.cu:73-82)
  * between two Linear<tile_mat>::forward calls, i.e. the LN1/LN2 steps of
- * Encoder<cfg>::forward (Encoder/Encoder.h:85-92).
+ * Encoder<cfg>::forward (Encoder/Encoder.h:85-92), with the reference's rounding
+ * points (Linear output and LayerNorm output in fp16).
  * et_linear_bsr16_fused_ln_supported returns 1 when both kernels take the shape
- * (the token strip, its statistics and the affine vectors must fit in LDS). */
+ * (the token strip, its statistics and the affine vectors must fit in LDS).
+ * Measured on MI355X at 1024 x 768 the pair costs as much as the LayerNorm
+ * kernel it removes (the producer gains 0.6-1.3 us, the consumer 2.2 us), so the
+ * class layer keeps et_skipln_linear_bsr16_f16 + et_skip_layernorm_f16; these
+ * entry points serve callers whose shapes make a separate pass over the
+ * activations the larger cost. */
 int et_linear_bsr16_fused_ln_supported(int T, int in, int out);
 int et_linear_bsr16_resid_stats_f16(const int32_t *row_ptr, const int32_t *col_idx,
                                     const et_f16 *tiles, const et_f16 *bias,
                                     const et_f16 *X, const et_f16 *resid, et_f16 *V,
                                     float *stats, int *stat_groups, int T, int in,
                                     int out, et_stream stream);
-int et_norm_linear_bsr16_f16(const et_f16 *V, const float *stats, int stat_groups,
-                             const et_f16 *gamma, const et_f16 *beta, float eps,
-                             et_f16 *ln_out, const int32_t *row_ptr,
+int et_norm_linear_bsr16_f16(const et_f16 *V, const et_f16 *skip, const float *stats,
+                             int stat_groups, const et_f16 *gamma, const et_f16 *beta,
+                             float eps, et_f16 *ln_out, const int32_t *row_ptr,
                              const int32_t *col_idx, const et_f16 *tiles,
                              const et_f16 *bias, et_f16 *Y, int T, int in, int out,
                              int act, et_stream stream);
-int et_norm_from_stats_f16(et_f16 *out, const et_f16 *V, const float *stats,
-                           int stat_groups, const et_f16 *gamma, const et_f16 *beta,
-                           int rows, int H, float eps, et_stream stream);
+int et_norm_from_stats_f16(et_f16 *out, const et_f16 *V, const et_f16 *skip,
+                           const float *stats, int stat_groups, const et_f16 *gamma,
+                           const et_f16 *beta, int rows, int H, float eps,
+                           et_stream stream);
 
 /* Tuning hook: et_linear_bsr16_f16 with an explicit launch geometry — mt in
  * {1,2,4} 16-token blocks per workgroup strip, stage != 0 keeps the strip of X

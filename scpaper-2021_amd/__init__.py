@@ -66,8 +66,8 @@ _SIGNATURES = {
     "et_skipln_linear_bsr16_f16": (_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_linear_bsr16_fused_ln_supported": (_i, _i, _i),
     "et_linear_bsr16_resid_stats_f16": (_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, C.POINTER(_i), _i, _i, _i, _vp),
-    "et_norm_linear_bsr16_f16": (_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
-    "et_norm_from_stats_f16": (_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _f, _vp),
+    "et_norm_linear_bsr16_f16": (_vp, _vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_norm_from_stats_f16": (_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _f, _vp),
     "et_linear_dense_f32": (_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_mha_fused_f32": (_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp),
     "et_skip_layernorm_f32": (_vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp),

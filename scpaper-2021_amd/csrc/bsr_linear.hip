@@ -47,14 +47,15 @@ struct BsrArgs {
     const _Float16 *ln_src, *ln_skip, *ln_gamma, *ln_beta;
     _Float16 *ln_out;
     float ln_eps;
-    // NORM prologue (kFxNorm): X holds v = (Linear output + residual) of a producer launched
-    // with kFxRes, st_in its per-row partial sums [st_groups][T][2] (sum, sum of squares); the
-    // strip is normalised with them, ln_gamma, ln_beta and ln_eps on its way into LDS and the
-    // workgroups of block-row group 0 write the normalised rows to ln_out.
+    // NORM prologue (kFxNorm): X holds the output of a producer launched with kFxRes, ln_skip
+    // the residual it was given and st_in its per-row partial sums [st_groups][T][2] (sum, sum
+    // of squares of output + residual); the strip X + ln_skip is normalised with them,
+    // ln_gamma, ln_beta and ln_eps on its way into LDS and the workgroups of block-row group 0
+    // write the normalised rows to ln_out.  The sum is never rounded to fp16.
     const float *st_in;
     int st_groups;
-    // RES epilogue (kFxRes): Y = X W^T + bias + resid, and st_out[group][token] = (sum, sum of
-    // squares) of the fp16 values this workgroup wrote for that token.
+    // RES epilogue (kFxRes): Y = X W^T + bias as usual, and st_out[group][token] = (sum, sum
+    // of squares) of (Y as stored + resid) over the features of this workgroup.
     const _Float16 *resid;
     float *st_out;
 };
@@ -138,6 +139,12 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
         // wait for it on the spot — a full memory round trip before the weight loads go out
 #pragma unroll
         for (int u = 0; u < kStageU; u++) sv[u] = src[min((int)threadIdx.x + u * nthr, total_vec - 1)];
+    }
+    const h8 *src_skip = NORM ? reinterpret_cast<const h8 *>(a.ln_skip + (size_t)tok0 * a.in) : nullptr;
+    h8 sk[NORM ? kStageU : 1];
+    if (NORM) {
+#pragma unroll
+        for (int u = 0; u < kStageU; u++) sk[u] = src_skip[min((int)threadIdx.x + u * nthr, total_vec - 1)];
     }
     // NORM: per-row (mean, rstd) and the affine vectors go to LDS behind the strip
     float2 *stat_lds = reinterpret_cast<float2 *>(xs + MT * 16 * lds_ld);
@@ -306,14 +313,15 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     // ---- strip copy: write the first batch, then the rest
     if (NORM) __syncthreads();  // statistics and affine vectors are in LDS
     // value written for strip vector (r, c): the loaded one, or its normalisation
-    auto strip_value = [&](h8 v, int r, int c) {
+    auto strip_value = [&](h8 v, h8 skp, int r, int c) {
         if (!NORM) return v;
         const float2 st = stat_lds[r];
         const h8 gm = *reinterpret_cast<const h8 *>(gam_lds + c * 8);
         const h8 bt = *reinterpret_cast<const h8 *>(bet_lds + c * 8);
         h8 o;
 #pragma unroll
-        for (int e = 0; e < 8; e++) o[e] = (_Float16)norm_value((float)v[e], st.x, st.y, (float)gm[e], (float)bt[e]);
+        for (int e = 0; e < 8; e++)
+            o[e] = (_Float16)norm_value((float)v[e] + (float)skp[e], st.x, st.y, (float)gm[e], (float)bt[e]);
         if (group == 0) *reinterpret_cast<h8 *>(a.ln_out + (size_t)(tok0 + r) * a.in + c * 8) = o;
         return o;
     };
@@ -323,7 +331,7 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
 #pragma unroll
         for (int u = 0; u < kStageU; u++) {
             const int idx = threadIdx.x + u * nthr;
-            if (idx < total_vec) *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) = strip_value(sv[u], r, c);
+            if (idx < total_vec) *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) = strip_value(sv[u], sk[NORM ? u : 0], r, c);
             r += dr;
             c += dc;
             if (c >= vec_per_row) {
@@ -334,10 +342,14 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
         for (int base = threadIdx.x + kStageU * nthr; base < total_vec; base += nthr * kStageU) {
 #pragma unroll
             for (int u = 0; u < kStageU; u++) sv[u] = src[min(base + u * nthr, total_vec - 1)];
+            if (NORM) {
+#pragma unroll
+                for (int u = 0; u < kStageU; u++) sk[u] = src_skip[min(base + u * nthr, total_vec - 1)];
+            }
 #pragma unroll
             for (int u = 0; u < kStageU; u++) {
                 const int idx = base + u * nthr;
-                if (idx < total_vec) *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) = strip_value(sv[u], r, c);
+                if (idx < total_vec) *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) = strip_value(sv[u], sk[NORM ? u : 0], r, c);
                 r += dr;
                 c += dc;
                 if (c >= vec_per_row) {
@@ -388,10 +400,10 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
                     const h4 rv = *reinterpret_cast<const h4 *>(a.resid + (size_t)tok * a.out + f0);
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
-                        o[j] = (_Float16)(acc[m][j] + (float)bv[j] + (float)rv[j]);
-                        const float w16 = (float)o[j];  // the statistics describe the stored values
-                        st1[m] += w16;
-                        st2[m] = __builtin_fmaf(w16, w16, st2[m]);
+                        o[j] = (_Float16)(acc[m][j] + (float)bv[j]);
+                        const float v = (float)o[j] + (float)rv[j];  // what the consumer will form
+                        st1[m] += v;
+                        st2[m] = __builtin_fmaf(v, v, st2[m]);
                     }
                 } else {
 #pragma unroll
@@ -780,14 +792,15 @@ int et_linear_bsr16_resid_stats_f16(const int32_t *row_ptr, const int32_t *col_i
     return dispatch_bsr_res(args, p, as_stream(stream));
 }
 
-int et_norm_linear_bsr16_f16(const et_f16 *V, const float *stats, int stat_groups, const et_f16 *gamma,
-                             const et_f16 *beta, float eps, et_f16 *ln_out, const int32_t *row_ptr,
+int et_norm_linear_bsr16_f16(const et_f16 *V, const et_f16 *skip, const float *stats, int stat_groups,
+                             const et_f16 *gamma, const et_f16 *beta, float eps, et_f16 *ln_out, const int32_t *row_ptr,
                              const int32_t *col_idx, const et_f16 *tiles, const et_f16 *bias, et_f16 *Y, int T,
                              int in, int out, int act, et_stream stream) {
-    ET_REQUIRE(stats && gamma && beta && ln_out, ET_ERR_INVALID_ARG, "et_norm_linear_bsr16_f16: NULL pointer");
+    ET_REQUIRE(skip && stats && gamma && beta && ln_out, ET_ERR_INVALID_ARG, "et_norm_linear_bsr16_f16: NULL pointer");
     ET_REQUIRE(stat_groups >= 1 && stat_groups <= kMaxStatGroups, ET_ERR_INVALID_ARG,
                "et_norm_linear_bsr16_f16: stat_groups=%d must be in [1, %d]", stat_groups, kMaxStatGroups);
-    ET_REQUIRE(ln_out != V, ET_ERR_INVALID_ARG, "et_norm_linear_bsr16_f16: ln_out must not alias V");
+    ET_REQUIRE(ln_out != V && ln_out != skip, ET_ERR_INVALID_ARG,
+               "et_norm_linear_bsr16_f16: ln_out must not alias V or skip");
     int s = bsr_check(row_ptr, col_idx, tiles, V, Y, T, in, out, act);
     if (s != ET_OK) return s;
     BsrPlan p = plan_bsr_fx(T, in, out, kFxNorm);
@@ -804,7 +817,8 @@ int et_norm_linear_bsr16_f16(const et_f16 *V, const float *stats, int stat_group
                  out,
                  p.rows_per_wg,
                  act,
-                 nullptr, nullptr,
+                 nullptr,
+                 reinterpret_cast<const _Float16 *>(skip),
                  reinterpret_cast<const _Float16 *>(gamma),
                  reinterpret_cast<const _Float16 *>(beta),
                  reinterpret_cast<_Float16 *>(ln_out),

@@ -123,10 +123,11 @@ __global__ __launch_bounds__(kWave *kRowsPerBlock) void layernorm_rows_kernel(
     }
 }
 
-// out = normalisation of V with the row statistics a producer kernel left behind: the
+// out = normalisation of V + skip with the row statistics a producer kernel left behind: the
 // stand-alone form of the NORM prologue of the tile-sparse Linear (same arithmetic, same bits).
 __global__ __launch_bounds__(256) void norm_from_stats_kernel(_Float16 *__restrict__ out,
                                                               const _Float16 *__restrict__ V,
+                                                              const _Float16 *__restrict__ skip,
                                                               const float *__restrict__ stats, int groups,
                                                               const _Float16 *__restrict__ gamma,
                                                               const _Float16 *__restrict__ beta, int rows,
@@ -137,13 +138,15 @@ __global__ __launch_bounds__(256) void norm_from_stats_kernel(_Float16 *__restri
     const float2 st = row_stats(stats, groups, rows, row, H, eps);
     const int vecs = H >> 3;
     const h8 *v = reinterpret_cast<const h8 *>(V + (size_t)row * H);
+    const h8 *k = reinterpret_cast<const h8 *>(skip + (size_t)row * H);
     h8 *o = reinterpret_cast<h8 *>(out + (size_t)row * H);
     for (int c = lane; c < vecs; c += kWave) {
-        const h8 x = v[c];
+        const h8 x = v[c], s = k[c];
         const h8 gm = reinterpret_cast<const h8 *>(gamma)[c], bt = reinterpret_cast<const h8 *>(beta)[c];
         h8 y;
 #pragma unroll
-        for (int e = 0; e < 8; e++) y[e] = (_Float16)norm_value((float)x[e], st.x, st.y, (float)gm[e], (float)bt[e]);
+        for (int e = 0; e < 8; e++)
+            y[e] = (_Float16)norm_value((float)x[e] + (float)s[e], st.x, st.y, (float)gm[e], (float)bt[e]);
         o[c] = y;
     }
 }
@@ -214,17 +217,18 @@ int et_layernorm_f16(et_f16 *out, const et_f16 *src, const et_f16 *gamma, const 
         H, eps, as_stream(stream));
 }
 
-int et_norm_from_stats_f16(et_f16 *out, const et_f16 *V, const float *stats, int stat_groups,
+int et_norm_from_stats_f16(et_f16 *out, const et_f16 *V, const et_f16 *skip, const float *stats, int stat_groups,
                            const et_f16 *gamma, const et_f16 *beta, int rows, int H, float eps,
                            et_stream stream) {
-    ET_REQUIRE(out && V && stats && gamma && beta, ET_ERR_INVALID_ARG, "et_norm_from_stats_f16: NULL pointer");
+    ET_REQUIRE(out && V && skip && stats && gamma && beta, ET_ERR_INVALID_ARG, "et_norm_from_stats_f16: NULL pointer");
     ET_REQUIRE(rows >= 0 && H > 0, ET_ERR_INVALID_ARG, "et_norm_from_stats_f16: rows=%d H=%d", rows, H);
     ET_REQUIRE(stat_groups >= 1 && stat_groups <= kMaxStatGroups, ET_ERR_INVALID_ARG,
                "et_norm_from_stats_f16: stat_groups=%d must be in [1, %d]", stat_groups, kMaxStatGroups);
     ET_REQUIRE(H % 8 == 0, ET_ERR_UNSUPPORTED, "et_norm_from_stats_f16: H=%d must be a multiple of 8", H);
     if (rows == 0) return ET_OK;
     norm_from_stats_kernel<<<(rows + kRowsPerBlock - 1) / kRowsPerBlock, kWave * kRowsPerBlock, 0, as_stream(stream)>>>(
-        reinterpret_cast<_Float16 *>(out), reinterpret_cast<const _Float16 *>(V), stats, stat_groups,
+        reinterpret_cast<_Float16 *>(out), reinterpret_cast<const _Float16 *>(V),
+        reinterpret_cast<const _Float16 *>(skip), stats, stat_groups,
         reinterpret_cast<const _Float16 *>(gamma), reinterpret_cast<const _Float16 *>(beta), rows, H, eps);
     return check_launch("norm_from_stats_kernel");
 }

@@ -255,9 +255,9 @@ def test_skipln_linear_bsr16_in_place_falls_back(et):
                                                      (48, 256, 512, 64, 0.5, 1), (16, 32, 16, 16, 0.0, 0),
                                                      (2048, 4096, 1024, 4096, 0.9, 2), (272, 160, 208, 800, 0.5, 0)])
 def test_split_layernorm_between_two_tile_linears(et, T, n_in, n_mid, n_out, sp, act):
-    """Producer Linear (+ residual, row statistics) -> consumer Linear (normalises while staging):
-    V, the statistics, the normalised rows and Y against the oracle; the stand-alone
-    normalisation from the same statistics is bit-identical to the fused one."""
+    """Producer Linear (row statistics of output + residual) -> consumer Linear (adds the two and
+    normalises while staging): V, the statistics, the normalised rows and Y against the oracle;
+    the stand-alone normalisation from the same statistics is bit-identical to the fused one."""
     import ctypes as C
     lib = et.lib()
     w1 = Hn.BsrWeight(n_mid, n_in, sp, seed=41, bias_std=0.05).upload(et)
@@ -267,36 +267,38 @@ def test_split_layernorm_between_two_tile_linears(et, T, n_in, n_mid, n_out, sp,
     beta = Hn.randn((n_mid,), 50, 0.1)
     d_v = et.DeviceBuffer.empty((T, n_mid), np.float16)
     d_stats = et.DeviceBuffer.empty((16, T, 2), np.float32)
+    d_resid = up(et, resid)
     groups = C.c_int(0)
     assert lib.et_linear_bsr16_fused_ln_supported(T, n_in, n_mid) == 1
     et.check(lib.et_linear_bsr16_resid_stats_f16(w1.d_row_ptr.ptr, w1.d_col_idx.ptr, w1.d_tiles.ptr, w1.d_bias.ptr,
-                                                 up(et, x).ptr, up(et, resid).ptr, d_v.ptr, d_stats.ptr,
+                                                 up(et, x).ptr, d_resid.ptr, d_v.ptr, d_stats.ptr,
                                                  C.byref(groups), T, n_in, n_mid, None))
     G = groups.value
     assert 1 <= G <= 16
     v = d_v.numpy()
-    want_v = (L.linear(Hn.f32(x), Hn.f32(w1.dense), Hn.f32(w1.bias), None, None) + Hn.f32(resid)).half().numpy()
-    assert Hn.max_abs(v, want_v) <= 8e-3  # one fp16 rounding of an O(8) value
+    want_v = L.linear(Hn.f32(x), Hn.f32(w1.dense), Hn.f32(w1.bias), None, torch.float16).numpy()
+    assert Hn.max_abs(v, want_v) <= 4e-3  # the plain Linear output
     st = d_stats.numpy()[:G].astype(np.float64).sum(0)
-    v64 = v.astype(np.float64)
-    assert np.allclose(st[:, 0], v64.sum(1), rtol=1e-5, atol=1e-3)
-    assert np.allclose(st[:, 1], (v64 * v64).sum(1), rtol=1e-5, atol=1e-3)
+    s64 = v.astype(np.float64) + resid.astype(np.float64)
+    assert np.allclose(st[:, 0], s64.sum(1), rtol=1e-5, atol=1e-3)
+    assert np.allclose(st[:, 1], (s64 * s64).sum(1), rtol=1e-5, atol=1e-3)
 
     d_ln = et.DeviceBuffer.empty((T, n_mid), np.float16)
     d_y = et.DeviceBuffer.empty((T, n_out), np.float16)
     d_g, d_b = up(et, gamma), up(et, beta)
-    et.check(lib.et_norm_linear_bsr16_f16(d_v.ptr, d_stats.ptr, G, d_g.ptr, d_b.ptr, 1e-5, d_ln.ptr, w2.d_row_ptr.ptr,
-                                          w2.d_col_idx.ptr, w2.d_tiles.ptr, w2.d_bias.ptr, d_y.ptr, T, n_mid, n_out,
-                                          act, None))
+    et.check(lib.et_norm_linear_bsr16_f16(d_v.ptr, d_resid.ptr, d_stats.ptr, G, d_g.ptr, d_b.ptr, 1e-5, d_ln.ptr,
+                                          w2.d_row_ptr.ptr, w2.d_col_idx.ptr, w2.d_tiles.ptr, w2.d_bias.ptr, d_y.ptr,
+                                          T, n_mid, n_out, act, None))
     ln = d_ln.numpy()
-    want_ln = L.layernorm(Hn.f32(v), Hn.f32(gamma), Hn.f32(beta), 1e-5, torch.float16).numpy()
+    want_ln = L.skip_layernorm(Hn.f32(v), Hn.f32(resid), Hn.f32(gamma), Hn.f32(beta), 1e-5, torch.float16).numpy()
     assert Hn.max_abs(ln, want_ln) <= 4e-3
     want_y = L.linear(Hn.f32(ln), Hn.f32(w2.dense), Hn.f32(w2.bias), {0: None, 1: "relu", 2: "gelu"}[act],
                       torch.float16).numpy()
     assert Hn.max_abs(d_y.numpy(), want_y) <= 5e-3
 
     d_ln2 = et.DeviceBuffer.empty((T, n_mid), np.float16)
-    et.check(lib.et_norm_from_stats_f16(d_ln2.ptr, d_v.ptr, d_stats.ptr, G, d_g.ptr, d_b.ptr, T, n_mid, 1e-5, None))
+    et.check(lib.et_norm_from_stats_f16(d_ln2.ptr, d_v.ptr, d_resid.ptr, d_stats.ptr, G, d_g.ptr, d_b.ptr, T, n_mid,
+                                        1e-5, None))
     assert np.array_equal(d_ln2.numpy().view(np.uint16), ln.view(np.uint16))
 
 
@@ -307,8 +309,8 @@ def test_split_layernorm_rejects_unsupported(et):
     assert lib.et_linear_bsr16_fused_ln_supported(64, 60, 64) == 0
     d = et.DeviceBuffer.empty((64, 64), np.float16)
     g = C.c_int(0)
-    st = lib.et_norm_linear_bsr16_f16(d.ptr, d.ptr, 17, d.ptr, d.ptr, 1e-5, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr,
-                                      64, 64, 64, 0, None)
+    st = lib.et_norm_linear_bsr16_f16(d.ptr, d.ptr, d.ptr, 17, d.ptr, d.ptr, 1e-5, d.ptr, d.ptr, d.ptr, d.ptr, d.ptr,
+                                      d.ptr, 64, 64, 64, 0, None)
     assert st == et.ET_ERR_INVALID_ARG
 
 
