@@ -267,7 +267,8 @@ int et_fill_rows_bias_f16(et_f16 *C, const et_f16 *bias, int rows, int cols,
  * mask: optional additive [S x S] binary16 matrix shared by all sequences and
  * heads (-inf removes a key).  lens: optional int32[B]; keys >= lens[b] of
  * sequence b get probability exactly 0 (right padding).  Scores, softmax and
- * both contractions are fp32-accumulated.  S % 16 == 0, hd in {32, 64, 128}.
+ * both contractions are fp32-accumulated.  S % 16 == 0; hd a multiple of 16 (the
+ * reference's own constraint, Fused_attention/test/testfused.cu:22), at most 128.
  *
  * Replaces Multihead_atttion<OTF_attn_full> (Attention/Attention.cu:80-95,
  * Attention/OTFkernel_full.h:15-125), the single-buffer form
@@ -369,7 +370,7 @@ int et_bias_add_f16(et_f16 *data, const et_f16 *bias, int rows, int cols,
  * CPU fp32 forward to max-abs 1e-4 — and have no counterpart in the reference,
  * whose kernels are binary16 only (Linear/Linear.h:9, lib/mma.hpp:6-13).
  * et_linear_dense_f32: in % 16 == 0, out % 4 == 0, any T.
- * et_mha_fused_f32: S % 16 == 0, hd in {32, 64, 128}, 16*S floats of scores
+ * et_mha_fused_f32: S % 16 == 0, hd a multiple of 16 up to 128, 16*S floats of scores
  * must fit on chip (S <= 2048); mask is a float [S x S] matrix.
  * ------------------------------------------------------------------------ */
 int et_linear_dense_f32(const float *W, const float *bias, const float *X, float *Y,

@@ -33,6 +33,7 @@ struct MhaArgs {
     const int32_t *lens;   // [B] or nullptr
     int ldq, ldk, ldv, ldz;
     int S, nh;
+    int hd;             // head size, a multiple of 16; the kernel template is the next of 32, 64, 128
     int nbh;            // sequences * heads
     float scale_log2e;  // scale * log2(e)
     int causal;
@@ -98,21 +99,25 @@ __global__ __launch_bounds__(64 * NW) void mha_fused_kernel(const MhaArgs a) {
     // under a causal mask no query of this strip sees a key past the strip's last query
     if (a.causal) klimit = min(klimit, (qstrip + 1) * kStripQ);
     // compact-V: this head's surviving V columns
-    int vc0 = 0, vlive = HD;
+    // head sizes between the template sizes: columns [hd, HD) of Q, K and V read as zero
+    // (no effect on scores or outputs) and are not written
+    const int hd = a.hd;
+    int vc0 = 0, vlive = hd;
     if (COMPACT) {
         vc0 = a.v_head_ptr[h];
-        vlive = min(a.v_head_ptr[h + 1] - vc0, HD);
+        vlive = min(a.v_head_ptr[h + 1] - vc0, hd);
     }
 
     // Q fragments: B operand, lane supplies Q[q][32*ks + 8g .. +7]
     h8 qf[QT][KS];
 #pragma unroll
     for (int t = 0; t < QT; t++) {
-        const _Float16 *qp = a.Q + (row0 + (q_ok[t] ? q[t] : 0)) * a.ldq + h * HD + 8 * g;
+        const _Float16 *qp = a.Q + (row0 + (q_ok[t] ? q[t] : 0)) * a.ldq + h * hd + 8 * g;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
-            qf[t][ks] = *reinterpret_cast<const h8 *>(qp + 32 * ks);
-            if (!q_ok[t]) qf[t][ks] = h8{0, 0, 0, 0, 0, 0, 0, 0};
+            const bool live = q_ok[t] && 32 * ks + 8 * g < hd;
+            qf[t][ks] = *reinterpret_cast<const h8 *>(qp + (live ? 32 * ks : 0));
+            if (!live) qf[t][ks] = h8{0, 0, 0, 0, 0, 0, 0, 0};
         }
     }
 
@@ -145,8 +150,8 @@ __global__ __launch_bounds__(64 * NW) void mha_fused_kernel(const MhaArgs a) {
             const int v = threadIdx.x + i * nthr;
             const int r = v / vec_per_row, c = v - r * vec_per_row;
             kreg[i] = h8{0, 0, 0, 0, 0, 0, 0, 0};
-            if (k0 + r < S)
-                kreg[i] = *reinterpret_cast<const h8 *>(a.K + (row0 + k0 + r) * a.ldk + h * HD + c * 8);
+            if (k0 + r < S && c * 8 < hd)
+                kreg[i] = *reinterpret_cast<const h8 *>(a.K + (row0 + k0 + r) * a.ldk + h * hd + c * 8);
         }
 #pragma unroll
         for (int j = 0; j < VU; j++) {
@@ -164,8 +169,8 @@ __global__ __launch_bounds__(64 * NW) void mha_fused_kernel(const MhaArgs a) {
                         for (int d = 0; d < 8; d++)
                             if (dg * 8 + d < vlive) vreg[j][i][d] = vp[d];
                     }
-                } else if (key < S) {
-                    vreg[j][i] = *reinterpret_cast<const h8 *>(a.V + (row0 + key) * a.ldv + h * HD + dg * 8);
+                } else if (key < S && dg * 8 < hd) {
+                    vreg[j][i] = *reinterpret_cast<const h8 *>(a.V + (row0 + key) * a.ldv + h * hd + dg * 8);
                 }
             }
         }
@@ -309,7 +314,7 @@ __global__ __launch_bounds__(64 * NW) void mha_fused_kernel(const MhaArgs a) {
                 }
 #pragma unroll
                 for (int d = 0; d < DB; d++) {
-                    if (COMPACT && d * 16 >= vlive) continue;  // no surviving column in this block
+                    if (d * 16 >= vlive) continue;  // no (surviving) column in this block: wave-uniform
                     const _Float16 *vp = Vt + (d * 16 + r16) * L::ldvt + s2 * 32 + 4 * g;
                     const h4 v0 = *reinterpret_cast<const h4 *>(vp);
                     const h4 v1 = *reinterpret_cast<const h4 *>(vp + 16);
@@ -339,9 +344,10 @@ __global__ __launch_bounds__(64 * NW) void mha_fused_kernel(const MhaArgs a) {
 #pragma unroll
         for (int t = 0; t < QT; t++) {
             if (!q_ok[t]) continue;
-            _Float16 *zp = a.Z + (row0 + q[t]) * a.ldz + h * HD + 4 * g;
+            _Float16 *zp = a.Z + (row0 + q[t]) * a.ldz + h * hd + 4 * g;
 #pragma unroll
             for (int d = 0; d < DB; d++) {
+                if (16 * d >= hd) continue;  // wave-uniform
                 h4 out;
 #pragma unroll
                 for (int j = 0; j < 4; j++) out[j] = (_Float16)(o[t][d][j] * inv[t]);
@@ -359,7 +365,8 @@ __global__ __launch_bounds__(64 * NW) void mha_fused_kernel(const MhaArgs a) {
                 _Float16 *zrow = a.Z + (row0 + q[t]) * a.ldz;
                 const h4 z4 = {0, 0, 0, 0};
 #pragma unroll
-                for (int d = 0; d < DB; d++) *reinterpret_cast<h4 *>(zrow + h * HD + 16 * d + 4 * g) = z4;
+                for (int d = 0; d < DB; d++)
+                    if (16 * d < hd) *reinterpret_cast<h4 *>(zrow + h * hd + 16 * d + 4 * g) = z4;
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
@@ -427,8 +434,8 @@ int et_mha_fused_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V, int ldq,
                flags);
     ET_REQUIRE(S % 16 == 0, ET_ERR_UNSUPPORTED, "et_mha_fused_f16: S=%d must be a multiple of 16",
                S);
-    ET_REQUIRE(hd == 32 || hd == 64 || hd == 128, ET_ERR_UNSUPPORTED,
-               "et_mha_fused_f16: head dim %d not in {32, 64, 128}", hd);
+    ET_REQUIRE(hd % 16 == 0 && hd <= 128, ET_ERR_UNSUPPORTED,
+               "et_mha_fused_f16: head dim %d must be a multiple of 16, at most 128", hd);
     const int width = nh * hd;
     ET_REQUIRE(ldq >= width && ldk >= width && ldv >= width && ldz >= width, ET_ERR_INVALID_ARG,
                "et_mha_fused_f16: row strides (%d %d %d %d) smaller than nh*hd=%d", ldq, ldk, ldv,
@@ -454,16 +461,15 @@ int et_mha_fused_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V, int ldq,
     args.ldz = ldz;
     args.S = S;
     args.nh = nh;
+    args.hd = hd;
     args.nbh = B * nh;
     args.scale_log2e = scale * kLog2e;
     args.causal = (flags & ET_MHA_CAUSAL) ? 1 : 0;
     args.v_col_id = nullptr;
     args.v_head_ptr = nullptr;
-    switch (hd) {
-        case 32: return launch_mha<32, false>(args, B, as_stream(stream));
-        case 64: return launch_mha<64, false>(args, B, as_stream(stream));
-        default: return launch_mha<128, false>(args, B, as_stream(stream));
-    }
+    if (hd <= 32) return launch_mha<32, false>(args, B, as_stream(stream));
+    if (hd <= 64) return launch_mha<64, false>(args, B, as_stream(stream));
+    return launch_mha<128, false>(args, B, as_stream(stream));
 }
 
 int et_mha_compactv_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *Vc, int ldq, int ldk, int ldvc,
@@ -476,8 +482,8 @@ int et_mha_compactv_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *Vc, int 
                "et_mha_compactv_f16: B=%d S=%d nh=%d hd=%d nnz_col=%d", B, S, nh, hd, nnz_col);
     ET_REQUIRE((flags & ~ET_MHA_CAUSAL) == 0, ET_ERR_INVALID_ARG, "et_mha_compactv_f16: flags=%d", flags);
     ET_REQUIRE(S % 16 == 0, ET_ERR_UNSUPPORTED, "et_mha_compactv_f16: S=%d must be a multiple of 16", S);
-    ET_REQUIRE(hd == 32 || hd == 64 || hd == 128, ET_ERR_UNSUPPORTED,
-               "et_mha_compactv_f16: head dim %d not in {32, 64, 128}", hd);
+    ET_REQUIRE(hd % 16 == 0 && hd <= 128, ET_ERR_UNSUPPORTED,
+               "et_mha_compactv_f16: head dim %d must be a multiple of 16, at most 128", hd);
     ET_REQUIRE(vhd == hd, ET_ERR_UNSUPPORTED,
                "et_mha_compactv_f16: V head width %d must equal the Q/K head width %d", vhd, hd);
     ET_REQUIRE(ldq >= nh * hd && ldk >= nh * hd && ldz >= nh * vhd && ldvc >= nnz_col, ET_ERR_INVALID_ARG,
@@ -499,16 +505,15 @@ int et_mha_compactv_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *Vc, int 
     args.ldz = ldz;
     args.S = S;
     args.nh = nh;
+    args.hd = hd;
     args.nbh = B * nh;
     args.scale_log2e = scale * kLog2e;
     args.causal = (flags & ET_MHA_CAUSAL) ? 1 : 0;
     args.v_col_id = v_col_id;
     args.v_head_ptr = v_head_ptr;
-    switch (hd) {
-        case 32: return launch_mha<32, true>(args, B, as_stream(stream));
-        case 64: return launch_mha<64, true>(args, B, as_stream(stream));
-        default: return launch_mha<128, true>(args, B, as_stream(stream));
-    }
+    if (hd <= 32) return launch_mha<32, true>(args, B, as_stream(stream));
+    if (hd <= 64) return launch_mha<64, true>(args, B, as_stream(stream));
+    return launch_mha<128, true>(args, B, as_stream(stream));
 }
 
 }  // extern "C"

@@ -19,6 +19,7 @@ struct ProbsArgs {
     int S, nh;
     float scale_log2e;
     int causal;
+    int hd;  // head size, a multiple of 16; the kernel template is the next of 32, 64, 128
 };
 
 constexpr float kLog2e_ = 1.4426950408889634f;
@@ -45,9 +46,14 @@ __global__ __launch_bounds__(256) void mha_probs_kernel(const ProbsArgs a) {
 
     h8 qf[KS];
     {
-        const _Float16 *qp = a.Q + (row0 + q) * a.ldq + h * HD + 8 * g;
+        // columns [hd, HD) read as zero: no contribution to the scores
+        const _Float16 *qp = a.Q + (row0 + q) * a.ldq + h * a.hd + 8 * g;
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) qf[ks] = *reinterpret_cast<const h8 *>(qp + 32 * ks);
+        for (int ks = 0; ks < KS; ks++) {
+            const bool live = 32 * ks + 8 * g < a.hd;
+            qf[ks] = *reinterpret_cast<const h8 *>(qp + (live ? 32 * ks : 0));
+            if (!live) qf[ks] = h8{0, 0, 0, 0, 0, 0, 0, 0};
+        }
     }
     f4 sc[NKB];
     float m = -INFINITY;
@@ -56,10 +62,11 @@ __global__ __launch_bounds__(256) void mha_probs_kernel(const ProbsArgs a) {
         sc[kb] = f4{0.f, 0.f, 0.f, 0.f};
         if (kb < nkb) {
             if (kb * 16 < klimit) {
-                const _Float16 *kp = a.K + (row0 + kb * 16 + r16) * a.ldk + h * HD + 8 * g;
+                const _Float16 *kp = a.K + (row0 + kb * 16 + r16) * a.ldk + h * a.hd + 8 * g;
 #pragma unroll
                 for (int ks = 0; ks < KS; ks++) {
-                    const h8 kf = *reinterpret_cast<const h8 *>(kp + 32 * ks);
+                    // a dead column block multiplies the zeros of qf: any valid address will do
+                    const h8 kf = *reinterpret_cast<const h8 *>(kp + (32 * ks + 8 * g < a.hd ? 32 * ks : 0));
                     sc[kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[ks], sc[kb], 0, 0, 0);
                 }
             }
@@ -119,11 +126,9 @@ static int launch_probs_hd(const ProbsArgs &a, int B, hipStream_t stream) {
 }
 
 static int launch_probs(const ProbsArgs &a, int B, int hd, hipStream_t stream) {
-    switch (hd) {
-        case 32: return launch_probs_hd<32>(a, B, stream);
-        case 64: return launch_probs_hd<64>(a, B, stream);
-        default: return launch_probs_hd<128>(a, B, stream);
-    }
+    if (hd <= 32) return launch_probs_hd<32>(a, B, stream);
+    if (hd <= 64) return launch_probs_hd<64>(a, B, stream);
+    return launch_probs_hd<128>(a, B, stream);
 }
 
 static int check_probs_shape(const char *fn, int B, int S, int nh, int hd, int flags) {
@@ -132,8 +137,8 @@ static int check_probs_shape(const char *fn, int B, int S, int nh, int hd, int f
     ET_REQUIRE((flags & ~ET_MHA_CAUSAL) == 0, ET_ERR_INVALID_ARG, "%s: flags=%d", fn, flags);
     ET_REQUIRE(S % 16 == 0 && S <= 512, ET_ERR_UNSUPPORTED,
                "%s: S=%d must be a multiple of 16 and at most 512", fn, S);
-    ET_REQUIRE(hd == 32 || hd == 64 || hd == 128, ET_ERR_UNSUPPORTED,
-               "%s: head dim %d not in {32, 64, 128}", fn, hd);
+    ET_REQUIRE(hd % 16 == 0 && hd <= 128, ET_ERR_UNSUPPORTED,
+               "%s: head dim %d must be a multiple of 16, at most 128", fn, hd);
     ET_REQUIRE(B <= 65535 && nh <= 65535, ET_ERR_UNSUPPORTED, "%s: grid too large", fn);
     return ET_OK;
 }
@@ -157,7 +162,7 @@ int et_mha_probs_f16(const et_f16 *Q, const et_f16 *K, int ldq, int ldk, et_f16 
                "et_mha_probs_f16: bad row strides %d %d", ldq, ldk);
     if (B == 0) return ET_OK;
     ProbsArgs a{H(Q), H(K), H(P), H(mask), lens, ldq, ldk, nh * S, S, nh, scale * kLog2e_,
-                (flags & ET_MHA_CAUSAL) ? 1 : 0};
+                (flags & ET_MHA_CAUSAL) ? 1 : 0, hd};
     return launch_probs(a, B, hd, as_stream(stream));
 }
 

@@ -121,15 +121,18 @@ __global__ __launch_bounds__(256) void mha_fused_f32_kernel(const MhaF32Args a) 
     const size_t row0 = (size_t)b * a.S;
     constexpr int kF = HD / 16;  // output features per thread
 
-    float *zrow = a.Z + (row0 + q0 + q) * a.ldz + h * HD;
+    // head sizes between the template sizes: columns [hd, HD) are staged as zero, not written
+    const int hd = a.hd;
+    float *zrow = a.Z + (row0 + q0 + q) * a.ldz + h * hd;
     if (len == 0) {  // a sequence without keys: zeros
 #pragma unroll
-        for (int i = 0; i < kF; i++) zrow[c + 16 * i] = 0.0f;
+        for (int i = 0; i < kF; i++)
+            if (c + 16 * i < hd) zrow[c + 16 * i] = 0.0f;
         return;
     }
     for (int i = threadIdx.x; i < kAttQ * HD; i += 256) {
         const int r = i / HD, d = i - r * HD;
-        qs[i] = a.Q[(row0 + q0 + r) * a.ldq + h * HD + d] * a.scale;
+        qs[i] = d < hd ? a.Q[(row0 + q0 + r) * a.ldq + h * hd + d] * a.scale : 0.0f;
     }
     // keys this block of queries can see
     int kend = len;
@@ -141,7 +144,7 @@ __global__ __launch_bounds__(256) void mha_fused_f32_kernel(const MhaF32Args a) 
         __syncthreads();
         for (int i = threadIdx.x; i < kAttKeys * HD; i += 256) {
             const int r = i / HD, d = i - r * HD;
-            kv[r * (HD + 1) + d] = kb + r < kend ? a.K[(row0 + kb + r) * a.ldk + h * HD + d] : 0.0f;
+            kv[r * (HD + 1) + d] = (kb + r < kend && d < hd) ? a.K[(row0 + kb + r) * a.ldk + h * hd + d] : 0.0f;
         }
         __syncthreads();
 #pragma unroll
@@ -179,7 +182,7 @@ __global__ __launch_bounds__(256) void mha_fused_f32_kernel(const MhaF32Args a) 
         __syncthreads();
         for (int i = threadIdx.x; i < kAttKeys * HD; i += 256) {
             const int r = i / HD, d = i - r * HD;
-            kv[r * (HD + 1) + d] = kb + r < kend ? a.V[(row0 + kb + r) * a.ldv + h * HD + d] : 0.0f;
+            kv[r * (HD + 1) + d] = (kb + r < kend && d < hd) ? a.V[(row0 + kb + r) * a.ldv + h * hd + d] : 0.0f;
         }
         __syncthreads();
         const int nk = min(kAttKeys, kend - kb);
@@ -191,7 +194,8 @@ __global__ __launch_bounds__(256) void mha_fused_f32_kernel(const MhaF32Args a) 
     }
     const float inv = l > 0.0f ? 1.0f / l : 0.0f;
 #pragma unroll
-    for (int i = 0; i < kF; i++) zrow[c + 16 * i] = acc[i] * inv;
+    for (int i = 0; i < kF; i++)
+        if (c + 16 * i < hd) zrow[c + 16 * i] = acc[i] * inv;
 }
 
 template <int OP>
@@ -236,12 +240,13 @@ int et_mha_fused_f32(const float *Q, const float *K, const float *V, int ldq, in
     ET_REQUIRE(Q && K && V && Z, ET_ERR_INVALID_ARG, "et_mha_fused_f32: NULL pointer");
     ET_REQUIRE(B >= 0 && S > 0 && nh > 0, ET_ERR_INVALID_ARG, "et_mha_fused_f32: B=%d S=%d nh=%d", B, S, nh);
     ET_REQUIRE((flags & ~ET_MHA_CAUSAL) == 0, ET_ERR_INVALID_ARG, "et_mha_fused_f32: flags=%d", flags);
-    ET_REQUIRE(S % 16 == 0 && (hd == 32 || hd == 64 || hd == 128), ET_ERR_UNSUPPORTED,
-               "et_mha_fused_f32: S=%d must be a multiple of 16, hd=%d one of 32, 64, 128", S, hd);
+    ET_REQUIRE(S % 16 == 0 && hd > 0 && hd % 16 == 0 && hd <= 128, ET_ERR_UNSUPPORTED,
+               "et_mha_fused_f32: S=%d and hd=%d must be multiples of 16, hd at most 128", S, hd);
     const int width = nh * hd;
     ET_REQUIRE(ldq >= width && ldk >= width && ldv >= width && ldz >= width, ET_ERR_INVALID_ARG,
                "et_mha_fused_f32: row strides must cover nh*hd=%d", width);
-    const size_t lds = sizeof(float) * ((size_t)kAttQ * hd + (size_t)kAttKeys * (hd + 1) + (size_t)kAttQ * S);
+    const int hdt = hd <= 32 ? 32 : hd <= 64 ? 64 : 128;  // kernel template size
+    const size_t lds = sizeof(float) * ((size_t)kAttQ * hdt + (size_t)kAttKeys * (hdt + 1) + (size_t)kAttQ * S);
     ET_REQUIRE(lds <= 160 * 1024, ET_ERR_UNSUPPORTED, "et_mha_fused_f32: S=%d does not fit the on-chip score strip", S);
     if (B == 0) return ET_OK;
     MhaF32Args a{Q, K, V, Z, mask, lens, ldq, ldk, ldv, ldz, B, S, nh, hd, scale, (flags & ET_MHA_CAUSAL) ? 1 : 0};
@@ -255,7 +260,7 @@ int et_mha_fused_f32(const float *Q, const float *K, const float *V, int ldq, in
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));               \
         kern<<<grid, 256, lds, st>>>(a);                                                                     \
     }
-    if (hd == 32) ET_MHA32(32) else if (hd == 64) ET_MHA32(64) else ET_MHA32(128)
+    if (hdt == 32) ET_MHA32(32) else if (hdt == 64) ET_MHA32(64) else ET_MHA32(128)
 #undef ET_MHA32
     return check_launch("mha_fused_f32_kernel");
 }

@@ -46,7 +46,8 @@ def test_linear_dense_f32_no_bias_and_bad_args(et):
 
 @pytest.mark.parametrize("B,S,nh,hd,causal,lens,mask", [
     (1, 128, 12, 64, False, None, False), (3, 128, 12, 64, False, [128, 64, 97], False),
-    (2, 64, 4, 32, True, None, False), (2, 48, 2, 128, False, [0, 48], True), (1, 512, 2, 64, True, [300], False)])
+    (2, 64, 4, 32, True, None, False), (2, 48, 2, 128, False, [0, 48], True), (1, 512, 2, 64, True, [300], False),
+    (2, 64, 3, 48, False, [64, 20], False), (1, 32, 2, 16, True, None, False)])
 def test_mha_fused_f32(et, B, S, nh, hd, causal, lens, mask):
     H = nh * hd
     qkv = randf((B * S, 3 * H), 6)
