@@ -38,9 +38,67 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak (vendor figure)
 FFN_UP_TRAFFIC_BYTES = (5420.5 * 1.9989 + 7680.1 * 1.0) * 1024
 
 
-def build_layers(Hn):
-    return [Hn.LayerWeights(H, NH, FF, SPARSITY, seed=100 + i, attention_aware=ATTENTION_AWARE)
-            for i in range(NLAYER)]
+class TileWeight:
+    """One tile-sparse matrix of the workload, built with the library's own host routines
+    (seeded permutation, surviving-tile count) and numpy: nothing here touches the CPU oracle."""
+
+    def __init__(self, et, out, inp, seed, dead_block_rows=(), dead_block_cols=()):
+        import ctypes as C
+        lib = et.lib()
+        br, bc = out // 16, inp // 16
+        total = br * bc
+        ntile = lib.et_fmt_kept_count(total, SPARSITY)  # int(total * (1.0 - (double)sparsity))
+        perm = np.zeros(total, np.int64)
+        et.check(lib.et_fmt_permutation(total, seed, perm.ctypes.data))
+        ys, xs = perm // bc, perm % bc
+        live = ~np.isin(ys, list(dead_block_rows)) & ~np.isin(xs, list(dead_block_cols))
+        kept = perm[live][:ntile]  # surviving tiles among the live positions, in permuted order
+        ys, xs = kept // bc, kept % bc
+        order = np.argsort(ys, kind="stable")
+        self.row_ptr = np.concatenate([[0], np.cumsum(np.bincount(ys, minlength=br))]).astype(np.int32)
+        self.col_idx = xs[order].astype(np.int32)
+        rng = np.random.default_rng(seed)
+        self.tiles = (rng.standard_normal((len(kept), 256), dtype=np.float32) * 0.02).astype(np.float16)
+        self.bias = (rng.standard_normal(out, dtype=np.float32) * 0.02).astype(np.float16)
+        for r in dead_block_rows:  # a dead V feature has no weights and no bias
+            self.bias[16 * r:16 * r + 16] = 0
+        self.out, self.inp = out, inp
+
+    def upload(self, et):
+        D = et.DeviceBuffer.from_numpy
+        self.d_row_ptr, self.d_col_idx = D(self.row_ptr), D(self.col_idx)
+        self.d_tiles, self.d_bias = D(self.tiles), D(self.bias)
+        return self
+
+
+class LayerWeights:
+    def __init__(self, et, seed):
+        per_head = (H // NH) // 16
+        ndead = int(per_head * ATTENTION_AWARE)
+        dead = [h * per_head + (per_head - 1 - i) for h in range(NH) for i in range(ndead)]
+        self.qkv = TileWeight(et, 3 * H, H, seed * 100 + 1, dead_block_rows=[2 * (H // 16) + b for b in dead])
+        self.o = TileWeight(et, H, H, seed * 100 + 11, dead_block_cols=dead)
+        self.l1 = TileWeight(et, FF, H, seed * 100 + 21)
+        self.l2 = TileWeight(et, H, FF, seed * 100 + 31)
+        rng = np.random.default_rng(seed * 100 + 41)
+        g = lambda: (1.0 + 0.1 * rng.standard_normal(H, dtype=np.float32)).astype(np.float16)
+        b = lambda: (0.1 * rng.standard_normal(H, dtype=np.float32)).astype(np.float16)
+        self.g1, self.be1, self.g2, self.be2 = g(), b(), g(), b()
+
+
+def build_layers(et):
+    return [LayerWeights(et, 100 + i) for i in range(NLAYER)]
+
+
+def build_model(et, layers, use_graph):
+    m = et.Model(H, NH, FF, S, NLAYER, batch=B, act=et.ACT_GELU, eps=1e-5, causal=False, use_graph=use_graph)
+    for i, w in enumerate(layers):
+        for which, tw in ((et.W_QKV, w.qkv), (et.W_O, w.o), (et.W_FF1, w.l1), (et.W_FF2, w.l2)):
+            m.set_bsr16(i, which, tw.row_ptr, tw.col_idx, tw.tiles, tw.bias)
+        m.set_norm(i, 0, w.g1, w.be1)
+        m.set_norm(i, 1, w.g2, w.be2)
+    m.finalize()
+    return m
 
 
 def time_stack(et, model, d_out, d_in, steps, warmup):
@@ -95,17 +153,24 @@ def time_ffn_kernel(et, w, T, launches_per_graph=64, replays=8):
     return t.ms * 1e-3 / (launches_per_graph * replays)
 
 
-def cpu_baseline(Hn, layers, x, reps=3):
+def cpu_baseline(layers, x, gpu_out, reps=3):
     """The CPU oracle (PyTorch-CPU fp32 forward, pruned weights as masked dense matrices) on
-    the host cores: one warm-up, then `reps` forwards of the full 12-layer, batch-8 stack."""
+    the host cores: one warm-up, then `reps` forwards of the full 12-layer, batch-8 stack.
+    The only part of this file that uses oracle/: it also checks the GPU result of the same
+    workload against the oracle run with the engine's fp16 storage points."""
     import torch
+    from oracle import formats as F
     from oracle import layers as L
 
     threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
     torch.set_num_threads(threads)
-    params = [w.oracle_params() for w in layers]
+    f32 = lambda a: torch.from_numpy(np.asarray(a, np.float32))
+    dense = lambda w: f32(F.bsr16_to_dense(w.row_ptr, w.col_idx, w.tiles, w.inp))
+    params = [L.LayerParams(dense(w.qkv), f32(w.qkv.bias), dense(w.o), f32(w.o.bias), dense(w.l1), f32(w.l1.bias),
+                            dense(w.l2), f32(w.l2.bias), f32(w.g1), f32(w.be1), f32(w.g2), f32(w.be2))
+              for w in layers]
     cfg = L.LayerConfig(nh=NH, B=B, act="gelu", store=None)
-    xt = Hn.f32(x)
+    xt = f32(x)
     with torch.no_grad():
         L.encoder_stack(xt, params, cfg)
         times = []
@@ -113,11 +178,20 @@ def cpu_baseline(Hn, layers, x, reps=3):
             t0 = time.perf_counter()
             L.encoder_stack(xt, params, cfg)
             times.append(time.perf_counter() - t0)
+        want32 = L.encoder_stack(xt, params, cfg).numpy()
+        want16 = L.encoder_stack(xt, params, L.LayerConfig(nh=NH, B=B, act="gelu", store=torch.float16)).numpy()
     med = float(np.median(times))
+    got = gpu_out.astype(np.float32)
+    err32, err16 = float(np.max(np.abs(got - want32))), float(np.max(np.abs(got - want16)))
+    ref16 = float(np.max(np.abs(want16 - want32)))
     return {"value": round(B / med, 3), "unit": "seq/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"{reps} forwards of the full workload (12 layers, batch 8, seq 128) after 1 warm-up, "
                       f"median {med * 1e3:.1f} ms per forward, fp32 masked-dense PyTorch-CPU oracle",
-            "us_per_layer": round(med * 1e6 / NLAYER, 1)}
+            "us_per_layer": round(med * 1e6 / NLAYER, 1),
+            # max-abs over the [1024 x 768] output of layer 12: the GPU against the fp32 forward timed above,
+            # against the same forward with the engine's fp16 storage points, and those two against each other
+            "gpu_max_abs_err_vs_fp32_forward": round(err32, 6), "gpu_max_abs_err_vs_fp16_storage_forward": round(err16, 6),
+            "fp16_storage_forward_vs_fp32_forward": round(ref16, 6)}
 
 
 def main():
@@ -137,11 +211,10 @@ def main():
 
     et = entry.load_package()
     et.lib()  # fails loudly if the native library is missing
-    from tests import harness as Hn
 
-    layers = build_layers(Hn)
-    model = Hn.build_model(et, layers, S, B, act=et.ACT_GELU, use_graph=not args.eager)
-    x = Hn.randn((B * S, H), 4)
+    layers = build_layers(et)
+    model = build_model(et, layers, use_graph=not args.eager)
+    x = np.random.default_rng(4).standard_normal((B * S, H), dtype=np.float32).astype(np.float16)
     d_in = et.DeviceBuffer.from_numpy(x)
     d_out = et.DeviceBuffer.empty((B * S, H), np.float16)
 
@@ -179,7 +252,7 @@ def main():
             et.check(et.lib().et_relu_f16(dst.ptr, src.ptr, n, None))
         et.sync()
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(Hn, layers, x)
+        out["cpu_baseline"] = cpu_baseline(layers, x, d_out.numpy())
     print(json.dumps(out))
 
 
