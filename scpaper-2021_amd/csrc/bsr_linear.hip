@@ -509,14 +509,14 @@ static BsrPlan plan_bsr(int T, int in, int out) {
     if (32 * row_bytes <= lds_cap / 2) mt_fit = 2;
     else if (16 * row_bytes <= lds_cap) mt_fit = 1;
     struct Cand { int mt, threads; };
-    Cand cands[7];
+    Cand cands[5];
     int nc = 0;
     // many token rows: 64-row strips halve the weight traffic per row again (each tile fetch
     // feeds four MFMAs); they only pay once 64-row strips alone fill the device
     if (64 * row_bytes <= lds_cap && T >= 64 * 128) cands[nc++] = {4, 512};
-    if (mt_fit == 2 && T >= 32) { cands[nc++] = {2, 512}; cands[nc++] = {2, 256}; }
-    if (mt_fit >= 1) { cands[nc++] = {1, 512}; cands[nc++] = {1, 256}; cands[nc++] = {1, 128}; }
-    if (mt_fit == 0) { cands[nc++] = {2, 256}; }
+    if (mt_fit == 2 && T >= 32) cands[nc++] = {2, 512};
+    if (mt_fit >= 1) { cands[nc++] = {1, 512}; cands[nc++] = {1, 256}; }
+    if (mt_fit == 0) cands[nc++] = {2, 256};
     BsrPlan best{};
     int best_wgs = -1;
     for (int i = 0; i < nc; i++) {
@@ -527,10 +527,19 @@ static BsrPlan plan_bsr(int T, int in, int out) {
         const int nwave = p.threads / 64;
         const int strips = (T + p.mt * 16 - 1) / (p.mt * 16);
         const int groups = strips >= 256 ? 1 : 256 / strips;
-        int rpw = (nbr + groups - 1) / groups;
-        rpw = ((rpw + nwave - 1) / nwave) * nwave;
+        // block-rows per wave: the nearest whole number to an even split over `groups`
+        // workgroups, at least one (few token rows: one block-row per wave is the shortest
+        // dependent chain, and more, smaller workgroups fill the device)
+        int per_wave = (int)((double)nbr / ((double)groups * nwave) + 0.5);
+        if (per_wave < 1) per_wave = 1;
+        // heavy workgroups (several block-rows per wave) saturate a compute unit's path to the
+        // L2: more of them than compute units would run as a second, mostly empty round
+        while (per_wave >= 2 && per_wave < kMaxWaveRows &&
+               strips * ((nbr + per_wave * nwave - 1) / (per_wave * nwave)) > 256)
+            per_wave++;
+        if (per_wave > kMaxWaveRows) per_wave = kMaxWaveRows;
+        int rpw = per_wave * nwave;
         if (rpw > nbr) rpw = nbr;
-        if (rpw > kMaxWaveRows * nwave) rpw = kMaxWaveRows * nwave;
         p.rows_per_wg = rpw;
         p.lds = bsr_lds_bytes(p.mt, p.stage, in, rpw);
         const int wgs = strips * ((nbr + rpw - 1) / rpw);
@@ -550,15 +559,21 @@ static BsrPlan plan_bsr_ln(int T, int in, int out) {
     const int nbr = out / 16;
     BsrPlan p{};
     p.stage = 16 * row_bytes <= lds_cap;
-    p.mt = (T >= 32 && 32 * row_bytes <= lds_cap / 2) ? 2 : 1;
+    // 32-row strips once they give every compute unit work; 16-row strips below that (half
+    // the rows to normalise per workgroup, twice the workgroups)
+    p.mt = (T >= 512 && 32 * row_bytes <= lds_cap / 2) ? 2 : 1;
     p.threads = 512;
     const int nwave = 8;
     const int strips = (T + p.mt * 16 - 1) / (p.mt * 16);
     const int groups = strips >= 256 ? 1 : 256 / strips;
-    int rpw = (nbr + groups - 1) / groups;
-    rpw = ((rpw + nwave - 1) / nwave) * nwave;
+    int per_wave = (int)((double)nbr / ((double)groups * nwave) + 0.5);
+    if (per_wave < 1) per_wave = 1;
+    while (per_wave >= 2 && per_wave < kMaxWaveRows &&
+           strips * ((nbr + per_wave * nwave - 1) / (per_wave * nwave)) > 256)
+        per_wave++;
+    if (per_wave > kMaxWaveRows) per_wave = kMaxWaveRows;
+    int rpw = per_wave * nwave;
     if (rpw > nbr) rpw = nbr;
-    if (rpw > kMaxWaveRows * nwave) rpw = kMaxWaveRows * nwave;
     p.rows_per_wg = rpw;
     p.lds = bsr_lds_bytes(p.mt, p.stage, in, rpw);
     return p;
