@@ -194,6 +194,7 @@ static int launch_gemm_tile(const GemmArgs &g, int batch, bool trans_b, hipStrea
 
 // 128x128 tiles once they still give a few hundred workgroups, 64x64 otherwise.
 int launch_gemm(const GemmArgs &g, int batch, bool trans_b, hipStream_t stream) {
+    if (gemm_big_applies(g, batch, trans_b)) return launch_gemm_big(g, stream);
     const long long big = (long long)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
     if (big >= 512) return launch_gemm_tile<4, 4>(g, batch, trans_b, stream);
     return launch_gemm_tile<2, 2>(g, batch, trans_b, stream);
