@@ -6,10 +6,11 @@
 // peak.  Here a workgroup of 4 waves computes a 256 x 256 tile and each wave a 128 x 128
 // block as 4 x 4 v_mfma_f32_32x32x16_f16 tiles, accumulators in 256 AGPR/VGPRs: 1 byte
 // of LDS per 64 flops.  One wave per SIMD is resident, so the latencies are covered inside
-// the wave: K advances in stages of 64 through two LDS buffers, global loads run two stages
-// ahead (one in registers, one in LDS), the LDS writes of the next stage and the fragment
-// reads of the next K slice are issued ahead of the MFMAs that hide them, and the one
-// workgroup barrier of a stage sits before its last K slice.
+// the wave: K advances in stages of 64 through two LDS buffers, the next stage is loaded
+// straight from global memory into the idle buffer while the current one is multiplied
+// (staging through registers and ds_write costs a third of the rate: the LDS port is then
+// the bound), the fragment reads of the next K slice are issued ahead of the MFMAs that hide
+// them, and the one workgroup barrier of a stage sits before its last K slice.
 //
 // The MFMA A operand is the B matrix (output features) and vice versa, so a lane ends with
 // 4 consecutive features of one row of C per 8-row group of a tile; the epilogue transposes
@@ -20,19 +21,22 @@ namespace et {
 
 constexpr int kBigTile = 256;            // rows of A and rows of B per workgroup
 constexpr int kBigK = 64;                // K per stage: one 128-byte line of every row
-constexpr int kBigLd = kBigK + 8;        // halfs per LDS row (16-byte pad: conflict-free b128 reads)
-constexpr int kBigVec = kBigTile * (kBigK / 8) / 256;  // 16-byte vectors per thread, operand and stage
 constexpr int kBigXcds = 8;
 constexpr int kSbM = 4, kSbN = 8;        // tile block one XCD works on at a time
-constexpr size_t kBigLds = (size_t)2 * 2 * kBigTile * kBigLd * sizeof(_Float16);
+constexpr size_t kBigLds = (size_t)2 * 2 * kBigTile * kBigK * sizeof(_Float16);  // 128 KB
+// s_waitcnt immediate for vmcnt(0) alone on gfx9: vmcnt in bits 3:0 and 15:14, expcnt 6:4 and
+// lgkmcnt 11:8 left at their maxima
+constexpr int kWaitVm0 = 0x0F70;
+#define ET_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
+#define ET_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
 typedef float f16v __attribute__((ext_vector_type(16)));
 
 template <int ACT>
 __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
     extern __shared__ __align__(16) unsigned char big_smem[];
-    _Float16 *As = reinterpret_cast<_Float16 *>(big_smem);  // [2][256][kBigLd]
-    _Float16 *Bs = As + 2 * kBigTile * kBigLd;               // [2][256][kBigLd]
+    _Float16 *As = reinterpret_cast<_Float16 *>(big_smem);  // [2][256][kBigK], chunks swizzled
+    _Float16 *Bs = As + 2 * kBigTile * kBigK;                // [2][256][kBigK]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -59,37 +63,34 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-    // staging: vector v of a thread = row (tid + 256 v) / 8, 16-byte column (tid + 256 v) % 8:
-    // 8 lanes read one whole 128-byte line of a row, so no fetched line is used by halves
-    h8 ra[kBigVec], rb[kBigVec];
-    auto load_stage = [&](int k0) {
+    // Stage loads go straight from global memory to LDS (global_load_lds_dwordx4): a wave
+    // instruction fills 1 KB of consecutive LDS, 16 bytes per lane, from addresses the lanes
+    // choose.  Here that is 8 rows of 128 bytes, 8 lanes a row (whole lines of the operand);
+    // within the row the lane at position p fetches chunk p ^ swz(row), so that the fragment
+    // reads below, 16 rows apart by one chunk column, spread over all banks with no padding.
+    const int lrow = lane >> 3, lpos = lane & 7;
+    auto load_stage = [&](int buf, int k0) {
 #pragma unroll
-        for (int v = 0; v < kBigVec; v++) {
-            const int idx = tid + v * 256;
-            const int r = idx / (kBigK / 8), c = idx % (kBigK / 8);
-            ra[v] = *reinterpret_cast<const h8 *>(A + (size_t)r * g.lda + k0 + c * 8);
-            rb[v] = *reinterpret_cast<const h8 *>(B + (size_t)r * g.ldb + k0 + c * 8);
+        for (int v = 0; v < 8; v++) {
+            const int r0 = wave * 64 + v * 8, r = r0 + lrow;
+            const int c = lpos ^ ((r >> 1) & 7);
+            __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(A + (size_t)r * g.lda + k0 + c * 8),
+                                             ET_LDS_PTR(As + (buf * kBigTile + r0) * kBigK), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(B + (size_t)r * g.ldb + k0 + c * 8),
+                                             ET_LDS_PTR(Bs + (buf * kBigTile + r0) * kBigK), 16, 0, 0);
         }
     };
-    auto store_stage = [&](int buf) {
-        _Float16 *as = As + buf * kBigTile * kBigLd, *bs = Bs + buf * kBigTile * kBigLd;
-#pragma unroll
-        for (int v = 0; v < kBigVec; v++) {
-            const int idx = tid + v * 256;
-            const int r = idx / (kBigK / 8), c = idx % (kBigK / 8);
-            *reinterpret_cast<h8 *>(as + r * kBigLd + c * 8) = ra[v];
-            *reinterpret_cast<h8 *>(bs + r * kBigLd + c * 8) = rb[v];
-        }
-    };
-    // fragments of one 16-wide K slice: 4 token tiles and 4 feature tiles of the wave's block
+    // fragments of one 16-wide K slice: 4 token tiles and 4 feature tiles of the wave's block.
+    // Rows 128 wm + 32 i + l32: the swizzle term (row >> 1) & 7 depends on the lane only.
     struct Frag { h8 x[4], w[4]; };
+    const int swz = (l32 >> 1) & 7;
+    const _Float16 *a_rows = As + (wm * 128 + l32) * kBigK, *b_rows = Bs + (wn * 128 + l32) * kBigK;
     auto read_frag = [&](Frag &f, int buf, int ks) {
-        const _Float16 *as = As + buf * kBigTile * kBigLd + (wm * 128 + l32) * kBigLd + kg * 8 + ks * 16;
-        const _Float16 *bs = Bs + buf * kBigTile * kBigLd + (wn * 128 + l32) * kBigLd + kg * 8 + ks * 16;
+        const int off = buf * kBigTile * kBigK + (((ks * 2 + kg) ^ swz) * 8);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            f.x[i] = *reinterpret_cast<const h8 *>(as + i * 32 * kBigLd);
-            f.w[i] = *reinterpret_cast<const h8 *>(bs + i * 32 * kBigLd);
+            f.x[i] = *reinterpret_cast<const h8 *>(a_rows + off + i * 32 * kBigK);
+            f.w[i] = *reinterpret_cast<const h8 *>(b_rows + off + i * 32 * kBigK);
         }
     };
     auto multiply = [&](const Frag &f) {
@@ -101,31 +102,30 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
     };
 
     const int nstage = g.K / kBigK;
-    // Stage s is multiplied from LDS buffer s % 2.  prologue: stage 0 in buffer 0, stage 1 on its way
+    // Stage s is multiplied from LDS buffer s % 2.
     Frag f0, f1;
-    load_stage(0);
-    store_stage(0);
-    load_stage(min(1, nstage - 1) * kBigK);
+    load_stage(0, 0);
+    __builtin_amdgcn_s_waitcnt(kWaitVm0);  // the data of a direct-to-LDS load is in LDS when vmcnt says so
     __syncthreads();
     read_frag(f0, 0, 0);
     // One stage, with the matrix pipe fed across the barrier: every K slice is read from LDS
     // while the one before it is multiplied, the first slice of the next stage included, so the
-    // barrier of the stage sits before its last slice.  The next stage goes to the other LDS
-    // buffer at the start of the stage (its last readers passed the previous barrier) and the
-    // registers are reloaded with the stage after next, which so has a whole stage to arrive.
-    // The store, load and fragment read of the last stages that have no successor touch valid
-    // memory and are never used; the loop has a single exit (a second one in the middle makes
-    // the register allocator copy the 256 accumulators).
+    // barrier of the stage sits before its last slice.  The loads of the next stage are issued at
+    // the start of the stage into the other buffer (its last readers passed the previous
+    // barrier) and waited for just before the barrier.  The load and fragment read of the last
+    // stage, which has no successor, touch valid memory and are never used; the loop has a
+    // single exit (a second one in the middle makes the register allocator copy the 256
+    // accumulators).
     for (int s = 0; s < nstage; s++) {
         const int cur = s & 1, nxt = cur ^ 1;
-        store_stage(nxt);  // stage s + 1
-        load_stage(min(s + 2, nstage - 1) * kBigK);
+        load_stage(nxt, min(s + 1, nstage - 1) * kBigK);
         read_frag(f1, cur, 1);
         multiply(f0);
         read_frag(f0, cur, 2);
         multiply(f1);
         read_frag(f1, cur, 3);
         multiply(f0);
+        __builtin_amdgcn_s_waitcnt(kWaitVm0);
         __syncthreads();
         read_frag(f0, nxt, 0);
         multiply(f1);
