@@ -32,7 +32,8 @@ constexpr int kWaitVm0 = 0x0F70;
 
 typedef float f16v __attribute__((ext_vector_type(16)));
 
-template <int ACT>
+// IDX: the result columns are scattered (c_scatter) or their bias is gathered (bias_idx).
+template <int ACT, bool IDX>
 __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
     extern __shared__ __align__(16) unsigned char big_smem[];
     _Float16 *As = reinterpret_cast<_Float16 *>(big_smem);  // [2][256][kBigK], chunks swizzled
@@ -142,7 +143,7 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
     // unconditional loads (from B when there is no bias) and a select: a load under a branch
     // is waited for on the spot
     const bool has_bias = g.bias != nullptr;
-    const _Float16 *bias_src = has_bias ? g.bias + nbase : g.B;
+    const int32_t *col_idx = g.c_scatter ? g.c_scatter : g.bias_idx;  // bias index of result column n
     h4 bias4[4][4];
 #pragma unroll
     for (int j = 0; j < 4; j++)
@@ -150,9 +151,25 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
         for (int q = 0; q < 4; q++)
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const _Float16 bv = bias_src[j * 32 + q * 8 + kg * 4 + e];
+                const int n = nbase + j * 32 + q * 8 + kg * 4 + e;
+                _Float16 bv;
+                if (IDX) {
+                    const int bi = col_idx ? col_idx[n] : n;
+                    bv = (has_bias ? g.bias : g.B)[has_bias ? bi : 0];
+                } else {
+                    bv = (has_bias ? g.bias : g.B)[n];
+                }
                 bias4[j][q][e] = has_bias ? bv : (_Float16)0.0f;
             }
+    // the 8 output columns of the lane's 16-byte chunk of a stored row
+    int scat[8];
+    if (IDX) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int n = nbase + (lane % 16) * 8 + e;
+            scat[e] = g.c_scatter ? g.c_scatter[n] : n;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < 4; i++) {
 #pragma unroll
@@ -174,16 +191,41 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
         for (int v = 0; v < 8; v++) {
             const int idx = lane + v * 64, r = idx / 16, c = idx % 16;
             const h8 val = *reinterpret_cast<const h8 *>(ep + r * kEpLd + c * 8);
-            *reinterpret_cast<h8 *>(g.C + (size_t)(m0 + wm * 128 + i * 32 + r) * g.ldc + nbase + c * 8) = val;
+            _Float16 *crow = g.C + (size_t)(m0 + wm * 128 + i * 32 + r) * g.ldc;
+            if (IDX) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) crow[scat[e]] = val[e];
+            } else {
+                *reinterpret_cast<h8 *>(crow + nbase + c * 8) = val;
+            }
         }
         __syncthreads();
     }
 }
 
 bool gemm_big_applies(const GemmArgs &g, int batch, bool trans_b) {
-    return trans_b && batch == 1 && !g.a_gather && !g.c_scatter && !g.bias_idx && g.M % kBigTile == 0 &&
+    return trans_b && batch == 1 && !g.a_gather && g.M % kBigTile == 0 &&
            g.N % kBigTile == 0 && g.K % kBigK == 0 &&
            (long long)(g.M / kBigTile) * (g.N / kBigTile) >= 256;
+}
+
+template <int ACT, bool IDX>
+static int launch_big_variant(const GemmArgs &g, dim3 grid, hipStream_t stream) {
+    auto kernel = gemm_f16_big_kernel<ACT, IDX>;
+    static bool raised = false;  // 128 KB of dynamic LDS needs the attribute, once per kernel
+    if (!raised) {
+        ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBigLds));
+        raised = true;
+    }
+    kernel<<<grid, 256, kBigLds, stream>>>(g);
+    return check_launch("gemm_f16_big_kernel");
+}
+
+template <int ACT>
+static int launch_big_act(const GemmArgs &g, dim3 grid, hipStream_t stream) {
+    return (g.c_scatter || g.bias_idx) ? launch_big_variant<ACT, true>(g, grid, stream)
+                                       : launch_big_variant<ACT, false>(g, grid, stream);
 }
 
 int launch_gemm_big(const GemmArgs &g, hipStream_t stream) {
@@ -191,24 +233,11 @@ int launch_gemm_big(const GemmArgs &g, hipStream_t stream) {
     const int nsb = ((tiles_m + kSbM - 1) / kSbM) * ((tiles_n + kSbN - 1) / kSbN);
     const int rounds = (nsb + kBigXcds - 1) / kBigXcds;
     const dim3 grid((unsigned)(rounds * kBigXcds * kSbM * kSbN));
-#define ET_BIG(ACTV)                                                                                  \
-    {                                                                                                 \
-        auto kernel = gemm_f16_big_kernel<ACTV>;                                                      \
-        static bool raised = false;                                                                   \
-        if (!raised) {                                                                                \
-            ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),                        \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBigLds));   \
-            raised = true;                                                                            \
-        }                                                                                             \
-        kernel<<<grid, 256, kBigLds, stream>>>(g);                                                    \
-    }
     switch (g.act) {
-        case ET_ACT_RELU: ET_BIG(ET_ACT_RELU) break;
-        case ET_ACT_GELU: ET_BIG(ET_ACT_GELU) break;
-        default: ET_BIG(ET_ACT_NONE) break;
+        case ET_ACT_RELU: return launch_big_act<ET_ACT_RELU>(g, grid, stream);
+        case ET_ACT_GELU: return launch_big_act<ET_ACT_GELU>(g, grid, stream);
+        default: return launch_big_act<ET_ACT_NONE>(g, grid, stream);
     }
-#undef ET_BIG
-    return check_launch("gemm_f16_big_kernel");
 }
 
 }  // namespace et

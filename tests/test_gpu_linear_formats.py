@@ -67,7 +67,8 @@ def test_gemm_rejects_bad_args(et):
 
 
 @pytest.mark.parametrize("T,inp,out,sp,act", [(2048, 768, 768, 0.5, 0), (2048, 768, 3072, 0.5, 2),
-                                              (2048, 3072, 768, 0.5, 0), (64, 64, 100 * 16, 0.9, 1)])
+                                              (2048, 3072, 768, 0.5, 0), (64, 64, 100 * 16, 0.9, 1),
+                                              (8192, 128, 4096, 0.5, 2)])  # last: the 256 x 256-tile kernel
 def test_linear_rowpruned(et, T, inp, out, sp, act):
     row_id = F.gen_row_ids(out, sp, seed=8)
     rows, b, x = Hn.randn((len(row_id), inp), 9, 0.02), Hn.randn((out,), 10, 0.1), Hn.randn((T, inp), 11)
