@@ -1,43 +1,51 @@
-// Large dense GEMM for gfx950: C[M x N] = act(A[M x K] * B^T + bias), A and B both
-// K-contiguous (B stored [N x K]), M and N multiples of 256, K a multiple of 64.
+// Dense GEMM for gfx950 on direct-to-LDS loads: C[M x N] = act(A[M x K] * B^T + bias), A and B
+// both K-contiguous (B stored [N x K]), M and N multiples of the tile, K a multiple of 64.
 //
 // The 64x64-per-wave kernel in gemm.hip reads 1 byte of LDS per 32 flops, which at the
-// MFMA peak is the whole bandwidth of the LDS port; it tops out near a third of the matrix
-// peak.  Here a workgroup of 4 waves computes a 256 x 256 tile and each wave a 128 x 128
-// block as 4 x 4 v_mfma_f32_32x32x16_f16 tiles, accumulators in 256 AGPR/VGPRs: 1 byte
-// of LDS per 64 flops.  One wave per SIMD is resident, so the latencies are covered inside
-// the wave: K advances in stages of 64 through two LDS buffers, the next stage is loaded
-// straight from global memory into the idle buffer while the current one is multiplied
-// (staging through registers and ds_write costs a third of the rate: the LDS port is then
-// the bound), the fragment reads of the next K slice are issued ahead of the MFMAs that hide
-// them, and the one workgroup barrier of a stage sits before its last K slice.
+// MFMA peak is the whole bandwidth of the LDS port, and stages through registers; it tops
+// out near a third of the matrix peak.  Here a workgroup of 4 waves (2 x 2) computes a tile of
+// 64 TMW x 64 TNW and each wave a block of TMW x TNW v_mfma_f32_32x32x16_f16 tiles.  The
+// largest tile, 256 x 256 (a wave: 128 x 128, 256 accumulators in AGPRs, 1 byte of LDS per 64
+// flops, one wave per SIMD), is for problems that fill the device with it; smaller problems
+// take smaller tiles (more workgroups, several per compute unit) at the price of more operand
+// traffic from the L2 per flop.  Latencies are covered inside the wave: K advances in stages
+// of 64 through two LDS buffers, the next stage is loaded straight from global memory into
+// the idle buffer while the current one is multiplied (staging through registers and
+// ds_write costs a third of the rate: the LDS port is then the bound), the fragment reads of
+// the next K slice are issued ahead of the MFMAs that hide them, and the one workgroup barrier
+// of a stage sits before its last K slice.
 //
 // The MFMA A operand is the B matrix (output features) and vice versa, so a lane ends with
 // 4 consecutive features of one row of C per 8-row group of a tile; the epilogue transposes
-// through LDS to store whole 256-byte row segments.
+// through LDS to store whole row segments.
 #include "gemm.hip.h"
 
 namespace et {
 
-constexpr int kBigTile = 256;            // rows of A and rows of B per workgroup
 constexpr int kBigK = 64;                // K per stage: one 128-byte line of every row
 constexpr int kBigXcds = 8;
 constexpr int kSbM = 4, kSbN = 8;        // tile block one XCD works on at a time
-constexpr size_t kBigLds = (size_t)2 * 2 * kBigTile * kBigK * sizeof(_Float16);  // 128 KB
-// s_waitcnt immediate for vmcnt(0) alone on gfx9: vmcnt in bits 3:0 and 15:14, expcnt 6:4 and
+constexpr size_t big_lds_bytes(int tmw, int tnw, int nbuf) {  // buffers of (BM + BN) rows of 128 bytes
+    return (size_t)nbuf * 64 * (tmw + tnw) * kBigK * sizeof(_Float16);
+}
+// s_waitcnt immediate for vmcnt(n) alone on gfx9: vmcnt in bits 3:0 and 15:14, expcnt 6:4 and
 // lgkmcnt 11:8 left at their maxima
-constexpr int kWaitVm0 = 0x0F70;
+constexpr int wait_vm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
 #define ET_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 #define ET_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
 typedef float f16v __attribute__((ext_vector_type(16)));
 
-// IDX: the result columns are scattered (c_scatter) or their bias is gathered (bias_idx).
-template <int ACT, bool IDX>
+// TMW x TNW: 32 x 32 MFMA tiles per wave.  IDX: the result columns are scattered (c_scatter) or
+// their bias is gathered (bias_idx).
+template <int TMW, int TNW, int NBUF, bool IDX>
 __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
+    static_assert(NBUF >= 2 && NBUF <= 4 && (NBUF - 2) * (2 * TMW + 2 * TNW) <= 63, "vmcnt holds 63 loads");
+    constexpr int BM = 64 * TMW, BN = 64 * TNW;  // workgroup tile
+    constexpr int WM = 32 * TMW, WN = 32 * TNW;  // wave block
     extern __shared__ __align__(16) unsigned char big_smem[];
-    _Float16 *As = reinterpret_cast<_Float16 *>(big_smem);  // [2][256][kBigK], chunks swizzled
-    _Float16 *Bs = As + 2 * kBigTile * kBigK;                // [2][256][kBigK]
+    _Float16 *As = reinterpret_cast<_Float16 *>(big_smem);  // [NBUF][BM][kBigK], chunks swizzled
+    _Float16 *Bs = As + NBUF * BM * kBigK;                   // [NBUF][BN][kBigK]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -46,21 +54,21 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
     // Workgroup id -> tile, XCD-aware.  Workgroups go to the 8 XCDs round-robin by id and each
     // XCD runs 32 of them at a time; those 32 are given a 4 x 8 block of tiles (4 panels of A,
     // 8 of B), so the XCD's L2 serves 12 panels to 32 workgroups instead of up to 64.
-    const int tiles_m = g.M / kBigTile, tiles_n = g.N / kBigTile;
+    const int tiles_m = g.M / BM, tiles_n = g.N / BN;
     const int nsbx = (tiles_n + kSbN - 1) / kSbN;
     const int xcd = blockIdx.x % kBigXcds, j = blockIdx.x / kBigXcds;
     const int gsb = (j / (kSbM * kSbN)) * kBigXcds + xcd, within = j % (kSbM * kSbN);
     const int ty = (gsb / nsbx) * kSbM + within / kSbN, tx = (gsb % nsbx) * kSbN + within % kSbN;
     if (ty >= tiles_m || tx >= tiles_n) return;  // padding of the block grid (whole workgroup)
-    const int m0 = ty * kBigTile, n0 = tx * kBigTile;
+    const int m0 = ty * BM, n0 = tx * BN;
     const _Float16 *A = g.A + (size_t)m0 * g.lda;
     const _Float16 *B = g.B + (size_t)n0 * g.ldb;
 
-    f16v acc[4][4];  // [token tile][feature tile]
+    f16v acc[TMW][TNW];  // [token tile][feature tile]
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < TMW; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < TNW; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
@@ -72,81 +80,107 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
     const int lrow = lane >> 3, lpos = lane & 7;
     auto load_stage = [&](int buf, int k0) {
 #pragma unroll
-        for (int v = 0; v < 8; v++) {
-            const int r0 = wave * 64 + v * 8, r = r0 + lrow;
+        for (int v = 0; v < 2 * TMW; v++) {  // a wave loads a quarter of the rows of each operand
+            const int r0 = wave * (BM / 4) + v * 8, r = r0 + lrow;
             const int c = lpos ^ ((r >> 1) & 7);
             __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(A + (size_t)r * g.lda + k0 + c * 8),
-                                             ET_LDS_PTR(As + (buf * kBigTile + r0) * kBigK), 16, 0, 0);
+                                             ET_LDS_PTR(As + (buf * BM + r0) * kBigK), 16, 0, 0);
+        }
+#pragma unroll
+        for (int v = 0; v < 2 * TNW; v++) {
+            const int r0 = wave * (BN / 4) + v * 8, r = r0 + lrow;
+            const int c = lpos ^ ((r >> 1) & 7);
             __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(B + (size_t)r * g.ldb + k0 + c * 8),
-                                             ET_LDS_PTR(Bs + (buf * kBigTile + r0) * kBigK), 16, 0, 0);
+                                             ET_LDS_PTR(Bs + (buf * BN + r0) * kBigK), 16, 0, 0);
         }
     };
-    // fragments of one 16-wide K slice: 4 token tiles and 4 feature tiles of the wave's block.
-    // Rows 128 wm + 32 i + l32: the swizzle term (row >> 1) & 7 depends on the lane only.
-    struct Frag { h8 x[4], w[4]; };
+    // fragments of one 16-wide K slice: the token tiles and feature tiles of the wave's block.
+    // Rows WM wm + 32 i + l32: the swizzle term (row >> 1) & 7 depends on the lane only.
+    struct Frag { h8 x[TMW], w[TNW]; };
     const int swz = (l32 >> 1) & 7;
-    const _Float16 *a_rows = As + (wm * 128 + l32) * kBigK, *b_rows = Bs + (wn * 128 + l32) * kBigK;
+    const _Float16 *a_rows = As + (wm * WM + l32) * kBigK, *b_rows = Bs + (wn * WN + l32) * kBigK;
     auto read_frag = [&](Frag &f, int buf, int ks) {
-        const int off = buf * kBigTile * kBigK + (((ks * 2 + kg) ^ swz) * 8);
+        const int chunk = ((ks * 2 + kg) ^ swz) * 8;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            f.x[i] = *reinterpret_cast<const h8 *>(a_rows + off + i * 32 * kBigK);
-            f.w[i] = *reinterpret_cast<const h8 *>(b_rows + off + i * 32 * kBigK);
-        }
+        for (int i = 0; i < TMW; i++)
+            f.x[i] = *reinterpret_cast<const h8 *>(a_rows + buf * BM * kBigK + chunk + i * 32 * kBigK);
+#pragma unroll
+        for (int j = 0; j < TNW; j++)
+            f.w[j] = *reinterpret_cast<const h8 *>(b_rows + buf * BN * kBigK + chunk + j * 32 * kBigK);
     };
     auto multiply = [&](const Frag &f) {
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < TMW; i++)
 #pragma unroll
-            for (int j = 0; j < 4; j++)
+            for (int j = 0; j < TNW; j++)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.w[j], f.x[i], acc[i][j], 0, 0, 0);
     };
 
     const int nstage = g.K / kBigK;
-    // Stage s is multiplied from LDS buffer s % 2.
+    // Stage s is multiplied from LDS buffer s % NBUF; the loads of kAhead later stages are in
+    // flight meanwhile.  A direct-to-LDS load has landed when vmcnt says so, and vmcnt counts
+    // in issue order: "stage s + 1 has landed" is "at most the loads of the stages after it
+    // are outstanding".
+    constexpr int kAhead = NBUF - 1;
+    constexpr int kStageLoads = 2 * TMW + 2 * TNW;  // per wave
+    auto wait_stages = [&](int later) {  // wait until at most `later` whole stages are outstanding
+        if (later <= 0) __builtin_amdgcn_s_waitcnt(wait_vm(0));
+        else if (later == 1) __builtin_amdgcn_s_waitcnt(wait_vm(kStageLoads));
+        else __builtin_amdgcn_s_waitcnt(wait_vm(2 * kStageLoads));
+    };
+    // Workgroup barrier that orders LDS accesses only.  __syncthreads() carries a fence that
+    // waits for every outstanding global access, the direct-to-LDS loads of the later stages
+    // included, which is exactly what a deeper pipeline must not do; here this wave's LDS reads
+    // are waited for, the barrier is passed, and the compiler moves no memory access across.
+    auto lds_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
     Frag f0, f1;
-    load_stage(0, 0);
-    __builtin_amdgcn_s_waitcnt(kWaitVm0);  // the data of a direct-to-LDS load is in LDS when vmcnt says so
-    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < kAhead; p++)
+        if (p < nstage) load_stage(p, p * kBigK);
+    wait_stages(min(kAhead, nstage) - 1);
+    lds_barrier();
     read_frag(f0, 0, 0);
     // One stage, with the matrix pipe fed across the barrier: every K slice is read from LDS
     // while the one before it is multiplied, the first slice of the next stage included, so the
-    // barrier of the stage sits before its last slice.  The loads of the next stage are issued at
-    // the start of the stage into the other buffer (its last readers passed the previous
-    // barrier) and waited for just before the barrier.  The load and fragment read of the last
-    // stage, which has no successor, touch valid memory and are never used; the loop has a
-    // single exit (a second one in the middle makes the register allocator copy the 256
+    // barrier of the stage sits before its last slice.  The loads of stage s + kAhead are issued
+    // at the start of stage s into the buffer stage s - 1 was read from (its last readers passed
+    // the previous barrier); stage s + 1 is waited for just before the barrier.  The fragment
+    // read after the barrier of the last stage touches valid LDS and is never used; the loop
+    // has a single exit (a second one in the middle makes the register allocator copy the
     // accumulators).
+    int cur = 0;
     for (int s = 0; s < nstage; s++) {
-        const int cur = s & 1, nxt = cur ^ 1;
-        load_stage(nxt, min(s + 1, nstage - 1) * kBigK);
+        const int nxt = cur + 1 == NBUF ? 0 : cur + 1;
+        if (s + kAhead < nstage) load_stage(cur == 0 ? NBUF - 1 : cur - 1, (s + kAhead) * kBigK);
         read_frag(f1, cur, 1);
         multiply(f0);
         read_frag(f0, cur, 2);
         multiply(f1);
         read_frag(f1, cur, 3);
         multiply(f0);
-        __builtin_amdgcn_s_waitcnt(kWaitVm0);
-        __syncthreads();
+        wait_stages(min(kAhead - 1, nstage - 2 - s));
+        lds_barrier();
         read_frag(f0, nxt, 0);
         multiply(f1);
+        cur = nxt;
     }
     __syncthreads();  // the staging LDS becomes the transposition buffer of the epilogue
 
-    // Epilogue.  acc[i][j][e] is token 128 wm + 32 i + l32, feature 128 wn + 32 j + 8 (e / 4) +
+    // Epilogue.  acc[i][j][e] is token WM wm + 32 i + l32, feature WN wn + 32 j + 8 (e / 4) +
     // 4 kg + e % 4 of the tile: a lane holds 4 consecutive features of one row, 32 rows per
-    // instruction.  Each wave passes its 32 x 128 strip through its own LDS region and stores
-    // rows of 256 contiguous bytes.
-    constexpr int kEpLd = 128 + 8;
+    // instruction.  Each wave passes its 32 x WN strips through its own LDS region and stores
+    // rows of 2 WN contiguous bytes.
+    constexpr int kEpLd = WN + 8;
+    constexpr int kRowChunks = WN / 8;  // 16-byte chunks of a stored row: 4, 8 or 16
     _Float16 *ep = reinterpret_cast<_Float16 *>(big_smem) + wave * 32 * kEpLd;
-    const int nbase = n0 + wn * 128;
+    const int nbase = n0 + wn * WN;
     // unconditional loads (from B when there is no bias) and a select: a load under a branch
     // is waited for on the spot
     const bool has_bias = g.bias != nullptr;
     const int32_t *col_idx = g.c_scatter ? g.c_scatter : g.bias_idx;  // bias index of result column n
-    h4 bias4[4][4];
+    h4 bias4[TNW][4];
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < TNW; j++)
 #pragma unroll
         for (int q = 0; q < 4; q++)
 #pragma unroll
@@ -157,7 +191,7 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
                     const int bi = col_idx ? col_idx[n] : n;
                     bv = (has_bias ? g.bias : g.B)[has_bias ? bi : 0];
                 } else {
-                    bv = (has_bias ? g.bias : g.B)[n];
+                    bv = (has_bias ? g.bias : g.B)[has_bias ? n : 0];
                 }
                 bias4[j][q][e] = has_bias ? bv : (_Float16)0.0f;
             }
@@ -166,32 +200,29 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
     if (IDX) {
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            const int n = nbase + (lane % 16) * 8 + e;
+            const int n = nbase + (lane % kRowChunks) * 8 + e;
             scat[e] = g.c_scatter ? g.c_scatter[n] : n;
         }
     }
+    const int act = g.act;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < TMW; i++) {
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < TNW; j++)
 #pragma unroll
             for (int q = 0; q < 4; q++) {
                 h4 o;
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    float y = acc[i][j][q * 4 + e] + (float)bias4[j][q][e];
-                    if (ACT == ET_ACT_RELU) y = y > 0.0f ? y : 0.0f;
-                    if (ACT == ET_ACT_GELU) y = gelu_tanh(y);
-                    o[e] = (_Float16)y;
-                }
+                for (int e = 0; e < 4; e++)
+                    o[e] = (_Float16)apply_act(acc[i][j][q * 4 + e] + (float)bias4[j][q][e], act);
                 *reinterpret_cast<h4 *>(ep + l32 * kEpLd + j * 32 + q * 8 + kg * 4) = o;
             }
         __syncthreads();
 #pragma unroll
-        for (int v = 0; v < 8; v++) {
-            const int idx = lane + v * 64, r = idx / 16, c = idx % 16;
+        for (int v = 0; v < 32 * kRowChunks / 64; v++) {
+            const int idx = lane + v * 64, r = idx / kRowChunks, c = idx % kRowChunks;
             const h8 val = *reinterpret_cast<const h8 *>(ep + r * kEpLd + c * 8);
-            _Float16 *crow = g.C + (size_t)(m0 + wm * 128 + i * 32 + r) * g.ldc;
+            _Float16 *crow = g.C + (size_t)(m0 + wm * WM + i * 32 + r) * g.ldc;
             if (IDX) {
 #pragma unroll
                 for (int e = 0; e < 8; e++) crow[scat[e]] = val[e];
@@ -203,40 +234,69 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
     }
 }
 
+// Tile choice, from measurements on dense Linears of 1024..16384 rows: a larger tile halves the
+// operand traffic from the L2 per flop but needs enough workgroups to keep every compute unit
+// busy through whole rounds (a 256 x 256 workgroup owns its compute unit; two 128 x 128, three
+// 128 x 64 or five 64 x 64 ones share it and cover each other's prologue and epilogue).
+// 256 x 128 tiles and a fourth LDS buffer were measured and never won.
+struct BigTile { int tmw, tnw, nbuf; };
+static bool pick_big_tile(const GemmArgs &g, BigTile *out) {
+    auto wgs = [&](int tmw, int tnw) -> long long {
+        const int bm = 64 * tmw, bn = 64 * tnw;
+        return (g.M % bm || g.N % bn) ? 0 : (long long)(g.M / bm) * (g.N / bn);
+    };
+    const long long w44 = wgs(4, 4), w11 = wgs(1, 1);
+    // whole rounds of one workgroup per compute unit, or so many that the last one hardly counts
+    if (w44 >= 256 && (w44 % 256 == 0 || w44 >= 1024)) { *out = {4, 4, 2}; return true; }
+    if (wgs(2, 2) >= 512) { *out = {2, 2, 2}; return true; }
+    if (wgs(2, 1) >= 512) { *out = {2, 1, 2}; return true; }
+    if (w11 == 0) return false;
+    // few workgroups with a long K loop are bound by the latency of a stage: a third buffer keeps
+    // two stages in flight (2048 x 3072 -> 768: 29.5 -> 24.7 us); elsewhere it only costs occupancy
+    *out = {1, 1, (w11 <= 512 && g.K / kBigK >= 24) ? 3 : 2};
+    return true;
+}
+
 bool gemm_big_applies(const GemmArgs &g, int batch, bool trans_b) {
-    return trans_b && batch == 1 && !g.a_gather && g.M % kBigTile == 0 &&
-           g.N % kBigTile == 0 && g.K % kBigK == 0 &&
-           (long long)(g.M / kBigTile) * (g.N / kBigTile) >= 256;
+    BigTile t;
+    return trans_b && batch == 1 && !g.a_gather && g.K % kBigK == 0 && pick_big_tile(g, &t);
 }
 
-template <int ACT, bool IDX>
-static int launch_big_variant(const GemmArgs &g, dim3 grid, hipStream_t stream) {
-    auto kernel = gemm_f16_big_kernel<ACT, IDX>;
-    static bool raised = false;  // 128 KB of dynamic LDS needs the attribute, once per kernel
-    if (!raised) {
-        ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBigLds));
-        raised = true;
-    }
-    kernel<<<grid, 256, kBigLds, stream>>>(g);
-    return check_launch("gemm_f16_big_kernel");
-}
-
-template <int ACT>
-static int launch_big_act(const GemmArgs &g, dim3 grid, hipStream_t stream) {
-    return (g.c_scatter || g.bias_idx) ? launch_big_variant<ACT, true>(g, grid, stream)
-                                       : launch_big_variant<ACT, false>(g, grid, stream);
-}
-
-int launch_gemm_big(const GemmArgs &g, hipStream_t stream) {
-    const int tiles_m = g.M / kBigTile, tiles_n = g.N / kBigTile;
+template <int TMW, int TNW, int NBUF, bool IDX>
+static int launch_big_variant(const GemmArgs &g, hipStream_t stream) {
+    constexpr int BM = 64 * TMW, BN = 64 * TNW;
+    constexpr size_t lds = big_lds_bytes(TMW, TNW, NBUF);
+    const int tiles_m = g.M / BM, tiles_n = g.N / BN;
     const int nsb = ((tiles_m + kSbM - 1) / kSbM) * ((tiles_n + kSbN - 1) / kSbN);
     const int rounds = (nsb + kBigXcds - 1) / kBigXcds;
     const dim3 grid((unsigned)(rounds * kBigXcds * kSbM * kSbN));
-    switch (g.act) {
-        case ET_ACT_RELU: return launch_big_act<ET_ACT_RELU>(g, grid, stream);
-        case ET_ACT_GELU: return launch_big_act<ET_ACT_GELU>(g, grid, stream);
-        default: return launch_big_act<ET_ACT_NONE>(g, grid, stream);
+    auto kernel = gemm_f16_big_kernel<TMW, TNW, NBUF, IDX>;
+    static bool raised = false;  // more than 64 KB of dynamic LDS needs the attribute, once per kernel
+    if (!raised) {
+        ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        raised = true;
+    }
+    kernel<<<grid, 256, lds, stream>>>(g);
+    return check_launch("gemm_f16_big_kernel");
+}
+
+template <int TMW, int TNW, int NBUF>
+static int launch_big_tile(const GemmArgs &g, hipStream_t stream) {
+    return (g.c_scatter || g.bias_idx) ? launch_big_variant<TMW, TNW, NBUF, true>(g, stream)
+                                       : launch_big_variant<TMW, TNW, NBUF, false>(g, stream);
+}
+
+int launch_gemm_big(const GemmArgs &g, hipStream_t stream) {
+    BigTile t{};
+    if (!pick_big_tile(g, &t)) return ET_ERR_UNSUPPORTED;
+    switch (t.tmw * 100 + t.tnw * 10 + t.nbuf) {
+        case 442: return launch_big_tile<4, 4, 2>(g, stream);
+        case 222: return launch_big_tile<2, 2, 2>(g, stream);
+        case 212: return launch_big_tile<2, 1, 2>(g, stream);
+        case 112: return launch_big_tile<1, 1, 2>(g, stream);
+        case 113: return launch_big_tile<1, 1, 3>(g, stream);
+        default: return ET_ERR_UNSUPPORTED;
     }
 }
 

@@ -16,12 +16,25 @@ up = Hn.up
 
 
 @pytest.mark.parametrize("T,inp,out,act", [(2048, 768, 768, 0), (1024, 768, 3072, 2), (128, 3072, 768, 0),
-                                           (16, 16, 16, 1), (48, 80, 112, 0), (2048, 1024, 1024, 0)])
+                                           (16, 16, 16, 1), (48, 80, 112, 0), (2048, 1024, 1024, 0),
+                                           # one shape per tile of the direct-to-LDS kernel: 256x256, 128x128,
+                                           # 128x64, 64x64 with three LDS buffers, a single K stage
+                                           (4096, 192, 4096, 2), (2048, 128, 4096, 1), (2048, 192, 2304, 0),
+                                           (512, 1536, 768, 2), (256, 64, 256, 0)])
 def test_linear_dense(et, T, inp, out, act):
     W, b, x = Hn.randn((out, inp), 1, 0.02), Hn.randn((out,), 2, 0.1), Hn.randn((T, inp), 3)
     d_y = et.DeviceBuffer.empty((T, out), np.float16)
     et.linear_dense(up(et, W), up(et, b), up(et, x), d_y, T, inp, out, act)
     want = L.linear(Hn.f32(x), Hn.f32(W), Hn.f32(b), ACT[act], torch.float16).numpy()
+    assert Hn.max_abs(d_y.numpy(), want) <= 4e-3
+
+
+@pytest.mark.parametrize("T,inp,out", [(4096, 128, 4096), (512, 768, 768)])
+def test_linear_dense_without_bias(et, T, inp, out):
+    W, x = Hn.randn((out, inp), 21, 0.02), Hn.randn((T, inp), 22)
+    d_y = et.DeviceBuffer.empty((T, out), np.float16)
+    et.check(et.lib().et_linear_dense_f16(up(et, W).ptr, None, up(et, x).ptr, d_y.ptr, T, inp, out, 0, None))
+    want = L.linear(Hn.f32(x), Hn.f32(W), None, None, torch.float16).numpy()
     assert Hn.max_abs(d_y.numpy(), want) <= 4e-3
 
 
