@@ -178,6 +178,37 @@ __global__ __launch_bounds__(256) void bias_rows_kernel(_Float16 *__restrict__ C
     }
 }
 
+// The same in 16-byte stores: a thread owns 8 consecutive columns (their values computed once)
+// and walks down the rows of its block row-group.  cols and ldc multiples of 8, C 16-byte aligned.
+__global__ __launch_bounds__(256) void bias_rows_vec_kernel(_Float16 *__restrict__ C,
+                                                            const _Float16 *__restrict__ bias, int rows,
+                                                            int cols, int ldc, int act, int rows_per_block) {
+    const int chunk = blockIdx.x * blockDim.x + threadIdx.x;
+    if (chunk * 8 >= cols) return;
+    h8 v;
+#pragma unroll
+    for (int e = 0; e < 8; e++) v[e] = (_Float16)apply_act(bias ? (float)bias[chunk * 8 + e] : 0.0f, act);
+    const int r0 = blockIdx.y * rows_per_block, r1 = min(rows, r0 + rows_per_block);
+    for (int r = r0; r < r1; r++) *reinterpret_cast<h8 *>(C + (size_t)r * ldc + chunk * 8) = v;
+}
+
+static int launch_bias_rows(_Float16 *C, const _Float16 *bias, int rows, int cols, int ldc, int act,
+                            hipStream_t st) {
+    if (cols % 8 == 0 && ldc % 8 == 0 && (reinterpret_cast<uintptr_t>(C) & 15) == 0) {
+        const int bx = (cols / 8 + 255) / 256;
+        int rpb = (int)(((long long)rows * bx + 1023) / 1024);  // about 1024 blocks, at least 4 rows each
+        if (rpb < 4) rpb = 4;
+        const dim3 grid((unsigned)bx, (unsigned)((rows + rpb - 1) / rpb));
+        bias_rows_vec_kernel<<<grid, 256, 0, st>>>(C, bias, rows, cols, ldc, act, rpb);
+        return check_launch("bias_rows_vec_kernel");
+    }
+    const size_t total = (size_t)rows * cols;
+    size_t blocks = (total + 255) / 256;
+    if (blocks > 2048) blocks = 2048;
+    bias_rows_kernel<<<(unsigned)blocks, 256, 0, st>>>(C, bias, rows, cols, ldc, act);
+    return check_launch("bias_rows_kernel");
+}
+
 template <int TM, int TN>
 static int launch_gemm_tile(const GemmArgs &g, int batch, bool trans_b, hipStream_t stream) {
     const dim3 grid((g.N + 32 * TN - 1) / (32 * TN), (g.M + 32 * TM - 1) / (32 * TM), batch);
@@ -292,11 +323,7 @@ int et_linear_rowpruned_f16(const et_f16 *rows, const int32_t *row_id, int nnz_r
     hipStream_t st = as_stream(stream);
     if (nnz_row < out) {
         // pruned features carry the bias alone; live ones are overwritten below
-        const size_t total = (size_t)T * out;
-        size_t blocks = (total + 255) / 256;
-        if (blocks > 2048) blocks = 2048;
-        bias_rows_kernel<<<(unsigned)blocks, 256, 0, st>>>(H(Y), H(bias), T, out, out, act);
-        s = check_launch("bias_rows_kernel");
+        s = launch_bias_rows(H(Y), H(bias), T, out, out, act, st);
         if (s != ET_OK) return s;
     }
     if (nnz_row == 0) return ET_OK;
@@ -327,11 +354,7 @@ int et_fill_rows_bias_f16(et_f16 *C, const et_f16 *bias, int rows, int cols, et_
     ET_REQUIRE(C != nullptr, ET_ERR_INVALID_ARG, "et_fill_rows_bias_f16: C is NULL");
     ET_REQUIRE(rows >= 0 && cols > 0, ET_ERR_INVALID_ARG, "et_fill_rows_bias_f16: rows=%d cols=%d", rows, cols);
     if (rows == 0) return ET_OK;
-    const size_t total = (size_t)rows * cols;
-    size_t blocks = (total + 255) / 256;
-    if (blocks > 2048) blocks = 2048;
-    bias_rows_kernel<<<(unsigned)blocks, 256, 0, as_stream(stream)>>>(H(C), H(bias), rows, cols, cols, ET_ACT_NONE);
-    return check_launch("bias_rows_kernel");
+    return launch_bias_rows(H(C), H(bias), rows, cols, cols, ET_ACT_NONE, as_stream(stream));
 }
 
 int et_linear_colpruned_f16(const et_f16 *cols, const int32_t *col_id, int nnz_col,
@@ -349,11 +372,7 @@ int et_linear_colpruned_f16(const et_f16 *cols, const int32_t *col_id, int nnz_c
     if (T == 0) return ET_OK;
     hipStream_t st = as_stream(stream);
     if (nnz_col == 0) {
-        const size_t total = (size_t)T * out;
-        size_t blocks = (total + 255) / 256;
-        if (blocks > 2048) blocks = 2048;
-        bias_rows_kernel<<<(unsigned)blocks, 256, 0, st>>>(H(Y), H(bias), T, out, out, act);
-        return check_launch("bias_rows_kernel");
+        return launch_bias_rows(H(Y), H(bias), T, out, out, act, st);
     }
     GemmArgs g = gemm_args(H(X), H(cols), H(Y), T, out, nnz_col, in, nnz_col, out);
     g.bias = H(bias);

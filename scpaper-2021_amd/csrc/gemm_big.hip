@@ -195,13 +195,19 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
                 }
                 bias4[j][q][e] = has_bias ? bv : (_Float16)0.0f;
             }
-    // the 8 output columns of the lane's 16-byte chunk of a stored row
-    int scat[8];
+    // Scattered columns are stored one 2-byte element per lane, kScLanes consecutive result
+    // columns of one row per group of lanes: ascending c_scatter keeps those stores within a
+    // few neighbouring sectors of the row of C.
+    constexpr int kScLanes = WN < 64 ? WN : 64;  // lanes per row
+    constexpr int kScCols = WN / kScLanes;       // column groups
+    constexpr int kScRows = 64 / kScLanes;       // rows per instruction
+    const bool scatter = IDX && g.c_scatter != nullptr;  // a gathered bias alone keeps the vector stores
+    int scat[kScCols];
     if (IDX) {
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const int n = nbase + (lane % kRowChunks) * 8 + e;
-            scat[e] = g.c_scatter ? g.c_scatter[n] : n;
+        for (int e = 0; e < kScCols; e++) {
+            const int n = nbase + e * kScLanes + lane % kScLanes;
+            scat[e] = scatter ? g.c_scatter[n] : n;
         }
     }
     const int act = g.act;
@@ -218,16 +224,20 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
                 *reinterpret_cast<h4 *>(ep + l32 * kEpLd + j * 32 + q * 8 + kg * 4) = o;
             }
         __syncthreads();
+        if (scatter) {
 #pragma unroll
-        for (int v = 0; v < 32 * kRowChunks / 64; v++) {
-            const int idx = lane + v * 64, r = idx / kRowChunks, c = idx % kRowChunks;
-            const h8 val = *reinterpret_cast<const h8 *>(ep + r * kEpLd + c * 8);
-            _Float16 *crow = g.C + (size_t)(m0 + wm * WM + i * 32 + r) * g.ldc;
-            if (IDX) {
+            for (int v = 0; v < 32 / kScRows; v++) {
+                const int r = v * kScRows + lane / kScLanes;
+                _Float16 *crow = g.C + (size_t)(m0 + wm * WM + i * 32 + r) * g.ldc;
 #pragma unroll
-                for (int e = 0; e < 8; e++) crow[scat[e]] = val[e];
-            } else {
-                *reinterpret_cast<h8 *>(crow + nbase + c * 8) = val;
+                for (int e = 0; e < kScCols; e++) crow[scat[e]] = ep[r * kEpLd + e * kScLanes + lane % kScLanes];
+            }
+        } else {
+#pragma unroll
+            for (int v = 0; v < 32 * kRowChunks / 64; v++) {
+                const int idx = lane + v * 64, r = idx / kRowChunks, c = idx % kRowChunks;
+                const h8 val = *reinterpret_cast<const h8 *>(ep + r * kEpLd + c * 8);
+                *reinterpret_cast<h8 *>(g.C + (size_t)(m0 + wm * WM + i * 32 + r) * g.ldc + nbase + c * 8) = val;
             }
         }
         __syncthreads();

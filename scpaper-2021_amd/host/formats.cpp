@@ -109,8 +109,13 @@ void validate_bsr16(const std::vector<int> &row_ptr, const std::vector<int> &col
         require(row_ptr[i] >= row_ptr[i - 1], "tile_mat: row_ptr must be non-decreasing");
     require((size_t)row_ptr.back() == ntile && column.size() == ntile,
             "tile_mat: row_ptr.back(), the column count and the tile count must agree");
-    for (int c : column)
-        require(c >= 0 && c < blk_col_num, "tile_mat: column-tile index out of range");
+    for (size_t t = 0; t < column.size(); t++) {
+        const int c = column[t];
+        if (c < 0 || c >= blk_col_num)
+            throw Error(ET_ERR_INVALID_ARG, "tile_mat: column-tile index out of range (tile " + std::to_string(t) +
+                                                " of " + std::to_string(ntile) + " has column " + std::to_string(c) +
+                                                ", the matrix has " + std::to_string(blk_col_num) + " column tiles)");
+    }
 }
 
 std::vector<int> gen_row_ids(int nrow, float sparsity, uint64_t seed) {
