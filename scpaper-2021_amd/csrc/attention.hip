@@ -60,8 +60,16 @@ struct MhaLds {
 
 // QT = 16-query tiles per wave: with QT = 2 every K and V^T fragment read from LDS feeds
 // two MFMAs and a workgroup covers 32*NW queries per staged key block.
+//
+// The variants that prefetch the next key block through registers (mha_prefetches) are held to
+// the 168 registers of three resident waves per SIMD; left alone the allocator takes a few more
+// and the third wave is lost, which costs more than the prefetch gains.
+template <int HD, int NW> constexpr bool mha_prefetches() { return HD <= 64 && NW == 4; }
+
 template <int HD, bool COMPACT, int NW, int QT>
-__global__ __launch_bounds__(64 * NW) void mha_fused_kernel(const MhaArgs a) {
+__global__ __launch_bounds__(64 * NW)
+    __attribute__((amdgpu_waves_per_eu(mha_prefetches<HD, NW>() ? 3 : 1, mha_prefetches<HD, NW>() ? 3 : 8))) void
+    mha_fused_kernel(const MhaArgs a) {
     using L = MhaLds<HD>;
     constexpr int KS = HD / 32;  // K=32 MFMA steps over the head dimension
     constexpr int DB = HD / 16;  // 16-wide output blocks of the head dimension
@@ -196,10 +204,10 @@ __global__ __launch_bounds__(64 * NW) void mha_fused_kernel(const MhaArgs a) {
         }
     };
 
-    // Holding the next block's loads in registers through the multiplication costs 32 or more
-    // VGPRs, i.e. one resident wave per SIMD; measured, the third wave hides the load latency
-    // better than the prefetch does, so it is off.
-    constexpr bool kPrefetch = false;
+    // Holding the next block's loads in registers through the multiplication costs 32 VGPRs: it
+    // is done where that still fits three resident waves per SIMD (3-4 % at 512 and 2048 keys);
+    // with fewer waves per workgroup or 128-wide heads it spills or loses a wave, and is off.
+    constexpr bool kPrefetch = mha_prefetches<HD, NW>();
     const int nblocks = (klimit + kKeyBlock - 1) / kKeyBlock;
     if (kPrefetch && nblocks > 0) load_block(0);
     for (int blk = 0; blk < nblocks; blk++) {
