@@ -4,8 +4,8 @@
 //   f  = act(linear1(y1))       out = SkipLN2(linear2(f), y1)
 // The activation is applied inside linear1's kernel epilogue (on the fp32
 // accumulator) rather than as a separate pass over [rows x dimFF]; act<>() is
-// still provided for callers that use it stand-alone.  forward() issues six
-// launches on one stream, never blocks the host and writes nothing to stdout.
+// still provided for callers that use it stand-alone.  forward() issues six or
+// seven launches on one stream, never blocks the host and writes nothing to stdout.
 #pragma once
 #include <memory>
 #include <type_traits>
@@ -81,16 +81,26 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
                 "Encoder: the Linear layers must be built for batch * seq_len rows");
     }
 
+    static constexpr int kFusedLnMaxRows = 256;
+
     attn_t &attention() { return *attn; }
     int token_rows() const { return rows; }
 
     void forward(half *out, half *src, stream_t stream = nullptr) {
         attn->forward(temp_attn.get(), src, src, src, stream);
+        bool fused_ln1 = false;
         if constexpr (std::is_same_v<linear1_t, Linear<tile_mat>>) {
-            // SkipLayerNorm rides in the prologue of the tile-sparse linear1
-            linear1->forward_skipln_act(temp_linear.get(), temp_LN.get(), temp_attn.get(), src, *LN1,
-                                        act_code<ACT_OP_t>(), stream);
-        } else {
+            // Up to kFusedLnMaxRows token rows SkipLayerNorm rides in the prologue of the tile-sparse
+            // linear1 (one launch fewer: 12-layer forward of one sequence 376 -> 358 us); above that
+            // every workgroup of a strip repeating the normalisation costs more than the launch
+            // (batch 8: 544 against 534 us, batch 32: 1240 against 1184 us).
+            if (rows <= kFusedLnMaxRows) {
+                linear1->forward_skipln_act(temp_linear.get(), temp_LN.get(), temp_attn.get(), src, *LN1,
+                                            act_code<ACT_OP_t>(), stream);
+                fused_ln1 = true;
+            }
+        }
+        if (!fused_ln1) {
             LN1->forward(temp_LN.get(), temp_attn.get(), src, rows, stream);
             linear1->forward_act(temp_linear.get(), temp_LN.get(), act_code<ACT_OP_t>(), stream);
         }

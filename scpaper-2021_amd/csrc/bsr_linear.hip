@@ -495,61 +495,50 @@ static size_t bsr_lds_bytes(int mt, bool stage, int in, int rows_per_wg) {
     return stage ? (size_t)mt * 16 * (in + kLdsPad) * sizeof(_Float16) : 0;
 }
 
-// Launch geometry.  The strip is staged in LDS whenever it fits next to a second
-// workgroup (half of the 160 KiB of a compute unit), else alone, else X is read
-// from global memory.  Measured on MI355X the kernel is fastest with about one
-// workgroup of 8 waves per compute unit (~200-256 workgroups): fewer, larger
-// workgroups re-read less of X and W through the L2.  Small problems that cannot
-// fill the device that way fall back to narrower strips and smaller workgroups.
+// Launch geometry, from sweeps over 128..16384 token rows of the BERT-base and BERT-large
+// matrices.  The kernel is bound by what one compute unit can fetch (its strip of X plus its
+// share of W, about 35 GB/s per unit whatever is in flight), so the fastest geometry is almost
+// always one workgroup per compute unit: strips of MT*16 rows, each split over
+// floor(256 / strips) groups of block-rows.  Wider strips fetch W fewer times but leave each
+// workgroup fewer block-rows; they pay once a workgroup still gets two per wave (64-row strips)
+// or about one (32-row strips).  6 waves instead of 8 where that deals the block-rows evenly
+// and as fast (6 or fewer, or 18, per workgroup).
 static BsrPlan plan_bsr(int T, int in, int out) {
     const size_t lds_cap = 160 * 1024;
     const size_t row_bytes = (size_t)(in + kLdsPad) * sizeof(_Float16);
     const int nbr = out / 16;
-    int mt_fit = 0;  // widest strip that can be staged
-    if (32 * row_bytes <= lds_cap / 2) mt_fit = 2;
-    else if (16 * row_bytes <= lds_cap) mt_fit = 1;
-    struct Cand { int mt, threads; };
-    Cand cands[5];
-    int nc = 0;
-    // many token rows: 64-row strips halve the weight traffic per row again (each tile fetch
-    // feeds four MFMAs); they only pay once 64-row strips alone fill the device
-    if (64 * row_bytes <= lds_cap && T >= 64 * 128) cands[nc++] = {4, 512};
-    if (mt_fit == 2 && T >= 32) cands[nc++] = {2, 512};
-    if (mt_fit >= 1) { cands[nc++] = {1, 512}; cands[nc++] = {1, 256}; }
-    if (mt_fit == 0) cands[nc++] = {2, 256};
-    BsrPlan best{};
-    int best_wgs = -1;
-    for (int i = 0; i < nc; i++) {
-        BsrPlan p;
-        p.mt = cands[i].mt;
-        p.stage = mt_fit != 0;
-        p.threads = cands[i].threads;
-        const int nwave = p.threads / 64;
-        const int strips = (T + p.mt * 16 - 1) / (p.mt * 16);
+    BsrPlan p{};
+    if (16 * row_bytes > lds_cap) {
+        // no strip fits the LDS: X fragments are read from global memory, 4 waves, two
+        // block-rows per wave or an even split over 256 workgroups, whichever is more
+        p.mt = 2;
+        p.stage = false;
+        p.threads = 256;
+        const int strips = (T + 31) / 32;
         const int groups = strips >= 256 ? 1 : 256 / strips;
-        // block-rows per wave: the nearest whole number to an even split over `groups`
-        // workgroups, at least one (few token rows: one block-row per wave is the shortest
-        // dependent chain, and more, smaller workgroups fill the device)
-        int per_wave = (int)((double)nbr / ((double)groups * nwave) + 0.5);
-        if (per_wave < 1) per_wave = 1;
-        // heavy workgroups (several block-rows per wave) saturate a compute unit's path to the
-        // L2: more of them than compute units would run as a second, mostly empty round
-        while (per_wave >= 2 && per_wave < kMaxWaveRows &&
-               strips * ((nbr + per_wave * nwave - 1) / (per_wave * nwave)) > 256)
-            per_wave++;
-        if (per_wave > kMaxWaveRows) per_wave = kMaxWaveRows;
-        int rpw = per_wave * nwave;
+        int rpw = (nbr + groups - 1) / groups;
+        if (rpw < 8) rpw = 8;
         if (rpw > nbr) rpw = nbr;
         p.rows_per_wg = rpw;
-        p.lds = bsr_lds_bytes(p.mt, p.stage, in, rpw);
-        const int wgs = strips * ((nbr + rpw - 1) / rpw);
-        if (wgs > best_wgs) {
-            best = p;
-            best_wgs = wgs;
-        }
-        if (wgs >= 160) break;  // enough to occupy the device: prefer the earlier candidate
+        p.lds = 0;
+        return p;
     }
-    return best;
+    auto rows_per_wg_for = [&](int mt) {
+        const int strips = (T + mt * 16 - 1) / (mt * 16);
+        const int groups = strips >= 256 ? 1 : 256 / strips;
+        return (nbr + groups - 1) / groups;
+    };
+    if (64 * row_bytes <= lds_cap && T >= 64 && rows_per_wg_for(4) >= 16) p.mt = 4;
+    else if (32 * row_bytes <= lds_cap / 2 && T >= 32 && rows_per_wg_for(2) >= 5) p.mt = 2;
+    else p.mt = 1;
+    p.stage = true;
+    int rpw = rows_per_wg_for(p.mt);
+    p.threads = (rpw <= 6 || rpw == 18) ? 384 : 512;
+    const int cap = kMaxWaveRows * (p.threads / 64);
+    if (rpw > cap) rpw = cap;
+    p.rows_per_wg = rpw;
+    p.lds = bsr_lds_bytes(p.mt, p.stage, in, rpw);
+    return p;
 }
 
 // Geometry of the kernels with the fused SkipLayerNorm prologue: 8 waves, staged strip.
@@ -563,17 +552,11 @@ static BsrPlan plan_bsr_ln(int T, int in, int out) {
     // the rows to normalise per workgroup, twice the workgroups)
     p.mt = (T >= 512 && 32 * row_bytes <= lds_cap / 2) ? 2 : 1;
     p.threads = 512;
-    const int nwave = 8;
+    // one workgroup per compute unit, as in plan_bsr
     const int strips = (T + p.mt * 16 - 1) / (p.mt * 16);
     const int groups = strips >= 256 ? 1 : 256 / strips;
-    int per_wave = (int)((double)nbr / ((double)groups * nwave) + 0.5);
-    if (per_wave < 1) per_wave = 1;
-    while (per_wave >= 2 && per_wave < kMaxWaveRows &&
-           strips * ((nbr + per_wave * nwave - 1) / (per_wave * nwave)) > 256)
-        per_wave++;
-    if (per_wave > kMaxWaveRows) per_wave = kMaxWaveRows;
-    int rpw = per_wave * nwave;
-    if (rpw > nbr) rpw = nbr;
+    int rpw = (nbr + groups - 1) / groups;
+    if (rpw > kMaxWaveRows * 8) rpw = kMaxWaveRows * 8;
     p.rows_per_wg = rpw;
     p.lds = bsr_lds_bytes(p.mt, p.stage, in, rpw);
     return p;
