@@ -114,8 +114,10 @@ int et_linear_bsr16_f16(const int32_t *row_ptr, const int32_t *col_idx,
  * in one kernel: the normalisation happens while the token strip is staged on
  * chip, so the Linear does not wait for a LayerNorm kernel to drain.  Same values
  * as et_skip_layernorm_f16 followed by et_linear_bsr16_f16 (which is what runs
- * when in > 1024).  Replaces LN1->forward + linear1->forward + act<>() of
- * Encoder<cfg>::forward (Encoder/Encoder.h:85-89). */
+ * when in > 1024).  It saves a launch and repeats the normalisation in every
+ * block-row group of a strip: the faster form up to about 256 token rows, the
+ * two separate calls above that.  Replaces LN1->forward + linear1->forward +
+ * act<>() of Encoder<cfg>::forward (Encoder/Encoder.h:85-89). */
 int et_skipln_linear_bsr16_f16(const et_f16 *src, const et_f16 *skip,
                                const et_f16 *gamma, const et_f16 *beta, float eps,
                                et_f16 *ln_out, const int32_t *row_ptr,
