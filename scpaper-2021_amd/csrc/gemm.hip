@@ -223,11 +223,12 @@ static int launch_gemm_tile(const GemmArgs &g, int batch, bool trans_b, hipStrea
     return check_launch("gemm_f16_kernel");
 }
 
-// 128x128 tiles once they still give a few hundred workgroups, 64x64 otherwise.
+// The direct-to-LDS kernel where it applies; else this file's kernel, with 128x128 tiles once
+// they still give a few hundred workgroups and 64x64 otherwise.
 int launch_gemm(const GemmArgs &g, int batch, bool trans_b, hipStream_t stream) {
-    if (gemm_big_applies(g, batch, trans_b)) return launch_gemm_big(g, stream);
-    const long long big = (long long)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
-    if (big >= 512) return launch_gemm_tile<4, 4>(g, batch, trans_b, stream);
+    if (gemm_dma_applies(g, batch, trans_b)) return launch_gemm_dma(g, stream);
+    const long long tiles128 = (long long)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
+    if (tiles128 >= 512) return launch_gemm_tile<4, 4>(g, batch, trans_b, stream);
     return launch_gemm_tile<2, 2>(g, batch, trans_b, stream);
 }
 

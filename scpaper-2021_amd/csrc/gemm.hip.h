@@ -25,9 +25,10 @@ struct GemmArgs {
 // Launches the MFMA GEMM kernel over batch_outer*batch_inner problems.
 int launch_gemm(const GemmArgs &g, int batch_total, bool trans_b, hipStream_t stream);
 
-// The 256 x 256-tile kernel for large, aligned, unbatched problems (gemm_big.hip).
-bool gemm_big_applies(const GemmArgs &g, int batch_total, bool trans_b);
-int launch_gemm_big(const GemmArgs &g, hipStream_t stream);
+// The direct-to-LDS kernel for unbatched problems with B transposed whose M, N and K are
+// multiples of 64 (gemm_dma.hip); launch_gemm tries it first.
+bool gemm_dma_applies(const GemmArgs &g, int batch_total, bool trans_b);
+int launch_gemm_dma(const GemmArgs &g, hipStream_t stream);
 
 inline GemmArgs gemm_args(const _Float16 *A, const _Float16 *B, _Float16 *C, int M, int N, int K, int lda,
                           int ldb, int ldc) {

@@ -22,11 +22,11 @@
 
 namespace et {
 
-constexpr int kBigK = 64;                // K per stage: one 128-byte line of every row
-constexpr int kBigXcds = 8;
+constexpr int kDmaK = 64;                // K per stage: one 128-byte line of every row
+constexpr int kDmaXcds = 8;
 constexpr int kSbM = 4, kSbN = 8;        // tile block one XCD works on at a time
-constexpr size_t big_lds_bytes(int tmw, int tnw, int nbuf) {  // buffers of (BM + BN) rows of 128 bytes
-    return (size_t)nbuf * 64 * (tmw + tnw) * kBigK * sizeof(_Float16);
+constexpr size_t dma_lds_bytes(int tmw, int tnw, int nbuf) {  // buffers of (BM + BN) rows of 128 bytes
+    return (size_t)nbuf * 64 * (tmw + tnw) * kDmaK * sizeof(_Float16);
 }
 // s_waitcnt immediate for vmcnt(n) alone on gfx9: vmcnt in bits 3:0 and 15:14, expcnt 6:4 and
 // lgkmcnt 11:8 left at their maxima
@@ -39,13 +39,13 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 // TMW x TNW: 32 x 32 MFMA tiles per wave.  IDX: the result columns are scattered (c_scatter) or
 // their bias is gathered (bias_idx).
 template <int TMW, int TNW, int NBUF, bool IDX>
-__global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
+__global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
     static_assert(NBUF >= 2 && NBUF <= 4 && (NBUF - 2) * (2 * TMW + 2 * TNW) <= 63, "vmcnt holds 63 loads");
     constexpr int BM = 64 * TMW, BN = 64 * TNW;  // workgroup tile
     constexpr int WM = 32 * TMW, WN = 32 * TNW;  // wave block
-    extern __shared__ __align__(16) unsigned char big_smem[];
-    _Float16 *As = reinterpret_cast<_Float16 *>(big_smem);  // [NBUF][BM][kBigK], chunks swizzled
-    _Float16 *Bs = As + NBUF * BM * kBigK;                   // [NBUF][BN][kBigK]
+    extern __shared__ __align__(16) unsigned char dma_smem[];
+    _Float16 *As = reinterpret_cast<_Float16 *>(dma_smem);  // [NBUF][BM][kDmaK], chunks swizzled
+    _Float16 *Bs = As + NBUF * BM * kDmaK;                   // [NBUF][BN][kDmaK]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -56,8 +56,8 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
     // 8 of B), so the XCD's L2 serves 12 panels to 32 workgroups instead of up to 64.
     const int tiles_m = g.M / BM, tiles_n = g.N / BN;
     const int nsbx = (tiles_n + kSbN - 1) / kSbN;
-    const int xcd = blockIdx.x % kBigXcds, j = blockIdx.x / kBigXcds;
-    const int gsb = (j / (kSbM * kSbN)) * kBigXcds + xcd, within = j % (kSbM * kSbN);
+    const int xcd = blockIdx.x % kDmaXcds, j = blockIdx.x / kDmaXcds;
+    const int gsb = (j / (kSbM * kSbN)) * kDmaXcds + xcd, within = j % (kSbM * kSbN);
     const int ty = (gsb / nsbx) * kSbM + within / kSbN, tx = (gsb % nsbx) * kSbN + within % kSbN;
     if (ty >= tiles_m || tx >= tiles_n) return;  // padding of the block grid (whole workgroup)
     const int m0 = ty * BM, n0 = tx * BN;
@@ -84,29 +84,29 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
             const int r0 = wave * (BM / 4) + v * 8, r = r0 + lrow;
             const int c = lpos ^ ((r >> 1) & 7);
             __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(A + (size_t)r * g.lda + k0 + c * 8),
-                                             ET_LDS_PTR(As + (buf * BM + r0) * kBigK), 16, 0, 0);
+                                             ET_LDS_PTR(As + (buf * BM + r0) * kDmaK), 16, 0, 0);
         }
 #pragma unroll
         for (int v = 0; v < 2 * TNW; v++) {
             const int r0 = wave * (BN / 4) + v * 8, r = r0 + lrow;
             const int c = lpos ^ ((r >> 1) & 7);
             __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(B + (size_t)r * g.ldb + k0 + c * 8),
-                                             ET_LDS_PTR(Bs + (buf * BN + r0) * kBigK), 16, 0, 0);
+                                             ET_LDS_PTR(Bs + (buf * BN + r0) * kDmaK), 16, 0, 0);
         }
     };
     // fragments of one 16-wide K slice: the token tiles and feature tiles of the wave's block.
     // Rows WM wm + 32 i + l32: the swizzle term (row >> 1) & 7 depends on the lane only.
     struct Frag { h8 x[TMW], w[TNW]; };
     const int swz = (l32 >> 1) & 7;
-    const _Float16 *a_rows = As + (wm * WM + l32) * kBigK, *b_rows = Bs + (wn * WN + l32) * kBigK;
+    const _Float16 *a_rows = As + (wm * WM + l32) * kDmaK, *b_rows = Bs + (wn * WN + l32) * kDmaK;
     auto read_frag = [&](Frag &f, int buf, int ks) {
         const int chunk = ((ks * 2 + kg) ^ swz) * 8;
 #pragma unroll
         for (int i = 0; i < TMW; i++)
-            f.x[i] = *reinterpret_cast<const h8 *>(a_rows + buf * BM * kBigK + chunk + i * 32 * kBigK);
+            f.x[i] = *reinterpret_cast<const h8 *>(a_rows + buf * BM * kDmaK + chunk + i * 32 * kDmaK);
 #pragma unroll
         for (int j = 0; j < TNW; j++)
-            f.w[j] = *reinterpret_cast<const h8 *>(b_rows + buf * BN * kBigK + chunk + j * 32 * kBigK);
+            f.w[j] = *reinterpret_cast<const h8 *>(b_rows + buf * BN * kDmaK + chunk + j * 32 * kDmaK);
     };
     auto multiply = [&](const Frag &f) {
 #pragma unroll
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.w[j], f.x[i], acc[i][j], 0, 0, 0);
     };
 
-    const int nstage = g.K / kBigK;
+    const int nstage = g.K / kDmaK;
     // Stage s is multiplied from LDS buffer s % NBUF; the loads of kAhead later stages are in
     // flight meanwhile.  A direct-to-LDS load has landed when vmcnt says so, and vmcnt counts
     // in issue order: "stage s + 1 has landed" is "at most the loads of the stages after it
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
     Frag f0, f1;
 #pragma unroll
     for (int p = 0; p < kAhead; p++)
-        if (p < nstage) load_stage(p, p * kBigK);
+        if (p < nstage) load_stage(p, p * kDmaK);
     wait_stages(min(kAhead, nstage) - 1);
     lds_barrier();
     read_frag(f0, 0, 0);
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
     int cur = 0;
     for (int s = 0; s < nstage; s++) {
         const int nxt = cur + 1 == NBUF ? 0 : cur + 1;
-        if (s + kAhead < nstage) load_stage(cur == 0 ? NBUF - 1 : cur - 1, (s + kAhead) * kBigK);
+        if (s + kAhead < nstage) load_stage(cur == 0 ? NBUF - 1 : cur - 1, (s + kAhead) * kDmaK);
         read_frag(f1, cur, 1);
         multiply(f0);
         read_frag(f0, cur, 2);
@@ -172,7 +172,7 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
     // rows of 2 WN contiguous bytes.
     constexpr int kEpLd = WN + 8;
     constexpr int kRowChunks = WN / 8;  // 16-byte chunks of a stored row: 4, 8 or 16
-    _Float16 *ep = reinterpret_cast<_Float16 *>(big_smem) + wave * 32 * kEpLd;
+    _Float16 *ep = reinterpret_cast<_Float16 *>(dma_smem) + wave * 32 * kEpLd;
     const int nbase = n0 + wn * WN;
     // unconditional loads (from B when there is no bias) and a select: a load under a branch
     // is waited for on the spot
@@ -249,8 +249,8 @@ __global__ __launch_bounds__(256) void gemm_f16_big_kernel(const GemmArgs g) {
 // busy through whole rounds (a 256 x 256 workgroup owns its compute unit; two 128 x 128, three
 // 128 x 64 or five 64 x 64 ones share it and cover each other's prologue and epilogue).
 // 256 x 128 tiles and a fourth LDS buffer were measured and never won.
-struct BigTile { int tmw, tnw, nbuf; };
-static bool pick_big_tile(const GemmArgs &g, BigTile *out) {
+struct DmaTile { int tmw, tnw, nbuf; };
+static bool pick_dma_tile(const GemmArgs &g, DmaTile *out) {
     auto wgs = [&](int tmw, int tnw) -> long long {
         const int bm = 64 * tmw, bn = 64 * tnw;
         return (g.M % bm || g.N % bn) ? 0 : (long long)(g.M / bm) * (g.N / bn);
@@ -263,24 +263,24 @@ static bool pick_big_tile(const GemmArgs &g, BigTile *out) {
     if (w11 == 0) return false;
     // few workgroups with a long K loop are bound by the latency of a stage: a third buffer keeps
     // two stages in flight (2048 x 3072 -> 768: 29.5 -> 24.7 us); elsewhere it only costs occupancy
-    *out = {1, 1, (w11 <= 512 && g.K / kBigK >= 24) ? 3 : 2};
+    *out = {1, 1, (w11 <= 512 && g.K / kDmaK >= 24) ? 3 : 2};
     return true;
 }
 
-bool gemm_big_applies(const GemmArgs &g, int batch, bool trans_b) {
-    BigTile t;
-    return trans_b && batch == 1 && !g.a_gather && g.K % kBigK == 0 && pick_big_tile(g, &t);
+bool gemm_dma_applies(const GemmArgs &g, int batch, bool trans_b) {
+    DmaTile t;
+    return trans_b && batch == 1 && !g.a_gather && g.K % kDmaK == 0 && pick_dma_tile(g, &t);
 }
 
 template <int TMW, int TNW, int NBUF, bool IDX>
-static int launch_big_variant(const GemmArgs &g, hipStream_t stream) {
+static int launch_dma_variant(const GemmArgs &g, hipStream_t stream) {
     constexpr int BM = 64 * TMW, BN = 64 * TNW;
-    constexpr size_t lds = big_lds_bytes(TMW, TNW, NBUF);
+    constexpr size_t lds = dma_lds_bytes(TMW, TNW, NBUF);
     const int tiles_m = g.M / BM, tiles_n = g.N / BN;
     const int nsb = ((tiles_m + kSbM - 1) / kSbM) * ((tiles_n + kSbN - 1) / kSbN);
-    const int rounds = (nsb + kBigXcds - 1) / kBigXcds;
-    const dim3 grid((unsigned)(rounds * kBigXcds * kSbM * kSbN));
-    auto kernel = gemm_f16_big_kernel<TMW, TNW, NBUF, IDX>;
+    const int rounds = (nsb + kDmaXcds - 1) / kDmaXcds;
+    const dim3 grid((unsigned)(rounds * kDmaXcds * kSbM * kSbN));
+    auto kernel = gemm_f16_dma_kernel<TMW, TNW, NBUF, IDX>;
     static bool raised = false;  // more than 64 KB of dynamic LDS needs the attribute, once per kernel
     if (!raised) {
         ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -288,24 +288,24 @@ static int launch_big_variant(const GemmArgs &g, hipStream_t stream) {
         raised = true;
     }
     kernel<<<grid, 256, lds, stream>>>(g);
-    return check_launch("gemm_f16_big_kernel");
+    return check_launch("gemm_f16_dma_kernel");
 }
 
 template <int TMW, int TNW, int NBUF>
-static int launch_big_tile(const GemmArgs &g, hipStream_t stream) {
-    return (g.c_scatter || g.bias_idx) ? launch_big_variant<TMW, TNW, NBUF, true>(g, stream)
-                                       : launch_big_variant<TMW, TNW, NBUF, false>(g, stream);
+static int launch_dma_tile(const GemmArgs &g, hipStream_t stream) {
+    return (g.c_scatter || g.bias_idx) ? launch_dma_variant<TMW, TNW, NBUF, true>(g, stream)
+                                       : launch_dma_variant<TMW, TNW, NBUF, false>(g, stream);
 }
 
-int launch_gemm_big(const GemmArgs &g, hipStream_t stream) {
-    BigTile t{};
-    if (!pick_big_tile(g, &t)) return ET_ERR_UNSUPPORTED;
+int launch_gemm_dma(const GemmArgs &g, hipStream_t stream) {
+    DmaTile t{};
+    if (!pick_dma_tile(g, &t)) return ET_ERR_UNSUPPORTED;
     switch (t.tmw * 100 + t.tnw * 10 + t.nbuf) {
-        case 442: return launch_big_tile<4, 4, 2>(g, stream);
-        case 222: return launch_big_tile<2, 2, 2>(g, stream);
-        case 212: return launch_big_tile<2, 1, 2>(g, stream);
-        case 112: return launch_big_tile<1, 1, 2>(g, stream);
-        case 113: return launch_big_tile<1, 1, 3>(g, stream);
+        case 442: return launch_dma_tile<4, 4, 2>(g, stream);
+        case 222: return launch_dma_tile<2, 2, 2>(g, stream);
+        case 212: return launch_dma_tile<2, 1, 2>(g, stream);
+        case 112: return launch_dma_tile<1, 1, 2>(g, stream);
+        case 113: return launch_dma_tile<1, 1, 3>(g, stream);
         default: return ET_ERR_UNSUPPORTED;
     }
 }
