@@ -119,6 +119,13 @@ BSR_CASES = [
     (2048, 4096, 1024, 0.9, 0),  # BERT-large FFN
     (64, 6144, 64, 0.5, 0),      # input too wide for an LDS-staged strip
     (8192, 768, 768, 0.8, 2),    # enough token rows for 64-row strips
+    # launch-geometry paths: 6-wave workgroups (5 and 18 block-rows each), 64-row strips at 4096
+    # rows, a ragged last strip with an uneven group split, one block-row per workgroup
+    (256, 768, 2304, 0.8, 0),
+    (4096, 768, 3072, 0.8, 2),
+    (1040, 768, 768, 0.8, 1),
+    (16, 768, 3072, 0.8, 0),
+    (80, 3072, 768, 0.8, 2),
 ]
 
 
