@@ -64,11 +64,11 @@ struct MhaLds {
 // The variants that prefetch the next key block through registers (mha_prefetches) are held to
 // the 168 registers of three resident waves per SIMD; left alone the allocator takes a few more
 // and the third wave is lost, which costs more than the prefetch gains.
-template <int HD, int NW> constexpr bool mha_prefetches() { return HD <= 64 && NW == 4; }
+template <int HD, int NW, bool COMPACT> constexpr bool mha_prefetches() { return HD <= 64 && NW == 4 && !COMPACT; }
 
 template <int HD, bool COMPACT, int NW, int QT>
 __global__ __launch_bounds__(64 * NW)
-    __attribute__((amdgpu_waves_per_eu(mha_prefetches<HD, NW>() ? 3 : 1, mha_prefetches<HD, NW>() ? 3 : 8))) void
+    __attribute__((amdgpu_waves_per_eu(mha_prefetches<HD, NW, COMPACT>() ? 3 : 1, mha_prefetches<HD, NW, COMPACT>() ? 3 : 8))) void
     mha_fused_kernel(const MhaArgs a) {
     using L = MhaLds<HD>;
     constexpr int KS = HD / 32;  // K=32 MFMA steps over the head dimension
@@ -111,9 +111,20 @@ __global__ __launch_bounds__(64 * NW)
     // (no effect on scores or outputs) and are not written
     const int hd = a.hd;
     int vc0 = 0, vlive = hd;
+    bool v_vec = false;  // this head's compact columns can be read as aligned 16-byte vectors
     if (COMPACT) {
         vc0 = a.v_head_ptr[h];
         vlive = min(a.v_head_ptr[h + 1] - vc0, hd);
+        v_vec = ((vc0 | vlive | a.ldv) & 7) == 0 && vlive > 0 && (reinterpret_cast<uintptr_t>(a.V) & 15) == 0;
+    }
+    // compact-V: the full-width positions of this head's surviving columns are requested now
+    // and used in the epilogue (kCid ids per thread cover the up to 128 columns of a head)
+    constexpr int kCid = COMPACT ? (128 + nthr - 1) / nthr : 1;
+    int my_cid[kCid];
+    if (COMPACT) {
+#pragma unroll
+        for (int i = 0; i < kCid; i++)
+            my_cid[i] = a.v_col_id[vc0 + min((int)threadIdx.x + i * nthr, max(vlive - 1, 0))];
     }
 
     // Q fragments: B operand, lane supplies Q[q][32*ks + 8g .. +7]
@@ -170,12 +181,22 @@ __global__ __launch_bounds__(64 * NW)
                 const int key = (u < v_units) ? k0 + kg * 4 + i : S;  // surplus threads load nothing
                 vreg[j][i] = h8{0, 0, 0, 0, 0, 0, 0, 0};
                 if (COMPACT) {
-                    // compact columns start at an arbitrary element: scalar loads
-                    if (key < S) {
-                        const _Float16 *vp = a.V + (row0 + key) * a.ldv + vc0 + dg * 8;
+                    // Every load is unconditional, from a clamped address, and the value is
+                    // selected afterwards: a load under a branch gets a basic block of its own and
+                    // is waited for on the spot, one memory round trip per element.
+                    const bool key_ok = key < S;
+                    const _Float16 *vp = a.V + (row0 + (key_ok ? key : 0)) * a.ldv + (vlive > 0 ? vc0 : 0);
+                    if (v_vec) {  // workgroup-uniform: 16-byte vectors of surviving columns
+                        const bool live = key_ok && dg * 8 < vlive;
+                        const h8 t = *reinterpret_cast<const h8 *>(vp + (live ? dg * 8 : 0));
+                        vreg[j][i] = live ? t : h8{0, 0, 0, 0, 0, 0, 0, 0};
+                    } else {  // compact columns that start at an arbitrary element
 #pragma unroll
-                        for (int d = 0; d < 8; d++)
-                            if (dg * 8 + d < vlive) vreg[j][i][d] = vp[d];
+                        for (int d = 0; d < 8; d++) {
+                            const bool live = key_ok && dg * 8 + d < vlive;
+                            const _Float16 t = vp[live ? dg * 8 + d : 0];
+                            vreg[j][i][d] = live ? t : (_Float16)0;
+                        }
                     }
                 } else if (key < S && dg * 8 < hd) {
                     vreg[j][i] = *reinterpret_cast<const h8 *>(a.V + (row0 + key) * a.ldv + h * hd + dg * 8);
@@ -207,7 +228,7 @@ __global__ __launch_bounds__(64 * NW)
     // Holding the next block's loads in registers through the multiplication costs 32 VGPRs: it
     // is done where that still fits three resident waves per SIMD (3-4 % at 512 and 2048 keys);
     // with fewer waves per workgroup or 128-wide heads it spills or loses a wave, and is off.
-    constexpr bool kPrefetch = mha_prefetches<HD, NW>();
+    constexpr bool kPrefetch = mha_prefetches<HD, NW, COMPACT>();
     const int nblocks = (klimit + kKeyBlock - 1) / kKeyBlock;
     if (kPrefetch && nblocks > 0) load_block(0);
     for (int blk = 0; blk < nblocks; blk++) {
@@ -364,20 +385,33 @@ __global__ __launch_bounds__(64 * NW)
         }
     }
     if (COMPACT) {
-        // Full-width Z: pruned columns of this head's slice are zero, surviving
-        // ones are scattered to v_col_id.  The zero fill is made visible before
-        // the scatter so that the scatter wins wherever both touch an element.
+        // Full-width Z: surviving columns are scattered to v_col_id, the pruned columns of this
+        // head's slice get zeros.  Every element of the slice is written exactly once (the
+        // liveness mask tells the two sets apart), so no store has to be ordered against another.
+        // The column ids were requested at the start of the kernel; mask and compact-to-full map
+        // go through LDS here, where every wave of the workgroup arrives.
+        __shared__ unsigned live_mask[4];  // bit c: column c of this head's slice of Z survives
+        __shared__ int full_col[128];      // compact column -> column of Z
+        if (threadIdx.x < 4) live_mask[threadIdx.x] = 0u;
+        __syncthreads();
 #pragma unroll
-        for (int t = 0; t < QT; t++) {
-            if (q_ok[t]) {
-                _Float16 *zrow = a.Z + (row0 + q[t]) * a.ldz;
-                const h4 z4 = {0, 0, 0, 0};
-#pragma unroll
-                for (int d = 0; d < DB; d++)
-                    if (16 * d < hd) *reinterpret_cast<h4 *>(zrow + h * hd + 16 * d + 4 * g) = z4;
+        for (int i = 0; i < kCid; i++) {
+            const int j = threadIdx.x + i * nthr;
+            if (j < vlive) {
+                full_col[j] = my_cid[i];
+                const int c = my_cid[i] - h * hd;
+                if (c >= 0 && c < HD) atomicOr(&live_mask[c >> 5], 1u << (c & 31));
             }
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        __syncthreads();
+        int zc[DB][4];
+#pragma unroll
+        for (int d = 0; d < DB; d++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) zc[d][j] = full_col[min(d * 16 + 4 * g + j, 127)];
+        unsigned live_w[4];
+#pragma unroll
+        for (int w = 0; w < 4; w++) live_w[w] = live_mask[w];
 #pragma unroll
         for (int t = 0; t < QT; t++) {
             if (q_ok[t]) {
@@ -386,8 +420,9 @@ __global__ __launch_bounds__(64 * NW)
                 for (int d = 0; d < DB; d++) {
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
-                        const int dc = d * 16 + 4 * g + j;
-                        if (dc < vlive) zrow[a.v_col_id[vc0 + dc]] = (_Float16)(o[t][d][j] * inv[t]);
+                        const int dc = d * 16 + 4 * g + j;  // as a compact index, and as a column of the slice
+                        if (dc < vlive) zrow[zc[d][j]] = (_Float16)(o[t][d][j] * inv[t]);
+                        if (dc < hd && !((live_w[dc >> 5] >> (dc & 31)) & 1u)) zrow[h * hd + dc] = (_Float16)0;
                     }
                 }
             }

@@ -162,6 +162,103 @@ class Bench:
                     2 * T * len(col_id) * n_out, "mfma")
 
 
+    def vec1x16(self, T, n_in, n_out, sparsity, launches):
+        et, lib = self.et, self.lib
+        cells = (n_out // 16) * (n_in // 16 + 1)
+        tile_idx = np.zeros(cells, np.int32)
+        row_idx = np.zeros(n_out * (n_in // 16) + 16, np.int32)
+        ntile = C.c_int()
+        et.check(lib.et_fmt_1x16_pattern(n_out, n_in, sparsity, 9, tile_idx.ctypes.data, row_idx.ctypes.data,
+                                         C.byref(ntile)))
+        n = ntile.value
+        data = self.dev(self.rnd((((n + 15) // 16) * 16 + 16, 16), 0.02))
+        d_ti, d_ri = self.dev(tile_idx), self.dev(row_idx[:max(n, 1)].copy())
+        bias = self.dev(np.zeros(n_out, np.float16))
+        x, y = self.dev(self.rnd((T, n_in))), self.empty((T, n_out))
+        us = self.time_us(lambda: et.check(lib.et_linear_vec1x16_f16(d_ti.ptr, d_ri.ptr, data.ptr, bias.ptr, x.ptr, y.ptr,
+                                                                    T, n_in, n_out, 0, self.stream)), launches)
+        self.record("linear_vec1x16", f"T{T} in{n_in} out{n_out} sparsity {sparsity}", us, 2 * 16 * n * T, "mfma")
+
+    def csr(self, T, n_in, n_out, sparsity, launches):
+        et, lib = self.et, self.lib
+        indptr = np.zeros(n_out + 1, np.int32)
+        indices = np.zeros(n_out * n_in, np.int32)
+        nnz = C.c_int()
+        et.check(lib.et_fmt_csr_pattern(n_out, n_in, sparsity, 10, indptr.ctypes.data, indices.ctypes.data, C.byref(nnz)))
+        n = nnz.value
+        d_ip, d_ix = self.dev(indptr), self.dev(indices[:max(n, 1)].copy())
+        data = self.dev(self.rnd((max(n, 1),), 0.02))
+        bias = self.dev(np.zeros(n_out, np.float16))
+        x, y = self.dev(self.rnd((T, n_in))), self.empty((T, n_out))
+        us = self.time_us(lambda: et.check(lib.et_linear_csr_f16(d_ip.ptr, d_ix.ptr, data.ptr, bias.ptr, x.ptr, y.ptr, T,
+                                                                n_in, n_out, 0, self.stream)), launches)
+        self.record("linear_csr", f"T{T} in{n_in} out{n_out} sparsity {sparsity}", us, 2 * n * T, "mfma")
+
+    def mha_compactv(self, B, S, nh, hd, live_per_head, launches):
+        """Attention-aware pruning: `live_per_head` of the hd value columns of every head survive."""
+        et, lib = self.et, self.lib
+        H = nh * hd
+        col_id = np.concatenate([h * hd + np.arange(live_per_head) for h in range(nh)]).astype(np.int32)
+        head_ptr = (np.arange(nh + 1) * live_per_head).astype(np.int32)
+        nnz = len(col_id)
+        qk, vc, z = self.dev(self.rnd((B * S, 2 * H))), self.dev(self.rnd((B * S, nnz))), self.empty((B * S, H))
+        d_cid, d_hp = self.dev(col_id), self.dev(head_ptr)
+        us = self.time_us(lambda: et.check(lib.et_mha_compactv_f16(qk.ptr, qk.offset(2 * H), vc.ptr, 2 * H, 2 * H, nnz,
+                                                                  d_cid.ptr, d_hp.ptr, nnz, z.ptr, H, None, None, B, S,
+                                                                  nh, hd, hd, hd ** -0.5, 0, self.stream)), launches)
+        self.record("mha_compactv", f"B{B} S{S} nh{nh} hd{hd} live {live_per_head}", us,
+                    2 * B * S * S * nh * (hd + live_per_head), "mfma")
+
+    def mha_vo(self, B, S, nh, hd, N, launches):
+        """Pre-multiplied value/output projection (Linear_VO) and the attention over it."""
+        et, lib = self.et, self.lib
+        H = nh * hd
+        W, x = self.dev(self.rnd((nh, H, N), 0.02)), self.dev(self.rnd((B * S, H)))
+        vo = self.empty((B * nh * S, N))
+        us = self.time_us(lambda: et.check(lib.et_linear_vo_f16(W.ptr, None, x.ptr, vo.ptr, B, S, H, N, nh, self.stream)),
+                          launches)
+        self.record("linear_vo", f"B{B} S{S} H{H} N{N} nh{nh}", us, 2 * B * S * H * N * nh, "mfma")
+        qk, p, out = self.dev(self.rnd((B * S, 2 * H))), self.empty((B * S, nh * S)), self.empty((B * S, N))
+        us = self.time_us(lambda: et.check(lib.et_mha_vo_f16(qk.ptr, qk.offset(2 * H), 2 * H, 2 * H, vo.ptr, p.ptr, out.ptr,
+                                                            None, None, None, None, B, S, nh, hd, N, N, hd ** -0.5, 0,
+                                                            self.stream)), launches)
+        self.record("mha_vo", f"B{B} S{S} nh{nh} hd{hd} N{N}", us, 2 * B * S * S * nh * (hd + N), "mfma")
+
+    def mha_unfused(self, B, S, nh, hd, launches):
+        """Scores through memory: batched GEMM, stand-alone softmax, batched GEMM (the comparison line)."""
+        et, lib = self.et, self.lib
+        H = nh * hd
+        qkv, z, p = self.dev(self.rnd((B * S, 3 * H))), self.empty((B * S, H)), self.empty((B * nh * S, S))
+        us = self.time_us(lambda: et.check(lib.et_mha_unfused_f16(qkv.ptr, qkv.offset(2 * H), qkv.offset(4 * H), 3 * H, 3 * H,
+                                                                 3 * H, z.ptr, H, p.ptr, None, None, B, S, nh, hd,
+                                                                 hd ** -0.5, 0, self.stream)), launches)
+        self.record("mha_unfused", f"B{B} S{S} nh{nh} hd{hd}", us, 4 * B * S * S * hd * nh, "mfma")
+
+    def f32_layer_kernels(self, B, S, H, nh, FF, launches):
+        """The binary32 twins at the shapes of the dense fp32 layer (fp32 matrix peak 157.3 TFLOP/s)."""
+        et, lib = self.et, self.lib
+        T = B * S
+        f = lambda *shape: et.DeviceBuffer.from_numpy(self.rng.standard_normal(shape, dtype=np.float32) * 0.05)
+        e = lambda *shape: et.DeviceBuffer.empty(shape, np.float32)
+        for n_in, n_out in ((H, 3 * H), (H, H), (H, FF), (FF, H)):
+            W, x, y = f(n_out, n_in), f(T, n_in), e(T, n_out)
+            us = self.time_us(lambda: et.check(lib.et_linear_dense_f32(W.ptr, None, x.ptr, y.ptr, T, n_in, n_out, 0,
+                                                                      self.stream)), launches)
+            self.record_f32("linear_dense_f32", f"T{T} in{n_in} out{n_out}", us, 2 * T * n_in * n_out)
+        qkv, z = f(T, 3 * H), e(T, H)
+        us = self.time_us(lambda: et.check(lib.et_mha_fused_f32(qkv.ptr, qkv.offset(4 * H), qkv.offset(8 * H), 3 * H, 3 * H,
+                                                               3 * H, z.ptr, H, None, None, B, S, nh, H // nh,
+                                                               (H // nh) ** -0.5, 0, self.stream)), launches)
+        self.record_f32("mha_fused_f32", f"B{B} S{S} nh{nh} hd{H // nh}", us, 4 * B * S * S * H)
+
+    def record_f32(self, kernel, shape, us, flops):
+        achieved, peak = flops / us / 1e6, 157.3
+        self.rows.append({"kernel": kernel, "shape": shape, "us": round(us, 2), "bound": "mfma_f32",
+                          "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s", "frac": round(achieved / peak, 4)})
+        print(f"{kernel:<22} {shape:<44} {us:10.1f} us  {achieved:8.2f} TFLOP/s {100 * achieved / peak:5.1f} % of fp32 mfma peak",
+              flush=True)
+
+
 def run_configs(b: Bench):
     rng = np.random.default_rng(1)
     for B in (1, 4, 16):  # attention block, right padding with lengths in [64, 128]
@@ -178,6 +275,15 @@ def run_configs(b: Bench):
     b.mha(4, 512, 16, 64, 20, lens=rng.integers(256, 513, 4))
     for n_in, n_out in ((1024, 1024), (1024, 3072), (1024, 4096), (4096, 1024)):
         b.bsr(2048, n_in, n_out, 0.9, 50)
+    # the other weight formats and attention variants at the same configurations
+    for n_in, n_out in ((768, 768), (768, 3072), (3072, 768)):
+        b.vec1x16(2048, n_in, n_out, 0.8, 20)
+        b.csr(2048, n_in, n_out, 0.8, 10)
+    b.mha_compactv(8, 128, 12, 64, 48, 50)  # 25 % of the value columns of every head pruned
+    b.mha_vo(1, 128, 12, 64, 768, 20)
+    b.mha_vo(4, 128, 12, 64, 384, 20)       # half of the VO columns pruned
+    b.mha_unfused(4, 128, 12, 64, 20)
+    b.f32_layer_kernels(1, 128, 768, 12, 3072, 20)
 
 
 def run_scale(b: Bench):
