@@ -133,7 +133,21 @@ __global__ __launch_bounds__(256) void csr_linear_kernel(const CsrArgs a) {
         float acc = 0.0f;
         if (o < o_end) {
             const int ks = a.indptr[o], ke = a.indptr[o + 1];
-            for (int k = ks; k < ke; k++) acc += (float)a.data[k] * (float)xrow[a.indices[k]];
+            // eight non-zeros per trip: their index and value loads are issued together instead
+            // of one dependent chain per non-zero
+            int k = ks;
+            for (; k + 8 <= ke; k += 8) {
+                int idx[8];
+                _Float16 val[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) {
+                    idx[u] = a.indices[k + u];
+                    val[u] = a.data[k + u];
+                }
+#pragma unroll
+                for (int u = 0; u < 8; u++) acc += (float)val[u] * (float)xrow[idx[u]];
+            }
+            for (; k < ke; k++) acc += (float)a.data[k] * (float)xrow[a.indices[k]];
             if (a.bias) acc += (float)a.bias[o];
             acc = apply_act(acc, a.act);
         }
@@ -202,7 +216,15 @@ int et_linear_csr_f16(const int32_t *indptr, const int32_t *indices, const et_f1
     a.rows_per_wg = rpw;
     const dim3 grid((out + rpw - 1) / rpw, strips);
     const size_t lds = (size_t)16 * (in + 2) * sizeof(_Float16);
-    if (lds <= 64 * 1024) {
+    if (lds <= 160 * 1024) {
+        if (lds > 64 * 1024) {
+            static bool raised = false;  // more than 64 KB of dynamic LDS needs the attribute, once
+            if (!raised) {
+                ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(csr_linear_kernel<true>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+                raised = true;
+            }
+        }
         csr_linear_kernel<true><<<grid, 256, lds, as_stream(stream)>>>(a);
     } else {
         csr_linear_kernel<false><<<grid, 256, 0, as_stream(stream)>>>(a);
