@@ -13,68 +13,90 @@ namespace et {
 // 32*wr.. and features 32*wc.. as 2x2 MFMA tiles.  The MFMA A operand is W and the B
 // operand is X, so a lane ends with 4 consecutive output features of one token
 // (one 16-byte store).
-constexpr int kF32Tile = 64;
-constexpr int kF32K = 16;       // k-values staged per step
+constexpr int kF32K = 64;       // k-values staged per step
 constexpr int kF32Ld = kF32K + 1;  // LDS row stride in floats (odd: conflict-free column reads)
 
-template <int ACT>
+// TILE x TILE outputs per workgroup (64 or 32), a wave TILE/2 x TILE/2 of them.  The small
+// tile is for problems that would leave compute units idle with the large one: the fp32 MFMA
+// rate of the waves that run is what bounds a small problem.
+template <int ACT, int TILE>
 __global__ __launch_bounds__(256) void linear_dense_f32_kernel(const float *__restrict__ W,
                                                                const float *__restrict__ bias,
                                                                const float *__restrict__ X,
                                                                float *__restrict__ Y, int T, int in,
                                                                int out) {
-    __shared__ float xs[kF32Tile * kF32Ld];
-    __shared__ float ws[kF32Tile * kF32Ld];
+    constexpr int WB = TILE / 2;          // wave block
+    constexpr int MI = WB / 16;           // 16 x 16 MFMA tiles per wave and dimension
+    constexpr int TPR = 256 / TILE;       // staging threads per row
+    constexpr int VPT = kF32K / 4 / TPR;  // float4 per thread, operand and step
+    __shared__ float xs[TILE * kF32Ld];
+    __shared__ float ws[TILE * kF32Ld];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int wr = wave >> 1, wc = wave & 1;
-    const int tok0 = blockIdx.y * kF32Tile, f0 = blockIdx.x * kF32Tile;
+    const int tok0 = blockIdx.y * TILE, f0 = blockIdx.x * TILE;
     const int r16 = lane & 15, kq = lane >> 4;
 
-    // staging: thread -> (row 0..63, 4 consecutive k)
-    const int srow = threadIdx.x >> 2, sk = (threadIdx.x & 3) << 2;
+    // staging: thread -> (row, 4 consecutive k at sk, sk + 4 TPR, ...)
+    const int srow = threadIdx.x / TPR, sk = (threadIdx.x % TPR) << 2;
     const bool x_ok = tok0 + srow < T, w_ok = f0 + srow < out;
-    const float *xp = X + (size_t)(tok0 + (x_ok ? srow : 0)) * in + sk;
-    const float *wp = W + (size_t)(f0 + (w_ok ? srow : 0)) * in + sk;
-
-    f4 acc[2][2];
+    const float *xp = X + (size_t)(tok0 + (x_ok ? srow : 0)) * in;
+    const float *wp = W + (size_t)(f0 + (w_ok ? srow : 0)) * in;
+    const float4 zero4 = float4{0.0f, 0.0f, 0.0f, 0.0f};
+    float4 xv[VPT], wv[VPT];
+    // unconditional loads from clamped addresses and a select (a load under a branch is waited
+    // for on the spot); `in` is a multiple of 16, so a group of 4 is inside or outside
+    auto load_step = [&](int k0) {
 #pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++) acc[i][j] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int j = 0; j < VPT; j++) {
+            const int k = k0 + sk + 4 * TPR * j;
+            const bool k_ok = k < in;
+            xv[j] = *reinterpret_cast<const float4 *>(xp + (k_ok ? k : 0));
+            wv[j] = *reinterpret_cast<const float4 *>(wp + (k_ok ? k : 0));
+            if (!(x_ok && k_ok)) xv[j] = zero4;
+            if (!(w_ok && k_ok)) wv[j] = zero4;
+        }
+    };
 
+    f4 acc[MI][MI];
+#pragma unroll
+    for (int i = 0; i < MI; i++)
+#pragma unroll
+        for (int j = 0; j < MI; j++) acc[i][j] = f4{0.0f, 0.0f, 0.0f, 0.0f};
+
+    load_step(0);
     for (int k0 = 0; k0 < in; k0 += kF32K) {
-        float4 xv = *reinterpret_cast<const float4 *>(xp + k0);
-        float4 wv = *reinterpret_cast<const float4 *>(wp + k0);
-        if (!x_ok) xv = float4{0.0f, 0.0f, 0.0f, 0.0f};
-        if (!w_ok) wv = float4{0.0f, 0.0f, 0.0f, 0.0f};
         __syncthreads();  // the previous step's reads are done
-        float *xd = xs + srow * kF32Ld + sk, *wd = ws + srow * kF32Ld + sk;
-        xd[0] = xv.x; xd[1] = xv.y; xd[2] = xv.z; xd[3] = xv.w;
-        wd[0] = wv.x; wd[1] = wv.y; wd[2] = wv.z; wd[3] = wv.w;
+#pragma unroll
+        for (int j = 0; j < VPT; j++) {
+            float *xd = xs + srow * kF32Ld + sk + 4 * TPR * j, *wd = ws + srow * kF32Ld + sk + 4 * TPR * j;
+            xd[0] = xv[j].x; xd[1] = xv[j].y; xd[2] = xv[j].z; xd[3] = xv[j].w;
+            wd[0] = wv[j].x; wd[1] = wv[j].y; wd[2] = wv[j].z; wd[3] = wv[j].w;
+        }
         __syncthreads();
+        load_step(k0 + kF32K);  // the next step travels while this one is multiplied (past the end: zeros)
 #pragma unroll
         for (int kk = 0; kk < kF32K; kk += 4) {
-            float a[2], b[2];
+            float a[MI], b[MI];
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                a[i] = ws[(wc * 32 + i * 16 + r16) * kF32Ld + kk + kq];  // A[m = feature][k]
-                b[i] = xs[(wr * 32 + i * 16 + r16) * kF32Ld + kk + kq];  // B[k][n = token]
+            for (int i = 0; i < MI; i++) {
+                a[i] = ws[(wc * WB + i * 16 + r16) * kF32Ld + kk + kq];  // A[m = feature][k]
+                b[i] = xs[(wr * WB + i * 16 + r16) * kF32Ld + kk + kq];  // B[k][n = token]
             }
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < MI; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++)
+                for (int j = 0; j < MI; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j], b[i], acc[i][j], 0, 0, 0);
         }
     }
-    // acc[i][j]: token tok0 + 32*wr + 16*i + r16, features f0 + 32*wc + 16*j + 4*kq .. +3
+    // acc[i][j]: token tok0 + WB*wr + 16*i + r16, features f0 + WB*wc + 16*j + 4*kq .. +3
 #pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int t = tok0 + wr * 32 + i * 16 + r16;
+    for (int i = 0; i < MI; i++) {
+        const int t = tok0 + wr * WB + i * 16 + r16;
         if (t >= T) continue;
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int f = f0 + wc * 32 + j * 16 + kq * 4;
+        for (int j = 0; j < MI; j++) {
+            const int f = f0 + wc * WB + j * 16 + kq * 4;
             if (f >= out) continue;  // out % 4 == 0: a group of 4 is inside or outside
             float4 o;
             float *po = reinterpret_cast<float *>(&o);
@@ -224,13 +246,22 @@ int et_linear_dense_f32(const float *W, const float *bias, const float *X, float
     ET_REQUIRE(((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(Y)) & 15) == 0,
                ET_ERR_UNSUPPORTED, "et_linear_dense_f32: W, X and Y must be 16-byte aligned");
     if (T == 0) return ET_OK;
-    const dim3 grid((out + kF32Tile - 1) / kF32Tile, (T + kF32Tile - 1) / kF32Tile);
     hipStream_t st = as_stream(stream);
-    switch (act) {
-        case ET_ACT_RELU: linear_dense_f32_kernel<ET_ACT_RELU><<<grid, 256, 0, st>>>(W, bias, X, Y, T, in, out); break;
-        case ET_ACT_GELU: linear_dense_f32_kernel<ET_ACT_GELU><<<grid, 256, 0, st>>>(W, bias, X, Y, T, in, out); break;
-        default: linear_dense_f32_kernel<ET_ACT_NONE><<<grid, 256, 0, st>>>(W, bias, X, Y, T, in, out); break;
+    // 64 x 64 tiles once they give every compute unit a workgroup, 32 x 32 below that
+    const bool small = (long long)((out + 63) / 64) * ((T + 63) / 64) < 256;
+    const int tile = small ? 32 : 64;
+    const dim3 grid((out + tile - 1) / tile, (T + tile - 1) / tile);
+#define ET_F32_LINEAR(ACTV)                                                                        \
+    {                                                                                              \
+        if (small) linear_dense_f32_kernel<ACTV, 32><<<grid, 256, 0, st>>>(W, bias, X, Y, T, in, out); \
+        else linear_dense_f32_kernel<ACTV, 64><<<grid, 256, 0, st>>>(W, bias, X, Y, T, in, out);       \
     }
+    switch (act) {
+        case ET_ACT_RELU: ET_F32_LINEAR(ET_ACT_RELU) break;
+        case ET_ACT_GELU: ET_F32_LINEAR(ET_ACT_GELU) break;
+        default: ET_F32_LINEAR(ET_ACT_NONE) break;
+    }
+#undef ET_F32_LINEAR
     return check_launch("linear_dense_f32_kernel");
 }
 
