@@ -37,8 +37,10 @@ constexpr int wait_vm(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0F70; }
 typedef float f16v __attribute__((ext_vector_type(16)));
 
 // TMW x TNW: 32 x 32 MFMA tiles per wave.  IDX: the result columns are scattered (c_scatter) or
-// their bias is gathered (bias_idx).
-template <int TMW, int TNW, int NBUF, bool IDX>
+// their bias is gathered (bias_idx).  RAGGED: M, N and K are multiples of 16 only; rows past the
+// end of an operand are loaded from its last row and never stored, the chunks of the last K
+// stage past the end of K are zeroed in LDS before they are read.
+template <int TMW, int TNW, int NBUF, bool IDX, bool RAGGED = false>
 __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
     static_assert(NBUF >= 2 && NBUF <= 4 && (NBUF - 2) * (2 * TMW + 2 * TNW) <= 63, "vmcnt holds 63 loads");
     constexpr int BM = 64 * TMW, BN = 64 * TNW;  // workgroup tile
@@ -54,15 +56,13 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
     // Workgroup id -> tile, XCD-aware.  Workgroups go to the 8 XCDs round-robin by id and each
     // XCD runs 32 of them at a time; those 32 are given a 4 x 8 block of tiles (4 panels of A,
     // 8 of B), so the XCD's L2 serves 12 panels to 32 workgroups instead of up to 64.
-    const int tiles_m = g.M / BM, tiles_n = g.N / BN;
+    const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     const int nsbx = (tiles_n + kSbN - 1) / kSbN;
     const int xcd = blockIdx.x % kDmaXcds, j = blockIdx.x / kDmaXcds;
     const int gsb = (j / (kSbM * kSbN)) * kDmaXcds + xcd, within = j % (kSbM * kSbN);
     const int ty = (gsb / nsbx) * kSbM + within / kSbN, tx = (gsb % nsbx) * kSbN + within % kSbN;
     if (ty >= tiles_m || tx >= tiles_n) return;  // padding of the block grid (whole workgroup)
     const int m0 = ty * BM, n0 = tx * BN;
-    const _Float16 *A = g.A + (size_t)m0 * g.lda;
-    const _Float16 *B = g.B + (size_t)n0 * g.ldb;
 
     f16v acc[TMW][TNW];  // [token tile][feature tile]
 #pragma unroll
@@ -83,15 +83,37 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
         for (int v = 0; v < 2 * TMW; v++) {  // a wave loads a quarter of the rows of each operand
             const int r0 = wave * (BM / 4) + v * 8, r = r0 + lrow;
             const int c = lpos ^ ((r >> 1) & 7);
-            __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(A + (size_t)r * g.lda + k0 + c * 8),
+            const int row = RAGGED ? min(m0 + r, g.M - 1) : m0 + r;
+            const int k = RAGGED ? min(k0 + c * 8, g.K - 8) : k0 + c * 8;
+            __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(g.A + (size_t)row * g.lda + k),
                                              ET_LDS_PTR(As + (buf * BM + r0) * kDmaK), 16, 0, 0);
         }
 #pragma unroll
         for (int v = 0; v < 2 * TNW; v++) {
             const int r0 = wave * (BN / 4) + v * 8, r = r0 + lrow;
             const int c = lpos ^ ((r >> 1) & 7);
-            __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(B + (size_t)r * g.ldb + k0 + c * 8),
+            const int row = RAGGED ? min(n0 + r, g.N - 1) : n0 + r;
+            const int k = RAGGED ? min(k0 + c * 8, g.K - 8) : k0 + c * 8;
+            __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(g.B + (size_t)row * g.ldb + k),
                                              ET_LDS_PTR(Bs + (buf * BN + r0) * kDmaK), 16, 0, 0);
+        }
+    };
+    // RAGGED: zeros over the chunks of the last stage that lie past the end of K, in the rows
+    // this wave loaded (after its loads have landed, before the barrier that releases the buffer)
+    const int ktail = g.K - (g.K - 1) / kDmaK * kDmaK;  // k-values of the last stage, 16..64
+    auto zero_tail = [&](int buf) {
+        const h8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int v = 0; v < 2 * TMW; v++) {
+            const int r = wave * (BM / 4) + v * 8 + lrow;
+            if ((lpos ^ ((r >> 1) & 7)) * 8 >= ktail)
+                *reinterpret_cast<h8 *>(As + (buf * BM + r) * kDmaK + lpos * 8) = zero8;
+        }
+#pragma unroll
+        for (int v = 0; v < 2 * TNW; v++) {
+            const int r = wave * (BN / 4) + v * 8 + lrow;
+            if ((lpos ^ ((r >> 1) & 7)) * 8 >= ktail)
+                *reinterpret_cast<h8 *>(Bs + (buf * BN + r) * kDmaK + lpos * 8) = zero8;
         }
     };
     // fragments of one 16-wide K slice: the token tiles and feature tiles of the wave's block.
@@ -116,7 +138,7 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.w[j], f.x[i], acc[i][j], 0, 0, 0);
     };
 
-    const int nstage = g.K / kDmaK;
+    const int nstage = RAGGED ? (g.K + kDmaK - 1) / kDmaK : g.K / kDmaK;
     // Stage s is multiplied from LDS buffer s % NBUF; the loads of kAhead later stages are in
     // flight meanwhile.  A direct-to-LDS load has landed when vmcnt says so, and vmcnt counts
     // in issue order: "stage s + 1 has landed" is "at most the loads of the stages after it
@@ -138,6 +160,7 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
     for (int p = 0; p < kAhead; p++)
         if (p < nstage) load_stage(p, p * kDmaK);
     wait_stages(min(kAhead, nstage) - 1);
+    if (RAGGED && nstage == 1 && ktail < kDmaK) zero_tail(0);
     lds_barrier();
     read_frag(f0, 0, 0);
     // One stage, with the matrix pipe fed across the barrier: every K slice is read from LDS
@@ -159,6 +182,7 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
         read_frag(f1, cur, 3);
         multiply(f0);
         wait_stages(min(kAhead - 1, nstage - 2 - s));
+        if (RAGGED && s + 2 == nstage && ktail < kDmaK) zero_tail(nxt);
         lds_barrier();
         read_frag(f0, nxt, 0);
         multiply(f1);
@@ -185,7 +209,8 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
         for (int q = 0; q < 4; q++)
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const int n = nbase + j * 32 + q * 8 + kg * 4 + e;
+                int n = nbase + j * 32 + q * 8 + kg * 4 + e;
+                if (RAGGED) n = min(n, g.N - 1);
                 _Float16 bv;
                 if (IDX) {
                     const int bi = col_idx ? col_idx[n] : n;
@@ -207,7 +232,7 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
 #pragma unroll
         for (int e = 0; e < kScCols; e++) {
             const int n = nbase + e * kScLanes + lane % kScLanes;
-            scat[e] = scatter ? g.c_scatter[n] : n;
+            scat[e] = scatter ? g.c_scatter[RAGGED ? min(n, g.N - 1) : n] : n;
         }
     }
     const int act = g.act;
@@ -228,16 +253,23 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
 #pragma unroll
             for (int v = 0; v < 32 / kScRows; v++) {
                 const int r = v * kScRows + lane / kScLanes;
-                _Float16 *crow = g.C + (size_t)(m0 + wm * WM + i * 32 + r) * g.ldc;
+                const int m = m0 + wm * WM + i * 32 + r;
+                _Float16 *crow = g.C + (size_t)m * g.ldc;
 #pragma unroll
-                for (int e = 0; e < kScCols; e++) crow[scat[e]] = ep[r * kEpLd + e * kScLanes + lane % kScLanes];
+                for (int e = 0; e < kScCols; e++) {
+                    const bool inside = !RAGGED || (m < g.M && nbase + e * kScLanes + lane % kScLanes < g.N);
+                    if (inside) crow[scat[e]] = ep[r * kEpLd + e * kScLanes + lane % kScLanes];
+                }
             }
         } else {
 #pragma unroll
             for (int v = 0; v < 32 * kRowChunks / 64; v++) {
                 const int idx = lane + v * 64, r = idx / kRowChunks, c = idx % kRowChunks;
                 const h8 val = *reinterpret_cast<const h8 *>(ep + r * kEpLd + c * 8);
-                *reinterpret_cast<h8 *>(g.C + (size_t)(m0 + wm * WM + i * 32 + r) * g.ldc + nbase + c * 8) = val;
+                const int m = m0 + wm * WM + i * 32 + r;
+                // N is a multiple of 16: a chunk of 8 columns is inside or outside as a whole
+                if (!RAGGED || (m < g.M && nbase + c * 8 < g.N))
+                    *reinterpret_cast<h8 *>(g.C + (size_t)m * g.ldc + nbase + c * 8) = val;
             }
         }
         __syncthreads();
@@ -249,38 +281,51 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
 // busy through whole rounds (a 256 x 256 workgroup owns its compute unit; two 128 x 128, three
 // 128 x 64 or five 64 x 64 ones share it and cover each other's prologue and epilogue).
 // 256 x 128 tiles and a fourth LDS buffer were measured and never won.
-struct DmaTile { int tmw, tnw, nbuf; };
+struct DmaTile { int tmw, tnw, nbuf; bool ragged; };
 static bool pick_dma_tile(const GemmArgs &g, DmaTile *out) {
+    const bool ragged = g.M % 64 || g.N % 64 || g.K % kDmaK;
+    if (ragged) {
+        // 64 x 64 tiles with the edges clamped and masked; large ragged problems are left to the
+        // 128 x 128 tiles of the register-staged kernel
+        const long long w = (long long)((g.M + 63) / 64) * ((g.N + 63) / 64);
+        if (g.M % 16 || g.N % 16 || g.K % 16 || w > 1536) return false;
+        *out = {1, 1, (w <= 512 && g.K / kDmaK >= 24) ? 3 : 2, true};  // third buffer: as below
+        return true;
+    }
     auto wgs = [&](int tmw, int tnw) -> long long {
         const int bm = 64 * tmw, bn = 64 * tnw;
         return (g.M % bm || g.N % bn) ? 0 : (long long)(g.M / bm) * (g.N / bn);
     };
     const long long w44 = wgs(4, 4), w11 = wgs(1, 1);
     // whole rounds of one workgroup per compute unit, or so many that the last one hardly counts
-    if (w44 >= 256 && (w44 % 256 == 0 || w44 >= 1024)) { *out = {4, 4, 2}; return true; }
-    if (wgs(2, 2) >= 512) { *out = {2, 2, 2}; return true; }
-    if (wgs(2, 1) >= 512) { *out = {2, 1, 2}; return true; }
-    if (w11 == 0) return false;
+    if (w44 >= 256 && (w44 % 256 == 0 || w44 >= 1024)) { *out = {4, 4, 2, false}; return true; }
+    if (wgs(2, 2) >= 512) { *out = {2, 2, 2, false}; return true; }
+    if (wgs(2, 1) >= 512) { *out = {2, 1, 2, false}; return true; }
     // few workgroups with a long K loop are bound by the latency of a stage: a third buffer keeps
     // two stages in flight (2048 x 3072 -> 768: 29.5 -> 24.7 us); elsewhere it only costs occupancy
-    *out = {1, 1, (w11 <= 512 && g.K / kDmaK >= 24) ? 3 : 2};
+    *out = {1, 1, (w11 <= 512 && g.K / kDmaK >= 24) ? 3 : 2, false};
     return true;
 }
 
+// The kernel moves 16 bytes at a time: operands and result 16-byte aligned, leading dimensions
+// multiples of 8.
 bool gemm_dma_applies(const GemmArgs &g, int batch, bool trans_b) {
     DmaTile t;
-    return trans_b && batch == 1 && !g.a_gather && g.K % kDmaK == 0 && pick_dma_tile(g, &t);
+    const auto misaligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; };
+    if (!trans_b || batch != 1 || g.a_gather || g.M <= 0) return false;
+    if (g.lda % 8 || g.ldb % 8 || g.ldc % 8 || misaligned(g.A) || misaligned(g.B) || misaligned(g.C)) return false;
+    return pick_dma_tile(g, &t);
 }
 
-template <int TMW, int TNW, int NBUF, bool IDX>
+template <int TMW, int TNW, int NBUF, bool IDX, bool RAGGED>
 static int launch_dma_variant(const GemmArgs &g, hipStream_t stream) {
     constexpr int BM = 64 * TMW, BN = 64 * TNW;
     constexpr size_t lds = dma_lds_bytes(TMW, TNW, NBUF);
-    const int tiles_m = g.M / BM, tiles_n = g.N / BN;
+    const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     const int nsb = ((tiles_m + kSbM - 1) / kSbM) * ((tiles_n + kSbN - 1) / kSbN);
     const int rounds = (nsb + kDmaXcds - 1) / kDmaXcds;
     const dim3 grid((unsigned)(rounds * kDmaXcds * kSbM * kSbN));
-    auto kernel = gemm_f16_dma_kernel<TMW, TNW, NBUF, IDX>;
+    auto kernel = gemm_f16_dma_kernel<TMW, TNW, NBUF, IDX, RAGGED>;
     static bool raised = false;  // more than 64 KB of dynamic LDS needs the attribute, once per kernel
     if (!raised) {
         ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -291,15 +336,16 @@ static int launch_dma_variant(const GemmArgs &g, hipStream_t stream) {
     return check_launch("gemm_f16_dma_kernel");
 }
 
-template <int TMW, int TNW, int NBUF>
+template <int TMW, int TNW, int NBUF, bool RAGGED = false>
 static int launch_dma_tile(const GemmArgs &g, hipStream_t stream) {
-    return (g.c_scatter || g.bias_idx) ? launch_dma_variant<TMW, TNW, NBUF, true>(g, stream)
-                                       : launch_dma_variant<TMW, TNW, NBUF, false>(g, stream);
+    return (g.c_scatter || g.bias_idx) ? launch_dma_variant<TMW, TNW, NBUF, true, RAGGED>(g, stream)
+                                       : launch_dma_variant<TMW, TNW, NBUF, false, RAGGED>(g, stream);
 }
 
 int launch_gemm_dma(const GemmArgs &g, hipStream_t stream) {
     DmaTile t{};
     if (!pick_dma_tile(g, &t)) return ET_ERR_UNSUPPORTED;
+    if (t.ragged) return t.nbuf == 3 ? launch_dma_tile<1, 1, 3, true>(g, stream) : launch_dma_tile<1, 1, 2, true>(g, stream);
     switch (t.tmw * 100 + t.tnw * 10 + t.nbuf) {
         case 442: return launch_dma_tile<4, 4, 2>(g, stream);
         case 222: return launch_dma_tile<2, 2, 2>(g, stream);

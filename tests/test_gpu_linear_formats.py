@@ -20,7 +20,10 @@ up = Hn.up
                                            # one shape per tile of the direct-to-LDS kernel: 256x256, 128x128,
                                            # 128x64, 64x64 with three LDS buffers, a single K stage
                                            (4096, 192, 4096, 2), (2048, 128, 4096, 1), (2048, 192, 2304, 0),
-                                           (512, 1536, 768, 2), (256, 64, 256, 0)])
+                                           (512, 1536, 768, 2), (256, 64, 256, 0),
+                                           # edges that are multiples of 16 only (clamped loads, zeroed K tail,
+                                           # masked stores): 16, 32 and 48 k-values in the last stage
+                                           (1008, 720, 400, 2), (80, 96, 2064, 1), (2032, 176, 48, 0)])
 def test_linear_dense(et, T, inp, out, act):
     W, b, x = Hn.randn((out, inp), 1, 0.02), Hn.randn((out,), 2, 0.1), Hn.randn((T, inp), 3)
     d_y = et.DeviceBuffer.empty((T, out), np.float16)
@@ -81,7 +84,8 @@ def test_gemm_rejects_bad_args(et):
 
 @pytest.mark.parametrize("T,inp,out,sp,act", [(2048, 768, 768, 0.5, 0), (2048, 768, 3072, 0.5, 2),
                                               (2048, 3072, 768, 0.5, 0), (64, 64, 100 * 16, 0.9, 1),
-                                              (8192, 128, 4096, 0.5, 2)])  # last: the 256 x 256-tile kernel
+                                              (8192, 128, 4096, 0.5, 2),  # the 256 x 256-tile kernel
+                                              (2048, 720, 784, 0.45, 1)])  # 432 surviving rows: a ragged tile edge
 def test_linear_rowpruned(et, T, inp, out, sp, act):
     row_id = F.gen_row_ids(out, sp, seed=8)
     rows, b, x = Hn.randn((len(row_id), inp), 9, 0.02), Hn.randn((out,), 10, 0.1), Hn.randn((T, inp), 11)
