@@ -185,6 +185,19 @@ def run_layer_case(et, H, nh, dimFF, S, B, sparsity, seed, lens=None, nlayers=1,
     return max_abs(got, want)
 
 
+def check_tile_pattern(bw, what):
+    """The generators cannot produce a column tile outside the matrix; one that shows up later
+    means the host array changed after it was built.  Says where and what, for the log."""
+    bc = bw.inp // 16
+    if len(bw.col_idx) and (bw.col_idx.min() < 0 or bw.col_idx.max() >= bc):
+        bad = np.nonzero((bw.col_idx < 0) | (bw.col_idx >= bc))[0]
+        lo = max(0, int(bad[0]) - 8)
+        raise AssertionError(
+            f"{what}: col_idx of {len(bw.col_idx)} tiles holds {len(bad)} values outside [0, {bc}) although it was "
+            f"generated inside: first at {bad[:8]}, values {bw.col_idx[bad[:8]]}, col_idx[{lo}:{lo + 40}] = "
+            f"{bw.col_idx[lo:lo + 40]}, array at {bw.col_idx.ctypes.data:#x} (owns its data: {bw.col_idx.flags.owndata})")
+
+
 def build_model(et, layers, S, B, act=2, lens=None, use_graph=True, causal=False, eps=1e-5):
     """Encoder stack through et_model_* from a list of LayerWeights (exact fp16 bits)."""
     w0 = layers[0]
@@ -192,6 +205,7 @@ def build_model(et, layers, S, B, act=2, lens=None, use_graph=True, causal=False
                  use_graph=use_graph)
     for i, w in enumerate(layers):
         for which, bw in ((et.W_QKV, w.qkv), (et.W_O, w.o), (et.W_FF1, w.l1), (et.W_FF2, w.l2)):
+            check_tile_pattern(bw, f"layer {i} matrix {which}")
             m.set_bsr16(i, which, bw.row_ptr, bw.col_idx, bw.tiles, bw.bias)
         m.set_norm(i, 0, w.g1, w.be1)
         m.set_norm(i, 1, w.g2, w.be2)
