@@ -226,7 +226,7 @@ static int launch_gemm_tile(const GemmArgs &g, int batch, bool trans_b, hipStrea
 // The direct-to-LDS kernel where it applies; else this file's kernel, with 128x128 tiles once
 // they still give a few hundred workgroups and 64x64 otherwise.
 int launch_gemm(const GemmArgs &g, int batch, bool trans_b, hipStream_t stream) {
-    if (gemm_dma_applies(g, batch, trans_b)) return launch_gemm_dma(g, stream);
+    if (gemm_dma_applies(g, batch, trans_b)) return launch_gemm_dma(g, batch, trans_b, stream);
     const long long tiles128 = (long long)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
     if (tiles128 >= 512) return launch_gemm_tile<4, 4>(g, batch, trans_b, stream);
     return launch_gemm_tile<2, 2>(g, batch, trans_b, stream);

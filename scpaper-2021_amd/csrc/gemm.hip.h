@@ -25,10 +25,10 @@ struct GemmArgs {
 // Launches the MFMA GEMM kernel over batch_outer*batch_inner problems.
 int launch_gemm(const GemmArgs &g, int batch_total, bool trans_b, hipStream_t stream);
 
-// The direct-to-LDS kernel for unbatched problems with B transposed whose M, N and K are
-// multiples of 64 (gemm_dma.hip); launch_gemm tries it first.
+// The direct-to-LDS kernel (gemm_dma.hip) for problems without an A-column gather whose M, N and K are
+// multiples of 16 and whose operands are 16-byte aligned; launch_gemm tries it first.
 bool gemm_dma_applies(const GemmArgs &g, int batch_total, bool trans_b);
-int launch_gemm_dma(const GemmArgs &g, hipStream_t stream);
+int launch_gemm_dma(const GemmArgs &g, int batch_total, bool trans_b, hipStream_t stream);
 
 inline GemmArgs gemm_args(const _Float16 *A, const _Float16 *B, _Float16 *C, int M, int N, int K, int lda,
                           int ldb, int ldc) {

@@ -40,9 +40,21 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 // their bias is gathered (bias_idx).  RAGGED: M, N and K are multiples of 16 only; rows past the
 // end of an operand are loaded from its last row and never stored, the chunks of the last K
 // stage past the end of K are zeroed in LDS before they are read.
-template <int TMW, int TNW, int NBUF, bool IDX, bool RAGGED = false>
-__global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
+// BT: B is stored [K x N] (N contiguous) instead of [N x K]; its stage lies in LDS as loaded, k-major,
+// and a lane gathers the 8 k-values of a fragment with 2-byte reads (64 x 64 tiles only).
+// Problem z = blockIdx.y of a batch uses the operand offsets of GemmArgs.
+template <int TMW, int TNW, int NBUF, bool IDX, bool RAGGED = false, bool BT = false>
+__global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
     static_assert(NBUF >= 2 && NBUF <= 4 && (NBUF - 2) * (2 * TMW + 2 * TNW) <= 63, "vmcnt holds 63 loads");
+    static_assert(!BT || (TMW == 1 && TNW == 1 && RAGGED), "the k-major B stage is written for the 64 x 64 tile");
+    GemmArgs g = ga;
+    {
+        const long long zo = blockIdx.y / g.batch_inner, zi = blockIdx.y % g.batch_inner;
+        g.A += zo * g.sAo + zi * g.sAi;
+        g.B += zo * g.sBo + zi * g.sBi;
+        g.C += zo * g.sCo + zi * g.sCi;
+        if (g.bias) g.bias += zo * g.sBias_o + zi * g.sBias_i;
+    }
     constexpr int BM = 64 * TMW, BN = 64 * TNW;  // workgroup tile
     constexpr int WM = 32 * TMW, WN = 32 * TNW;  // wave block
     extern __shared__ __align__(16) unsigned char dma_smem[];
@@ -91,11 +103,17 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
 #pragma unroll
         for (int v = 0; v < 2 * TNW; v++) {
             const int r0 = wave * (BN / 4) + v * 8, r = r0 + lrow;
-            const int c = lpos ^ ((r >> 1) & 7);
-            const int row = RAGGED ? min(n0 + r, g.N - 1) : n0 + r;
-            const int k = RAGGED ? min(k0 + c * 8, g.K - 8) : k0 + c * 8;
-            __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(g.B + (size_t)row * g.ldb + k),
-                                             ET_LDS_PTR(Bs + (buf * BN + r0) * kDmaK), 16, 0, 0);
+            if (BT) {  // LDS row r = k-value k0 + r of the stage, 64 columns of B from n0
+                const int krow = min(k0 + r, g.K - 1), n = min(n0 + lpos * 8, g.N - 8);
+                __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(g.B + (size_t)krow * g.ldb + n),
+                                                 ET_LDS_PTR(Bs + (buf * kDmaK + r0) * BN), 16, 0, 0);
+            } else {
+                const int c = lpos ^ ((r >> 1) & 7);
+                const int row = RAGGED ? min(n0 + r, g.N - 1) : n0 + r;
+                const int k = RAGGED ? min(k0 + c * 8, g.K - 8) : k0 + c * 8;
+                __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(g.B + (size_t)row * g.ldb + k),
+                                                 ET_LDS_PTR(Bs + (buf * BN + r0) * kDmaK), 16, 0, 0);
+            }
         }
     };
     // RAGGED: zeros over the chunks of the last stage that lie past the end of K, in the rows
@@ -112,8 +130,11 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
 #pragma unroll
         for (int v = 0; v < 2 * TNW; v++) {
             const int r = wave * (BN / 4) + v * 8 + lrow;
-            if ((lpos ^ ((r >> 1) & 7)) * 8 >= ktail)
+            if (BT) {  // whole k-rows past the end of K
+                if (r >= ktail) *reinterpret_cast<h8 *>(Bs + (buf * kDmaK + r) * BN + lpos * 8) = zero8;
+            } else if ((lpos ^ ((r >> 1) & 7)) * 8 >= ktail) {
                 *reinterpret_cast<h8 *>(Bs + (buf * BN + r) * kDmaK + lpos * 8) = zero8;
+            }
         }
     };
     // fragments of one 16-wide K slice: the token tiles and feature tiles of the wave's block.
@@ -127,8 +148,15 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
         for (int i = 0; i < TMW; i++)
             f.x[i] = *reinterpret_cast<const h8 *>(a_rows + buf * BM * kDmaK + chunk + i * 32 * kDmaK);
 #pragma unroll
-        for (int j = 0; j < TNW; j++)
-            f.w[j] = *reinterpret_cast<const h8 *>(b_rows + buf * BN * kDmaK + chunk + j * 32 * kDmaK);
+        for (int j = 0; j < TNW; j++) {
+            if (BT) {
+                const _Float16 *col = Bs + (buf * kDmaK + ks * 16 + kg * 8) * BN + wn * WN + l32;
+#pragma unroll
+                for (int e = 0; e < 8; e++) f.w[j][e] = col[e * BN];
+            } else {
+                f.w[j] = *reinterpret_cast<const h8 *>(b_rows + buf * BN * kDmaK + chunk + j * 32 * kDmaK);
+            }
+        }
     };
     auto multiply = [&](const Frag &f) {
 #pragma unroll
@@ -282,13 +310,19 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs g) {
 // 128 x 64 or five 64 x 64 ones share it and cover each other's prologue and epilogue).
 // 256 x 128 tiles and a fourth LDS buffer were measured and never won.
 struct DmaTile { int tmw, tnw, nbuf; bool ragged; };
-static bool pick_dma_tile(const GemmArgs &g, DmaTile *out) {
-    const bool ragged = g.M % 64 || g.N % 64 || g.K % kDmaK;
+static bool pick_dma_tile(const GemmArgs &g, int batch, bool trans_b, DmaTile *out) {
+    const bool ragged = g.M % 64 || g.N % 64 || g.K % kDmaK || batch != 1 || !trans_b;
     if (ragged) {
         // 64 x 64 tiles with the edges clamped and masked; large ragged problems are left to the
         // 128 x 128 tiles of the register-staged kernel
-        const long long w = (long long)((g.M + 63) / 64) * ((g.N + 63) / 64);
+        const long long w = (long long)((g.M + 63) / 64) * ((g.N + 63) / 64) * batch;
         if (g.M % 16 || g.N % 16 || g.K % 16 || w > 1536) return false;
+        // Batched problems and B stored k-major run on this instantiation too, where they are
+        // bound by the latency of a long K loop in few workgroups (the stacked VO product of the
+        // pre-computed-VO attention: 32 -> 22 us); gathering the k-major fragments with 2-byte LDS
+        // reads costs more than it saves elsewhere (Linear_VO 28 -> 78 us), those stay on the
+        // register-staged kernel.
+        if ((batch != 1 || !trans_b) && (w > 256 || g.K / kDmaK < 16)) return false;
         *out = {1, 1, (w <= 512 && g.K / kDmaK >= 24) ? 3 : 2, true};  // third buffer: as below
         return true;
     }
@@ -312,20 +346,21 @@ static bool pick_dma_tile(const GemmArgs &g, DmaTile *out) {
 bool gemm_dma_applies(const GemmArgs &g, int batch, bool trans_b) {
     DmaTile t;
     const auto misaligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; };
-    if (!trans_b || batch != 1 || g.a_gather || g.M <= 0) return false;
+    if (batch < 1 || batch > 65535 || g.a_gather || g.M <= 0) return false;
     if (g.lda % 8 || g.ldb % 8 || g.ldc % 8 || misaligned(g.A) || misaligned(g.B) || misaligned(g.C)) return false;
-    return pick_dma_tile(g, &t);
+    if (batch > 1 && ((g.sAo | g.sAi | g.sBo | g.sBi | g.sCo | g.sCi) & 7)) return false;  // every problem aligned
+    return pick_dma_tile(g, batch, trans_b, &t);
 }
 
-template <int TMW, int TNW, int NBUF, bool IDX, bool RAGGED>
-static int launch_dma_variant(const GemmArgs &g, hipStream_t stream) {
+template <int TMW, int TNW, int NBUF, bool IDX, bool RAGGED, bool BT = false>
+static int launch_dma_variant(const GemmArgs &g, int batch, hipStream_t stream) {
     constexpr int BM = 64 * TMW, BN = 64 * TNW;
     constexpr size_t lds = dma_lds_bytes(TMW, TNW, NBUF);
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     const int nsb = ((tiles_m + kSbM - 1) / kSbM) * ((tiles_n + kSbN - 1) / kSbN);
     const int rounds = (nsb + kDmaXcds - 1) / kDmaXcds;
-    const dim3 grid((unsigned)(rounds * kDmaXcds * kSbM * kSbN));
-    auto kernel = gemm_f16_dma_kernel<TMW, TNW, NBUF, IDX, RAGGED>;
+    const dim3 grid((unsigned)(rounds * kDmaXcds * kSbM * kSbN), (unsigned)batch);
+    auto kernel = gemm_f16_dma_kernel<TMW, TNW, NBUF, IDX, RAGGED, BT>;
     static bool raised = false;  // more than 64 KB of dynamic LDS needs the attribute, once per kernel
     if (!raised) {
         ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -336,22 +371,28 @@ static int launch_dma_variant(const GemmArgs &g, hipStream_t stream) {
     return check_launch("gemm_f16_dma_kernel");
 }
 
-template <int TMW, int TNW, int NBUF, bool RAGGED = false>
-static int launch_dma_tile(const GemmArgs &g, hipStream_t stream) {
-    return (g.c_scatter || g.bias_idx) ? launch_dma_variant<TMW, TNW, NBUF, true, RAGGED>(g, stream)
-                                       : launch_dma_variant<TMW, TNW, NBUF, false, RAGGED>(g, stream);
+template <int TMW, int TNW, int NBUF, bool RAGGED = false, bool BT = false>
+static int launch_dma_tile(const GemmArgs &g, int batch, hipStream_t stream) {
+    return (g.c_scatter || g.bias_idx) ? launch_dma_variant<TMW, TNW, NBUF, true, RAGGED, BT>(g, batch, stream)
+                                       : launch_dma_variant<TMW, TNW, NBUF, false, RAGGED, BT>(g, batch, stream);
 }
 
-int launch_gemm_dma(const GemmArgs &g, hipStream_t stream) {
+int launch_gemm_dma(const GemmArgs &g, int batch, bool trans_b, hipStream_t stream) {
     DmaTile t{};
-    if (!pick_dma_tile(g, &t)) return ET_ERR_UNSUPPORTED;
-    if (t.ragged) return t.nbuf == 3 ? launch_dma_tile<1, 1, 3, true>(g, stream) : launch_dma_tile<1, 1, 2, true>(g, stream);
+    if (!pick_dma_tile(g, batch, trans_b, &t)) return ET_ERR_UNSUPPORTED;
+    if (t.ragged) {
+        if (!trans_b)
+            return t.nbuf == 3 ? launch_dma_tile<1, 1, 3, true, true>(g, batch, stream)
+                               : launch_dma_tile<1, 1, 2, true, true>(g, batch, stream);
+        return t.nbuf == 3 ? launch_dma_tile<1, 1, 3, true>(g, batch, stream)
+                           : launch_dma_tile<1, 1, 2, true>(g, batch, stream);
+    }
     switch (t.tmw * 100 + t.tnw * 10 + t.nbuf) {
-        case 442: return launch_dma_tile<4, 4, 2>(g, stream);
-        case 222: return launch_dma_tile<2, 2, 2>(g, stream);
-        case 212: return launch_dma_tile<2, 1, 2>(g, stream);
-        case 112: return launch_dma_tile<1, 1, 2>(g, stream);
-        case 113: return launch_dma_tile<1, 1, 3>(g, stream);
+        case 442: return launch_dma_tile<4, 4, 2>(g, 1, stream);
+        case 222: return launch_dma_tile<2, 2, 2>(g, 1, stream);
+        case 212: return launch_dma_tile<2, 1, 2>(g, 1, stream);
+        case 112: return launch_dma_tile<1, 1, 2>(g, 1, stream);
+        case 113: return launch_dma_tile<1, 1, 3>(g, 1, stream);
         default: return ET_ERR_UNSUPPORTED;
     }
 }

@@ -52,7 +52,8 @@ def test_linear_dense_closed_form_ones(et):
 
 
 @pytest.mark.parametrize("trans_b", [True, False])
-@pytest.mark.parametrize("M,N,K,batch", [(128, 64, 128, 12), (256, 768, 1536, 1), (48, 32, 16, 3)])
+@pytest.mark.parametrize("M,N,K,batch", [(128, 64, 128, 12), (256, 768, 1536, 1), (48, 32, 16, 3),
+                                         (128, 192, 1040, 3)])  # long K in few tiles, 16 k-values in the last stage
 def test_gemm_batched(et, trans_b, M, N, K, batch):
     A = Hn.randn((batch, M, K), 4, 0.5)
     Bm = Hn.randn((batch, N, K) if trans_b else (batch, K, N), 5, 0.1)
