@@ -14,11 +14,22 @@
 #include "col_mat.hpp"
 
 namespace et {
-inline void linear_vo_forward(const half *W, const half *bias, const half *X, half *out, const Model_t &m,
+// Wt: the weights k-contiguous per head, [nh][N][H] (transposed_heads below)
+inline void linear_vo_forward(const half *Wt, const half *bias, const half *X, half *out, const Model_t &m,
                               int batch, int N, stream_t stream) {
-    etChk(et_linear_vo_f16(reinterpret_cast<const et_f16 *>(W), reinterpret_cast<const et_f16 *>(bias),
-                           reinterpret_cast<const et_f16 *>(X), reinterpret_cast<et_f16 *>(out), batch,
-                           m.seq_len, m.emdim, N, m.nhead, stream));
+    etChk(et_linear_vo_t_f16(reinterpret_cast<const et_f16 *>(Wt), reinterpret_cast<const et_f16 *>(bias),
+                             reinterpret_cast<const et_f16 *>(X), reinterpret_cast<et_f16 *>(out), batch,
+                             m.seq_len, m.emdim, N, m.nhead, stream));
+}
+
+// Device copy of W[nh][H][N] turned into [nh][N][H], made once at construction: the GEMM behind
+// the projection reads k-contiguous operands about twice as fast.
+inline DeviceBuffer<half> transposed_heads(const half *W_dev, int nhead, int H, int N) {
+    DeviceBuffer<half> t((std::size_t)nhead * H * N);
+    etChk(et_transpose_heads_f16(reinterpret_cast<et_f16 *>(t.get()), reinterpret_cast<const et_f16 *>(W_dev), nhead,
+                                 H, N, nullptr));
+    etChk(et_device_sync());
+    return t;
 }
 
 // W_VO[h] = W_V[h*hd:(h+1)*hd, :]^T * W_O[:, h*hd:(h+1)*hd]^T   ([H x N], N = emdim)
@@ -51,16 +62,22 @@ class Linear_VO {
     ptr_t bias;    // [nh][N]
     ptr_t weight;  // [nh][H][N] row-major
     std::shared_ptr<Model_t> model;
+    ptr_t weight_t;  // [nh][N][H]: what forward() reads
 
     Linear_VO(const ptr_t &_weight, const ptr_t &_bias, std::shared_ptr<Model_t> _model)
-        : bias(_bias), weight(_weight), model(std::move(_model)) {
-        et::require(weight.size == (std::size_t)model->nhead * model->emdim * model->emdim,
-                    "Linear_VO: weight must be [nhead][emdim][emdim]");
+        : bias(_bias), weight(_weight), model(std::move(_model)),
+          weight_t(checked_transpose(weight, *model)) {
         et::require(bias.size == (std::size_t)model->nhead * model->emdim, "Linear_VO: bias must be [nhead][emdim]");
     }
     int out_width() const { return model->emdim; }
     void forward(half *output, const half *input, et::stream_t stream = nullptr, int batch = 1) {
-        et::linear_vo_forward(weight.get(), bias.get(), input, output, *model, batch, model->emdim, stream);
+        et::linear_vo_forward(weight_t.get(), bias.get(), input, output, *model, batch, model->emdim, stream);
+    }
+
+  private:
+    static ptr_t checked_transpose(const ptr_t &w, const Model_t &m) {
+        et::require(w.size == (std::size_t)m.nhead * m.emdim * m.emdim, "Linear_VO: weight must be [nhead][emdim][emdim]");
+        return et::transposed_heads(w.get(), m.nhead, m.emdim, m.emdim);
     }
 };
 
@@ -73,16 +90,23 @@ class Linear_VO_prune {
     ptr_t bias;
     col_mat weight;
     std::shared_ptr<Model_t> model;
+    ptr_t weight_t;  // [nh][len(col_id)][H]: what forward() reads
 
     Linear_VO_prune(const col_mat &_weight, const ptr_t &_bias, std::shared_ptr<Model_t> _model)
-        : bias(_bias), weight(_weight), model(std::move(_model)) {
-        const std::size_t n = weight.col_id->size;
-        et::require(weight.cols->size == (std::size_t)model->nhead * model->emdim * n,
-                    "Linear_VO_prune: weight must be [nhead][emdim][len(col_id)]");
-        et::require(bias.size == (std::size_t)model->nhead * n, "Linear_VO_prune: bias must be [nhead][len(col_id)]");
+        : bias(_bias), weight(_weight), model(std::move(_model)), weight_t(checked_transpose(weight, *model)) {
+        et::require(bias.size == (std::size_t)model->nhead * weight.col_id->size,
+                    "Linear_VO_prune: bias must be [nhead][len(col_id)]");
     }
     int out_width() const { return (int)weight.col_id->size; }
     void forward(half *output, const half *input, et::stream_t stream = nullptr, int batch = 1) {
-        et::linear_vo_forward(weight.cols->get(), bias.get(), input, output, *model, batch, out_width(), stream);
+        et::linear_vo_forward(weight_t.get(), bias.get(), input, output, *model, batch, out_width(), stream);
+    }
+
+  private:
+    static ptr_t checked_transpose(const col_mat &w, const Model_t &m) {
+        const std::size_t n = w.col_id->size;
+        et::require(w.cols->size == (std::size_t)m.nhead * m.emdim * n,
+                    "Linear_VO_prune: weight must be [nhead][emdim][len(col_id)]");
+        return et::transposed_heads(w.cols->get(), m.nhead, m.emdim, (int)n);
     }
 };

@@ -146,6 +146,21 @@ static int check_probs_shape(const char *fn, int B, int S, int nh, int hd, int f
 static inline const _Float16 *H(const et_f16 *p) { return reinterpret_cast<const _Float16 *>(p); }
 static inline _Float16 *H(et_f16 *p) { return reinterpret_cast<_Float16 *>(p); }
 
+// dst[h][n][k] = src[h][k][n]: the per-head weights of Linear_VO turned k-contiguous, once, at
+// construction (32 x 32 tiles through LDS, both sides coalesced).
+__global__ __launch_bounds__(256) void transpose_heads_kernel(_Float16 *__restrict__ dst,
+                                                              const _Float16 *__restrict__ src, int Hk, int N) {
+    __shared__ _Float16 tile[32][33];
+    const size_t head = (size_t)blockIdx.z * Hk * N;
+    const int k0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    for (int r = ty; r < 32; r += 8)
+        if (k0 + r < Hk && n0 + tx < N) tile[r][tx] = src[head + (size_t)(k0 + r) * N + n0 + tx];
+    __syncthreads();
+    for (int r = ty; r < 32; r += 8)
+        if (n0 + r < N && k0 + tx < Hk) dst[head + (size_t)(n0 + r) * Hk + k0 + tx] = tile[tx][r];
+}
+
 }  // namespace et
 
 using namespace et;
@@ -208,6 +223,40 @@ int et_linear_vo_f16(const et_f16 *W, const et_f16 *bias, const et_f16 *X, et_f1
     g.sBias_o = 0;
     g.sBias_i = N;
     return launch_gemm(g, B * nh, false, as_stream(stream));
+}
+
+int et_transpose_heads_f16(et_f16 *dst, const et_f16 *src, int nh, int H_, int N, et_stream stream) {
+    ET_REQUIRE(dst && src && dst != src, ET_ERR_INVALID_ARG, "et_transpose_heads_f16: NULL or aliasing pointers");
+    ET_REQUIRE(nh > 0 && nh <= 65535 && H_ > 0 && N > 0, ET_ERR_INVALID_ARG,
+               "et_transpose_heads_f16: nh=%d H=%d N=%d", nh, H_, N);
+    const dim3 grid((unsigned)((N + 31) / 32), (unsigned)((H_ + 31) / 32), (unsigned)nh);
+    ET_REQUIRE(grid.y <= 65535, ET_ERR_UNSUPPORTED, "et_transpose_heads_f16: H=%d too large", H_);
+    transpose_heads_kernel<<<grid, 256, 0, as_stream(stream)>>>(H(dst), H(src), H_, N);
+    return check_launch("transpose_heads_kernel");
+}
+
+int et_linear_vo_t_f16(const et_f16 *Wt, const et_f16 *bias, const et_f16 *X, et_f16 *VO, int B, int S,
+                       int H_, int N, int nh, et_stream stream) {
+    ET_REQUIRE(Wt && X && VO, ET_ERR_INVALID_ARG, "et_linear_vo_t_f16: NULL pointer");
+    ET_REQUIRE(B >= 0 && S > 0 && H_ > 0 && N > 0 && nh > 0, ET_ERR_INVALID_ARG,
+               "et_linear_vo_t_f16: B=%d S=%d H=%d N=%d nh=%d", B, S, H_, N, nh);
+    ET_REQUIRE(S % 16 == 0 && H_ % 16 == 0 && N % 16 == 0, ET_ERR_UNSUPPORTED,
+               "et_linear_vo_t_f16: S=%d H=%d N=%d must be multiples of 16", S, H_, N);
+    ET_REQUIRE((long long)B * nh <= 65535, ET_ERR_UNSUPPORTED, "et_linear_vo_t_f16: batch*nhead too large");
+    if (B == 0) return ET_OK;
+    // VO[b][h] (S x N) = X[b] (S x H) * Wt[h]^T (Wt[h] is N x H) + bias[h]
+    GemmArgs g = gemm_args(H(X), H(Wt), H(VO), S, N, H_, H_, H_, N);
+    g.batch_inner = nh;
+    g.sAo = (long long)S * H_;
+    g.sAi = 0;
+    g.sBo = 0;
+    g.sBi = (long long)N * H_;
+    g.sCo = (long long)nh * S * N;
+    g.sCi = (long long)S * N;
+    g.bias = H(bias);
+    g.sBias_o = 0;
+    g.sBias_i = N;
+    return launch_gemm(g, B * nh, true, as_stream(stream));
 }
 
 int et_mha_vo_f16(const et_f16 *Q, const et_f16 *K, int ldq, int ldk, const et_f16 *VO, et_f16 *P,

@@ -215,7 +215,9 @@ class Bench:
         H = nh * hd
         W, x = self.dev(self.rnd((nh, H, N), 0.02)), self.dev(self.rnd((B * S, H)))
         vo = self.empty((B * nh * S, N))
-        us = self.time_us(lambda: et.check(lib.et_linear_vo_f16(W.ptr, None, x.ptr, vo.ptr, B, S, H, N, nh, self.stream)),
+        wt = self.empty((nh, N, H))  # k-contiguous per head, as the Linear_VO classes keep it
+        et.check(lib.et_transpose_heads_f16(wt.ptr, W.ptr, nh, H, N, self.stream))
+        us = self.time_us(lambda: et.check(lib.et_linear_vo_t_f16(wt.ptr, None, x.ptr, vo.ptr, B, S, H, N, nh, self.stream)),
                           launches)
         self.record("linear_vo", f"B{B} S{S} H{H} N{N} nh{nh}", us, 2 * B * S * H * N * nh, "mfma")
         qk, p, out = self.dev(self.rnd((B * S, 2 * H))), self.empty((B * S, nh * S)), self.empty((B * S, N))

@@ -72,6 +72,13 @@ def test_vo_attention(et, B, S, H, nh, pruned):
     want_vo = (x.astype(np.float32).reshape(B, 1, S, H) @ Wvo.astype(np.float32)[None] +
                bvo.astype(np.float32)[None, :, None, :]).astype(np.float16)
     assert Hn.max_abs(d_vo.numpy(), want_vo) <= 4e-3
+    # the same projection from weights transposed per head on the device (what the classes use)
+    d_wt = et.DeviceBuffer.empty((nh, N, H), np.float16)
+    et.check(et.lib().et_transpose_heads_f16(d_wt.ptr, up(et, Wvo).ptr, nh, H, N, None))
+    assert np.array_equal(d_wt.numpy(), np.ascontiguousarray(Wvo.transpose(0, 2, 1)))
+    d_vo_t = et.DeviceBuffer.empty((B, nh, S, N), np.float16)
+    et.check(et.lib().et_linear_vo_t_f16(d_wt.ptr, up(et, bvo).ptr, d_x.ptr, d_vo_t.ptr, B, S, H, N, nh, None))
+    assert Hn.max_abs(d_vo_t.numpy(), want_vo) <= 4e-3
     d_p = et.DeviceBuffer.empty((T, nh * S), np.float16)
     d_out = et.DeviceBuffer.empty((T, H), np.float16)
     et.check(et.lib().et_fill_f16(d_out.ptr, T * H, 0x7E00, None))
