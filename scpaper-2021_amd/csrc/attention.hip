@@ -58,6 +58,27 @@ struct MhaLds {
     static constexpr size_t bytes = (size_t)(k_halfs + vt_halfs) * sizeof(_Float16);
 };
 
+// Layout of a V^T row (one head dimension, kKeyBlock keys) in LDS.
+//
+// Order of the keys.  The P*V product contracts 32 keys per MFMA and lane (r16, g) supplies, as
+// its 8 values, the scores it holds from two 16x16 score tiles: keys 4g..4g+3 of the first and
+// of the second.  Key k = 32s + 16a + 4g + j is therefore stored at position 32s + 8g + 4a + j:
+// the 8 values of a lane are consecutive and one 16-byte read fetches them (two 8-byte reads
+// cost 1.55x as much LDS time).
+//
+// Swizzle.  The rows are written transposed, 8 bytes (4 keys of one dimension) per lane, and
+// the lanes of one store instruction differ in the dimension group dg = row / 8: rows 16 apart
+// fall in the same banks (4-way conflict, 3x the store time).  Bits of row / 16 are XORed into
+// the position bits that the lanes of a store pass do not vary themselves (which bits depends on
+// how many dimension groups a head has); a reader applies the same XOR, which for it is uniform
+// over the wave: a swap of the two 4-key halves (bit 2), of 16-key chunks (bit 4) or of 32-key
+// groups (bit 5).  With it stores and fragment reads are both conflict-free.
+template <int HD> __device__ __forceinline__ constexpr int vt_swizzle(int row16) {
+    if (HD <= 32) return (row16 & 1) << 5;
+    if (HD <= 64) return ((row16 & 1) << 2) | (((row16 >> 1) & 1) << 5);
+    return ((row16 & 1) << 2) | (((row16 >> 1) & 1) << 4) | (((row16 >> 2) & 1) << 5);
+}
+
 // QT = 16-query tiles per wave: with QT = 2 every K and V^T fragment read from LDS feeds
 // two MFMAs and a workgroup covers 32*NW queries per staged key block.
 //
@@ -216,10 +237,12 @@ __global__ __launch_bounds__(64 * NW)
             const int u = threadIdx.x + j * nthr;
             const int kg = u / dgroups, dg = u - kg * dgroups;
             if (u < v_units) {
+                // keys 4kg..4kg+3 = (s, a, g) = (kg / 8, (kg / 4) % 2, kg % 4); rows 8dg..8dg+7 share row / 16
+                const int pos = (32 * (kg >> 3) + 8 * (kg & 3) + 4 * ((kg >> 2) & 1)) ^ vt_swizzle<HD>(dg >> 1);
 #pragma unroll
                 for (int d = 0; d < 8; d++) {
                     h4 col = {vreg[j][0][d], vreg[j][1][d], vreg[j][2][d], vreg[j][3][d]};
-                    *reinterpret_cast<h4 *>(Vt + (dg * 8 + d) * L::ldvt + kg * 4) = col;
+                    *reinterpret_cast<h4 *>(Vt + (dg * 8 + d) * L::ldvt + pos) = col;
                 }
             }
         }
@@ -344,10 +367,11 @@ __global__ __launch_bounds__(64 * NW)
 #pragma unroll
                 for (int d = 0; d < DB; d++) {
                     if (d * 16 >= vlive) continue;  // no (surviving) column in this block: wave-uniform
-                    const _Float16 *vp = Vt + (d * 16 + r16) * L::ldvt + s2 * 32 + 4 * g;
-                    const h4 v0 = *reinterpret_cast<const h4 *>(vp);
-                    const h4 v1 = *reinterpret_cast<const h4 *>(vp + 16);
-                    const h8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                    constexpr int kSwzMask = vt_swizzle<HD>(7);
+                    const int swz = vt_swizzle<HD>(d);  // a constant once d is unrolled
+                    const h8 vr = *reinterpret_cast<const h8 *>(Vt + (d * 16 + r16) * L::ldvt +
+                                                                 ((s2 * 32 + 8 * g) ^ (swz & kSwzMask & ~4)));
+                    const h8 vf = (swz & 4) ? h8{vr[4], vr[5], vr[6], vr[7], vr[0], vr[1], vr[2], vr[3]} : vr;
 #pragma unroll
                     for (int t = 0; t < QT; t++)
                         o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[t], o[t][d], 0, 0, 0);

@@ -65,7 +65,11 @@ constexpr int kFxRes = 2;
 
 constexpr int kXcds = 8;      // accelerator dies, each with a private L2
 constexpr int kLdsPad = 8;    // halfs
-constexpr int kSlots = 8;     // slots per row group held in registers (two groups resident)
+constexpr int kSlots = 8;     // slots per row group held in registers
+#ifndef ET_BSR_NB
+#define ET_BSR_NB 2
+#endif
+constexpr int kNB = ET_BSR_NB;  // row groups resident (requested ahead) per wave
 constexpr int kStageU = 8;    // 16-byte strip vectors a thread keeps in flight
 constexpr int kMaxWaveRows = 64;  // block-rows one wave can own (one lane each)
 
@@ -190,11 +194,11 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
 
     // ---- row-group stream of this wave.  An item is up to kSlots slots of one
     // block-row; (it_row, it_part) is the next item to request.
-    h8 w[2][kSlots];
-    int col[2][kSlots];
-    h4 bias_v[2];
-    int g_row[2], g_nsl[2];  // resident items: wave row index (-1 = none), slots in the item
-    bool g_last[2];          // item ends its block-row
+    h8 w[kNB][kSlots];
+    int col[kNB][kSlots];
+    h4 bias_v[kNB];
+    int g_row[kNB], g_nsl[kNB];  // resident items: wave row index (-1 = none), slots in the item
+    bool g_last[kNB];            // item ends its block-row
     int it_row = 0, it_part = 0;
     // skip rows without tiles (they are written at the end)
     auto skip_empty = [&]() {
@@ -249,8 +253,8 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
             it_part++;
         }
     };
-    issue_item(0);
-    issue_item(1);
+#pragma unroll
+    for (int buf = 0; buf < kNB; buf++) issue_item(buf);
 
     // ---- fused SkipLayerNorm: statistics in fp32 per row (wave64 butterflies), the
     // normalised row goes to LDS as fp16 — the value a separate LayerNorm kernel would
@@ -417,7 +421,7 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
 
     while (g_row[0] >= 0) {
 #pragma unroll
-        for (int buf = 0; buf < 2; buf++) {
+        for (int buf = 0; buf < kNB; buf++) {
             if (g_row[buf] >= 0) {
                 const int nsl = g_nsl[buf];
 #pragma unroll
