@@ -69,14 +69,21 @@ struct MhaLds {
 // Swizzle.  The rows are written transposed, 8 bytes (4 keys of one dimension) per lane, and
 // the lanes of one store instruction differ in the dimension group dg = row / 8: rows 16 apart
 // fall in the same banks (4-way conflict, 3x the store time).  Bits of row / 16 are XORed into
-// the position bits that the lanes of a store pass do not vary themselves (which bits depends on
-// how many dimension groups a head has); a reader applies the same XOR, which for it is uniform
-// over the wave: a swap of the two 4-key halves (bit 2), of 16-key chunks (bit 4) or of 32-key
-// groups (bit 5).  With it stores and fragment reads are both conflict-free.
+// the position bits that the 32 lanes of a store pass do not vary themselves: bit 4 (16-key
+// chunks, g ^ 2) and bit 5 (32-key groups); 128-wide heads have a third bit to place, which
+// swaps the two 4-key halves of a lane's 8 values (bit 2).  For 64-wide heads the 4-key groups
+// are dealt to the lanes of a wave with bits 1 and 2 of their index exchanged (vt_unit_keys), so
+// that a pass varies g's low bit and a instead of both bits of g.  A reader applies the same XOR,
+// which for it is uniform over the wave.  Stores and fragment reads are then conflict-free.
 template <int HD> __device__ __forceinline__ constexpr int vt_swizzle(int row16) {
     if (HD <= 32) return (row16 & 1) << 5;
-    if (HD <= 64) return ((row16 & 1) << 2) | (((row16 >> 1) & 1) << 5);
-    return ((row16 & 1) << 2) | (((row16 >> 1) & 1) << 4) | (((row16 >> 2) & 1) << 5);
+    if (HD <= 64) return ((row16 & 1) << 4) | (((row16 >> 1) & 1) << 5);
+    return ((row16 & 1) << 4) | (((row16 >> 1) & 1) << 5) | (((row16 >> 2) & 1) << 2);
+}
+// 4-key group staged by unit number kg (units are dealt to consecutive threads)
+template <int HD> __device__ __forceinline__ constexpr int vt_unit_keys(int kg) {
+    if (HD > 32 && HD <= 64) return (kg & ~6) | ((kg & 2) << 1) | ((kg & 4) >> 1);
+    return kg;
 }
 
 // QT = 16-query tiles per wave: with QT = 2 every K and V^T fragment read from LDS feeds
@@ -196,7 +203,7 @@ __global__ __launch_bounds__(64 * NW)
 #pragma unroll
         for (int j = 0; j < VU; j++) {
             const int u = threadIdx.x + j * nthr;
-            const int kg = u / dgroups, dg = u - kg * dgroups;
+            const int dg = u % dgroups, kg = vt_unit_keys<HD>(u / dgroups);
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int key = (u < v_units) ? k0 + kg * 4 + i : S;  // surplus threads load nothing
@@ -235,7 +242,7 @@ __global__ __launch_bounds__(64 * NW)
 #pragma unroll
         for (int j = 0; j < VU; j++) {
             const int u = threadIdx.x + j * nthr;
-            const int kg = u / dgroups, dg = u - kg * dgroups;
+            const int dg = u % dgroups, kg = vt_unit_keys<HD>(u / dgroups);
             if (u < v_units) {
                 // keys 4kg..4kg+3 = (s, a, g) = (kg / 8, (kg / 4) % 2, kg % 4); rows 8dg..8dg+7 share row / 16
                 const int pos = (32 * (kg >> 3) + 8 * (kg & 3) + 4 * ((kg >> 2) & 1)) ^ vt_swizzle<HD>(dg >> 1);
@@ -320,8 +327,7 @@ __global__ __launch_bounds__(64 * NW)
                         }
                     }
                 }
-                m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 16, kWave));
-                m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, kWave));
+                m_blk = rows_max(m_blk);
 
                 const float m_new = fmaxf(m_run[t], m_blk);
                 // all keys so far masked: keep everything at zero without inf - inf
@@ -339,42 +345,53 @@ __global__ __launch_bounds__(64 * NW)
 
             // ---- probabilities (fp32 sum, fp16 operands) and O^T += V^T P^T
             const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+            const int g8 = 8 * g, g8x = (8 * g) ^ 16;  // the lane's 8-key chunk of a 32-key group, plain and swizzled
 #pragma unroll
             for (int s2 = 0; s2 < kNKB / 2; s2++) {
                 if (!FAST && k0 + s2 * 32 >= klimit) continue;  // both key blocks fully padded
                 h8 pf[QT];
 #pragma unroll
                 for (int t = 0; t < QT; t++) {
+                    // the lane's 8 values: keys 4g..4g+3 of score tile 2*s2, then of tile 2*s2+1;
+                    // each fp16 pair is formed once and feeds both the MFMA and the row sum
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
+                    for (int pr = 0; pr < 4; pr++) {
+                        const int kb = 2 * s2 + (pr >> 1), j = 2 * (pr & 1);
                         float e0, e1;
                         if (FAST) {
-                            e0 = sc[t][2 * s2][j] * a.scale_log2e - m_use[t];
-                            e1 = sc[t][2 * s2 + 1][j] * a.scale_log2e - m_use[t];
+                            e0 = sc[t][kb][j] * a.scale_log2e - m_use[t];
+                            e1 = sc[t][kb][j + 1] * a.scale_log2e - m_use[t];
                         } else {
-                            e0 = sc[t][2 * s2][j] - m_use[t];
-                            e1 = sc[t][2 * s2 + 1][j] - m_use[t];
+                            e0 = sc[t][kb][j] - m_use[t];
+                            e1 = sc[t][kb][j + 1] - m_use[t];
                         }
                         // raw v_exp_f32: results below the normal range flush to zero, which
                         // the conversion to fp16 would do anyway
                         const h2 hp = {(_Float16)__builtin_amdgcn_exp2f(e0), (_Float16)__builtin_amdgcn_exp2f(e1)};
                         // the row sum uses the values that enter the MFMA
                         l_part[t] = __builtin_amdgcn_fdot2(hp, ones, l_part[t], false);
-                        pf[t][j] = hp[0];
-                        pf[t][4 + j] = hp[1];
+                        pf[t][2 * pr] = hp[0];
+                        pf[t][2 * pr + 1] = hp[1];
                     }
+                }
+                // The V^T fragments of the step are read unconditionally (dimension blocks past the
+                // head size or the surviving columns hold zeros) so that the reads go out together;
+                // a read under a branch is waited for on the spot.  Only compact V skips the
+                // products of dead blocks (wave-uniform).
+                h8 vf[DB];
+#pragma unroll
+                for (int d = 0; d < DB; d++) {
+                    const int swz = vt_swizzle<HD>(d);  // a constant once d is unrolled
+                    const h8 vr = *reinterpret_cast<const h8 *>(Vt + (d * 16 + r16) * L::ldvt +
+                                                                 ((s2 * 32) ^ (swz & 32)) + ((swz & 16) ? g8x : g8));
+                    vf[d] = (swz & 4) ? h8{vr[4], vr[5], vr[6], vr[7], vr[0], vr[1], vr[2], vr[3]} : vr;
                 }
 #pragma unroll
                 for (int d = 0; d < DB; d++) {
-                    if (d * 16 >= vlive) continue;  // no (surviving) column in this block: wave-uniform
-                    constexpr int kSwzMask = vt_swizzle<HD>(7);
-                    const int swz = vt_swizzle<HD>(d);  // a constant once d is unrolled
-                    const h8 vr = *reinterpret_cast<const h8 *>(Vt + (d * 16 + r16) * L::ldvt +
-                                                                 ((s2 * 32 + 8 * g) ^ (swz & kSwzMask & ~4)));
-                    const h8 vf = (swz & 4) ? h8{vr[4], vr[5], vr[6], vr[7], vr[0], vr[1], vr[2], vr[3]} : vr;
+                    if (COMPACT && d * 16 >= vlive) continue;
 #pragma unroll
                     for (int t = 0; t < QT; t++)
-                        o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf[t], o[t][d], 0, 0, 0);
+                        o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[d], pf[t], o[t][d], 0, 0, 0);
                 }
             }
         };
@@ -389,8 +406,7 @@ __global__ __launch_bounds__(64 * NW)
 #pragma unroll
     for (int t = 0; t < QT; t++) {
         float l = l_part[t];
-        l += __shfl_xor(l, 16, kWave);
-        l += __shfl_xor(l, 32, kWave);
+        l = rows_sum(l);
         inv[t] = l > 0.0f ? 1.0f / l : 0.0f;
     }
     if (!COMPACT) {

@@ -70,6 +70,30 @@ __device__ __forceinline__ float wave_max(float v) {
     return fmaxf(fmaxf(lane_value(v, 0), lane_value(v, 16)), fmaxf(lane_value(v, 32), lane_value(v, 48)));
 }
 
+// Butterflies across the four 16-lane rows of a wave (lane ^ 16, then lane ^ 32) with the gfx950
+// row-swap instructions: v_permlane16_swap exchanges the odd rows of its first operand with the
+// even rows of its second, v_permlane32_swap the upper half of the first with the lower half of
+// the second.  Given the same value twice they return (this lane's row pair, the partner's), so
+// one swap and one VALU operation make a butterfly step without the LDS crossbar a
+// ds_bpermute-based shuffle goes through.  Every lane of a column (lane % 16) ends with the
+// result over the column's four lanes.
+__device__ __forceinline__ float rows_max(float v) {
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const float m = fmaxf(__builtin_bit_cast(float, (unsigned)a[0]), __builtin_bit_cast(float, (unsigned)a[1]));
+    const unsigned w = __builtin_bit_cast(unsigned, m);
+    auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+    return fmaxf(__builtin_bit_cast(float, (unsigned)b[0]), __builtin_bit_cast(float, (unsigned)b[1]));
+}
+__device__ __forceinline__ float rows_sum(float v) {
+    const unsigned u = __builtin_bit_cast(unsigned, v);
+    auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const float m = __builtin_bit_cast(float, (unsigned)a[0]) + __builtin_bit_cast(float, (unsigned)a[1]);
+    const unsigned w = __builtin_bit_cast(unsigned, m);
+    auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+    return __builtin_bit_cast(float, (unsigned)b[0]) + __builtin_bit_cast(float, (unsigned)b[1]);
+}
+
 // tanh-form GELU, x*(0.5 + 0.5*tanh(x*(0.035677408*x^2 + 0.7978845608)))
 // (the form the reference evaluates, Encoder/Encoder.cu:25-37).
 __device__ __forceinline__ float gelu_tanh(float x) {
