@@ -89,14 +89,19 @@ template <int HD> __device__ __forceinline__ constexpr int vt_unit_keys(int kg) 
 // QT = 16-query tiles per wave: with QT = 2 every K and V^T fragment read from LDS feeds
 // two MFMAs and a workgroup covers 32*NW queries per staged key block.
 //
-// The variants that prefetch the next key block through registers (mha_prefetches) are held to
-// the 168 registers of three resident waves per SIMD; left alone the allocator takes a few more
-// and the third wave is lost, which costs more than the prefetch gains.
-template <int HD, int NW, bool COMPACT> constexpr bool mha_prefetches() { return HD <= 64 && NW == 4 && !COMPACT; }
+// Some variants prefetch the next key block through registers (mha_prefetches).  The 4-wave one
+// is held to the 168 registers of three resident waves per SIMD; left alone the allocator takes
+// a few more and the third wave is lost, which costs more than the prefetch gains.
+template <int HD, int NW, bool COMPACT, int QT> constexpr bool mha_prefetches() {
+    return HD <= 64 && !COMPACT && ((NW == 4 && QT == 1) || (NW == 8 && QT == 2));
+}
+template <int HD, int NW, bool COMPACT, int QT> constexpr bool mha_three_waves() {
+    return mha_prefetches<HD, NW, COMPACT, QT>() && NW == 4;
+}
 
 template <int HD, bool COMPACT, int NW, int QT>
 __global__ __launch_bounds__(64 * NW)
-    __attribute__((amdgpu_waves_per_eu(mha_prefetches<HD, NW, COMPACT>() ? 3 : 1, mha_prefetches<HD, NW, COMPACT>() ? 3 : 8))) void
+    __attribute__((amdgpu_waves_per_eu(mha_three_waves<HD, NW, COMPACT, QT>() ? 3 : 1, mha_three_waves<HD, NW, COMPACT, QT>() ? 3 : 8))) void
     mha_fused_kernel(const MhaArgs a) {
     using L = MhaLds<HD>;
     constexpr int KS = HD / 32;  // K=32 MFMA steps over the head dimension
@@ -256,9 +261,9 @@ __global__ __launch_bounds__(64 * NW)
     };
 
     // Holding the next block's loads in registers through the multiplication costs 32 VGPRs: it
-    // is done where that still fits three resident waves per SIMD (3-4 % at 512 and 2048 keys);
-    // with fewer waves per workgroup or 128-wide heads it spills or loses a wave, and is off.
-    constexpr bool kPrefetch = mha_prefetches<HD, NW, COMPACT>();
+    // is done where that still fits the resident waves the variant runs with anyway (3-4 % at
+    // 512 and 2048 keys); elsewhere it spills or loses a wave, and is off.
+    constexpr bool kPrefetch = mha_prefetches<HD, NW, COMPACT, QT>();
     const int nblocks = (klimit + kKeyBlock - 1) / kKeyBlock;
     if (kPrefetch && nblocks > 0) load_block(0);
     for (int blk = 0; blk < nblocks; blk++) {
@@ -488,14 +493,23 @@ static int launch_mha_nw(const MhaArgs &args, hipStream_t stream) {
     return check_launch("mha_fused_kernel");
 }
 
-// 4 waves per workgroup; 2 or 1 waves when that would leave a half-empty strip
-// (S = 32, 96, 16, ...).  One query tile per wave: two tiles (QT = 2) halve the LDS and
-// L2 traffic per flop but need 256 registers, and the lost third resident wave costs
-// more than that saves (measured 13 % slower at S = 512 and S = 2048).
+// 4 waves per workgroup and one 16-query tile per wave; 2 or 1 waves when 4 would leave a
+// half-empty strip (S = 32, 96, 16, ...).  Larger workgroups stage each key block for more
+// queries and pay once the grid still fills the chip: 8 waves (128 queries) from 256 such
+// workgroups on (2048 keys, 16 x 16 heads: 546 -> 516 us; 128-wide heads 592 -> 570 us), and 8
+// waves with two query tiles each (256 queries; every K and V^T fragment read from LDS feeds two
+// MFMAs) from 512 on (-> 464 us; it needs 214 registers, two waves per SIMD, so 64-wide heads
+// only).  Two tiles on 4 waves lose more to the missing third wave than they save (735 us).
 template <int HD, bool COMPACT>
 static int launch_mha(const MhaArgs &args, int B, hipStream_t stream) {
     (void)B;
     const int qblocks = args.S / 16;
+    if (!COMPACT) {
+        if (HD == 64 && qblocks % 16 == 0 && (long)args.nbh * (qblocks / 16) >= 512)
+            return launch_mha_nw<(HD == 64 ? HD : 64), COMPACT, 8, 2>(args, stream);
+        if (HD >= 64 && qblocks % 8 == 0 && (long)args.nbh * (qblocks / 8) >= 256)
+            return launch_mha_nw<HD, COMPACT, 8, 1>(args, stream);
+    }
     if (qblocks % 4 == 0) return launch_mha_nw<HD, COMPACT, 4, 1>(args, stream);
     if (qblocks % 2 == 0) return launch_mha_nw<HD, COMPACT, 2, 1>(args, stream);
     return launch_mha_nw<HD, COMPACT, 1, 1>(args, stream);

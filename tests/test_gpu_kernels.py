@@ -406,6 +406,16 @@ def test_mha_many_strips_with_padding(et):
     assert Hn.max_abs(got, want) <= 2e-3
 
 
+@pytest.mark.parametrize("causal,padded", [(False, False), (True, False), (False, True)])
+def test_mha_large_grid(et, causal, padded):
+    """Enough (sequence, head) pairs and queries that workgroups of 8 waves with two query tiles per
+    wave (256 queries) are used; branch-free and masked key blocks, partial last blocks."""
+    B, S, nh, hd = 32, 256, 16, 64
+    lens = ([256, 3, 0, 129, 128, 250, 255, 17] * 4) if padded else None
+    got, want = run_mha(et, B, S, nh, hd, seed=63, lens=lens, causal=causal)
+    assert Hn.max_abs(got, want) <= 2e-3
+
+
 def test_mha_additive_mask_and_lens(et):
     B, S, nh, hd = 2, 128, 4, 64
     mask = Hn.randn((S, S), 70, 1.0, np.float32)
