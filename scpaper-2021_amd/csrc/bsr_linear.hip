@@ -23,8 +23,8 @@
 // immediate offsets from per-row base pointers, one LDS read and one MFMA per
 // 16-token block) and keeps loads in flight across rows: the row pointers of all
 // rows of a wave are fetched with one load, and the weights, indices and bias of
-// the next row group (up to kSlots slots) are requested before the current one is
-// multiplied.  Several workgroups per compute unit cover the rest.
+// the next kNB - 1 row groups (up to kSlots slots each) are requested before the
+// current one is multiplied.
 //
 // Tile order inside a block-row is free (the sum commutes), as in the
 // reference kernel (Linear/SPMM_tile.cu:277-283).
@@ -66,10 +66,13 @@ constexpr int kFxRes = 2;
 constexpr int kXcds = 8;      // accelerator dies, each with a private L2
 constexpr int kLdsPad = 8;    // halfs
 constexpr int kSlots = 8;     // slots per row group held in registers
-#ifndef ET_BSR_NB
-#define ET_BSR_NB 2
-#endif
-constexpr int kNB = ET_BSR_NB;  // row groups resident (requested ahead) per wave
+// Row groups a wave has requested ahead of the one it multiplies.  Inside a stack of layers every
+// kernel starts on weights that have left the caches, and four groups in flight instead of two
+// shorten a 12-layer forward by 3 % (the stand-alone kernel, whose weights stay in L2, gains 0-5 %).
+// Five would spill (4 groups = 225 registers of the 256 that 8 waves per compute unit leave), and
+// so would four in the kernels whose prologue normalises the strip: those keep two.
+constexpr int kGroupsAhead = 4;
+constexpr int kGroupsAheadNorm = 2;
 constexpr int kStageU = 8;    // 16-byte strip vectors a thread keeps in flight
 constexpr int kMaxWaveRows = 64;  // block-rows one wave can own (one lane each)
 
@@ -91,6 +94,7 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     static_assert(!(FX & kFxNorm) || (STAGE && !LN), "the NORM prologue writes the strip to LDS");
     constexpr bool NORM = (FX & kFxNorm) != 0;
     constexpr bool RES = (FX & kFxRes) != 0;
+    constexpr int kNB = (LN || NORM) ? kGroupsAheadNorm : kGroupsAhead;  // row groups resident per wave
     extern __shared__ __align__(16) unsigned char smem_raw[];
     _Float16 *xs = reinterpret_cast<_Float16 *>(smem_raw);
 
