@@ -35,7 +35,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak (vendor figure)
 # HBM-side bytes per launch of the FFN down-projection kernel: rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a streaming
 # kernel of known size (profiles/encoder_stack_bert_base_b8_s128_hbm_traffic.txt).
-FFN_DOWN_TRAFFIC_BYTES = (6880.0 * 1.9989 + 1536.0 * 1.0) * 1024
+FFN_DOWN_TRAFFIC_BYTES = (6926.0 * 1.9989 + 1536.0 * 1.0) * 1024
 
 
 class TileWeight:
