@@ -274,8 +274,9 @@ __global__ __launch_bounds__(64 * NW)
         __syncthreads();
         if (kPrefetch && blk + 1 < nblocks) load_block(k0 + kKeyBlock);
 
-        // The multiplication of one staged block.  FAST (wave-uniform) = every key of the
-        // block is live for every query of the workgroup and nothing is added to the scores:
+        // The multiplication of one staged block.  FAST (wave-uniform) = nothing is added to the
+        // scores and every key of the block is live for every query of the workgroup, or dead
+        // for every query (right padding):
         // no per-16-key branches (the LDS reads of the whole block can be issued ahead of
         // the MFMAs) and the softmax costs one max, one multiply-add, one exp2, half a
         // conversion and half a dot-accumulate per score.
@@ -299,6 +300,20 @@ __global__ __launch_bounds__(64 * NW)
                 }
             }
 
+            if (FAST && k0 + kKeyBlock > klimit) {  // wave-uniform
+                // The block ends in padded keys: their raw scores become -inf, in place.  Key
+                // 16kb + 4g + j is padded when 16kb + j >= klimit - k0 - 4g (the left side a
+                // constant once unrolled).  (A separate instantiation of this lambda for the
+                // case made the allocator spill in the variants held to 168 registers.)
+                const int lim = klimit - k0 - 4 * g;
+#pragma unroll
+                for (int t = 0; t < QT; t++)
+#pragma unroll
+                    for (int kb = 0; kb < kNKB; kb++)
+#pragma unroll
+                        for (int j = 0; j < 4; j++)
+                            sc[t][kb][j] = (kb * 16 + j >= lim) ? -INFINITY : sc[t][kb][j];
+            }
             // ---- scale, mask, block max, running max (FAST keeps the raw scores: the scale
             // is positive there, so the max commutes with it, and it is applied inside the
             // exponent's multiply-add)
@@ -400,9 +415,9 @@ __global__ __launch_bounds__(64 * NW)
                 }
             }
         };
-        const bool fast = k0 + kKeyBlock <= klimit && a.mask == nullptr && a.scale_log2e > 0.0f &&
+        const bool plain = a.mask == nullptr && a.scale_log2e > 0.0f &&
                           (!a.causal || k0 + kKeyBlock <= qstrip * kStripQ + 1);
-        if (fast) multiply(std::true_type{});
+        if (plain) multiply(std::true_type{});
         else multiply(std::false_type{});
     }
 
