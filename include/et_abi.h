@@ -285,7 +285,9 @@ int et_mha_fused_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V,
 /* Attention-aware pruning: W_V is row-pruned, so V arrives compact,
  * Vc[T x nnz_col] (row stride ldvc), holding only the surviving V columns.
  * v_col_id[nnz_col] (ascending) are their full-width positions and
- * v_head_ptr[nh+1] splits them by head.  P*V runs over the surviving columns
+ * v_head_ptr[nh+1] splits them by head (the columns of head h lie in its own
+ * slice [h*vhd, (h+1)*vhd), as col_mat::set_metadata produces them,
+ * mat_type/col_mat/col_mat.cu:34-58).  P*V runs over the surviving columns
  * only; Z is written full width [T x nh*vhd] with zeros in pruned columns.
  * Completes Multihead_atttion<Prune_attn> (Attention/Attention.cu:54-78), whose
  * reference kernel never stores Z (Attention/kernels.cu:453-458). */

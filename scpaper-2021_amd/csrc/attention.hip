@@ -452,8 +452,10 @@ __global__ __launch_bounds__(64 * NW)
         // go through LDS here, where every wave of the workgroup arrives.
         __shared__ unsigned live_mask[4];  // bit c: column c of this head's slice of Z survives
         __shared__ int full_col[128];      // compact column -> column of Z
+        __shared__ int n_outside;          // surviving columns that lie outside this head's slice
         if (threadIdx.x < 4) live_mask[threadIdx.x] = 0u;
-        __syncthreads();
+        if (threadIdx.x == 4) n_outside = 0;
+        __syncthreads();  // also: every wave is done with the staged K and V
 #pragma unroll
         for (int i = 0; i < kCid; i++) {
             const int j = threadIdx.x + i * nthr;
@@ -461,9 +463,49 @@ __global__ __launch_bounds__(64 * NW)
                 full_col[j] = my_cid[i];
                 const int c = my_cid[i] - h * hd;
                 if (c >= 0 && c < HD) atomicOr(&live_mask[c >> 5], 1u << (c & 31));
+                if (c < 0 || c >= hd) atomicAdd(&n_outside, 1);
             }
         }
         __syncthreads();
+        if (n_outside == 0) {
+            // The usual case, every surviving column inside the head's own slice: the wave
+            // assembles its 16 queries x hd slice in LDS (zeros, then the surviving columns at
+            // their places) and stores whole 8-byte pieces of rows, 4 per lane and tile, instead
+            // of up to 32 two-byte stores.  One wave's LDS instructions complete in order, so
+            // the three steps need no barrier.
+            constexpr int ldt = HD + 8;
+            _Float16 *zt = Ks + wave * 16 * ldt;  // the K stage is free: NW * 16 rows <= 128
+            static_assert(NW * 16 <= kKeyBlock && HD + 8 <= MhaLds<HD>::ldk, "slice tiles fit the K stage");
+            int zl[DB][4];
+#pragma unroll
+            for (int d = 0; d < DB; d++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) zl[d][j] = full_col[min(d * 16 + 4 * g + j, 127)] - h * hd;
+#pragma unroll
+            for (int t = 0; t < QT; t++) {
+                const h4 zero4 = {0, 0, 0, 0};
+#pragma unroll
+                for (int i = 0; i < HD / 16; i++) {
+                    const int v = lane + 64 * i;  // 8-byte piece of the 16 x HD tile
+                    *reinterpret_cast<h4 *>(zt + (v / (HD / 4)) * ldt + (v % (HD / 4)) * 4) = zero4;
+                }
+#pragma unroll
+                for (int d = 0; d < DB; d++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        if (d * 16 + 4 * g + j < vlive) zt[r16 * ldt + zl[d][j]] = (_Float16)(o[t][d][j] * inv[t]);
+                const int qbase = qstrip * kStripQ + (wave * QT + t) * 16;
+#pragma unroll
+                for (int i = 0; i < HD / 16; i++) {
+                    const int v = lane + 64 * i;
+                    const int rr = v / (HD / 4), cc = (v % (HD / 4)) * 4;
+                    const h4 piece = *reinterpret_cast<const h4 *>(zt + rr * ldt + cc);
+                    if (qbase + rr < S && cc < hd)
+                        *reinterpret_cast<h4 *>(a.Z + (row0 + qbase + rr) * a.ldz + h * hd + cc) = piece;
+                }
+            }
+            return;
+        }
         int zc[DB][4];
 #pragma unroll
         for (int d = 0; d < DB; d++)
