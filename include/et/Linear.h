@@ -203,7 +203,11 @@ template <> class Linear<csr_mat> {
 };
 
 // 1x16 vector pruning — Linear/Linear.h:153-167 (the reference's kernel is a stub,
-// Linear/SPMM1x16.cu:35-124; this one computes y = x W^T + b)
+// Linear/SPMM1x16.cu:35-124; this one computes y = x W^T + b).  A matrix core multiplies whole
+// 16x16 cells and up to about 95 % vector sparsity nearly every cell holds a vector, so no
+// product can be skipped: the weight is expanded to its dense image once, on the device, and
+// forward runs the dense GEMM on it (et_linear_vec1x16_f16 works on the vectors directly and
+// is 3-5 times slower at 80 %).
 template <> class Linear<mat1x16> {
   public:
     const uint32_t in_size;
@@ -211,19 +215,31 @@ template <> class Linear<mat1x16> {
     const int size;
     mat1x16 weight;
     et::DeviceBuffer<half> bias;
+    et::DeviceBuffer<half> dense;  // [out x in] image of weight
 
     Linear(int _in_size, int _out_size, const mat1x16 &w, const half *b, int _size)
-        : in_size(_in_size), out_size(_out_size), size(_size), weight(w), bias(b, (std::size_t)_out_size) {}
+        : in_size(_in_size), out_size(_out_size), size(_size), weight(w), bias(b, (std::size_t)_out_size),
+          dense((std::size_t)_in_size * (std::size_t)_out_size) {
+        expand();
+    }
     Linear(int _in_size, int _out_size, mat1x16 &&w, const half *b, int _size)
         : in_size(_in_size), out_size(_out_size), size(_size), weight(std::move(w)),
-          bias(b, (std::size_t)_out_size) {}
+          bias(b, (std::size_t)_out_size), dense((std::size_t)_in_size * (std::size_t)_out_size) {
+        expand();
+    }
     void forward(half *output, const half *input, et::stream_t stream = nullptr) {
         forward_act(output, input, ET_ACT_NONE, stream);
     }
     void forward_act(half *output, const half *input, int act, et::stream_t stream = nullptr) {
-        etChk(et_linear_vec1x16_f16(weight.tile_idx.get(), weight.row_idx.get(), et::f16(weight.data.get()),
-                                    et::f16(bias.get()), et::f16(input), et::f16(output), size,
-                                    (int)in_size, (int)out_size, act, stream));
+        etChk(et_linear_dense_f16(et::f16(dense.get()), et::f16(bias.get()), et::f16(input), et::f16(output),
+                                  size, (int)in_size, (int)out_size, act, stream));
+    }
+
+  private:
+    void expand() {
+        etChk(et_vec1x16_to_dense_f16(weight.tile_idx.get(), weight.row_idx.get(), et::f16(weight.data.get()),
+                                      et::f16(dense.get()), (int)in_size, (int)out_size, nullptr));
+        etChk(et_device_sync());
     }
 };
 

@@ -247,6 +247,16 @@ int et_linear_vec1x16_f16(const int32_t *tile_idx, const int32_t *row_idx,
                           const et_f16 *X, et_f16 *Y, int T, int in, int out,
                           int act, et_stream stream);
 
+/* Dense image W[out x in] of a 1x16 weight, written on the device.  A matrix
+ * core multiplies whole 16x16 cells, and below about 95 % vector sparsity nearly
+ * every cell holds a vector, so the products cannot be skipped: Linear<mat1x16>
+ * expands its weight once at construction and runs et_linear_dense_f16 on the
+ * image (3-5 times faster than et_linear_vec1x16_f16 at 80 %).  No counterpart
+ * in the reference. */
+int et_vec1x16_to_dense_f16(const int32_t *tile_idx, const int32_t *row_idx,
+                            const et_f16 *data, et_f16 *W, int in, int out,
+                            et_stream stream);
+
 /* Unstructured CSR weight over [out x in] (indices need not be sorted inside a
  * row).  T may be any size; out % 4 == 0.  Replaces Linear<csr_mat>::forward
  * (Linear/cusp.cu:23-82, cusparseSpMM + bias map); no workspace is allocated. */

@@ -92,6 +92,31 @@ __global__ __launch_bounds__(256) void vec1x16_linear_kernel(const V16Args a) {
     }
 }
 
+// Dense [out x in] image of a 1x16 weight.  One wave per (row-set, part) cell:
+// it clears the cell's 16x16 block of W (two lanes per row, 16 bytes each),
+// then the lanes that have a vector (two per vector) copy its halves to the
+// row it names.  A wave's stores to one address complete in issue order.
+__global__ __launch_bounds__(256) void vec1x16_expand_kernel(const int32_t *tile_idx, const int32_t *row_idx,
+                                                             const _Float16 *data, _Float16 *W, int in,
+                                                             int ncell) {
+    const int lane = threadIdx.x & 63;
+    const int cellno = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (cellno >= ncell) return;
+    const int npart = in >> 4;
+    const int rset = cellno / npart, part = cellno - rset * npart;
+    const int32_t *cell = tile_idx + (size_t)rset * (npart + 1) + part;
+    const int s = cell[0], e = cell[1];
+    _Float16 *blk = W + (size_t)rset * 16 * in + part * 16;
+    const h8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (lane < 32) *reinterpret_cast<h8 *>(blk + (size_t)(lane >> 1) * in + (lane & 1) * 8) = zero8;
+    // a cell holds at most 16 vectors (one per row of the set); more would name a row twice
+    for (int idx = s + (lane >> 1); idx < e; idx += 32) {
+        const int row = row_idx[idx] & 15;
+        *reinterpret_cast<h8 *>(blk + (size_t)row * in + (lane & 1) * 8) =
+            *reinterpret_cast<const h8 *>(data + (size_t)idx * 16 + (lane & 1) * 8);
+    }
+}
+
 // ------------------------------------------------------------------- CSR ----
 struct CsrArgs {
     const int32_t *indptr, *indices;
@@ -176,6 +201,20 @@ static inline _Float16 *H(et_f16 *p) { return reinterpret_cast<_Float16 *>(p); }
 using namespace et;
 
 extern "C" {
+
+int et_vec1x16_to_dense_f16(const int32_t *tile_idx, const int32_t *row_idx, const et_f16 *data,
+                            et_f16 *W, int in, int out, et_stream stream) {
+    ET_REQUIRE(tile_idx && row_idx && data && W, ET_ERR_INVALID_ARG, "et_vec1x16_to_dense_f16: NULL pointer");
+    ET_REQUIRE(in > 0 && out > 0 && in % 16 == 0 && out % 16 == 0, ET_ERR_UNSUPPORTED,
+               "et_vec1x16_to_dense_f16: in=%d out=%d must be positive multiples of 16", in, out);
+    ET_REQUIRE((reinterpret_cast<uintptr_t>(W) & 15) == 0 && (reinterpret_cast<uintptr_t>(data) & 15) == 0,
+               ET_ERR_UNSUPPORTED, "et_vec1x16_to_dense_f16: W and data must be 16-byte aligned");
+    const long ncell = (long)(out / 16) * (in / 16);
+    ET_REQUIRE(ncell <= 0x7fffffffL, ET_ERR_UNSUPPORTED, "et_vec1x16_to_dense_f16: %ld cells", ncell);
+    vec1x16_expand_kernel<<<dim3((unsigned)((ncell + 3) / 4)), 256, 0, as_stream(stream)>>>(
+        tile_idx, row_idx, H(data), H(W), in, (int)ncell);
+    return check_launch("vec1x16_expand_kernel");
+}
 
 int et_linear_vec1x16_f16(const int32_t *tile_idx, const int32_t *row_idx, const et_f16 *data,
                           const et_f16 *bias, const et_f16 *X, et_f16 *Y, int T, int in, int out,

@@ -178,6 +178,14 @@ class Bench:
         us = self.time_us(lambda: et.check(lib.et_linear_vec1x16_f16(d_ti.ptr, d_ri.ptr, data.ptr, bias.ptr, x.ptr, y.ptr,
                                                                     T, n_in, n_out, 0, self.stream)), launches)
         self.record("linear_vec1x16", f"T{T} in{n_in} out{n_out} sparsity {sparsity}", us, 2 * 16 * n * T, "mfma")
+        # what the Linear<mat1x16> class runs: the dense image, written once, and the dense GEMM on it
+        w = self.empty((n_out, n_in))
+        us = self.time_us(lambda: et.check(lib.et_vec1x16_to_dense_f16(d_ti.ptr, d_ri.ptr, data.ptr, w.ptr, n_in, n_out,
+                                                                      self.stream)), launches)
+        self.record("vec1x16_to_dense", f"in{n_in} out{n_out} sparsity {sparsity}", us, 2 * n_in * n_out + 32 * n, "hbm")
+        us = self.time_us(lambda: et.check(lib.et_linear_dense_f16(w.ptr, bias.ptr, x.ptr, y.ptr, T, n_in, n_out, 0,
+                                                                  self.stream)), launches)
+        self.record("linear_vec1x16 image", f"T{T} in{n_in} out{n_out} sparsity {sparsity}", us, 2 * 16 * n * T, "mfma")
 
     def csr(self, T, n_in, n_out, sparsity, launches):
         et, lib = self.et, self.lib

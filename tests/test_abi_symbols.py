@@ -16,7 +16,7 @@ def test_header_declares_the_expected_surface():
     names = declared_symbols()
     for must in ("et_linear_bsr16_f16", "et_mha_fused_f16", "et_skip_layernorm_f16", "et_model_forward",
                  "et_linear_dense_f16", "et_linear_rowpruned_f16", "et_linear_colpruned_f16",
-                 "et_linear_vec1x16_f16", "et_linear_csr_f16", "et_mha_compactv_f16", "et_mha_vo_f16",
+                 "et_linear_vec1x16_f16", "et_vec1x16_to_dense_f16", "et_linear_csr_f16", "et_mha_compactv_f16", "et_mha_vo_f16",
                  "et_fmt_dense_to_bsr16", "et_graph_launch"):
         assert must in names
     assert len(names) >= 70

@@ -144,6 +144,12 @@ def test_linear_vec1x16(et, T, inp, out, sp, act):
                                             up(et, x).ptr, d_y.ptr, T, inp, out, act, None))
     want = L.linear(Hn.f32(x), Hn.f32(W), Hn.f32(b), ACT[act], torch.float16).numpy()
     assert Hn.max_abs(d_y.numpy(), want) <= 4e-3
+    # the dense image written on the device (what Linear<mat1x16> multiplies with) is exact
+    d_w = et.DeviceBuffer.empty((out, inp), np.float16)
+    et.check(et.lib().et_fill_f16(d_w.ptr, out * inp, 0x7E00, None))
+    et.check(et.lib().et_vec1x16_to_dense_f16(up(et, tile_idx).ptr, up(et, row_idx_d).ptr, up(et, data).ptr, d_w.ptr,
+                                              inp, out, None))
+    assert np.array_equal(d_w.numpy(), W)  # as values: the masked W of this test holds -0.0 where the image has +0.0
 
 
 def test_linear_vec1x16_unsorted_rows_in_a_cell(et):
@@ -159,6 +165,10 @@ def test_linear_vec1x16_unsorted_rows_in_a_cell(et):
                                             up(et, x).ptr, d_y.ptr, T, inp, out, 0, None))
     want = L.linear(Hn.f32(x), Hn.f32(W), None, None, torch.float16).numpy()
     assert Hn.max_abs(d_y.numpy(), want) <= 4e-3
+    d_w = et.DeviceBuffer.empty((out, inp), np.float16)
+    et.check(et.lib().et_vec1x16_to_dense_f16(up(et, tile_idx).ptr, up(et, row_idx).ptr, up(et, data).ptr, d_w.ptr,
+                                              inp, out, None))
+    assert np.array_equal(d_w.numpy(), W.astype(np.float16))
 
 
 @pytest.mark.parametrize("T,inp,out,sp,act", [(1024, 768, 768, 0.9, 0), (100, 768, 3072, 0.95, 2), (7, 40, 12, 0.5, 1),
