@@ -165,6 +165,96 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const GemmArgs g) {
     }
 }
 
+// Small results with a long K (one sequence through a pruned or dense Linear: 128 x 80 x 768):
+// the tiled kernels would run a handful of workgroups, each stepping through K stage by stage —
+// 12 dependent round trips for K = 768.  Here a workgroup owns one 16x16 tile of the result and
+// its four waves split K between them; a wave requests all its fragments of up to STEPS K-steps
+// of 32 straight from global memory (L2) before the first product, so the whole kernel is one
+// or two memory round trips plus an LDS reduction of three partial tiles.  B is [N x K]
+// (transposed form), no A-column gather; rows 16-byte aligned.  Every tile reads its 16 rows of
+// A and of B in full, so this only pays while the tiles are few (used up to 1024 of them where
+// the 64x64 tiling has fewer than 64 workgroups; 128 x 768 -> 80 / 384 / 768: 7.1 -> 3.9 / 4.0 /
+// 5.3 us, 256 x 768 -> 768: 7.5 -> 6.8, 128 x 3072 -> 768: 18.6 -> 14.6).  STEPS = 6 when that
+// covers a wave's share of K: fragments requested for steps a wave does not have cost as much
+// as real ones (with 12 where 6 were live the first three shapes took 5.6 / 5.8 / 8.4 us).
+template <int STEPS>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs g) {
+    constexpr int kSkinnySteps = STEPS;
+    __shared__ f4 part[3][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, grp = lane >> 4;
+    const int ntn = g.N >> 4;
+    const int tm = blockIdx.x / ntn, tn = blockIdx.x - tm * ntn;
+    const long long zo = blockIdx.z / g.batch_inner, zi = blockIdx.z % g.batch_inner;
+    const _Float16 *A = g.A + zo * g.sAo + zi * g.sAi + (size_t)(tm * 16 + r16) * g.lda;  // this lane's token row
+    const _Float16 *B = g.B + zo * g.sBo + zi * g.sBi + (size_t)(tn * 16 + r16) * g.ldb;  // ... and feature row
+    _Float16 *Cm = g.C + zo * g.sCo + zi * g.sCi;
+    const _Float16 *bias = g.bias ? g.bias + zo * g.sBias_o + zi * g.sBias_i : nullptr;
+    const h8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    // K-steps of this wave: [s_begin, s_end) of ceil(K / 32), a quarter each
+    const int nsteps = (g.K + 31) >> 5;
+    const int per = (nsteps + 3) >> 2;
+    const int s_begin = wave * per, s_end = min(nsteps, s_begin + per);
+    f4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = s_begin; s0 < s_end; s0 += kSkinnySteps) {
+        // unconditional loads from clamped addresses; values past K or past this wave's share
+        // are selected away (a load under a branch would be waited for on the spot)
+        h8 fa[kSkinnySteps], fb[kSkinnySteps];
+#pragma unroll
+        for (int i = 0; i < kSkinnySteps; i++) {
+            const int k = (s0 + i) * 32 + 8 * grp;
+            const int kc = min(k, g.K - 8);
+            fa[i] = *reinterpret_cast<const h8 *>(A + kc);
+            fb[i] = *reinterpret_cast<const h8 *>(B + kc);
+        }
+#pragma unroll
+        for (int i = 0; i < kSkinnySteps; i++) {
+            const int k = (s0 + i) * 32 + 8 * grp;
+            const bool live = s0 + i < s_end && k < g.K;
+            // features are the A operand: the lane ends with four consecutive features of its token
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(live ? fb[i] : zero8, live ? fa[i] : zero8, acc, 0, 0, 0);
+        }
+    }
+    if (wave > 0) part[wave - 1][lane] = acc;
+    __syncthreads();
+    if (wave > 0) return;
+    acc += part[0][lane] + part[1][lane] + part[2][lane];
+
+    const int m = tm * 16 + r16, n = tn * 16 + 4 * grp;
+    if (g.c_scatter) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int col = g.c_scatter[n + e];
+            float y = acc[e];
+            if (bias) y += (float)bias[col];
+            Cm[(size_t)m * g.ldc + col] = (_Float16)apply_act(y, g.act);
+        }
+    } else {
+        h4 o;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float y = acc[e];
+            if (bias) y += (float)bias[g.bias_idx ? g.bias_idx[n + e] : n + e];
+            o[e] = (_Float16)apply_act(y, g.act);
+        }
+        *reinterpret_cast<h4 *>(Cm + (size_t)m * g.ldc + n) = o;
+    }
+}
+
+// The small-result kernel applies when the 64x64 tiling would leave most of the chip idle.
+static bool gemm_skinny_applies(const GemmArgs &g, int batch, bool trans_b) {
+    const auto misaligned = [](const void *p, int a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; };
+    if (!trans_b || g.a_gather || batch < 1 || batch > 65535) return false;
+    if (g.M <= 0 || g.M % 16 || g.N % 16 || g.K % 16 || g.K < 256) return false;
+    if (g.lda % 8 || g.ldb % 8 || misaligned(g.A, 16) || misaligned(g.B, 16)) return false;
+    if (!g.c_scatter && (g.ldc % 4 || misaligned(g.C, 8))) return false;
+    if (batch > 1 && (((g.sAo | g.sAi | g.sBo | g.sBi) & 7) || ((g.sCo | g.sCi) & 3))) return false;
+    const long long tiles64 = (long long)((g.M + 63) / 64) * ((g.N + 63) / 64) * batch;
+    const long long tiles16 = (long long)(g.M / 16) * (g.N / 16);
+    return tiles64 < 64 && tiles16 <= 1024;
+}
+
 // C[r][c] = act(bias[c]) for the columns a row-pruned weight does not produce.
 __global__ __launch_bounds__(256) void bias_rows_kernel(_Float16 *__restrict__ C,
                                                         const _Float16 *__restrict__ bias, int rows,
@@ -226,6 +316,12 @@ static int launch_gemm_tile(const GemmArgs &g, int batch, bool trans_b, hipStrea
 // The direct-to-LDS kernel where it applies; else this file's kernel, with 128x128 tiles once
 // they still give a few hundred workgroups and 64x64 otherwise.
 int launch_gemm(const GemmArgs &g, int batch, bool trans_b, hipStream_t stream) {
+    if (gemm_skinny_applies(g, batch, trans_b)) {
+        const dim3 grid((unsigned)((g.M / 16) * (g.N / 16)), 1, (unsigned)batch);
+        if (g.K <= 6 * 4 * 32) gemm_skinny_kernel<6><<<grid, 256, 0, stream>>>(g);  // at most 6 K-steps per wave
+        else gemm_skinny_kernel<12><<<grid, 256, 0, stream>>>(g);
+        return check_launch("gemm_skinny_kernel");
+    }
     if (gemm_dma_applies(g, batch, trans_b)) return launch_gemm_dma(g, batch, trans_b, stream);
     const long long tiles128 = (long long)((g.M + 127) / 128) * ((g.N + 127) / 128) * batch;
     if (tiles128 >= 512) return launch_gemm_tile<4, 4>(g, batch, trans_b, stream);

@@ -23,7 +23,10 @@ up = Hn.up
                                            (512, 1536, 768, 2), (256, 64, 256, 0),
                                            # edges that are multiples of 16 only (clamped loads, zeroed K tail,
                                            # masked stores): 16, 32 and 48 k-values in the last stage
-                                           (1008, 720, 400, 2), (80, 96, 2064, 1), (2032, 176, 48, 0)])
+                                           (1008, 720, 400, 2), (80, 96, 2064, 1), (2032, 176, 48, 0),
+                                           # few 64x64 tiles and a long K: one 16x16 tile per workgroup, K split over
+                                           # its waves (K a multiple of 32, of 16 only, more than one round of loads)
+                                           (128, 768, 768, 2), (16, 272, 16, 0), (128, 3072, 80, 1), (32, 6160, 48, 0)])
 def test_linear_dense(et, T, inp, out, act):
     W, b, x = Hn.randn((out, inp), 1, 0.02), Hn.randn((out,), 2, 0.1), Hn.randn((T, inp), 3)
     d_y = et.DeviceBuffer.empty((T, out), np.float16)
@@ -53,7 +56,8 @@ def test_linear_dense_closed_form_ones(et):
 
 @pytest.mark.parametrize("trans_b", [True, False])
 @pytest.mark.parametrize("M,N,K,batch", [(128, 64, 128, 12), (256, 768, 1536, 1), (48, 32, 16, 3),
-                                         (128, 192, 1040, 3)])  # long K in few tiles, 16 k-values in the last stage
+                                         (128, 192, 1040, 3),  # long K in few tiles, 16 k-values in the last stage
+                                         (32, 48, 400, 3)])    # batched small results
 def test_gemm_batched(et, trans_b, M, N, K, batch):
     A = Hn.randn((batch, M, K), 4, 0.5)
     Bm = Hn.randn((batch, N, K) if trans_b else (batch, K, N), 5, 0.1)
@@ -86,7 +90,8 @@ def test_gemm_rejects_bad_args(et):
 @pytest.mark.parametrize("T,inp,out,sp,act", [(2048, 768, 768, 0.5, 0), (2048, 768, 3072, 0.5, 2),
                                               (2048, 3072, 768, 0.5, 0), (64, 64, 100 * 16, 0.9, 1),
                                               (8192, 128, 4096, 0.5, 2),  # the 256 x 256-tile kernel
-                                              (2048, 720, 784, 0.45, 1)])  # 432 surviving rows: a ragged tile edge
+                                              (2048, 720, 784, 0.45, 1),  # 432 surviving rows: a ragged tile edge
+                                              (128, 768, 768, 0.9, 2)])  # one sequence: the small-result kernel, scattered
 def test_linear_rowpruned(et, T, inp, out, sp, act):
     row_id = F.gen_row_ids(out, sp, seed=8)
     rows, b, x = Hn.randn((len(row_id), inp), 9, 0.02), Hn.randn((out,), 10, 0.1), Hn.randn((T, inp), 11)
@@ -109,7 +114,7 @@ def test_linear_rowpruned(et, T, inp, out, sp, act):
 
 
 @pytest.mark.parametrize("T,inp,out,sp,act", [(2048, 768, 768, 0.5, 0), (2048, 768, 3072, 0.5, 2),
-                                              (2048, 3072, 768, 0.5, 0), (32, 160, 48, 0.3, 1)])
+                                              (2048, 3072, 768, 0.5, 0), (32, 160, 48, 0.3, 1), (128, 3072, 768, 0.9, 0)])
 def test_linear_colpruned(et, T, inp, out, sp, act):
     col_id = F.gen_col_ids(inp, sp, seed=12)  # unsorted, as the reference generator leaves them
     cols, b, x = Hn.randn((out, len(col_id)), 13, 0.02), Hn.randn((out,), 14, 0.1), Hn.randn((T, inp), 15)
