@@ -261,6 +261,36 @@ class Bench:
                                                                (H // nh) ** -0.5, 0, self.stream)), launches)
         self.record_f32("mha_fused_f32", f"B{B} S{S} nh{nh} hd{H // nh}", us, 4 * B * S * S * H)
 
+    def stack(self, name, H, nh, FF, S, B, nlayer, sparsity, lens, replays=20):
+        """A whole encoder stack through the model handle (one HIP-graph replay per forward): every
+        Linear tile-sparse at `sparsity` with its own seeded pattern, right padding `lens` or None."""
+        et = self.et
+        m = et.Model(H, nh, FF, S, nlayer, batch=B, act=et.ACT_GELU, eps=1e-5, causal=False, use_graph=True)
+        flops = 0
+        for i in range(nlayer):
+            for which, (o, n_in) in ((et.W_QKV, (3 * H, H)), (et.W_O, (H, H)), (et.W_FF1, (FF, H)), (et.W_FF2, (H, FF))):
+                row_ptr, col, ntile = self.tile_pattern(o, n_in, sparsity, 1000 * i + which + 1)
+                m.set_bsr16(i, which, row_ptr, col, self.rnd((max(ntile, 1), 256), 0.02), self.rnd((o,), 0.02))
+                flops += 2 * 256 * ntile * B * S
+            for which in (0, 1):
+                m.set_norm(i, which, (1.0 + self.rnd((H,), 0.1).astype(np.float32)).astype(np.float16), self.rnd((H,), 0.1))
+        pairs = B * S * S if lens is None else int(sum(int(n) * int(n) for n in lens))
+        flops += nlayer * 4 * pairs * H
+        if lens is not None:
+            m.set_lens(lens)
+        m.finalize()
+        x, y = self.dev(self.rnd((B * S, H))), self.empty((B * S, H))
+        for _ in range(3):
+            m.forward(y, x)
+        m.sync()
+        import time
+        t0 = time.perf_counter()
+        for _ in range(replays):
+            m.forward(y, x)
+        m.sync()
+        us = (time.perf_counter() - t0) * 1e6 / replays
+        self.record("encoder_stack", f"{name}: {B / us * 1e6:.0f} seq/s, {us / nlayer:.1f} us per layer", us, flops, "mfma")
+
     def record_f32(self, kernel, shape, us, flops):
         achieved, peak = flops / us / 1e6, 157.3
         self.rows.append({"kernel": kernel, "shape": shape, "us": round(us, 2), "bound": "mfma_f32",
@@ -294,6 +324,10 @@ def run_configs(b: Bench):
     b.mha_vo(4, 128, 12, 64, 384, 20)       # half of the VO columns pruned
     b.mha_unfused(4, 128, 12, 64, 20)
     b.f32_layer_kernels(1, 128, 768, 12, 3072, 20)
+    # whole stacks: 12-layer BERT-base at batch 8 (80 %), 24-layer BERT-large shape at batch 4, 512 tokens,
+    # right padding with lengths in [256, 512] (90 %)
+    b.stack("BERT-base 12 layers S128 B8 80%", 768, 12, 3072, 128, 8, 12, 0.8, None)
+    b.stack("BERT-large 24 layers S512 B4 90% padded", 1024, 16, 4096, 512, 4, 24, 0.9, rng.integers(256, 513, 4))
 
 
 def run_scale(b: Bench):
