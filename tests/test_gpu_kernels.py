@@ -416,6 +416,16 @@ def test_mha_large_grid(et, causal, padded):
     assert Hn.max_abs(got, want) <= 2e-3
 
 
+@pytest.mark.parametrize("B,S,nh,hd,causal", [(6, 768, 32, 64, False),    # 8 waves x 2 tiles, three query strips, six key blocks
+                                              (6, 768, 32, 64, True),
+                                              (16, 128, 16, 128, False),  # 8 waves x 1 tile with 128-wide heads
+                                              (4, 384, 24, 128, True)])
+def test_mha_large_grid_shapes(et, B, S, nh, hd, causal):
+    lens = [S - (37 * b) % (S // 2) for b in range(B)]
+    got, want = run_mha(et, B, S, nh, hd, seed=64, lens=lens, causal=causal)
+    assert Hn.max_abs(got, want) <= 2e-3
+
+
 def test_mha_additive_mask_and_lens(et):
     B, S, nh, hd = 2, 128, 4, 64
     mask = Hn.randn((S, S), 70, 1.0, np.float32)
