@@ -226,6 +226,11 @@ def main():
                 "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 5), "us_per_launch": round(ksec * 1e6, 3),
                 "flop_per_launch": flops, "traffic": round(FFN_DOWN_TRAFFIC_BYTES)}
+    # The same launch against the other roof: algorithmic bytes 2T(in+out) + 516 ntile + 4(out/16+1) + 2 out.
+    # At 109 flop per byte the shape sits below the ridge of the machine (312 flop/B), i.e. on the HBM roof.
+    alg_bytes = 2.0 * T * (FF + H) + 516.0 * ntile + 4.0 * (H // 16 + 1) + 2.0 * H
+    roofline["hbm_view"] = {"bound": "hbm", "achieved": round(alg_bytes / ksec / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
+                            "frac": round(alg_bytes / ksec / 8e12, 5), "bytes_per_launch": alg_bytes}
 
     out = {
         "metric": "BERT-base encoder seqs/sec + per-layer latency µs, seq128 fp16 80% tile-sparse",
