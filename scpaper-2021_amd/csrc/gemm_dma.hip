@@ -336,8 +336,9 @@ static bool pick_dma_tile(const GemmArgs &g, int batch, bool trans_b, DmaTile *o
     if (wgs(2, 2) >= 512) { *out = {2, 2, 2, false}; return true; }
     if (wgs(2, 1) >= 512) { *out = {2, 1, 2, false}; return true; }
     // few workgroups with a long K loop are bound by the latency of a stage: a third buffer keeps
-    // two stages in flight (2048 x 3072 -> 768: 29.5 -> 24.7 us); elsewhere it only costs occupancy
-    *out = {1, 1, (w11 <= 512 && g.K / kDmaK >= 24) ? 3 : 2, false};
+    // two stages in flight (2048 x 3072 -> 768: 29.5 -> 24.7 us; from 12 stages on it still gives
+    // 3-5 %: 2048 x 768 -> 768 9.6 -> 9.1 us); elsewhere it only costs occupancy
+    *out = {1, 1, (w11 <= 512 && g.K / kDmaK >= 12) ? 3 : 2, false};
     return true;
 }
 
