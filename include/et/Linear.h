@@ -171,15 +171,23 @@ template <> class Linear<tile_mat> {
     }
 };
 
-// unstructured CSR — Linear/Linear.h:88-112, Linear/cusp.cu:23-82
+// unstructured CSR — Linear/Linear.h:88-112, Linear/cusp.cu:23-82.  Single non-zeros give a
+// matrix core nothing to skip, and the scalar CSR kernel (et_linear_csr_f16) is 10-25 times slower
+// than the dense GEMM at 80-95 % sparsity.  Where the shapes allow the GEMM (token rows and both
+// widths multiples of 16) and at least kDenseFromDensity of the elements are non-zero, the
+// constructor therefore sums the non-zeros into a dense image on the host (duplicates of one
+// position add up, as they do in the sparse product) and forward multiplies with that; sparser
+// or odd-shaped weights stay on the CSR kernel.
 template <> class Linear<csr_mat> {
   public:
+    static constexpr double kDenseFromDensity = 0.02;
     const uint32_t in_size;
     const uint32_t out_size;
     const int size;
     std::unique_ptr<et::DeviceBuffer<int>> indptr;
     std::unique_ptr<et::DeviceBuffer<int>> indices;
     std::unique_ptr<et::DeviceBuffer<half>> data;
+    std::unique_ptr<et::DeviceBuffer<half>> dense;  // [out x in] image, or empty
     et::DeviceBuffer<half> bias;
 
     Linear(int _in_size, int _out_size, const csr_mat &w, const half *b, int _size)
@@ -190,12 +198,32 @@ template <> class Linear<csr_mat> {
         indptr = std::make_unique<et::DeviceBuffer<int>>(w.indptr);
         indices = std::make_unique<et::DeviceBuffer<int>>(w.indices);
         data = std::make_unique<et::DeviceBuffer<half>>(h);
+        const double cells = (double)_in_size * (double)_out_size;
+        if (_size % 16 == 0 && _in_size % 16 == 0 && _out_size % 16 == 0 && _size > 0 &&
+            (double)w.data.size() >= kDenseFromDensity * cells) {
+            std::vector<float> img((std::size_t)_in_size * (std::size_t)_out_size, 0.0f);
+            for (int r = 0; r < _out_size; r++)
+                for (int k = w.indptr[(std::size_t)r]; k < w.indptr[(std::size_t)r + 1]; k++) {
+                    const int c = w.indices[(std::size_t)k];
+                    et::require(c >= 0 && c < _in_size, "Linear<csr_mat>: column index out of range");
+                    // the value as the CSR kernel sees it: rounded to binary16 first
+                    img[(std::size_t)r * (std::size_t)_in_size + (std::size_t)c] += static_cast<float>(h[(std::size_t)k]);
+                }
+            std::vector<half> himg(img.size());
+            for (std::size_t i = 0; i < img.size(); i++) himg[i] = static_cast<half>(img[i]);
+            dense = std::make_unique<et::DeviceBuffer<half>>(himg);
+        }
     }
     Linear(Linear<csr_mat> &&other) = default;
     void forward(half *output, const half *input, et::stream_t stream = nullptr) {
         forward_act(output, input, ET_ACT_NONE, stream);
     }
     void forward_act(half *output, const half *input, int act, et::stream_t stream = nullptr) {
+        if (dense) {
+            etChk(et_linear_dense_f16(et::f16(dense->get()), et::f16(bias.get()), et::f16(input), et::f16(output),
+                                      size, (int)in_size, (int)out_size, act, stream));
+            return;
+        }
         etChk(et_linear_csr_f16(indptr->get(), indices->get(), et::f16(data->get()), et::f16(bias.get()),
                                 et::f16(input), et::f16(output), size, (int)in_size, (int)out_size, act,
                                 stream));

@@ -234,6 +234,21 @@ static int run_factories(const std::string &dir) {
         ln->forward(O.get(), A.get(), B.get(), T);
         out.push_back(first_value(O, 100));                             // 0.2
     }
+    // Linear<csr_mat> multiplies with a dense image from 2 % density on and with the CSR kernel below:
+    // both against a direct call of the CSR kernel (weights and inputs are ones: sums are exact)
+    for (float sp : {0.8f, 0.99f}) {
+        auto lin = gen_sparse_linear<csr_mat>(128, 256, T, sp);
+        lin->forward(Y.get(), X256.get());
+        et::DeviceBuffer<half> Y2((std::size_t)T * 128);
+        etChk(et_linear_csr_f16(lin->indptr->get(), lin->indices->get(), et::f16(lin->data->get()), et::f16(lin->bias.get()),
+                                et::f16(X256.get()), et::f16(Y2.get()), T, 256, 128, ET_ACT_NONE, nullptr));
+        etChk(et_device_sync());
+        auto a = Y.to_host(), b = Y2.to_host();
+        bool same = true;
+        for (std::size_t i = 0; i < (std::size_t)T * 128; i++) same = same && static_cast<float>(a[i]) == static_cast<float>(b[i]);
+        out.push_back(same ? 1.0f : 0.0f);
+        out.push_back(lin->dense ? 1.0f : 0.0f);  // 1 at 80 %, 0 at 99 %
+    }
     // DeviceBuffer value semantics: deep copy, move, clear, set
     {
         et::DeviceBuffer<half> a(8, static_cast<half>(3.0f));

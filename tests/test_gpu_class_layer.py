@@ -135,4 +135,6 @@ def test_factories_closed_forms(tmp_path):
     assert col_v == 64.5 and csr_v == 256.5 and v16 == 256.5
     assert vo == 205.0  # the reference driver's expected value (Fused_attention/test/testVO.cu:10-16)
     assert abs(ln - 0.2) < 1e-3
-    assert db == [3.0, 4.0, 0.0, 1.0]
+    # Linear<csr_mat>: dense-image path (80 %) and CSR-kernel path (99 %) both equal the CSR kernel called directly
+    assert db[:4] == [1.0, 1.0, 1.0, 0.0]
+    assert db[4:] == [3.0, 4.0, 0.0, 1.0]
