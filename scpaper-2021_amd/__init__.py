@@ -347,6 +347,14 @@ class Model:
         bias = None if bias is None else np.ascontiguousarray(bias, data.dtype)
         fn = lib().et_model_set_bsr16_f16 if data.dtype == np.float16 else lib().et_model_set_bsr16
         assert data.dtype in (np.float16, np.float32)
+        # the library reads out/16+1 row pointers, len(column) tiles of 256 values and out biases
+        d = self.desc
+        n_out = {W_QKV: 2 * d.kdim + d.vdim, W_O: d.emdim, W_FF1: d.dimFF, W_FF2: d.emdim}.get(which)
+        if n_out is not None:
+            if row_ptr.size != n_out // 16 + 1 or data.size != column.size * 256 or (
+                    bias is not None and bias.size != n_out):
+                raise ValueError(f"set_bsr16: row_ptr[{row_ptr.size}], column[{column.size}], data[{data.size}] or "
+                                 f"bias do not fit a matrix of {n_out} output features")
         check(fn(self.handle, layer, which, _np_ptr(row_ptr), _np_ptr(column), _np_ptr(data), len(column),
                  _np_ptr(bias)))
 

@@ -161,7 +161,7 @@ std::vector<half> to_half(const float *src, size_t n) {
 }
 std::vector<half> to_half(const et_f16 *src, size_t n) {
     std::vector<half> v(n);
-    std::memcpy(v.data(), src, n * sizeof(half));
+    if (n) std::memcpy(v.data(), src, n * sizeof(half));  // an empty vector's data() may be null
     return v;
 }
 

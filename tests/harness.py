@@ -2,6 +2,7 @@
 seeded synthetic weights, upload/download, and oracle comparison."""
 from __future__ import annotations
 
+import hashlib
 import math
 import sys
 from pathlib import Path
@@ -55,6 +56,15 @@ class BsrWeight:
         self.out, self.inp = out, inp
         self._pattern_args = (out, inp, sparsity, seed, tuple(dead_block_rows), tuple(dead_block_cols))
         self.row_ptr, self.col_idx = self._pattern()
+        # The structure is frozen the moment it exists: numpy refuses any later write through
+        # these arrays, and the digest taken here is compared again at every hand-over to the
+        # library (check_tile_pattern), so a change made behind numpy's back cannot go unseen.
+        bc = inp // 16
+        assert len(self.col_idx) == 0 or (self.col_idx.min() >= 0 and self.col_idx.max() < bc), \
+            "pattern generator produced a column tile outside the matrix"
+        self.row_ptr.flags.writeable = False
+        self.col_idx.flags.writeable = False
+        self._pattern_digest = pattern_digest(self.row_ptr, self.col_idx)
         n = len(self.col_idx)
         self.tiles = randn((n, 256), seed + 1, std)
         self.bias = randn((out,), seed + 2, bias_std) if bias_std else np.zeros(out, np.float16)
@@ -65,11 +75,6 @@ class BsrWeight:
         if dead_rows or dead_cols:
             return dead_aware_pattern(out, inp, sparsity, seed, dead_rows, dead_cols)
         return F.gen_tile_pattern(out, inp, sparsity, seed)
-
-    def rebuild_pattern(self):
-        """Generates the (deterministic) pattern and the masked dense matrix again."""
-        self.row_ptr, self.col_idx = self._pattern()
-        self.dense = F.bsr16_to_dense(self.row_ptr, self.col_idx, self.tiles, self.inp)
 
     def upload(self, et):
         check_tile_pattern(self, f"weight {self.out} x {self.inp}")
@@ -194,23 +199,27 @@ def run_layer_case(et, H, nh, dimFF, S, B, sparsity, seed, lens=None, nlayers=1,
     return max_abs(got, want)
 
 
+def pattern_digest(row_ptr, col_idx) -> str:
+    return hashlib.sha1(row_ptr.tobytes() + col_idx.tobytes()).hexdigest()
+
+
 def check_tile_pattern(bw, what):
-    """The generators cannot produce a column tile outside the matrix; one that shows up later
-    means the host array changed after it was built (seen twice in some forty runs of the whole
-    suite, cause unknown).  Says where and what in a warning, for the log, and generates the
-    pattern again, so that the parity checks of the test still run — on weights known to be good."""
+    """A tile pattern must reach the library exactly as it was generated.  The arrays are
+    read-only for numpy from the moment they exist, so a difference here means that memory
+    was written behind numpy's back; the test stops and says where and what."""
+    if pattern_digest(bw.row_ptr, bw.col_idx) == bw._pattern_digest:
+        return
     bc = bw.inp // 16
-    if len(bw.col_idx) and (bw.col_idx.min() < 0 or bw.col_idx.max() >= bc):
-        import warnings
-        bad = np.nonzero((bw.col_idx < 0) | (bw.col_idx >= bc))[0]
-        lo = max(0, int(bad[0]) - 8)
-        warnings.warn(
-            f"{what}: col_idx of {len(bw.col_idx)} tiles holds {len(bad)} values outside [0, {bc}) although it was "
-            f"generated inside: first at {bad[:8]}, values {bw.col_idx[bad[:8]]}, col_idx[{lo}:{lo + 40}] = "
-            f"{bw.col_idx[lo:lo + 40]}, array at {bw.col_idx.ctypes.data:#x} (owns its data: "
-            f"{bw.col_idx.flags.owndata}); pattern generated again")
-        bw.rebuild_pattern()
-        assert bw.col_idx.min() >= 0 and bw.col_idx.max() < bc
+    fresh_rp, fresh_ci = bw._pattern()
+    bad = np.nonzero(bw.col_idx != fresh_ci)[0]
+    bad_rp = np.nonzero(bw.row_ptr != fresh_rp)[0]
+    lo = max(0, int(bad[0]) - 8) if len(bad) else 0
+    raise AssertionError(
+        f"{what}: the tile pattern changed after it was generated ({len(bad)} of {len(bw.col_idx)} column ids, "
+        f"{len(bad_rp)} of {len(bw.row_ptr)} row pointers; {bc} column tiles): first at {bad[:8]}, values "
+        f"{bw.col_idx[bad[:8]]} instead of {fresh_ci[bad[:8]]}, col_idx[{lo}:{lo + 40}] = {bw.col_idx[lo:lo + 40]}, "
+        f"bytes {bw.col_idx[lo:lo + 40].tobytes().hex()}, array at {bw.col_idx.ctypes.data:#x} "
+        f"(owns its data: {bw.col_idx.flags.owndata}, writeable: {bw.col_idx.flags.writeable})")
 
 
 def build_model(et, layers, S, B, act=2, lens=None, use_graph=True, causal=False, eps=1e-5):
