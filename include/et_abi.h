@@ -236,6 +236,21 @@ int et_linear_colpruned_ws_f16(const et_f16 *cols, const int32_t *col_id,
                                et_f16 *Y, et_f16 *workspace, int T, int in,
                                int out, int act, et_stream stream);
 
+/* et_linear_colpruned_ws_f16 without a workspace argument and without any
+ * allocation: the gathered activations [T x nnz_col] go to a buffer built into
+ * the library (a file-scope device array of 8 MiB per GPU, held until the
+ * process ends).  No counterpart in the reference; it is for callers that
+ * cannot allocate device memory or pass a workspace: code under HIP-graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  Same result,
+ * bit for bit, as the _ws form.  T * nnz_col * 2 bytes must fit 8 MiB
+ * (ET_ERR_UNSUPPORTED otherwise).  All calls on one GPU share the buffer: calls
+ * that may overlap on one GPU (different streams, or one graph replayed while
+ * another call runs) race on it and must be ordered by the caller. */
+int et_linear_colpruned_static_f16(const et_f16 *cols, const int32_t *col_id,
+                                   int nnz_col, const et_f16 *bias, const et_f16 *X,
+                                   et_f16 *Y, int T, int in, int out, int act,
+                                   et_stream stream);
+
 /* 1x16 vector-sparse weight (mat1x16): for row-set r (16 output features) and
  * part p (16 input features) the surviving 1x16 vectors are idx in
  * [tile_idx[r*(in/16+1)+p], tile_idx[r*(in/16+1)+p+1]); row_idx[idx] % 16 is

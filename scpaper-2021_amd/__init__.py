@@ -76,6 +76,7 @@ _SIGNATURES = {
     "et_relu_f32": (_vp, _vp, _sz, _vp),
     "et_gather_cols_f16": (_vp, _vp, _vp, _i, _i, _i, _vp),
     "et_linear_colpruned_ws_f16": (_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_linear_colpruned_static_f16": (_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_linear_dense_f16": (_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_gemm_f16": (_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _ll, _ll, _ll, _vp),
     "et_linear_rowpruned_f16": (_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp),

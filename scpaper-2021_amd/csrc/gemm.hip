@@ -19,6 +19,9 @@
 //   c_scatter: column n of the result is written to C[:, c_scatter[n]]
 //              (row_mat Linear: replaces the scatter pass, Linear/SPMM_row.cu:14-30)
 //   bias/act : y = act(acc + bias[column]) on the fp32 accumulator.
+#include <atomic>
+#include <mutex>
+
 #include "gemm.hip.h"
 
 namespace et {
@@ -363,6 +366,45 @@ __global__ __launch_bounds__(256) void gather_cols_kernel(_Float16 *__restrict__
 
 }  // namespace et
 
+
+// ---------------------------------------------------------------------------
+// Scratch for the allocation-free column-pruned Linear: the gathered activations
+// [T x nnz_col] live in this file-scope device array instead of a caller's or
+// an allocated workspace.  Every GPU the library runs on holds its own copy at
+// its own address until the process ends; the array's name below is only the
+// host-side handle of the symbol, the device address comes from
+// hipGetSymbolAddress, once per device, with that device current.
+// ---------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = (size_t)8 << 20;  // 8 MiB: e.g. 2048 rows x 2048 kept columns
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace et {
+
+constexpr int kMaxDevices = 64;
+static std::atomic<void *> g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device (looked up on first use).
+static int static_scratch(void **out) {
+    int dev = -1;
+    ET_HIP(hipGetDevice(&dev));
+    ET_REQUIRE(dev >= 0 && dev < kMaxDevices, ET_ERR_UNSUPPORTED, "static scratch: device ordinal %d", dev);
+    void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+        if (!p) {
+            ET_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+            ET_REQUIRE(p != nullptr, ET_ERR_LAUNCH, "static scratch: hipGetSymbolAddress returned NULL");
+            g_scratch_ptr[dev].store(p, std::memory_order_release);
+        }
+    }
+    *out = p;
+    return ET_OK;
+}
+
+}  // namespace et
+
 using namespace et;
 
 extern "C" {
@@ -507,6 +549,24 @@ int et_linear_colpruned_ws_f16(const et_f16 *cols, const int32_t *col_id, int nn
     int s = et_gather_cols_f16(workspace, X, col_id, T, in, nnz_col, stream);
     if (s != ET_OK) return s;
     return et_linear_dense_f16(cols, bias, workspace, Y, T, nnz_col, out, act, stream);
+}
+
+int et_linear_colpruned_static_f16(const et_f16 *cols, const int32_t *col_id, int nnz_col, const et_f16 *bias,
+                                   const et_f16 *X, et_f16 *Y, int T, int in, int out, int act,
+                                   et_stream stream) {
+    ET_REQUIRE(T >= 0 && nnz_col >= 0, ET_ERR_INVALID_ARG, "et_linear_colpruned_static_f16: T=%d nnz_col=%d", T,
+               nnz_col);
+    const size_t need = (size_t)T * (size_t)nnz_col * sizeof(et_f16);
+    ET_REQUIRE(need <= kStaticScratchBytes, ET_ERR_UNSUPPORTED,
+               "et_linear_colpruned_static_f16: T x nnz_col = %d x %d needs %zu bytes of scratch, the built-in "
+               "buffer holds %zu; use et_linear_colpruned_ws_f16 with a workspace of your own",
+               T, nnz_col, need, kStaticScratchBytes);
+    void *ws = nullptr;
+    int s = static_scratch(&ws);
+    if (s != ET_OK) return s;
+    // the gather overwrites every element of the [T x nnz_col] prefix it then reads: nothing to clear
+    return et_linear_colpruned_ws_f16(cols, col_id, nnz_col, bias, X, Y, static_cast<et_f16 *>(ws), T, in, out,
+                                      act, stream);
 }
 
 }  // extern "C"
