@@ -5,7 +5,12 @@ of activations: ``None`` keeps fp32 throughout (the plain mathematics);
 ``torch.float16`` rounds to fp16 exactly where the GPU engine writes fp16 to
 memory (after each Linear incl. its fused bias/activation, after the attention
 output, after each LayerNorm) and where it feeds fp16 operands to the matrix
-cores (the un-normalised softmax probabilities).
+cores (the un-normalised softmax probabilities).  ``LayerConfig.resid`` selects
+the storage of the residual stream separately: with ``resid=torch.float32`` and
+``store=torch.float16`` (the engine's mixed-precision mode) the outputs of the
+two projections that feed a SkipLayerNorm and the SkipLayerNorm results stay
+fp32, and fp16 rounding happens only where a value becomes a matrix-core
+operand.
 
 Weights are applied as masked dense ``[out, in]`` matrices; sparse containers
 are expanded with ``oracle.formats.*_to_dense`` first.
@@ -208,31 +213,40 @@ class LayerConfig:
     mask: Optional[torch.Tensor] = None
     lens: Optional[torch.Tensor] = None
     store: object = None
+    resid: object = "same"  # storage of the residual stream; "same" = as ``store``
     fused_act: bool = True  # activation applied on the fp32 accumulator of linear1
     extras: dict = field(default_factory=dict)
 
 
+def _resid_store(cfg: LayerConfig):
+    return cfg.store if isinstance(cfg.resid, str) else cfg.resid
+
+
 def attention_block(x, P: LayerParams, cfg: LayerConfig):
     """One Linear H -> 3H, attention over column slices, output Linear
-    (Attention/Attention.h:246-265)."""
+    (Attention/Attention.h:246-265).  x is rounded to the operand type on its
+    way into the projection; the output projection is stored as the residual
+    stream is."""
     H = P.Wo.shape[1]
-    qkv = linear(x, P.Wqkv, P.bqkv, store=cfg.store)
+    qkv = linear(_store(x, cfg.store), P.Wqkv, P.bqkv, store=cfg.store)
     q, k, v = qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:]
     z = mha(q, k, v, cfg.nh, cfg.B, mask=cfg.mask, lens=cfg.lens, causal=cfg.causal, store=cfg.store)
-    return linear(z, P.Wo, P.bo, store=cfg.store)
+    return linear(z, P.Wo, P.bo, store=_resid_store(cfg))
 
 
 def encoder_layer(x, P: LayerParams, cfg: LayerConfig):
     """attn -> SkipLN(attn, x) -> L1 -> act -> L2 -> SkipLN(L2, LN1)
     (Encoder/Encoder.h:81-96)."""
+    rs = _resid_store(cfg)
     a = attention_block(x, P, cfg)
-    y1 = skip_layernorm(a, x, P.g1, P.be1, cfg.eps, cfg.store)
+    y1 = skip_layernorm(a, x, P.g1, P.be1, cfg.eps, rs)
+    y1_op = _store(y1, cfg.store)  # what linear1's matrix cores see
     if cfg.fused_act:
-        f = linear(y1, P.W1, P.b1, act=cfg.act, store=cfg.store)
+        f = linear(y1_op, P.W1, P.b1, act=cfg.act, store=cfg.store)
     else:
-        f = _store(ACTS[cfg.act](linear(y1, P.W1, P.b1, store=cfg.store)), cfg.store)
-    f2 = linear(f, P.W2, P.b2, store=cfg.store)
-    return skip_layernorm(f2, y1, P.g2, P.be2, cfg.eps, cfg.store)
+        f = _store(ACTS[cfg.act](linear(y1_op, P.W1, P.b1, store=cfg.store)), cfg.store)
+    f2 = linear(f, P.W2, P.b2, store=rs)
+    return skip_layernorm(f2, y1, P.g2, P.be2, cfg.eps, rs)
 
 
 def encoder_stack(x, layers, cfg: LayerConfig):
