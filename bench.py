@@ -91,7 +91,9 @@ def build_layers(et):
 
 
 def build_model(et, layers, use_graph):
-    m = et.Model(H, NH, FF, S, NLAYER, batch=B, act=et.ACT_GELU, eps=1e-5, causal=False, use_graph=use_graph)
+    # mixed precision: fp16 matrix-core operands, fp32 accumulation, fp32 residual stream / LayerNorm / softmax
+    m = et.Model(H, NH, FF, S, NLAYER, batch=B, act=et.ACT_GELU, eps=1e-5, causal=False, use_graph=use_graph,
+                 mixed=True)
     for i, w in enumerate(layers):
         for which, tw in ((et.W_QKV, w.qkv), (et.W_O, w.o), (et.W_FF1, w.l1), (et.W_FF2, w.l2)):
             m.set_bsr16(i, which, tw.row_ptr, tw.col_idx, tw.tiles, tw.bias)
@@ -148,45 +150,66 @@ def time_ffn_down_kernel(et, w, T, launches_per_graph=64, replays=8):
     return t.ms * 1e-3 / (launches_per_graph * replays)
 
 
-def cpu_baseline(layers, x, gpu_out, reps=3):
-    """The CPU oracle (PyTorch-CPU fp32 forward, pruned weights as masked dense matrices) on
-    the host cores: one warm-up, then `reps` forwards of the full 12-layer, batch-8 stack.
-    The only part of this file that uses oracle/: it also checks the GPU result of the same
-    workload against the oracle run with the engine's fp16 storage points."""
+def oracle_params(layers):
     import torch
     from oracle import formats as F
+    from oracle import layers as L
+    f32 = lambda a: torch.from_numpy(np.asarray(a, np.float32))
+    dense = lambda w: f32(F.bsr16_to_dense(w.row_ptr, w.col_idx, w.tiles, w.inp))
+    return [L.LayerParams(dense(w.qkv), f32(w.qkv.bias), dense(w.o), f32(w.o.bias), dense(w.l1), f32(w.l1.bias),
+                          dense(w.l2), f32(w.l2.bias), f32(w.g1), f32(w.be1), f32(w.g2), f32(w.be2))
+            for w in layers]
+
+
+def oracle_forwards(layers, x):
+    """(fp32 forward, forward with the engine's mixed-precision rounding points) of the workload."""
+    import torch
+    from oracle import layers as L
+    params = oracle_params(layers)
+    xt = torch.from_numpy(np.asarray(x, np.float32))
+    with torch.no_grad():
+        want32 = L.encoder_stack(xt, params, L.LayerConfig(nh=NH, B=B, act="gelu", store=None)).numpy()
+        want_mixed = L.encoder_stack(xt, params, L.LayerConfig(nh=NH, B=B, act="gelu", store=torch.float16,
+                                                               resid=torch.float32)).numpy()
+    return want32, want_mixed
+
+
+def cpu_baseline(layers, x, gpu_out, warmups=2, reps=5):
+    """The CPU oracle (PyTorch-CPU fp32 forward, pruned weights as masked dense matrices) on
+    the host cores: `warmups` untimed forwards, then the median of `reps` forwards of the full
+    12-layer, batch-8 stack.  The only part of this file that uses oracle/: it also checks the GPU
+    result of the same workload against the oracle."""
+    import torch
     from oracle import layers as L
 
     threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
     torch.set_num_threads(threads)
-    f32 = lambda a: torch.from_numpy(np.asarray(a, np.float32))
-    dense = lambda w: f32(F.bsr16_to_dense(w.row_ptr, w.col_idx, w.tiles, w.inp))
-    params = [L.LayerParams(dense(w.qkv), f32(w.qkv.bias), dense(w.o), f32(w.o.bias), dense(w.l1), f32(w.l1.bias),
-                            dense(w.l2), f32(w.l2.bias), f32(w.g1), f32(w.be1), f32(w.g2), f32(w.be2))
-              for w in layers]
+    params = oracle_params(layers)
     cfg = L.LayerConfig(nh=NH, B=B, act="gelu", store=None)
-    xt = f32(x)
+    xt = torch.from_numpy(np.asarray(x, np.float32))
     with torch.no_grad():
-        L.encoder_stack(xt, params, cfg)
+        for _ in range(warmups):
+            L.encoder_stack(xt, params, cfg)
         times = []
         for _ in range(reps):
             t0 = time.perf_counter()
             L.encoder_stack(xt, params, cfg)
             times.append(time.perf_counter() - t0)
-        want32 = L.encoder_stack(xt, params, cfg).numpy()
-        want16 = L.encoder_stack(xt, params, L.LayerConfig(nh=NH, B=B, act="gelu", store=torch.float16)).numpy()
+    want32, want_mixed = oracle_forwards(layers, x)
     med = float(np.median(times))
     got = gpu_out.astype(np.float32)
-    err32, err16 = float(np.max(np.abs(got - want32))), float(np.max(np.abs(got - want16)))
-    ref16 = float(np.max(np.abs(want16 - want32)))
+    err32, errm = float(np.max(np.abs(got - want32))), float(np.max(np.abs(got - want_mixed)))
+    refm = float(np.max(np.abs(want_mixed - want32)))
     return {"value": round(B / med, 3), "unit": "seq/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"{reps} forwards of the full workload (12 layers, batch 8, seq 128) after 1 warm-up, "
+            "sample": f"{reps} forwards of the full workload (12 layers, batch 8, seq 128) after {warmups} warm-ups, "
                       f"median {med * 1e3:.1f} ms per forward, fp32 masked-dense PyTorch-CPU oracle",
             "us_per_layer": round(med * 1e6 / NLAYER, 1),
-            # max-abs over the [1024 x 768] output of layer 12: the GPU against the fp32 forward timed above,
-            # against the same forward with the engine's fp16 storage points, and those two against each other
-            "gpu_max_abs_err_vs_fp32_forward": round(err32, 6), "gpu_max_abs_err_vs_fp16_storage_forward": round(err16, 6),
-            "fp16_storage_forward_vs_fp32_forward": round(ref16, 6)}
+            # max-abs over the [1024 x 768] output of layer 12: the GPU (fp16 result) against the fp32 forward
+            # timed above, against the same forward with the engine's rounding points (fp16 operands, fp32
+            # residual stream), and those two against each other
+            "gpu_max_abs_err_vs_fp32_forward": round(err32, 6),
+            "gpu_max_abs_err_vs_mixed_precision_forward": round(errm, 6),
+            "mixed_precision_forward_vs_fp32_forward": round(refm, 6)}
 
 
 def main():

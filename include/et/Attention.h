@@ -238,6 +238,20 @@ class Attention<_config, std::enable_if_t<!_config::isSingleKernel>> : public et
             linearO->forward(out, mat_z->get(), stream);
         }
     }
+
+    // the same with the output projection stored as binary32 (mixed-precision layer);
+    // scratch16 [rows x emdim] is used when linearO's container has no binary32 store
+    void forward_f32(float *out, half *query, half *key, half *value, half *scratch16,
+                     et::stream_t stream = nullptr) {
+        static_assert(!std::is_same<OTF_attn_Ofused, typename config::attn_t>::value,
+                      "the O-fused form has no binary32 output");
+        linearQ->forward(mat_q->get(), query, stream);
+        linearK->forward(mat_k->get(), key, stream);
+        linearV->forward(mat_v->get(), value, stream);
+        Multihead_atttion<typename config::attn_t>(mat_q.get(), mat_k.get(), mat_v.get(), mat_qk.get(), nullptr,
+                                                   mat_z.get(), model, run(stream));
+        et::linear_forward_f32(*linearO, out, mat_z->get(), scratch16, stream);
+    }
 };
 
 // one projection H -> (2*kdim + vdim), attention over column slices of its output
@@ -273,5 +287,18 @@ class Attention<_config, std::enable_if_t<_config::isSingleKernel>> : public et:
         half *V = K + model->kdim;
         et::fused_mha(Q, K, V, ldm, ldm, ldm, mat_z->get(), model->vdim, *model, run(stream));
         linearO->forward(out, mat_z->get(), stream);
+    }
+
+    // the same with the output projection stored as binary32 (mixed-precision layer)
+    void forward_f32(float *out, half *query, half *key, half *value, half *scratch16,
+                     et::stream_t stream = nullptr) {
+        et::require(query == key && key == value, "single-projection attention is self-attention");
+        linearQKV->forward(mat_qkv->get(), query, stream);
+        const int ldm = model->kdim * 2 + model->vdim;
+        half *Q = mat_qkv->get();
+        half *K = Q + model->kdim;
+        half *V = K + model->kdim;
+        et::fused_mha(Q, K, V, ldm, ldm, ldm, mat_z->get(), model->vdim, *model, run(stream));
+        et::linear_forward_f32(*linearO, out, mat_z->get(), scratch16, stream);
     }
 };

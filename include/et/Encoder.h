@@ -69,6 +69,8 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
     DeviceBuffer<half> temp_linear;  // [rows x dimFF]
     DeviceBuffer<half> temp_attn;    // [rows x emdim]
     DeviceBuffer<half> temp_LN;      // [rows x emdim]
+    // binary32 twins of temp_attn and temp_LN, present after enable_mixed()
+    std::unique_ptr<DeviceBuffer<float>> temp_attn32, temp_LN32;
 
     EncoderLayer(std::unique_ptr<attn_t> _attn, std::unique_ptr<SkipLayerNorm> _LN1,
                  std::unique_ptr<SkipLayerNorm> _LN2, std::unique_ptr<linear1_t> _linear1,
@@ -106,6 +108,43 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
         }
         linear2->forward(temp_attn.get(), temp_linear.get(), stream);
         LN2->forward(out, temp_attn.get(), temp_LN.get(), rows, stream);
+    }
+
+    // Mixed precision.  The residual stream — the layer input, both projections that feed a
+    // SkipLayerNorm, and both SkipLayerNorm results — is binary32; binary16 appears only where a
+    // value is a matrix-core operand (the layer input and LN1's result as Linear inputs, Q/K/V,
+    // the probabilities, the attention output, the activated FFN hidden layer).  Without it the
+    // rounding of the residual stream to binary16 after every sublayer is what a deep stack's
+    // error consists of (12 BERT-base layers: 2e-2 against the fp32 mathematics; mixed: 1e-3).
+    //   src32 / src16: the layer input in both forms;  out32 / out16: the result in both forms
+    //   (either may be null).  Call enable_mixed() once before the first forward_mixed().
+    void enable_mixed() {
+        if (!temp_attn32) temp_attn32 = std::make_unique<DeviceBuffer<float>>((std::size_t)rows * model->emdim);
+        if (!temp_LN32) temp_LN32 = std::make_unique<DeviceBuffer<float>>((std::size_t)rows * model->emdim);
+    }
+    void forward_mixed(float *out32, half *out16, const float *src32, half *src16, stream_t stream = nullptr) {
+        require(temp_attn32 && temp_LN32, "Encoder: call enable_mixed() before forward_mixed()");
+        attn_forward_f32(temp_attn32->get(), src16, stream);
+        LN1->forward_mixed(temp_LN32->get(), temp_LN.get(), temp_attn32->get(), src32, rows, stream);
+        linear1->forward_act(temp_linear.get(), temp_LN.get(), act_code<ACT_OP_t>(), stream);
+        linear_forward_f32(*linear2, temp_attn32->get(), temp_linear.get(), temp_attn.get(), stream);
+        LN2->forward_mixed(out32, out16, temp_attn32->get(), temp_LN32->get(), rows, stream);
+    }
+
+  private:
+    template <typename A, typename = void> struct attn_has_f32 : std::false_type {};
+    template <typename A>
+    struct attn_has_f32<A, std::void_t<decltype(std::declval<A &>().forward_f32(
+                               static_cast<float *>(nullptr), static_cast<half *>(nullptr),
+                               static_cast<half *>(nullptr), static_cast<half *>(nullptr),
+                               static_cast<half *>(nullptr), static_cast<stream_t>(nullptr)))>> : std::true_type {};
+    void attn_forward_f32(float *out32, half *src16, stream_t stream) {
+        if constexpr (attn_has_f32<attn_t>::value) {
+            attn->forward_f32(out32, src16, src16, src16, temp_attn.get(), stream);
+        } else {  // attention forms without a binary32 output projection: widen their result
+            attn->forward(temp_attn.get(), src16, src16, src16, stream);
+            etChk(et_f16_to_f32(out32, f16(temp_attn.get()), (std::size_t)rows * model->emdim, stream));
+        }
     }
 };
 

@@ -8,6 +8,7 @@
 // GEMM instead of the reference's extra passes.  Nothing blocks the host.
 #pragma once
 #include <memory>
+#include <type_traits>
 #include <utility>
 #include <vector>
 
@@ -149,6 +150,13 @@ template <> class Linear<tile_mat> {
                                   et::f16(bias.get()), et::f16(input), et::f16(output), size, (int)in_size,
                                   (int)out_size, act, stream));
     }
+    // binary32 result (fp16 operands, fp32 accumulator stored unrounded): what the
+    // mixed-precision encoder layer adds to its fp32 residual stream
+    void forward_f32(float *output, const half *input, et::stream_t stream = nullptr) {
+        etChk(et_linear_bsr16_f16_f32out(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
+                                         et::f16(bias.get()), et::f16(input), output, size, (int)in_size,
+                                         (int)out_size, ET_ACT_NONE, stream));
+    }
     // ln_out = ln(src + skip); output = act(ln_out * W^T + bias) in one launch: the
     // SkipLayerNorm -> Linear -> activation sequence of Encoder/Encoder.h:85-89.  LN_t is
     // SkipLayerNorm (gamma(), beta(), epsilon(), width()).
@@ -272,3 +280,26 @@ template <> class Linear<mat1x16> {
 };
 
 #include "gen_linear.hpp"
+
+namespace et {
+
+// binary32 output of any Linear: its own forward_f32 where the container's kernel can store
+// the accumulator unrounded (tile_mat), else the binary16 result widened (one rounding of the
+// projection's output; the residual stream it is added to stays binary32 either way).
+template <typename L, typename = void> struct has_forward_f32 : std::false_type {};
+template <typename L>
+struct has_forward_f32<L, std::void_t<decltype(std::declval<L &>().forward_f32(
+                              static_cast<float *>(nullptr), static_cast<const half *>(nullptr),
+                              static_cast<stream_t>(nullptr)))>> : std::true_type {};
+
+template <typename L>
+void linear_forward_f32(L &lin, float *out32, const half *in, half *scratch16, stream_t stream) {
+    if constexpr (has_forward_f32<L>::value) {
+        lin.forward_f32(out32, in, stream);
+    } else {
+        lin.forward(scratch16, in, stream);
+        etChk(et_f16_to_f32(out32, f16(scratch16), (std::size_t)lin.size * (std::size_t)lin.out_size, stream));
+    }
+}
+
+}  // namespace et

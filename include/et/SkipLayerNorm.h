@@ -24,6 +24,15 @@ class SkipLayerNorm {
                                     reinterpret_cast<const et_f16 *>(weight.get()),
                                     reinterpret_cast<const et_f16 *>(bias.get()), num, size, eps, stream));
     }
+    // mixed precision: src and skip binary32 (a projection's unrounded output and the residual
+    // stream), result written as binary32 (out32, the next residual) and rounded to binary16
+    // (out16, the next projection's operand); either output may be null
+    void forward_mixed(float *out32, half *out16, const float *src, const float *skip, int num,
+                       et::stream_t stream = nullptr) const {
+        etChk(et_skip_layernorm_mixed(out32, reinterpret_cast<et_f16 *>(out16), src, skip,
+                                      reinterpret_cast<const et_f16 *>(weight.get()),
+                                      reinterpret_cast<const et_f16 *>(bias.get()), num, size, eps, stream));
+    }
     int width() const { return size; }
     const half *gamma() const { return weight.get(); }
     const half *beta() const { return bias.get(); }

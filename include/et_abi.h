@@ -28,7 +28,7 @@ extern "C" {
 typedef uint16_t et_f16;  /* IEEE binary16 bit pattern */
 typedef void *et_stream;  /* hipStream_t; NULL = the null stream */
 typedef void *et_event;   /* hipEvent_t */
-typedef void *et_graph;   /* an instantiated HIP graph (hipGraphExec_t) */
+typedef void *et_graph;   /* a captured HIP graph with its executable instance (opaque) */
 
 enum et_status {
     ET_OK = 0,
@@ -107,6 +107,17 @@ int et_linear_bsr16_f16(const int32_t *row_ptr, const int32_t *col_idx,
                         const et_f16 *tiles, const et_f16 *bias,
                         const et_f16 *X, et_f16 *Y, int T, int in, int out,
                         int act, et_stream stream);
+
+/* et_linear_bsr16_f16 with the result stored as binary32 [T x out]: the fp32
+ * accumulator after bias and activation, unrounded (Y 16-byte aligned).  The
+ * projections that feed a SkipLayerNorm use it in the mixed-precision layer
+ * (fp16 matrix-core operands, fp32 residual stream); the reference's mixed
+ * kernels (Attention/mixed-precision/mixed_attn.cu:10-124) widen only the
+ * score accumulation. */
+int et_linear_bsr16_f16_f32out(const int32_t *row_ptr, const int32_t *col_idx,
+                               const et_f16 *tiles, const et_f16 *bias,
+                               const et_f16 *X, float *Y, int T, int in, int out,
+                               int act, et_stream stream);
 
 /* SkipLayerNorm fused into the tile-sparse Linear that consumes it:
  *   ln_out = LayerNorm(src + skip) * gamma + beta      (written, [T x in])
@@ -385,6 +396,17 @@ int et_skip_layernorm_f16(et_f16 *out, const et_f16 *src, const et_f16 *skip,
                           const et_f16 *gamma, const et_f16 *beta, int rows,
                           int H, float eps, et_stream stream);
 
+/* Mixed-precision SkipLayerNorm: src and skip are binary32 [rows x H] (a
+ * projection's unrounded output and the residual stream), gamma and beta the
+ * model's binary16 parameters; the result is written as binary32 to out32 (the
+ * next residual) and, rounded once, as binary16 to out16 (the next
+ * projection's operand).  Either output may be NULL.  Same statistics as
+ * et_skip_layernorm_f16 (SkipLayerNorm/SkipLayerNorm.cu:22-63). */
+int et_skip_layernorm_mixed(float *out32, et_f16 *out16, const float *src,
+                            const float *skip, const et_f16 *gamma,
+                            const et_f16 *beta, int rows, int H, float eps,
+                            et_stream stream);
+
 /* out[r] = LayerNorm(src[r]) * gamma + beta.
  * Replaces LayerNorm::forward (LayerNorm/LayerNorm.cu:51-57). */
 int et_layernorm_f16(et_f16 *out, const et_f16 *src, const et_f16 *gamma,
@@ -447,6 +469,11 @@ typedef struct et_model_desc {
     float eps;     /* LayerNorm epsilon; <= 0 selects 1e-5                        */
     int causal;    /* != 0: causal mask (the reference's hard-wired one)          */
     int use_graph; /* != 0: replay a captured HIP graph; 0: launch kernel by kernel */
+    int mixed;     /* != 0: mixed precision — the residual stream (layer inputs, the two
+                    * projections that feed a SkipLayerNorm, both SkipLayerNorm results)
+                    * is kept in binary32 inside the stack, binary16 only as matrix-core
+                    * operands; input and output of et_model_forward stay binary16.
+                    * 0: every activation is stored as binary16 (the reference's storage) */
 } et_model_desc;
 
 /* which matrix of a layer */

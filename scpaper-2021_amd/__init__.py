@@ -62,6 +62,8 @@ _SIGNATURES = {
     "et_event_sync": (_vp,),
     "et_event_elapsed_ms": (C.POINTER(_f), _vp, _vp),
     "et_linear_bsr16_f16": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_linear_bsr16_f16_f32out": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_skip_layernorm_mixed": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp),
     "et_linear_bsr16_f16_geom": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp),
     "et_skipln_linear_bsr16_f16": (_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_linear_bsr16_fused_ln_supported": (_i, _i, _i),
@@ -138,7 +140,7 @@ W_QKV, W_O, W_FF1, W_FF2 = 0, 1, 2, 3
 
 class ModelDesc(C.Structure):
     _fields_ = [("kdim", _i), ("vdim", _i), ("seq_len", _i), ("nhead", _i), ("dimFF", _i), ("emdim", _i),
-                ("nlayer", _i), ("batch", _i), ("act", _i), ("eps", _f), ("causal", _i), ("use_graph", _i)]
+                ("nlayer", _i), ("batch", _i), ("act", _i), ("eps", _f), ("causal", _i), ("use_graph", _i), ("mixed", _i)]
 _RESTYPES = {"et_status_string": C.c_char_p, "et_last_error": C.c_char_p}
 
 _lib = None
@@ -322,8 +324,9 @@ class Model:
     """Encoder stack assembled from host weights; forward replays one HIP graph."""
 
     def __init__(self, H, nh, dimFF, S, nlayer, batch=1, act=ACT_GELU, eps=1e-5, causal=False, use_graph=True,
-                 handle=None):
-        self.desc = ModelDesc(H, H, S, nh, dimFF, H, nlayer, batch, act, eps, int(causal), int(use_graph))
+                 handle=None, mixed=False):
+        self.desc = ModelDesc(H, H, S, nh, dimFF, H, nlayer, batch, act, eps, int(causal), int(use_graph),
+                              int(mixed))
         self.rows, self.H = batch * S, H
         if handle is None:
             h = _vp()

@@ -58,6 +58,9 @@ struct BsrArgs {
     // of squares) of (Y as stored + resid) over the features of this workgroup.
     const _Float16 *resid;
     float *st_out;
+    // binary32 result: when set, act(acc + bias) is stored here unrounded (16 bytes per lane)
+    // and Y is not written — the mixed-precision layer keeps its residual stream in fp32
+    float *Y32;
 };
 
 constexpr int kFxNorm = 1;
@@ -413,6 +416,13 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
                         st1[m] += v;
                         st2[m] = __builtin_fmaf(v, v, st2[m]);
                     }
+                } else if (a.Y32) {  // wave-uniform (a kernel argument)
+                    f4 o32;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) o32[j] = act_fixed<ACT>(acc[m][j] + (float)bv[j]);
+                    *reinterpret_cast<f4 *>(a.Y32 + (size_t)tok * a.out + f0) = o32;
+                    acc[m] = f4{0.f, 0.f, 0.f, 0.f};
+                    continue;
                 } else {
 #pragma unroll
                     for (int j = 0; j < 4; j++) o[j] = (_Float16)act_fixed<ACT>(acc[m][j] + (float)bv[j]);
@@ -527,6 +537,9 @@ static BsrPlan plan_bsr(int T, int in, int out) {
         int rpw = (nbr + groups - 1) / groups;
         if (rpw < 8) rpw = 8;
         if (rpw > nbr) rpw = nbr;
+        // a wave keeps one block-row's [lo, hi) per lane: at most kMaxWaveRows block-rows per wave
+        const int cap = kMaxWaveRows * (p.threads / 64);
+        if (rpw > cap) rpw = cap;
         p.rows_per_wg = rpw;
         p.lds = 0;
         return p;
@@ -669,6 +682,9 @@ static int dispatch_bsr_res(const BsrArgs &args, const BsrPlan &p, hipStream_t s
 }
 
 static int dispatch_bsr(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
+    ET_REQUIRE(p.rows_per_wg >= 1 && p.rows_per_wg <= kMaxWaveRows * (p.threads / 64), ET_ERR_UNSUPPORTED,
+               "tile-sparse Linear: %d block-rows per workgroup of %d waves exceed %d per wave", p.rows_per_wg,
+               p.threads / 64, kMaxWaveRows);
     if (p.stage) {
         switch (p.mt) {
             case 4: return launch_bsr<4, true>(args, p, stream);
@@ -720,6 +736,30 @@ int et_linear_bsr16_f16(const int32_t *row_ptr, const int32_t *col_idx, const et
                  0,
                  act,
                  nullptr, nullptr, nullptr, nullptr, nullptr, 0.0f, nullptr, 0, nullptr, nullptr};
+    BsrPlan p = plan_bsr(T, in, out);
+    args.rows_per_wg = p.rows_per_wg;
+    return dispatch_bsr(args, p, as_stream(stream));
+}
+
+int et_linear_bsr16_f16_f32out(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles,
+                               const et_f16 *bias, const et_f16 *X, float *Y, int T, int in, int out,
+                               int act, et_stream stream) {
+    int s = bsr_check(row_ptr, col_idx, tiles, X, reinterpret_cast<et_f16 *>(Y), T, in, out, act);
+    if (s != ET_OK) return s;
+    ET_REQUIRE((reinterpret_cast<uintptr_t>(Y) & 15) == 0, ET_ERR_UNSUPPORTED,
+               "et_linear_bsr16_f16_f32out: Y must be 16-byte aligned");
+    if (T == 0) return ET_OK;
+    BsrArgs args{};
+    args.row_ptr = row_ptr;
+    args.col_idx = col_idx;
+    args.tiles = reinterpret_cast<const _Float16 *>(tiles);
+    args.bias = reinterpret_cast<const _Float16 *>(bias);
+    args.X = reinterpret_cast<const _Float16 *>(X);
+    args.T = T;
+    args.in = in;
+    args.out = out;
+    args.act = act;
+    args.Y32 = Y;
     BsrPlan p = plan_bsr(T, in, out);
     args.rows_per_wg = p.rows_per_wg;
     return dispatch_bsr(args, p, as_stream(stream));

@@ -123,6 +123,77 @@ __global__ __launch_bounds__(kWave *kRowsPerBlock) void layernorm_rows_kernel(
     }
 }
 
+// Mixed-precision SkipLayerNorm: the residual stream (src = a projection's fp32 output, skip = the
+// fp32 residual) stays binary32 end to end; the result is written twice, as binary32 (the next
+// residual) and rounded to binary16 (the operand the next projection's matrix cores read).
+// gamma and beta are the model's binary16 parameters.  Same structure as layernorm_rows_kernel.
+template <int NIT>
+__global__ __launch_bounds__(kWave *kRowsPerBlock) void skip_layernorm_mixed_kernel(
+    float *__restrict__ out32, _Float16 *__restrict__ out16, const float *__restrict__ src,
+    const float *__restrict__ skip, const _Float16 *__restrict__ gamma, const _Float16 *__restrict__ beta,
+    int rows, int H, float eps) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int row = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int chunks = H >> 2;
+    const float4 *s = reinterpret_cast<const float4 *>(src + (size_t)row * H);
+    const float4 *k = reinterpret_cast<const float4 *>(skip + (size_t)row * H);
+    const uint2 *g = reinterpret_cast<const uint2 *>(gamma);
+    const uint2 *b = reinterpret_cast<const uint2 *>(beta);
+    float4 rs[NIT], rk[NIT];
+    uint2 rg[NIT], rb[NIT];
+#pragma unroll
+    for (int i = 0; i < NIT; i++) {
+        const int c = min(lane + kWave * i, chunks - 1);
+        rs[i] = s[c];
+        rk[i] = k[c];
+        rg[i] = g[c];
+        rb[i] = b[c];
+    }
+    float x[NIT][4];
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NIT; i++) {
+        const bool ok = lane + kWave * i < chunks;
+        float y[4];
+        unpack4(rs[i], x[i]);
+        unpack4(rk[i], y);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            x[i][j] = ok ? x[i][j] + y[j] : 0.0f;
+            sum += x[i][j];
+        }
+    }
+    const float inv_h = 1.0f / (float)H;
+    const float mean = wave_sum(sum) * inv_h;
+    float sq = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NIT; i++) {
+        const bool ok = lane + kWave * i < chunks;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float d = ok ? x[i][j] - mean : 0.0f;
+            sq += d * d;
+        }
+    }
+    const float rstd = rsqrtf(wave_sum(sq) * inv_h + eps);
+    float4 *o32 = out32 ? reinterpret_cast<float4 *>(out32 + (size_t)row * H) : nullptr;
+    uint2 *o16 = out16 ? reinterpret_cast<uint2 *>(out16 + (size_t)row * H) : nullptr;
+#pragma unroll
+    for (int i = 0; i < NIT; i++) {
+        const int c = lane + kWave * i;
+        if (c < chunks) {
+            float gg[4], bb[4], y[4];
+            unpack4(rg[i], gg);
+            unpack4(rb[i], bb);
+#pragma unroll
+            for (int j = 0; j < 4; j++) y[j] = (x[i][j] - mean) * rstd * gg[j] + bb[j];
+            if (o32) o32[c] = float4{y[0], y[1], y[2], y[3]};
+            if (o16) o16[c] = pack4(y);
+        }
+    }
+}
+
 // out = normalisation of V + skip with the row statistics a producer kernel left behind: the
 // stand-alone form of the NORM prologue of the tile-sparse Linear (same arithmetic, same bits).
 __global__ __launch_bounds__(256) void norm_from_stats_kernel(_Float16 *__restrict__ out,
@@ -176,6 +247,33 @@ static int launch_layernorm(T *out, const T *src, const T *skip, const T *gamma,
     }
 #undef ET_LN_CASE
     return check_launch("layernorm_rows_kernel");
+}
+
+static int launch_skip_layernorm_mixed(float *out32, _Float16 *out16, const float *src, const float *skip,
+                                       const _Float16 *gamma, const _Float16 *beta, int rows, int H, float eps,
+                                       hipStream_t stream) {
+    const int chunks = H / 4;
+    const int nit = (chunks + kWave - 1) / kWave;
+    const dim3 grid((rows + kRowsPerBlock - 1) / kRowsPerBlock), block(kWave * kRowsPerBlock);
+#define ET_LNM_CASE(N)                                                                                       \
+    case N:                                                                                                  \
+        skip_layernorm_mixed_kernel<N><<<grid, block, 0, stream>>>(out32, out16, src, skip, gamma, beta, rows, H, \
+                                                                   eps);                                     \
+        break;
+    switch (nit) {
+        ET_LNM_CASE(1) ET_LNM_CASE(2) ET_LNM_CASE(3) ET_LNM_CASE(4)
+        ET_LNM_CASE(5) ET_LNM_CASE(6) ET_LNM_CASE(7) ET_LNM_CASE(8)
+        default:
+            if (nit <= 16) {
+                skip_layernorm_mixed_kernel<16><<<grid, block, 0, stream>>>(out32, out16, src, skip, gamma, beta,
+                                                                            rows, H, eps);
+            } else {
+                skip_layernorm_mixed_kernel<32><<<grid, block, 0, stream>>>(out32, out16, src, skip, gamma, beta,
+                                                                            rows, H, eps);
+            }
+    }
+#undef ET_LNM_CASE
+    return check_launch("skip_layernorm_mixed_kernel");
 }
 
 static int check_ln_args(const char *fn, const void *out, const void *src, const void *gamma,
@@ -248,6 +346,19 @@ int et_layernorm_f32(float *out, const float *src, const float *gamma, const flo
     if (s != ET_OK) return s;
     if (rows == 0) return ET_OK;
     return launch_layernorm<false, float>(out, src, nullptr, gamma, beta, rows, H, eps, as_stream(stream));
+}
+
+int et_skip_layernorm_mixed(float *out32, et_f16 *out16, const float *src, const float *skip,
+                            const et_f16 *gamma, const et_f16 *beta, int rows, int H, float eps,
+                            et_stream stream) {
+    int s = check_ln_args("et_skip_layernorm_mixed", out32 ? (const void *)out32 : (const void *)out16, src, gamma,
+                          beta, rows, H);
+    if (s != ET_OK) return s;
+    ET_REQUIRE(skip != nullptr, ET_ERR_INVALID_ARG, "et_skip_layernorm_mixed: skip is NULL");
+    if (rows == 0) return ET_OK;
+    return launch_skip_layernorm_mixed(out32, reinterpret_cast<_Float16 *>(out16), src, skip,
+                                       reinterpret_cast<const _Float16 *>(gamma),
+                                       reinterpret_cast<const _Float16 *>(beta), rows, H, eps, as_stream(stream));
 }
 
 }  // extern "C"

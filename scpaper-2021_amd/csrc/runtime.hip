@@ -1,6 +1,8 @@
 // Device buffers, streams, events, fills and fp32<->fp16 conversion behind the
 // C ABI, plus the status/error plumbing shared by every entry point.
 #include <stdarg.h>
+
+#include <new>
 #include <string.h>
 
 #include "common.hip.h"
@@ -214,6 +216,14 @@ int et_graph_begin_capture(et_stream stream) {
     return ET_OK;
 }
 
+// An et_graph keeps the captured template together with its executable instance and destroys
+// them in that order (instance first) at et_graph_destroy: the instance is never left referring
+// to a template that is already gone.
+struct GraphPair {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
 int et_graph_end_capture(et_stream stream, et_graph *graph) {
     ET_REQUIRE(stream != nullptr && graph != nullptr, ET_ERR_INVALID_ARG,
                "et_graph_end_capture: NULL argument");
@@ -222,21 +232,39 @@ int et_graph_end_capture(et_stream stream, et_graph *graph) {
     ET_HIP(hipStreamEndCapture(as_stream(stream), &g));
     hipGraphExec_t exec = nullptr;
     int s = check_hip(hipGraphInstantiate(&exec, g, nullptr, nullptr, 0), "hipGraphInstantiate");
-    (void)hipGraphDestroy(g);
-    if (s != ET_OK) return s;
-    *graph = exec;
+    if (s != ET_OK) {
+        (void)hipGraphDestroy(g);
+        return s;
+    }
+    GraphPair *pair = new (std::nothrow) GraphPair;
+    if (!pair) {
+        (void)hipGraphExecDestroy(exec);
+        (void)hipGraphDestroy(g);
+        return fail(ET_ERR_ALLOC, "et_graph_end_capture: out of host memory");
+    }
+    pair->graph = g;
+    pair->exec = exec;
+    *graph = pair;
     return ET_OK;
 }
 
 int et_graph_launch(et_graph graph, et_stream stream) {
     ET_REQUIRE(graph != nullptr, ET_ERR_INVALID_ARG, "et_graph_launch: graph is NULL");
-    ET_HIP(hipGraphLaunch(reinterpret_cast<hipGraphExec_t>(graph), as_stream(stream)));
+    ET_HIP(hipGraphLaunch(static_cast<GraphPair *>(graph)->exec, as_stream(stream)));
     return ET_OK;
 }
 
 int et_graph_destroy(et_graph graph) {
     if (!graph) return ET_OK;
-    ET_HIP(hipGraphExecDestroy(reinterpret_cast<hipGraphExec_t>(graph)));
+    GraphPair *pair = static_cast<GraphPair *>(graph);
+    // replays still in flight hold the instance's kernel arguments: drain before it goes
+    hipError_t e0 = hipDeviceSynchronize();
+    hipError_t e1 = hipGraphExecDestroy(pair->exec);
+    hipError_t e2 = hipGraphDestroy(pair->graph);
+    delete pair;
+    ET_HIP(e0);
+    ET_HIP(e1);
+    ET_HIP(e2);
     return ET_OK;
 }
 

@@ -18,6 +18,8 @@ using et::stream_t;
 struct ILayer {
     virtual ~ILayer() = default;
     virtual void forward(half *out, half *src, stream_t stream) = 0;
+    virtual void enable_mixed() = 0;
+    virtual void forward_mixed(float *out32, half *out16, const float *src32, half *src16, stream_t stream) = 0;
     virtual et::AttnState &attn() = 0;
 };
 
@@ -25,6 +27,10 @@ template <typename EncoderT> struct LayerOf final : ILayer {
     std::unique_ptr<EncoderT> enc;
     explicit LayerOf(std::unique_ptr<EncoderT> e) : enc(std::move(e)) {}
     void forward(half *out, half *src, stream_t stream) override { enc->forward(out, src, stream); }
+    void enable_mixed() override { enc->enable_mixed(); }
+    void forward_mixed(float *out32, half *out16, const float *src32, half *src16, stream_t stream) override {
+        enc->forward_mixed(out32, out16, src32, src16, stream);
+    }
     et::AttnState &attn() override { return enc->attention(); }
 };
 
@@ -56,6 +62,8 @@ struct et_model_s {
     std::vector<HostLayer> host;
     std::vector<std::unique_ptr<ILayer>> layers;
     std::unique_ptr<et::DeviceBuffer<half>> pp[2];
+    std::unique_ptr<et::DeviceBuffer<float>> pp32[2];  // mixed precision: the residual stream between layers
+    std::unique_ptr<et::DeviceBuffer<half>> warm;      // result of the eager pass that precedes a capture
     std::vector<int> lens;   // empty = no padding
     std::vector<half> mask;  // empty = no additive mask
     bool finalized = false;
@@ -144,7 +152,26 @@ void check_layer_index(const et_model_s *m, int layer) {
     et::require(layer >= 0 && layer < m->desc.nlayer, "et_model: layer index out of range");
 }
 
+// Mixed precision: the binary16 input is widened once, every layer hands the next one its result
+// in both forms (binary32 residual, binary16 operand), the last one writes binary16 to `out`.
+void run_layers_mixed(et_model_s &m, half *out, half *in, stream_t stream) {
+    const int n = (int)m.layers.size();
+    const std::size_t elems = (std::size_t)m.rows() * m.desc.emdim;
+    etChk(et_f16_to_f32(m.pp32[1]->get(), et::f16(in), elems, stream));
+    const float *src32 = m.pp32[1]->get();
+    half *src16 = in;
+    for (int i = 0; i < n; i++) {
+        const bool last = i == n - 1;
+        float *dst32 = last ? nullptr : m.pp32[i % 2]->get();
+        half *dst16 = last ? out : m.pp[i % 2]->get();
+        m.layers[(size_t)i]->forward_mixed(dst32, dst16, src32, src16, stream);
+        src32 = dst32;
+        src16 = dst16;
+    }
+}
+
 void run_layers(et_model_s &m, half *out, half *in, stream_t stream) {
+    if (m.desc.mixed) return run_layers_mixed(m, out, in, stream);
     const int n = (int)m.layers.size();
     half *src = in;
     for (int i = 0; i < n; i++) {
@@ -311,6 +338,12 @@ int et_model_finalize(et_model m) {
         const size_t act_elems = (size_t)m->rows() * m->desc.emdim;
         m->pp[0] = std::make_unique<et::DeviceBuffer<half>>(act_elems);
         m->pp[1] = std::make_unique<et::DeviceBuffer<half>>(act_elems);
+        m->warm = std::make_unique<et::DeviceBuffer<half>>(act_elems);
+        if (m->desc.mixed) {
+            m->pp32[0] = std::make_unique<et::DeviceBuffer<float>>(act_elems);
+            m->pp32[1] = std::make_unique<et::DeviceBuffer<float>>(act_elems);
+            for (auto &l : m->layers) l->enable_mixed();
+        }
         etChk(et_stream_create(&m->own_stream));
         apply_attention_state(*m);
         m->host.clear();
@@ -325,8 +358,14 @@ int et_model_forward_layer(et_model m, int layer, et_f16 *out, const et_f16 *in,
         check_layer_index(m, layer);
         et::require(m->finalized, "et_model_forward_layer: call et_model_finalize first");
         et::require(out && in, "et_model_forward_layer: NULL pointer");
-        m->layers[(size_t)layer]->forward(reinterpret_cast<half *>(out),
-                                          reinterpret_cast<half *>(const_cast<et_f16 *>(in)), stream);
+        half *o = reinterpret_cast<half *>(out);
+        half *i = reinterpret_cast<half *>(const_cast<et_f16 *>(in));
+        if (m->desc.mixed) {  // one layer between binary16 buffers: the residual starts from the binary16 input
+            etChk(et_f16_to_f32(m->pp32[1]->get(), in, (std::size_t)m->rows() * m->desc.emdim, stream));
+            m->layers[(size_t)layer]->forward_mixed(nullptr, o, m->pp32[1]->get(), i, stream);
+        } else {
+            m->layers[(size_t)layer]->forward(o, i, stream);
+        }
         return ET_OK;
     });
 }
@@ -343,10 +382,12 @@ int et_model_forward(et_model m, et_f16 *out, const et_f16 *in, et_stream stream
             return ET_OK;
         }
         if (!m->graph || m->graph_in != in || m->graph_out != out) {
-            // (Re)capture for this pair of buffers.  The first eager pass runs
-            // every kernel once outside capture (lazy one-time kernel setup).
+            // (Re)capture for this pair of buffers.  An eager pass first runs every kernel once
+            // outside capture (lazy one-time kernel setup); its result goes to a buffer of the
+            // model's own, so that a caller who normalises in place (out == in) still has the
+            // untouched input when the graph runs.
             m->drop_graph();
-            run_layers(*m, o, i, s);
+            run_layers(*m, m->warm->get(), i, s);
             etChk(et_stream_sync(s));
             etChk(et_graph_begin_capture(s));
             try {

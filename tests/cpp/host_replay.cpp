@@ -62,6 +62,7 @@ struct Case {
     float sparsity;
     int act, use_graph;
     bool lens;
+    int mixed = 0;
 };
 
 void run_case(const Case &c, uint64_t seed) {
@@ -75,6 +76,7 @@ void run_case(const Case &c, uint64_t seed) {
     d.act = c.act;
     d.eps = 1e-5f;
     d.use_graph = c.use_graph;
+    d.mixed = c.mixed;
     et_model m = nullptr;
     OK(et_model_create(&d, &m));
     if (!m) return;
@@ -100,6 +102,7 @@ void run_case(const Case &c, uint64_t seed) {
     OK(et_malloc(&out2, bytes));
     for (int rep = 0; rep < 3; rep++) OK(et_model_forward(m, (et_f16 *)out, (const et_f16 *)in, nullptr));
     OK(et_model_forward(m, (et_f16 *)out2, (const et_f16 *)in, nullptr));  // other buffers: recapture
+    OK(et_model_forward(m, (et_f16 *)out2, (const et_f16 *)out2, nullptr)); // in place
     OK(et_model_set_lens(m, lens.data()));
     OK(et_model_forward(m, (et_f16 *)out, (const et_f16 *)in, nullptr));
     std::vector<et_f16> mask((size_t)c.S * c.S, 0);
@@ -179,6 +182,8 @@ int main(int argc, char **argv) {
         {128, 2, 256, 32, 2, 1, 0.5f, ET_ACT_GELU, 1, false},   // recapture for new buffers and lengths
         {256, 4, 512, 48, 1, 3, 0.7f, ET_ACT_RELU, 1, false},   // layer by layer (QKV: 230 tiles)
         {768, 12, 3072, 128, 8, 2, 0.8f, ET_ACT_GELU, 1, false},  // headline shape, two layers
+        {128, 2, 256, 32, 2, 3, 0.5f, ET_ACT_GELU, 1, true, 1},    // mixed precision, graph
+        {256, 4, 512, 48, 1, 1, 0.7f, ET_ACT_RELU, 0, false, 1},   // mixed precision, one layer, eager
     };
     uint64_t seed = 4000;
     for (const Case &c : cases) run_case(c, seed += 100);

@@ -55,10 +55,12 @@ class BsrWeight:
                  dead_block_cols=()):
         self.out, self.inp = out, inp
         self._pattern_args = (out, inp, sparsity, seed, tuple(dead_block_rows), tuple(dead_block_cols))
-        self.row_ptr, self.col_idx = self._pattern()
-        # The structure is frozen the moment it exists: numpy refuses any later write through
-        # these arrays, and the digest taken here is compared again at every hand-over to the
-        # library (check_tile_pattern), so a change made behind numpy's back cannot go unseen.
+        # The index arrays live in anonymous mappings of their own, outside the malloc heap (see
+        # isolated()).  The structure is frozen the moment it exists: numpy refuses any later
+        # write through these arrays, and the digest taken here is compared again at every
+        # hand-over to the library (check_tile_pattern), so a change made behind numpy's back
+        # cannot go unseen.
+        self.row_ptr, self.col_idx = (isolated(a) for a in self._pattern())
         bc = inp // 16
         assert len(self.col_idx) == 0 or (self.col_idx.min() >= 0 and self.col_idx.max() < bc), \
             "pattern generator produced a column tile outside the matrix"
@@ -199,6 +201,22 @@ def run_layer_case(et, H, nh, dimFF, S, B, sparsity, seed, lens=None, nlayers=1,
     return max_abs(got, want)
 
 
+def isolated(arr: np.ndarray) -> np.ndarray:
+    """Copy of an index array in an anonymous private mapping of its own (whole pages, fresh from
+    the kernel, never part of the malloc heap).  Twice a run of the GPU suite found a pattern
+    changed after generation: two 8-byte words of a 920-byte numpy buffer, 736 bytes apart, each
+    lower by exactly 6 — what decrements of a counter through dangling pointers into a freed and
+    recycled heap block look like (both addresses were former 16-byte-aligned allocations with
+    the word at offset 8).  This library has no such counter and its host code is clean under
+    AddressSanitizer, so the writer is another component of the process; small numpy buffers come
+    from the recycled heap, a private mapping cannot be the target of a pointer into it."""
+    import mmap
+    mm = mmap.mmap(-1, max(arr.nbytes, 1))
+    out = np.frombuffer(mm, dtype=arr.dtype, count=arr.size)
+    out[...] = arr
+    return out
+
+
 def pattern_digest(row_ptr, col_idx) -> str:
     return hashlib.sha1(row_ptr.tobytes() + col_idx.tobytes()).hexdigest()
 
@@ -222,11 +240,11 @@ def check_tile_pattern(bw, what):
         f"(owns its data: {bw.col_idx.flags.owndata}, writeable: {bw.col_idx.flags.writeable})")
 
 
-def build_model(et, layers, S, B, act=2, lens=None, use_graph=True, causal=False, eps=1e-5):
+def build_model(et, layers, S, B, act=2, lens=None, use_graph=True, causal=False, eps=1e-5, mixed=False):
     """Encoder stack through et_model_* from a list of LayerWeights (exact fp16 bits)."""
     w0 = layers[0]
     m = et.Model(w0.H, w0.nh, w0.dimFF, S, len(layers), batch=B, act=act, eps=eps, causal=causal,
-                 use_graph=use_graph)
+                 use_graph=use_graph, mixed=mixed)
     for i, w in enumerate(layers):
         for which, bw in ((et.W_QKV, w.qkv), (et.W_O, w.o), (et.W_FF1, w.l1), (et.W_FF2, w.l2)):
             check_tile_pattern(bw, f"layer {i} matrix {which}")
@@ -239,7 +257,9 @@ def build_model(et, layers, S, B, act=2, lens=None, use_graph=True, causal=False
     return m
 
 
-def oracle_stack(x, layers, B, lens=None, act="gelu", causal=False, eps=1e-5, store=torch.float16):
+def oracle_stack(x, layers, B, lens=None, act="gelu", causal=False, eps=1e-5, store=torch.float16, resid="same"):
+    """store=None: the fp32 mathematics; store=float16: fp16 at the engine's storage points;
+    store=float16 with resid=float32: the engine's mixed-precision mode."""
     cfg = L.LayerConfig(nh=layers[0].nh, B=B, act=act, eps=eps, causal=causal,
-                        lens=None if lens is None else torch.as_tensor(np.asarray(lens)), store=store)
+                        lens=None if lens is None else torch.as_tensor(np.asarray(lens)), store=store, resid=resid)
     return L.encoder_stack(f32(x), [w.oracle_params() for w in layers], cfg).numpy()

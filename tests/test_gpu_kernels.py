@@ -61,6 +61,27 @@ def test_skip_layernorm(et, rows, H):
     assert Hn.max_abs(d_out.numpy(), want.numpy()) <= 4e-3
 
 
+@pytest.mark.parametrize("rows,H", [(1024, 768), (2048, 1024), (128, 800), (7, 64), (5, 4100)])
+def test_skip_layernorm_mixed(et, rows, H):
+    """binary32 in (a projection's output and the residual), binary32 and binary16 out."""
+    src, skip = Hn.randn((rows, H), 1, 0.5, np.float32), Hn.randn((rows, H), 2, 1.0, np.float32)
+    gamma = (1 + Hn.randn((H,), 3, 0.1, np.float32)).astype(np.float16)
+    beta = Hn.randn((H,), 4, 0.1)
+    d32, d16 = et.DeviceBuffer.empty((rows, H), np.float32), et.DeviceBuffer.empty((rows, H), np.float16)
+    args = (up(et, src).ptr, up(et, skip).ptr, up(et, gamma).ptr, up(et, beta).ptr, rows, H, 1e-5, None)
+    et.check(et.lib().et_skip_layernorm_mixed(d32.ptr, d16.ptr, *args))
+    want = L.skip_layernorm(Hn.f32(src), Hn.f32(skip), Hn.f32(gamma), Hn.f32(beta), 1e-5, None).numpy()
+    assert want.dtype == np.float32
+    got32, got16 = d32.numpy(), d16.numpy()
+    assert Hn.max_abs(got32, want) <= 2e-5          # fp32 statistics on both sides
+    assert np.array_equal(got16, got32.astype(np.float16))  # the operand copy is the rounded residual
+    # either output alone
+    e32, e16 = et.DeviceBuffer.empty((rows, H), np.float32), et.DeviceBuffer.empty((rows, H), np.float16)
+    et.check(et.lib().et_skip_layernorm_mixed(e32.ptr, None, *args))
+    et.check(et.lib().et_skip_layernorm_mixed(None, e16.ptr, *args))
+    assert np.array_equal(e32.numpy(), got32) and np.array_equal(e16.numpy(), got16)
+
+
 @pytest.mark.parametrize("rows,H", [(1024, 768), (16, 1024), (3, 800)])
 def test_layernorm(et, rows, H):
     src = Hn.randn((rows, H), 5, 2.0)
@@ -126,6 +147,12 @@ BSR_CASES = [
     (1040, 768, 768, 0.8, 1),
     (16, 768, 3072, 0.8, 0),
     (80, 3072, 768, 0.8, 2),
+    # the 90 % rows of the tile-sparse Linear configuration at 2048 token rows
+    (2048, 768, 3072, 0.9, 0),
+    (2048, 3072, 768, 0.9, 0),
+    # unstaged strips (input too wide for LDS) with more block-rows per workgroup than one wave
+    # can own before the cap: 320 block-rows, 4 waves
+    (16384, 5120, 5120, 0.98, 0),
 ]
 
 
@@ -141,6 +168,35 @@ def test_linear_bsr16(et, T, inp, out, sp, act):
     print(f"bsr T={T} in={inp} out={out} sp={sp}: ntile={len(w.col_idx)} max-abs={err:.2e}")
     # |y| stays below ~4 here: one fp16 rounding (<= 2e-3) plus accumulation-order noise
     assert err <= 4e-3
+
+
+@pytest.mark.parametrize("T,inp,out,sp,act", [(1024, 768, 768, 0.8, 0), (1024, 3072, 768, 0.8, 0), (2048, 4096, 1024, 0.9, 0),
+                                              (48, 64, 32, 0.3, 2), (64, 6144, 64, 0.5, 1), (4096, 768, 3072, 0.8, 2)])
+def test_linear_bsr16_f32_output(et, T, inp, out, sp, act):
+    """The binary32 store of the accumulator (mixed-precision residual stream): no rounding of
+    the result, so the bound is accumulation-order noise only; and rounding it gives the
+    binary16 entry point's result bit for bit."""
+    w = Hn.BsrWeight(out, inp, sp, seed=21, bias_std=0.1).upload(et)
+    x = Hn.randn((T, inp), 22)
+    d_x = up(et, x)
+    d_y32 = et.DeviceBuffer.empty((T, out), np.float32)
+    d_y16 = et.DeviceBuffer.empty((T, out), np.float16)
+    et.check(et.lib().et_linear_bsr16_f16_f32out(w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, w.d_bias.ptr,
+                                                 d_x.ptr, d_y32.ptr, T, inp, out, act, None))
+    w.forward(et, d_x, d_y16, T, act)
+    want = L.linear(Hn.f32(x), Hn.f32(w.dense), Hn.f32(w.bias), {0: None, 1: "relu", 2: "gelu"}[act], None).numpy()
+    got = d_y32.numpy()
+    assert Hn.max_abs(got, want) <= 5e-5 * max(1.0, float(np.abs(want).max()))
+    a, b = got.astype(np.float16), d_y16.numpy()
+    if act != 2:
+        assert np.array_equal(a, b)
+    else:
+        # tanh-GELU is evaluated by two instantiations of the epilogue, whose fused multiply-adds
+        # the compiler may contract differently: the last binary32 bit, hence rarely the binary16
+        # rounding, can differ — by one unit in the last place at most
+        ulp = np.spacing(np.maximum(np.abs(a), np.abs(b)).astype(np.float16)).astype(np.float32)
+        assert np.all(np.abs(a.astype(np.float32) - b.astype(np.float32)) <= ulp)
+        assert np.mean(a != b) < 1e-3
 
 
 def test_linear_bsr16_closed_form_all_ones(et):
