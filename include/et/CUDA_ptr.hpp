@@ -1,13 +1,12 @@
 // Device buffer with value semantics — the role culib::CUDA_ptr<T> plays in the
 // reference (lib/CUDA_ptr.hpp:10-69), over et_malloc/et_free of the C ABI:
 //   DeviceBuffer(n)            n zero-filled elements
-//   DeviceBuffer(ptr, n)       copy of n elements from a host pointer
+//   DeviceBuffer(ptr, n)       copy of n elements from a host or a device pointer
 //   DeviceBuffer(vector)       copy of a host vector
 //   DeviceBuffer(n, value)     n elements set to value
 //   copy = deep device-to-device copy, move = steal; get/size/dump/clear/set.
-// Unlike the reference, the pointer constructor takes HOST memory only (HIP has
-// no cudaMemcpyDefault-style inference through this ABI); use the copy
-// constructor or from_device() for device sources.
+// As in the reference (cudaMemcpyDefault, lib/CUDA_ptr.hpp:18-31) the pointer
+// constructor takes host or device memory: the runtime tells them apart by the address.
 #pragma once
 #include <cstddef>
 #include <type_traits>
@@ -26,9 +25,9 @@ template <typename T> class DeviceBuffer {
 
     DeviceBuffer() = delete;
     explicit DeviceBuffer(std::size_t n) : size(n) { etChk(et_malloc(&raw_, bytes())); }
-    DeviceBuffer(const T *host, std::size_t n) : size(n) {
+    DeviceBuffer(const T *host_or_device, std::size_t n) : size(n) {
         etChk(et_malloc(&raw_, bytes()));
-        etChk(et_memcpy_h2d(raw_, host, bytes()));
+        etChk(et_memcpy_auto(raw_, host_or_device, bytes()));
     }
     DeviceBuffer(const std::vector<T> &host) : DeviceBuffer(host.data(), host.size()) {}
     DeviceBuffer(std::size_t n, T value) : size(n) {

@@ -201,6 +201,9 @@ template <> class Linear<csr_mat> {
     Linear(int _in_size, int _out_size, const csr_mat &w, const half *b, int _size)
         : in_size(_in_size), out_size(_out_size), size(_size), bias(b, (std::size_t)_out_size) {
         et::require(w.nrow == _out_size && w.ncol == _in_size, "Linear<csr_mat>: weight shape mismatch");
+        // both paths below (the dense image and the CSR kernel, which indexes its LDS strip with the
+        // column ids) rely on a consistent structure
+        et::fmt::validate_csr(w.indptr, w.indices, w.data.size(), w.nrow, w.ncol);
         std::vector<half> h(w.data.size());
         for (std::size_t i = 0; i < h.size(); i++) h[i] = static_cast<half>(w.data[i]);
         indptr = std::make_unique<et::DeviceBuffer<int>>(w.indptr);

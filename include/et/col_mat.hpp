@@ -31,14 +31,23 @@ class col_mat {
         if (!f) throw et::Error(ET_ERR_IO, "cannot open " + filename);
         int32_t meta[3];
         f.read(reinterpret_cast<char *>(meta), sizeof meta);
+        if (!f) throw et::Error(ET_ERR_IO, filename + ": truncated header");
         nrow = meta[0];
         ncol = meta[1];
         nnz_col = meta[2];
+        f.seekg(0, std::ios::end);
+        const std::size_t file_bytes = (std::size_t)f.tellg();
+        f.seekg(12, std::ios::beg);
+        if (nrow <= 0 || ncol <= 0 || nnz_col < 0 || nnz_col > ncol || file_bytes < 12 + 4 * (std::size_t)nnz_col ||
+            (nnz_col > 0 && (file_bytes - 12 - 4 * (std::size_t)nnz_col) / 4 / (std::size_t)nnz_col < (std::size_t)nrow))
+            throw et::Error(ET_ERR_IO, filename + ": header does not match the file size");
         std::vector<int> ids((std::size_t)nnz_col);
         std::vector<float> vals((std::size_t)nrow * nnz_col);
         f.read(reinterpret_cast<char *>(ids.data()), (std::streamsize)(ids.size() * 4));
         f.read(reinterpret_cast<char *>(vals.data()), (std::streamsize)(vals.size() * 4));
         if (!f) throw et::Error(ET_ERR_IO, filename + ": truncated");
+        for (int id : ids)
+            if (id < 0 || id >= ncol) throw et::Error(ET_ERR_IO, filename + ": column id outside the matrix");
         std::vector<half> h(vals.size());
         for (std::size_t i = 0; i < h.size(); i++) h[i] = static_cast<half>(vals[i]);
         col_id = std::make_unique<et::DeviceBuffer<int>>(ids);

@@ -48,6 +48,11 @@ std::vector<float> bsr16_to_dense(const int *row_ptr, const int *column, const f
 void validate_bsr16(const std::vector<int> &row_ptr, const std::vector<int> &column,
                     std::size_t ntile, int blk_col_num);
 
+// CSR consistency: indptr[nrow+1] starting at 0 and non-decreasing, indptr.back() == index count
+// == value count, every column inside [0, ncol).  Throws et::Error otherwise.
+void validate_csr(const std::vector<int> &indptr, const std::vector<int> &indices, std::size_t ndata, int nrow,
+                  int ncol);
+
 // row_mat::gen_sparse_mat ids (mat_type/row_mat/row_mat.cu:14-25): ascending.
 std::vector<int> gen_row_ids(int nrow, float sparsity, uint64_t seed);
 // col_mat::gen_sparse_mat ids (mat_type/col_mat/col_mat.cu:22-32): permuted order.

@@ -25,14 +25,25 @@ class row_mat {
         if (!f) throw et::Error(ET_ERR_IO, "cannot open " + filename);
         uint32_t meta[3];
         f.read(reinterpret_cast<char *>(meta), sizeof meta);
+        if (!f) throw et::Error(ET_ERR_IO, filename + ": truncated header");
         nrow = (int)meta[0];
         ncol = (int)meta[1];
         const std::size_t len = meta[2];
+        // the header must describe the file: counts that do not fit its size are refused before
+        // anything is allocated from them
+        f.seekg(0, std::ios::end);
+        const std::size_t file_bytes = (std::size_t)f.tellg();
+        f.seekg(12, std::ios::beg);
+        if (nrow <= 0 || ncol <= 0 || len > (std::size_t)nrow ||
+            file_bytes < 12 + 4 * len || (file_bytes - 12 - 4 * len) / 4 / (std::size_t)ncol < len)
+            throw et::Error(ET_ERR_IO, filename + ": header does not match the file size");
         std::vector<int> ids(len);
         std::vector<float> vals(len * (std::size_t)ncol);
         f.read(reinterpret_cast<char *>(ids.data()), (std::streamsize)(ids.size() * 4));
         f.read(reinterpret_cast<char *>(vals.data()), (std::streamsize)(vals.size() * 4));
         if (!f) throw et::Error(ET_ERR_IO, filename + ": truncated");
+        for (int id : ids)
+            if (id < 0 || id >= nrow) throw et::Error(ET_ERR_IO, filename + ": row id outside the matrix");
         std::vector<half> h(vals.size());
         for (std::size_t i = 0; i < h.size(); i++) h[i] = static_cast<half>(vals[i]);
         row_id = std::make_unique<et::DeviceBuffer<int>>(ids);

@@ -66,6 +66,9 @@ int et_memset(void *ptr, int byte, size_t bytes, et_stream stream);
 int et_memcpy_h2d(void *dst, const void *src_host, size_t bytes);
 int et_memcpy_d2h(void *dst_host, const void *src, size_t bytes);
 int et_memcpy_d2d(void *dst, const void *src, size_t bytes, et_stream stream);
+/* dst device; src host OR device memory, told apart by the address, like the
+ * cudaMemcpyDefault copy of CUDA_ptr(ptr, n) (lib/CUDA_ptr.hpp:18-31).  Blocking. */
+int et_memcpy_auto(void *dst, const void *src, size_t bytes);
 int et_fill_f16(et_f16 *dst, size_t n, et_f16 value, et_stream stream);
 int et_fill_i32(int32_t *dst, size_t n, int32_t value, et_stream stream);
 int et_f32_to_f16(et_f16 *dst, const float *src, size_t n, et_stream stream); /* RN-even */

@@ -48,6 +48,7 @@ _SIGNATURES = {
     "et_memcpy_h2d": (_vp, _vp, _sz),
     "et_memcpy_d2h": (_vp, _vp, _sz),
     "et_memcpy_d2d": (_vp, _vp, _sz, _vp),
+    "et_memcpy_auto": (_vp, _vp, _sz),
     "et_fill_f16": (_vp, _sz, _u16, _vp),
     "et_fill_i32": (_vp, _sz, C.c_int32, _vp),
     "et_f32_to_f16": (_vp, _vp, _sz, _vp),

@@ -42,6 +42,7 @@ struct MhaArgs {
     // for the full-width columns v_col_id[.] (all inside head h's slice of Z).
     const int32_t *v_col_id;
     const int32_t *v_head_ptr;
+    int v_nnz = 0;  // entries of v_col_id (> 0 in the compact-V form)
 };
 
 constexpr int kXcds = 8;                // accelerator dies, each with a private L2
@@ -157,7 +158,8 @@ __global__ __launch_bounds__(64 * NW)
     if (COMPACT) {
 #pragma unroll
         for (int i = 0; i < kCid; i++)
-            my_cid[i] = a.v_col_id[vc0 + min((int)threadIdx.x + i * nthr, max(vlive - 1, 0))];
+            // clamped into the array also for a head without surviving columns that sits at its end
+            my_cid[i] = a.v_col_id[min(vc0 + min((int)threadIdx.x + i * nthr, max(vlive - 1, 0)), a.v_nnz - 1)];
     }
 
     // Q fragments: B operand, lane supplies Q[q][32*ks + 8g .. +7]
@@ -646,7 +648,12 @@ int et_mha_compactv_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *Vc, int 
                "et_mha_compactv_f16: row strides must keep 16-byte alignment");
     ET_REQUIRE((long long)B * nh * (S / 16) < (1LL << 30), ET_ERR_UNSUPPORTED, "et_mha_compactv_f16: grid too large");
     if (B == 0) return ET_OK;
+    if (nnz_col == 0) {  // every V column pruned: Z is zero
+        ET_REQUIRE(ldz == nh * vhd, ET_ERR_UNSUPPORTED, "et_mha_compactv_f16: nnz_col = 0 needs a contiguous Z");
+        return et_fill_f16(Z, (size_t)B * S * ldz, 0, stream);
+    }
     MhaArgs args;
+    args.v_nnz = nnz_col;
     args.Q = reinterpret_cast<const _Float16 *>(Q);
     args.K = reinterpret_cast<const _Float16 *>(K);
     args.V = reinterpret_cast<const _Float16 *>(Vc);

@@ -148,6 +148,14 @@ int et_memcpy_d2h(void *dst_host, const void *src, size_t bytes) {
     return ET_OK;
 }
 
+int et_memcpy_auto(void *dst, const void *src, size_t bytes) {
+    ET_REQUIRE((dst && src) || bytes == 0, ET_ERR_INVALID_ARG, "et_memcpy_auto: NULL pointer");
+    if (bytes == 0) return ET_OK;
+    // the runtime tells host from device memory by the address (unified addressing)
+    ET_HIP(hipMemcpy(dst, src, bytes, hipMemcpyDefault));
+    return ET_OK;
+}
+
 int et_memcpy_d2d(void *dst, const void *src, size_t bytes, et_stream stream) {
     ET_REQUIRE((dst && src) || bytes == 0, ET_ERR_INVALID_ARG, "et_memcpy_d2d: NULL pointer");
     if (bytes == 0) return ET_OK;

@@ -118,6 +118,17 @@ void validate_bsr16(const std::vector<int> &row_ptr, const std::vector<int> &col
     }
 }
 
+void validate_csr(const std::vector<int> &indptr, const std::vector<int> &indices, std::size_t ndata, int nrow,
+                  int ncol) {
+    require(nrow >= 0 && ncol >= 0 && indptr.size() == (size_t)nrow + 1, "csr_mat: indptr must hold nrow + 1 entries");
+    require(indptr.front() == 0, "csr_mat: indptr must start at 0");
+    for (size_t i = 1; i < indptr.size(); i++)
+        require(indptr[i] >= indptr[i - 1], "csr_mat: indptr must be non-decreasing");
+    require((size_t)indptr.back() == indices.size() && ndata == indices.size(),
+            "csr_mat: indptr.back(), the index count and the value count must agree");
+    for (int c : indices) require(c >= 0 && c < ncol, "csr_mat: column index out of range");
+}
+
 std::vector<int> gen_row_ids(int nrow, float sparsity, uint64_t seed) {
     int nn = kept_count(nrow, sparsity);
     nn = ((nn / 16) + ((nn % 16) != 0)) * 16;
@@ -260,6 +271,13 @@ Csr read_csr(const std::string &path) {
     m.nrow = (int)head[0];
     m.ncol = (int)head[1];
     m.nnz = (int)head[2];
+    // the header must describe the file before anything is sized from it
+    f.seekg(0, std::ios::end);
+    const uint64_t file_bytes = (uint64_t)f.tellg();
+    f.seekg(12, std::ios::beg);
+    if (m.nrow < 0 || m.ncol < 0 || m.nnz < 0 ||
+        file_bytes != 12 + 4 * ((uint64_t)head[0] + 1) + 8 * (uint64_t)head[2])
+        throw Error(ET_ERR_IO, path + ": header does not match the file size");
     m.indptr.resize((size_t)m.nrow + 1);
     m.indices.resize((size_t)m.nnz);
     m.data.resize((size_t)m.nnz);
@@ -267,6 +285,7 @@ Csr read_csr(const std::string &path) {
     f.read(reinterpret_cast<char *>(m.indices.data()), (std::streamsize)(m.indices.size() * 4));
     f.read(reinterpret_cast<char *>(m.data.data()), (std::streamsize)(m.data.size() * 4));
     if (!f) throw Error(ET_ERR_IO, path + ": truncated body");
+    validate_csr(m.indptr, m.indices, m.data.size(), m.nrow, m.ncol);
     return m;
 }
 

@@ -103,8 +103,17 @@ Array parse_npy(const char *buf, std::size_t len, const std::string &what) {
         a.shape.push_back((std::size_t)std::stoull(shape.substr(i, e - i)));
         i = e;
     }
-    const std::size_t nbytes = a.num_vals() * a.word_size;
-    if (hoff + hlen + nbytes > len) bad(what, "npy data shorter than its shape");
+    // the element count times the word size must not wrap: a shape whose product overflows would
+    // pass the length test below
+    const std::size_t avail = len - hoff - hlen;
+    if (a.word_size == 0 || a.word_size > 16) bad(what, "unsupported element size");
+    std::size_t count = 1;
+    for (std::size_t d : a.shape) {
+        if (d != 0 && count > avail / d) bad(what, "npy data shorter than its shape");
+        count *= d;
+    }
+    if (count > avail / a.word_size) bad(what, "npy data shorter than its shape");
+    const std::size_t nbytes = count * a.word_size;
     a.bytes.assign(buf + hoff + hlen, buf + hoff + hlen + nbytes);
     return a;
 }
@@ -157,36 +166,47 @@ npz_t npz_load(const std::string &path) {
         // zip64: locator sits right before the end record
         if (eocd < 20 || rd32(p + eocd - 20) != 0x07064b50u) bad(path, "zip64 locator missing");
         const uint64_t e64 = rd64(p + eocd - 20 + 8);
-        if (e64 + 56 > n || rd32(p + e64) != 0x06064b50u) bad(path, "zip64 end record missing");
+        if (e64 > n || n - e64 < 56 || rd32(p + e64) != 0x06064b50u) bad(path, "zip64 end record missing");
         entries = rd64(p + e64 + 32);
         cd_off = rd64(p + e64 + 48);
     }
     npz_t out;
+    if (cd_off > n) bad(path, "zip central directory lies outside the file");
     std::size_t pos = (std::size_t)cd_off;
     for (uint64_t e = 0; e < entries; e++) {
-        if (pos + 46 > n || rd32(p + pos) != 0x02014b50u) bad(path, "zip central directory is corrupt");
+        if (pos > n || n - pos < 46 || rd32(p + pos) != 0x02014b50u) bad(path, "zip central directory is corrupt");
         const uint16_t method = rd16(p + pos + 10);
         uint64_t csize = rd32(p + pos + 20), usize = rd32(p + pos + 24);
         const uint16_t nlen = rd16(p + pos + 28), xlen = rd16(p + pos + 30), clen = rd16(p + pos + 32);
         uint64_t lho = rd32(p + pos + 42);
+        // name, extra field and comment of this entry must lie inside the file
+        if (n - pos - 46 < (std::size_t)nlen + xlen + clen) bad(path, "zip central directory is corrupt");
         std::string name(file.data() + pos + 46, nlen);
         // zip64 extra field (id 1): the 64-bit values appear for each 32-bit field that is saturated
         std::size_t x = pos + 46 + nlen;
         const std::size_t xend = x + xlen;
         while (x + 4 <= xend) {
             const uint16_t id = rd16(p + x), sz = rd16(p + x + 2);
+            if (x + 4 + (std::size_t)sz > xend) bad(path, "zip extra field is corrupt");
             if (id == 0x0001) {
                 std::size_t q = x + 4;
-                if (usize == 0xFFFFFFFFu) { usize = rd64(p + q); q += 8; }
-                if (csize == 0xFFFFFFFFu) { csize = rd64(p + q); q += 8; }
-                if (lho == 0xFFFFFFFFu) { lho = rd64(p + q); q += 8; }
+                const std::size_t qend = x + 4 + sz;
+                auto take64 = [&](uint64_t &v) {
+                    if (q + 8 > qend) bad(path, "zip64 extra field is too short");
+                    v = rd64(p + q);
+                    q += 8;
+                };
+                if (usize == 0xFFFFFFFFu) take64(usize);
+                if (csize == 0xFFFFFFFFu) take64(csize);
+                if (lho == 0xFFFFFFFFu) take64(lho);
             }
             x += 4 + (std::size_t)sz;
         }
         pos = xend + clen;
-        if (lho + 30 > n || rd32(p + lho) != 0x04034b50u) bad(path, "zip local header is corrupt");
+        if (lho > n || n - lho < 30 || rd32(p + lho) != 0x04034b50u) bad(path, "zip local header is corrupt");
         const std::size_t data = (std::size_t)lho + 30 + rd16(p + lho + 26) + rd16(p + lho + 28);
-        if (data + csize > n) bad(path, "zip member runs past the end of the file");
+        if (data > n || csize > n - data) bad(path, "zip member runs past the end of the file");
+        if (usize > ((uint64_t)1 << 40)) bad(path, "zip member claims an implausible size");
         std::vector<char> raw;
         if (method == 0) {
             raw.assign(file.data() + data, file.data() + data + csize);

@@ -7,6 +7,11 @@
 //   fused_attn    FusedAttention<NOTF_fused_attn> with the W_VO built by et::build_vo_weight
 //   fused_prune   FusedAttention<NOTF_fused_prune_attn> over a column-pruned W_VO
 //   factories     the gen_* test factories: closed forms of the reference drivers
+//   attn_variants Attention<> with separate Q/K/V projections under the tags OTF_attn_full,
+//                 OTF_attn_full_mixed, OTF_attn_Ofused (tile-sparse) and Norm_attn (dense)
+//   encoder_fuse  Encoder_fuse<NOTF_fused_attn> (pre-computed VO attention + tile-sparse FFN), in both
+//                 the all-fp16 and the mixed-precision form
+//   file_ctors    row_mat / col_mat / csr_mat built from their raw files
 #include <algorithm>
 #include <cstdio>
 #include <cstring>
@@ -260,9 +265,170 @@ static int run_factories(const std::string &dir) {
         c.clear();
         out.push_back(first_value(c));                                  // 0
         out.push_back((float)(a.get() == nullptr));                     // 1: moved-from
+        // the pointer constructor takes device memory as well as host memory (lib/CUDA_ptr.hpp:18-31)
+        et::DeviceBuffer<half> src(8, static_cast<half>(7.0f));
+        et::DeviceBuffer<half> from_dev(src.get(), 8);
+        src.set(static_cast<half>(1.0f));
+        out.push_back(first_value(from_dev, 5));                        // 7 (copied, not aliased)
+        const std::vector<half> host8(8, static_cast<half>(6.0f));
+        et::DeviceBuffer<half> from_host(host8.data(), 8);
+        out.push_back(first_value(from_host, 5));                       // 6
     }
     etChk(et_device_sync());
     npy_save(dir + "/factories.npy", out.data(), "<f4", 4, {out.size()});
+    return 0;
+}
+
+// ---- Attention<> with separate projections under every tag that has not been built elsewhere ------
+template <typename MAT, typename tag>
+static void run_attn_variant(const std::string &dir, const std::string &out_name, bool as_f32 = false) {
+    using attn_config = Attention_config<MAT, MAT, MAT, MAT, tag, false, true>;
+    const auto meta = read_meta(dir);  // H seq nhead batch
+    const int H = meta[0], S = meta[1], nh = meta[2], batch = meta[3], rows = batch * S;
+    auto para = std::make_shared<Model_t>(Model_t{H, H, S, nh, 4 * H, H, 1});
+    auto make = [&](const std::string &t) {
+        auto b = load_half(dir + "/b" + t + ".npy");
+        if constexpr (std::is_same<MAT, tile_mat>::value) {
+            auto W = npy_load(dir + "/W" + t + ".npy").as_vector<float>();
+            return std::make_unique<Linear<tile_mat>>(H, H, tile_mat::from_dense(W.data(), H, H), b.data(), rows);
+        } else {
+            auto W = load_half(dir + "/W" + t + ".npy");
+            return std::make_unique<Linear<base_mat>>(H, H, base_mat(W), b.data(), rows);
+        }
+    };
+    Attention<attn_config> attn(make("q"), make("k"), make("v"), make("o"), para, batch);
+    auto lens = load_int(dir + "/lens.npy");
+    attn.set_lens(lens.data());
+    et::DeviceBuffer<half> X(load_half(dir + "/input.npy")), OUT((std::size_t)rows * H);
+    if (as_f32) {
+        if constexpr (!std::is_same<tag, OTF_attn_Ofused>::value) {
+            et::DeviceBuffer<float> OUT32((std::size_t)rows * H);
+            et::DeviceBuffer<half> scratch((std::size_t)rows * H);
+            attn.forward_f32(OUT32.get(), X.get(), X.get(), X.get(), scratch.get());
+            etChk(et_device_sync());
+            auto f = OUT32.to_host();
+            npy_save(dir + "/" + out_name, f.data(), "<f4", 4, {(std::size_t)rows, (std::size_t)H});
+        }
+        return;
+    }
+    attn.forward(OUT.get(), X.get(), X.get(), X.get());
+    etChk(et_device_sync());
+    save_half(dir + "/" + out_name, OUT, (std::size_t)rows, (std::size_t)H);
+}
+
+static int run_attn_variants(const std::string &dir) {
+    run_attn_variant<tile_mat, OTF_attn_full>(dir, "out_full.npy");
+    run_attn_variant<tile_mat, OTF_attn_full_mixed>(dir, "out_full_mixed.npy");
+    run_attn_variant<tile_mat, OTF_attn_Ofused>(dir, "out_ofused.npy");
+    run_attn_variant<tile_mat, OTF_attn>(dir, "out_otf.npy");
+    run_attn_variant<base_mat, Norm_attn>(dir, "out_norm.npy");
+    run_attn_variant<tile_mat, OTF_attn_full>(dir, "out_full_f32.npy", true);   // binary32 output projection
+    run_attn_variant<base_mat, OTF_attn_full>(dir, "out_dense_f32.npy", true);  // widened binary16 projection
+    // the free function of Attention/kernel_fuseO.h:6-9 called directly on Q = K = V = input
+    {
+        const auto meta = read_meta(dir);
+        const int H = meta[0], S = meta[1], nh = meta[2], batch = meta[3], rows = batch * S;
+        auto para = std::make_shared<Model_t>(Model_t{H, H, S, nh, 4 * H, H, 1});
+        auto Wo = npy_load(dir + "/Wo.npy").as_vector<float>();
+        tile_mat wo = tile_mat::from_dense(Wo.data(), H, H);
+        et::DeviceBuffer<half> bo(load_half(dir + "/bo.npy"));
+        et::DeviceBuffer<half> X(load_half(dir + "/input.npy")), Z((std::size_t)rows * H), OUT((std::size_t)rows * H);
+        et::AttnRun run;
+        run.batch = batch;
+        Multihead_atttion_fuseO(X.get(), X.get(), X.get(), nullptr, Z.get(), wo.row_ptr.get(), wo.row_offset.get(),
+                                wo.data.get(), bo.get(), para, OUT.get(), run);
+        etChk(et_device_sync());
+        save_half(dir + "/out_fuseO_free.npy", OUT, (std::size_t)rows, (std::size_t)H);
+    }
+    return 0;
+}
+
+// ---- Encoder_fuse (Encoder/Encoder.h:99-139) ------------------------------------------------------
+static int run_encoder_fuse(const std::string &dir) {
+    using attn_config = Attention_config<base_mat, base_mat, base_mat, base_mat, NOTF_fused_attn, false, true>;
+    const auto meta = read_meta(dir);  // H seq nhead batch FF
+    const int H = meta[0], S = meta[1], nh = meta[2], batch = meta[3], FF = meta[4], rows = batch * S;
+    auto para = std::make_shared<Model_t>(Model_t{H, H, S, nh, FF, H, 1});
+    auto build = [&]() {
+        auto dense_linear = [&](const std::string &t) {
+            auto W = load_half(dir + "/W" + t + ".npy");
+            auto b = load_half(dir + "/b" + t + ".npy");
+            return std::make_unique<Linear<base_mat>>(H, H, base_mat(W), b.data(), rows);
+        };
+        auto Wv = npy_load(dir + "/Wv.npy").as_vector<float>(), bv = npy_load(dir + "/bv.npy").as_vector<float>();
+        auto Wo = npy_load(dir + "/Wo.npy").as_vector<float>();
+        std::vector<float> Wvo, bvo;
+        et::build_vo_weight(Wv.data(), bv.data(), Wo.data(), H, H, H, nh, Wvo, bvo);
+        auto LVO = std::make_unique<Linear_VO>(et::DeviceBuffer<half>(vec_F2H(Wvo)), et::DeviceBuffer<half>(vec_F2H(bvo)), para);
+        et::DeviceBuffer<half> biasO(load_half(dir + "/bo.npy"));
+        auto attn = std::make_unique<FusedAttention<attn_config>>(dense_linear("q"), dense_linear("k"), std::move(LVO), biasO,
+                                                                 para, batch);
+        auto lens = load_int(dir + "/lens.npy");
+        attn->set_lens(lens.data());
+        auto ln = [&](const std::string &t) {
+            return std::make_unique<SkipLayerNorm>(load_half(dir + "/g" + t + ".npy").data(),
+                                                   load_half(dir + "/be" + t + ".npy").data(), H);
+        };
+        auto W1 = npy_load(dir + "/W1.npy").as_vector<float>(), W2 = npy_load(dir + "/W2.npy").as_vector<float>();
+        auto L1 = std::make_unique<Linear<tile_mat>>(H, FF, tile_mat::from_dense(W1.data(), FF, H),
+                                                     load_half(dir + "/b1.npy").data(), rows);
+        auto L2 = std::make_unique<Linear<tile_mat>>(FF, H, tile_mat::from_dense(W2.data(), H, FF),
+                                                     load_half(dir + "/b2.npy").data(), rows);
+        return std::make_unique<Encoder_fuse<attn_config>>(std::move(attn), ln("1"), ln("2"), std::move(L1), std::move(L2),
+                                                           para);
+    };
+    auto enc = build();
+    et::DeviceBuffer<half> X(load_half(dir + "/input.npy")), OUT((std::size_t)rows * H);
+    enc->forward(OUT.get(), X.get());
+    etChk(et_device_sync());
+    save_half(dir + "/out.npy", OUT, (std::size_t)rows, (std::size_t)H);
+    // mixed precision: binary32 residual stream around the same sublayers
+    enc->enable_mixed();
+    et::DeviceBuffer<float> X32((std::size_t)rows * H), OUT32((std::size_t)rows * H);
+    etChk(et_f16_to_f32(X32.get(), et::f16(X.get()), (std::size_t)rows * H, nullptr));
+    enc->forward_mixed(OUT32.get(), OUT.get(), X32.get(), X.get());
+    etChk(et_device_sync());
+    auto f = OUT32.to_host();
+    npy_save(dir + "/out_mixed32.npy", f.data(), "<f4", 4, {(std::size_t)rows, (std::size_t)H});
+    save_half(dir + "/out_mixed16.npy", OUT, (std::size_t)rows, (std::size_t)H);
+    return 0;
+}
+
+// ---- raw-file constructors (row_mat.hpp:15-29, col_mat.hpp:22-36, csr_mat.h:19-35) ------------------
+static int run_file_ctors(const std::string &dir) {
+    auto save_ints = [&](const std::string &name, const std::vector<int> &v) {
+        npy_save(dir + "/" + name, v.data(), "<i4", 4, {v.size()});
+    };
+    auto save_halfs = [&](const std::string &name, const std::vector<half> &h) {
+        std::vector<float> f(h.size());
+        for (std::size_t i = 0; i < h.size(); i++) f[i] = static_cast<float>(h[i]);
+        npy_save(dir + "/" + name, f.data(), "<f4", 4, {f.size()});
+    };
+    row_mat r(dir + "/small.row");
+    save_ints("row_meta.npy", {r.nrow, r.ncol, r.nnz_row()});
+    save_ints("row_id.npy", r.row_id->to_host());
+    save_halfs("rows.npy", r.rows->to_host());
+    col_mat c(dir + "/small.col");
+    save_ints("col_meta.npy", {c.nrow, c.ncol, c.nnz_col, c.ldm});
+    save_ints("col_id.npy", c.col_id->to_host());
+    save_halfs("cols.npy", c.cols->to_host());
+    csr_mat m(dir + "/small.csr");
+    save_ints("csr_meta.npy", {m.nrow, m.ncol, m.nnz});
+    save_ints("csr_indptr.npy", m.indptr);
+    save_ints("csr_indices.npy", m.indices);
+    npy_save(dir + "/csr_data.npy", m.data.data(), "<f4", 4, {m.data.size()});
+    // damaged headers are refused
+    int refused = 0;
+    for (const char *name : {"/bad.row", "/bad.col", "/bad.csr"}) {
+        try {
+            if (std::string(name) == "/bad.row") row_mat bad(dir + name);
+            else if (std::string(name) == "/bad.col") col_mat bad(dir + name);
+            else csr_mat bad(dir + name);
+        } catch (const et::Error &e) {
+            if (e.status() == ET_ERR_IO) refused++;
+        }
+    }
+    save_ints("refused.npy", {refused});
     return 0;
 }
 
@@ -278,6 +444,9 @@ int main(int argc, char **argv) {
         if (which == "fused_attn") return run_fused<NOTF_fused_attn>(dir);
         if (which == "fused_prune") return run_fused<NOTF_fused_prune_attn>(dir);
         if (which == "factories") return run_factories(dir);
+        if (which == "attn_variants") return run_attn_variants(dir);
+        if (which == "encoder_fuse") return run_encoder_fuse(dir);
+        if (which == "file_ctors") return run_file_ctors(dir);
         std::fprintf(stderr, "unknown case %s\n", which.c_str());
         return 2;
     } catch (const et::Error &e) {

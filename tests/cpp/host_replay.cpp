@@ -9,6 +9,9 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <filesystem>
+#include <fstream>
+#include <iterator>
 #include <string>
 #include <vector>
 
@@ -173,6 +176,59 @@ void load_archives(const std::string &dir) {
     OK(et_free(out));
 }
 
+// Damaged archives must be refused with a status, never read out of bounds: the first archive
+// of the model is truncated at many lengths and has single bytes of its zip directory, local
+// header and npy header overwritten; every variant goes through et_model_load.
+void corrupt_archives(const std::string &dir) {
+    namespace fs = std::filesystem;
+    const fs::path work = fs::path(dir) / "damaged";
+    fs::create_directories(work);
+    for (const auto &e : fs::directory_iterator(dir))
+        if (e.is_regular_file()) fs::copy_file(e.path(), work / e.path().filename(), fs::copy_options::overwrite_existing);
+    std::ifstream list((work / "weights.txt").string());
+    std::string first;
+    std::getline(list, first);
+    const fs::path victim = work / first;
+    std::ifstream in(victim.string(), std::ios::binary);
+    const std::vector<char> good((std::istreambuf_iterator<char>(in)), std::istreambuf_iterator<char>());
+    EXPECT(good.size() > 200);
+    et_model_desc d{};
+    d.kdim = d.vdim = d.emdim = 128;
+    d.seq_len = 32;
+    d.nhead = 2;
+    d.dimFF = 256;
+    d.nlayer = 2;
+    d.batch = 1;
+    d.act = ET_ACT_GELU;
+    int refused = 0, tried = 0;
+    auto attempt = [&](const std::vector<char> &bytes) {
+        std::ofstream out(victim.string(), std::ios::binary | std::ios::trunc);
+        out.write(bytes.data(), (std::streamsize)bytes.size());
+        out.close();
+        et_model m = nullptr;
+        const int s = et_model_load((work / "weights.txt").string().c_str(), (work.string() + "/").c_str(), &d, &m);
+        tried++;
+        if (s != ET_OK) refused++;
+        if (m) OK(et_model_destroy(m));
+    };
+    for (std::size_t cut : {std::size_t(0), std::size_t(10), std::size_t(21), std::size_t(22), std::size_t(45), good.size() / 3,
+                            good.size() / 2, good.size() - 100, good.size() - 23, good.size() - 22, good.size() - 1})
+        attempt(std::vector<char>(good.begin(), good.begin() + (std::ptrdiff_t)std::min(cut, good.size())));
+    uint64_t rng = 0x9E3779B97F4A7C15ull;
+    for (int k = 0; k < 400; k++) {
+        rng = rng * 6364136223846793005ull + 1442695040888963407ull;
+        std::vector<char> bad = good;
+        // half of the hits in the last 400 bytes (central directory and end record), the rest anywhere
+        const std::size_t span = (k & 1) ? std::min<std::size_t>(400, bad.size()) : bad.size();
+        const std::size_t pos = bad.size() - 1 - (std::size_t)((rng >> 20) % span);
+        bad[pos] = (char)(rng >> 56);
+        if (k % 5 == 0) bad[(pos + 1) % bad.size()] = (char)0xFF;
+        attempt(bad);
+    }
+    EXPECT(refused >= 11);  // every truncation at least; damaged payload bytes may still load
+    printf("host_replay: %d damaged archives, %d refused\n", tried, refused);
+}
+
 }  // namespace
 
 int main(int argc, char **argv) {
@@ -188,7 +244,10 @@ int main(int argc, char **argv) {
     uint64_t seed = 4000;
     for (const Case &c : cases) run_case(c, seed += 100);
     error_paths();
-    if (argc > 1) load_archives(argv[1]);
+    if (argc > 1) {
+        load_archives(argv[1]);
+        corrupt_archives(argv[1]);
+    }
     if (g_failures) {
         fprintf(stderr, "host_replay: %d check(s) failed\n", g_failures);
         return 1;

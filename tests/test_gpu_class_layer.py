@@ -26,11 +26,13 @@ def run_case(case, d):
     return res
 
 
-def test_example_model_from_npz(tmp_path):
+@pytest.mark.parametrize("TEXT", [1024, 28800])
+def test_example_model_from_npz(tmp_path, TEXT):
     """Two ReLU encoder layers + decoder, the reference example's shape family (emdim 800 is not a
     multiple of the head size the kernels take, so 768 / 4 heads x 192 is not used either): H 512,
-    4 heads x 128, FFN 208, decoder 1024 wide, batch 2 x seq 64."""
-    H, nh, FF, S, B, TEXT, NL = 512, 4, 208, 64, 2, 1024, 2
+    4 heads x 128, FFN 208, batch 2 x seq 64; the decoder 1024 wide, and 28 800 wide as in the
+    reference example (example/main.cu:29,164)."""
+    H, nh, FF, S, B, NL = 512, 4, 208, 64, 2, 2
     layers = [Hn.LayerWeights(H, nh, FF, 0.6, seed=70 + i) for i in range(NL)]
     dec = Hn.BsrWeight(TEXT, H, 0.7, seed=90, bias_std=0.02)
     names = []
@@ -137,4 +139,81 @@ def test_factories_closed_forms(tmp_path):
     assert abs(ln - 0.2) < 1e-3
     # Linear<csr_mat>: dense-image path (80 %) and CSR-kernel path (99 %) both equal the CSR kernel called directly
     assert db[:4] == [1.0, 1.0, 1.0, 0.0]
-    assert db[4:] == [3.0, 4.0, 0.0, 1.0]
+    assert db[4:8] == [3.0, 4.0, 0.0, 1.0]
+    assert db[8:] == [7.0, 6.0]  # DeviceBuffer(ptr, n) from a device pointer and from a host pointer
+
+
+def test_attention_tags_with_separate_projections(tmp_path):
+    """Attention<> with separate Q/K/V projections under OTF_attn_full, OTF_attn_full_mixed, OTF_attn,
+    OTF_attn_Ofused (tile-sparse weights) and Norm_attn (dense weights, scores through memory), the
+    binary32-output form, and the free Multihead_atttion_fuseO: all the standard attention block."""
+    H, nh, S, B = 256, 4, 64, 2
+    W, b, x, lens = attention_inputs(tmp_path, H, nh, S, B, 130)
+    run_case("attn_variants", tmp_path)
+    st = torch.float16
+    lin = lambda t, inp, store=st: L.linear(inp, Hn.f32(W[t]), Hn.f32(b[t]), store=store)
+    xf = Hn.f32(x)
+    z = L.mha(lin("q", xf), lin("k", xf), lin("v", xf), nh, B, lens=lens, store=st)
+    want = lin("o", z).numpy()
+    full = np.load(tmp_path / "out_full.npy")
+    assert Hn.max_abs(full, want) <= 4e-3
+    for name in ("out_full_mixed.npy", "out_ofused.npy", "out_otf.npy"):
+        assert np.array_equal(np.load(tmp_path / name), full), name  # one fused kernel behind every on-the-fly tag
+    assert Hn.max_abs(np.load(tmp_path / "out_norm.npy"), want) <= 6e-3  # probabilities rounded to fp16 in memory
+    want32 = lin("o", z, None).numpy()
+    assert Hn.max_abs(np.load(tmp_path / "out_full_f32.npy"), want32) <= 1e-3
+    assert np.array_equal(np.load(tmp_path / "out_full_f32.npy").astype(np.float16), full.astype(np.float16))
+    assert Hn.max_abs(np.load(tmp_path / "out_dense_f32.npy"), want) <= 4e-3
+    # free function: attention over Q = K = V = x without projections, no padding, then the O projection
+    z0 = L.mha(xf, xf, xf, nh, B, store=st)
+    assert Hn.max_abs(np.load(tmp_path / "out_fuseO_free.npy"), lin("o", z0).numpy()) <= 6e-3
+
+
+def test_encoder_fuse_class(tmp_path):
+    """Encoder_fuse: pre-computed-VO attention, SkipLayerNorm, tile-sparse FFN with GELU — equals the
+    standard layer (the E.T. identity); and the same layer with a binary32 residual stream."""
+    H, nh, S, B, FF = 256, 4, 64, 2, 512
+    W, b, x, lens = attention_inputs(tmp_path, H, nh, S, B, 140)
+    w1 = Hn.BsrWeight(FF, H, 0.5, seed=141, bias_std=0.02)
+    w2 = Hn.BsrWeight(H, FF, 0.5, seed=142, bias_std=0.02)
+    g = {k: (1 + Hn.randn((H,), 143 + i, 0.1, np.float32)).astype(np.float16) for i, k in enumerate("12")}
+    be = {k: Hn.randn((H,), 146 + i, 0.1) for i, k in enumerate("12")}
+    for k in "12":
+        np.save(tmp_path / f"g{k}.npy", g[k].astype(np.float32))
+        np.save(tmp_path / f"be{k}.npy", be[k].astype(np.float32))
+    np.save(tmp_path / "W1.npy", w1.dense.astype(np.float32)); np.save(tmp_path / "b1.npy", w1.bias.astype(np.float32))
+    np.save(tmp_path / "W2.npy", w2.dense.astype(np.float32)); np.save(tmp_path / "b2.npy", w2.bias.astype(np.float32))
+    np.save(tmp_path / "meta.npy", np.array([H, S, nh, B, FF], np.int32))
+    run_case("encoder_fuse", tmp_path)
+    Wqkv = np.concatenate([W["q"], W["k"], W["v"]]); bqkv = np.concatenate([b["q"], b["k"], b["v"]])
+    P = L.LayerParams(Hn.f32(Wqkv), Hn.f32(bqkv), Hn.f32(W["o"]), Hn.f32(b["o"]), Hn.f32(w1.dense), Hn.f32(w1.bias),
+                      Hn.f32(w2.dense), Hn.f32(w2.bias), Hn.f32(g["1"]), Hn.f32(be["1"]), Hn.f32(g["2"]), Hn.f32(be["2"]))
+    cfg = lambda **kw: L.LayerConfig(nh=nh, B=B, act="gelu", lens=torch.as_tensor(lens), **kw)
+    want32 = L.encoder_layer(Hn.f32(x), P, cfg(store=None)).numpy()
+    # the VO form rounds different intermediates than the standard layer: both within the layer tolerance
+    assert Hn.max_abs(np.load(tmp_path / "out.npy"), want32) <= 2e-2
+    m32, m16 = np.load(tmp_path / "out_mixed32.npy"), np.load(tmp_path / "out_mixed16.npy")
+    assert Hn.max_abs(m32, want32) <= 1e-2
+    assert np.array_equal(m16.astype(np.float16), m32.astype(np.float16))
+
+
+def test_raw_file_constructors(tmp_path):
+    """row_mat(std::string), col_mat(std::string), csr_mat(std::string) on hand-written byte strings
+    (tests/golden/pruned_files.json) and on files whose header does not describe them."""
+    import json
+    g = json.loads((Path(__file__).resolve().parent / "golden" / "pruned_files.json").read_text())
+    raw = {k: bytes.fromhex(g[k]["hex"].replace(" ", "")) for k in ("row", "col", "csr")}
+    for k in raw:
+        (tmp_path / f"small.{k}").write_bytes(raw[k])
+        bad = bytearray(raw[k]); bad[8:12] = (100000).to_bytes(4, "little")  # len_id / nnz far beyond the file
+        (tmp_path / f"bad.{k}").write_bytes(bytes(bad))
+    run_case("file_ctors", tmp_path)
+    ld = lambda n: np.load(tmp_path / n)
+    r, c, s = g["row"], g["col"], g["csr"]
+    assert ld("row_meta.npy").tolist() == [r["nrow"], r["ncol"], 2] and ld("row_id.npy").tolist() == r["row_id"]
+    assert ld("rows.npy").tolist() == np.array(r["rows"]).ravel().tolist()
+    assert ld("col_meta.npy").tolist() == [c["nrow"], c["ncol"], 2, 2] and ld("col_id.npy").tolist() == c["col_id"]
+    assert ld("cols.npy").tolist() == np.array(c["cols"]).ravel().tolist()
+    assert ld("csr_meta.npy").tolist() == [2, 3, 3] and ld("csr_indptr.npy").tolist() == s["indptr"]
+    assert ld("csr_indices.npy").tolist() == s["indices"] and ld("csr_data.npy").tolist() == s["data"]
+    assert ld("refused.npy").tolist() == [3]

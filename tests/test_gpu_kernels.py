@@ -420,6 +420,43 @@ def run_mha(et, B, S, nh, hd, seed, lens=None, causal=False, mask=None, single_b
 
 
 @pytest.mark.parametrize("B", [1, 4, 16])
+def test_attention_block_dense_projections_padded(et, B):
+    """The fused self-attention block composed as a caller composes it: dense Q, K, V and O
+    projections (768 x 768, N(0, 0.02)) around the fused attention core, S128, 12 heads x 64,
+    inputs N(0,1), right padding with lengths in [64, 128] — against the oracle's attention block."""
+    H, nh, S = 768, 12, 128
+    T, hd = B * S, 64
+    g = Hn.rng(300 + B)
+    W = {k: (torch.randn(H, H, generator=g) * 0.02).numpy().astype(np.float16) for k in "qkvo"}
+    x = Hn.randn((T, H), 310 + B)
+    lens = torch.randint(64, 129, (B,), generator=Hn.rng(320 + B)).numpy().astype(np.int32)
+    d_x, d_lens = up(et, x), up(et, lens)
+    d = {k: et.DeviceBuffer.empty((T, H), np.float16) for k in ("q", "k", "v", "z", "out")}
+    for k in "qkv":
+        et.linear_dense(up(et, W[k]), None, d_x, d[k], T, H, H)
+    et.mha_fused(d["q"], d["k"], d["v"], H, H, H, d["z"], H, None, d_lens, B, S, nh, hd, 1.0 / math.sqrt(hd))
+    et.linear_dense(up(et, W["o"]), None, d["z"], d["out"], T, H, H)
+    Wqkv = np.concatenate([W["q"], W["k"], W["v"]])
+    zeros = torch.zeros
+    P = L.LayerParams(Hn.f32(Wqkv), zeros(3 * H), Hn.f32(W["o"]), zeros(H), None, None, None, None, None, None, None, None)
+    want16 = L.attention_block(Hn.f32(x), P, L.LayerConfig(nh=nh, B=B, lens=torch.as_tensor(lens), store=torch.float16))
+    want32 = L.attention_block(Hn.f32(x), P, L.LayerConfig(nh=nh, B=B, lens=torch.as_tensor(lens), store=None))
+    got = d["out"].numpy()
+    e16, e32 = Hn.max_abs(got, want16.numpy()), Hn.max_abs(got, want32.numpy())
+    print(f"attention block B={B} lens={lens.tolist()}: vs fp16-storage oracle {e16:.2e}, vs fp32 {e32:.2e}")
+    assert e16 <= 2e-3 and e32 <= 2e-2
+    # rows of padded queries are computed too (only keys are masked), and padding never leaks:
+    # each sequence alone gives the same rows
+    b = B - 1
+    d1 = {k: et.DeviceBuffer.empty((S, H), np.float16) for k in ("z", "out")}
+    off = b * S * H * 2
+    et.mha_fused(d["q"].offset(off), d["k"].offset(off), d["v"].offset(off), H, H, H, d1["z"], H, None,
+                 up(et, lens[b:b + 1]), 1, S, nh, hd, 1.0 / math.sqrt(hd))
+    et.linear_dense(up(et, W["o"]), None, d1["z"], d1["out"], S, H, H)
+    assert Hn.max_abs(d1["out"].numpy(), got[b * S:(b + 1) * S]) <= 1e-3
+
+
+@pytest.mark.parametrize("B", [1, 4, 16])
 def test_mha_block_config(et, B):
     """Attention core of the BERT-base block: S128, 12 heads x 64, right padding U{64..128}."""
     lens = torch.randint(64, 129, (B,), generator=Hn.rng(100 + B)).numpy()
