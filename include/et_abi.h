@@ -122,6 +122,30 @@ int et_linear_bsr16_f16_f32out(const int32_t *row_ptr, const int32_t *col_idx,
                                const et_f16 *X, float *Y, int T, int in, int out,
                                int act, et_stream stream);
 
+/* Tile-sparse Linear through a plan.  et_bsr16_plan_create re-orders the weight
+ * once (device pointers in the reference layout in, a device-side copy grouped by
+ * K chunk and workgroup out; blocking) for T token rows; the planned call then
+ * streams token strips and weight tiles through LDS chunk by chunk, which lifts
+ * the limit the plain call has on the input width and lets one weight tile serve
+ * 16*mt token rows.  mt (1, 2, 4, 8 sixteen-row blocks per strip), kc (128, 256,
+ * 512 columns per chunk) and rows_per_wg (block-rows per workgroup, at most 32)
+ * select the launch geometry; 0 picks it from T.  A plan may be used with any T
+ * that is a multiple of 16.  Exactly one of Y (binary16) and Y32 (binary32, the
+ * accumulator unrounded) is non-NULL.  Same results as et_linear_bsr16_f16 up to
+ * the order of the fp32 accumulation.  Replaces Linear<tile_mat>::forward
+ * (Linear/SPMM_tile.cu:312-324) for callers that keep a Linear object. */
+typedef struct et_bsr_plan_s *et_bsr_plan;
+int et_bsr16_plan_create(const int32_t *row_ptr, const int32_t *col_idx,
+                         const et_f16 *tiles, int T, int in, int out, int mt,
+                         int kc, int rows_per_wg, et_bsr_plan *plan);
+int et_bsr16_plan_destroy(et_bsr_plan plan);
+/* the geometry a plan was built with, and the LDS bytes of a workgroup */
+int et_bsr16_plan_info(et_bsr_plan plan, int *mt, int *kc, int *rows_per_wg,
+                       int *lds_bytes);
+int et_linear_bsr16_planned_f16(et_bsr_plan plan, const et_f16 *bias,
+                                const et_f16 *X, et_f16 *Y, float *Y32, int T,
+                                int act, et_stream stream);
+
 /* SkipLayerNorm fused into the tile-sparse Linear that consumes it:
  *   ln_out = LayerNorm(src + skip) * gamma + beta      (written, [T x in])
  *   Y      = act(ln_out * W^T + bias)

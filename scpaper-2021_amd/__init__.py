@@ -65,6 +65,10 @@ _SIGNATURES = {
     "et_linear_bsr16_f16": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_linear_bsr16_f16_f32out": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_skip_layernorm_mixed": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp),
+    "et_bsr16_plan_create": (_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, C.POINTER(_vp)),
+    "et_bsr16_plan_destroy": (_vp,),
+    "et_bsr16_plan_info": (_vp, C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)),
+    "et_linear_bsr16_planned_f16": (_vp, _vp, _vp, _vp, _vp, _i, _i, _vp),
     "et_linear_bsr16_f16_geom": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp),
     "et_skipln_linear_bsr16_f16": (_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_linear_bsr16_fused_ln_supported": (_i, _i, _i),

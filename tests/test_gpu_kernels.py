@@ -199,6 +199,80 @@ def test_linear_bsr16_f32_output(et, T, inp, out, sp, act):
         assert np.mean(a != b) < 1e-3
 
 
+PLANNED_CASES = [
+    # T, in, out, sparsity, act, (mt, kc, rows_per_wg) or None for the automatic geometry
+    (1024, 768, 2304, 0.8, 0, None),
+    (1024, 768, 768, 0.8, 0, None),
+    (1024, 768, 3072, 0.8, 2, None),
+    (1024, 3072, 768, 0.8, 0, None),
+    (2048, 4096, 1024, 0.9, 0, None),
+    (2048, 768, 3072, 0.9, 1, None),
+    (8192, 768, 768, 0.8, 2, None),       # 128-row strips
+    (128, 800, 208, 0.5, 1, None),        # widths that are no multiple of the chunk, 13 block-rows
+    (64, 6144, 64, 0.5, 0, None),         # an input no LDS strip of the plain kernel holds
+    (1040, 768, 768, 0.8, 1, None),       # ragged last strip
+    (16, 128, 16, 0.0, 0, None),
+    (48, 256, 32, 0.3, 2, (1, 128, 1)),
+    (2048, 768, 3072, 0.0, 0, (4, 128, 12)),   # dense structure, two block-rows per wave in half of the waves
+    (512, 3072, 768, 0.8, 0, (2, 512, 3)),
+    (512, 3072, 768, 0.8, 0, (8, 128, 24)),
+    (256, 1024, 1024, 0.95, 0, (1, 512, 20)),  # block-rows without tiles in most chunks
+]
+
+
+@pytest.mark.parametrize("T,inp,out,sp,act,geom", PLANNED_CASES)
+def test_linear_bsr16_planned(et, T, inp, out, sp, act, geom):
+    """The streaming kernel behind a plan: same Linear as the plain call, for binary16 and
+    binary32 results, at the automatic and at forced launch geometries."""
+    import ctypes as C
+    lib = et.lib()
+    w = Hn.BsrWeight(out, inp, sp, seed=31, bias_std=0.1).upload(et)
+    x = Hn.randn((T, inp), 32)
+    d_x = up(et, x)
+    mt, kc, rpw = geom or (0, 0, 0)
+    plan = C.c_void_p()
+    et.check(lib.et_bsr16_plan_create(w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, T, inp, out, mt, kc, rpw,
+                                      C.byref(plan)))
+    try:
+        g = [C.c_int() for _ in range(4)]
+        et.check(lib.et_bsr16_plan_info(plan, *[C.byref(v) for v in g]))
+        d_y16 = et.DeviceBuffer.empty((T, out), np.float16)
+        d_y32 = et.DeviceBuffer.empty((T, out), np.float32)
+        et.check(lib.et_fill_f16(d_y16.ptr, T * out, 0x7E00, None))
+        et.check(lib.et_linear_bsr16_planned_f16(plan, w.d_bias.ptr, d_x.ptr, d_y16.ptr, None, T, act, None))
+        et.check(lib.et_linear_bsr16_planned_f16(plan, w.d_bias.ptr, d_x.ptr, None, d_y32.ptr, T, act, None))
+        name = {0: None, 1: "relu", 2: "gelu"}[act]
+        want32 = L.linear(Hn.f32(x), Hn.f32(w.dense), Hn.f32(w.bias), name, None).numpy()
+        want16 = L.linear(Hn.f32(x), Hn.f32(w.dense), Hn.f32(w.bias), name, torch.float16).numpy()
+        e16, e32 = Hn.max_abs(d_y16.numpy(), want16), Hn.max_abs(d_y32.numpy(), want32)
+        print(f"planned T={T} in={inp} out={out} sp={sp} geometry mt={g[0].value} kc={g[1].value} rows={g[2].value} "
+              f"lds={g[3].value}: max-abs fp16 {e16:.2e} fp32 {e32:.2e}")
+        assert e16 <= 4e-3
+        assert e32 <= 5e-5 * max(1.0, float(np.abs(want32).max()))
+        # a plan serves other row counts too (here: the first 16 rows only)
+        d_y = et.DeviceBuffer.empty((16, out), np.float16)
+        et.check(lib.et_linear_bsr16_planned_f16(plan, w.d_bias.ptr, d_x.ptr, d_y.ptr, None, 16, act, None))
+        assert Hn.max_abs(d_y.numpy(), want16[:16]) <= 4e-3
+    finally:
+        et.check(lib.et_bsr16_plan_destroy(plan))
+
+
+def test_bsr16_plan_rejects_what_it_cannot_do(et):
+    import ctypes as C
+    lib = et.lib()
+    w = Hn.BsrWeight(64, 64, 0.5, seed=33).upload(et)
+    plan = C.c_void_p()
+    args = (w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr)
+    assert lib.et_bsr16_plan_create(*args, 64, 64, 64, 0, 0, 0, C.byref(plan)) == et.ET_ERR_UNSUPPORTED  # in < 128
+    assert lib.et_bsr16_plan_create(*args, 64, 64, 64, 3, 0, 0, C.byref(plan)) != et.ET_OK
+    w2 = Hn.BsrWeight(512, 2048, 0.0, seed=34).upload(et)
+    # 32 dense block-rows of 512 columns per chunk: 512 slots = 512 KB of LDS per buffer
+    st = lib.et_bsr16_plan_create(w2.d_row_ptr.ptr, w2.d_col_idx.ptr, w2.d_tiles.ptr, 64, 2048, 512, 1, 512, 32,
+                                  C.byref(plan))
+    assert st == et.ET_ERR_UNSUPPORTED and b"LDS" in lib.et_last_error()
+    assert plan.value is None
+
+
 def test_linear_bsr16_closed_form_all_ones(et):
     """All-ones input and all-ones tiles: Y[t][o] = 16 * tiles_in_block_row(o/16) + bias
     (the only closed form the reference's driver offers, Linear/test/test_tile.cu:56-75)."""

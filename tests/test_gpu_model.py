@@ -192,6 +192,20 @@ def test_mixed_small_stack_graph_eager_inplace_and_single_layers(et, use_graph):
     assert Hn.max_abs(bufs[1].numpy(np.float16, (B * S, H)), ref.numpy()) <= 4e-3
 
 
+@pytest.mark.parametrize("mixed", [False, True])
+def test_layer_at_4096_rows_uses_the_streaming_linear(et, mixed):
+    """32 sequences of 128 tokens: the FFN down-projection (3072 inputs, 4096 token rows) runs on the
+    planned streaming kernel inside the class layer; binary16 and binary32 results of it."""
+    H, nh, FF, S, B = 768, 12, 3072, 128, 32
+    layers = [Hn.LayerWeights(H, nh, FF, 0.8, seed=400)]
+    m = Hn.build_model(et, layers, S, B, mixed=mixed)
+    x = Hn.randn((B * S, H), 401)
+    got = run_model(et, m, x, reps=2)
+    want = Hn.oracle_stack(x, layers, B, store=torch.float16, resid=torch.float32 if mixed else "same")
+    assert Hn.max_abs(got[0], want) <= 4e-3
+    assert np.array_equal(got[0], got[1])
+
+
 def test_in_place_forward_with_graph_all_fp16(et):
     H, nh, FF, S, B = 128, 2, 256, 32, 1
     layers = [Hn.LayerWeights(H, nh, FF, 0.5, seed=70 + i) for i in range(2)]
