@@ -5,10 +5,14 @@ seq 128, batch 8, 80 % 16x16 tile sparsity with attention-aware V/O pruning.
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 One "step" is one forward of the whole encoder stack over one batch of synthetic
-token embeddings that already sit in HBM (one HIP-graph replay through the C ABI).
+token embeddings that already sit in HBM (one HIP-graph replay through the C ABI),
+in the engine's mixed-precision mode: fp16 matrix-core operands, fp32 accumulation,
+fp32 softmax, LayerNorm and residual stream.
 Prints ONE JSON line: sequences/s (value), ms per step, per-layer latency, the
-roofline of the dominant kernel (SkipLayerNorm + tile-sparse FFN up-projection + GELU in
-one launch, timed with HIP events on its own stream) and the CPU oracle timed on the host cores.
+roofline of the dominant kernel (the tile-sparse FFN down-projection, 768 x 3072 at
+80 %, binary32 result; timed with HIP events on its own stream over launches that
+rotate through the twelve layers' weights and twelve activation buffers, so that no
+launch finds its operands in the L2s) and the CPU oracle timed on the host cores.
 """
 from __future__ import annotations
 
@@ -32,10 +36,24 @@ SPARSITY = 0.8
 ATTENTION_AWARE = 0.25
 
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak (vendor figure)
-# HBM-side bytes per launch of the FFN down-projection kernel: rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a streaming
-# kernel of known size (profiles/encoder_stack_bert_base_b8_s128_hbm_traffic.txt).
-FFN_DOWN_TRAFFIC_BYTES = (6926.0 * 1.9989 + 1536.0 * 1.0) * 1024
+# HBM-side bytes per launch of the FFN down-projection kernel come from the committed PMC summary:
+# rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (KiB per dispatch), each scaled by what the same
+# counter reads for a streaming kernel of known size.  The summary ends in one machine-readable
+# line, "bench.py reads: {json}", which is all this file takes from it.
+TRAFFIC_PROFILE = ROOT / "profiles" / "encoder_stack_bert_base_b8_s128_hbm_traffic.txt"
+DOMINANT_KERNEL = "bsr16_linear_kernel<1,true,NONE> FFN down-projection 768x3072 @80%, T=1024, binary32 result"
+
+
+def traffic_from_profile():
+    """(bytes per launch, source note) of the dominant kernel, or (None, reason)."""
+    try:
+        for line in TRAFFIC_PROFILE.read_text().splitlines():
+            if line.startswith("bench.py reads:"):
+                d = json.loads(line.split(":", 1)[1])
+                return (d["fetch_kib"] * d["fetch_factor"] + d["write_kib"] * d["write_factor"]) * 1024.0, d["kernel"]
+    except (OSError, ValueError, KeyError) as e:
+        return None, f"{TRAFFIC_PROFILE.name}: {e}"
+    return None, f"{TRAFFIC_PROFILE.name}: no 'bench.py reads:' line"
 
 
 class TileWeight:
@@ -116,28 +134,34 @@ def time_stack(et, model, d_out, d_in, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
-def time_ffn_down_kernel(et, w, T, launches_per_graph=64, replays=8):
+def time_ffn_down_kernel(et, weights, T, rounds_per_graph=6, replays=8):
     """Average duration of the layer's longest kernel at the workload's shape — the FFN
-    down-projection through the tile-sparse W2 (768 x 3072 at 80 %), T token rows:
-    `launches_per_graph` launches recorded into one HIP graph, replayed between two HIP
-    events on the same stream, so no host launch latency is in the figure."""
+    down-projection through the tile-sparse W2 (768 x 3072 at 80 %), T token rows, binary32
+    result as the mixed-precision stack launches it.  One graph holds `rounds_per_graph` rounds
+    over the twelve layers' weights, each launch with an input and an output buffer of its own
+    (12 x 6 MB + 12 x 3 MB), so that — as inside the stack — no launch finds its weights or its
+    activations where the previous launch left them.  Replayed between two HIP events on the
+    launch stream: no host launch latency is in the figure."""
     import ctypes as C
     lib = et.lib()
     stream = C.c_void_p()
     et.check(lib.et_stream_create(C.byref(stream)))
     rng = np.random.default_rng(0)
-    x = et.DeviceBuffer.from_numpy(rng.standard_normal((T, FF)).astype(np.float16))
-    y = et.DeviceBuffer.empty((T, H), np.float16)
+    xs = [et.DeviceBuffer.from_numpy(rng.standard_normal((T, FF), dtype=np.float32).astype(np.float16))
+          for _ in weights]
+    ys = [et.DeviceBuffer.empty((T, H), np.float32) for _ in weights]
 
-    def launch():
-        et.check(lib.et_linear_bsr16_f16(w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, w.d_bias.ptr, x.ptr, y.ptr,
-                                         T, FF, H, et.ACT_NONE, stream))
+    def launch(i):
+        w = weights[i]
+        et.check(lib.et_linear_bsr16_f16_f32out(w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, w.d_bias.ptr,
+                                                xs[i].ptr, ys[i].ptr, T, FF, H, et.ACT_NONE, stream))
 
-    launch()  # eager once (one-time kernel setup)
+    launch(0)  # eager once (one-time kernel setup)
     et.check(lib.et_stream_sync(stream))
     et.check(lib.et_graph_begin_capture(stream))
-    for _ in range(launches_per_graph):
-        launch()
+    for _ in range(rounds_per_graph):
+        for i in range(len(weights)):
+            launch(i)
     graph = C.c_void_p()
     et.check(lib.et_graph_end_capture(stream, C.byref(graph)))
     et.check(lib.et_graph_launch(graph, stream))  # warm
@@ -147,7 +171,7 @@ def time_ffn_down_kernel(et, w, T, launches_per_graph=64, replays=8):
             et.check(lib.et_graph_launch(graph, stream))
     et.check(lib.et_graph_destroy(graph))
     et.check(lib.et_stream_destroy(stream))
-    return t.ms * 1e-3 / (launches_per_graph * replays)
+    return t.ms * 1e-3 / (rounds_per_graph * len(weights) * replays)
 
 
 def oracle_params(layers):
@@ -238,20 +262,23 @@ def main():
 
     sec = time_stack(et, model, d_out, d_in, args.steps, args.warmup)
 
-    # dominant kernel: FFN down-projection (768x3072 BSR at 80 %, T = 1024)
+    # dominant kernel: FFN down-projection (768x3072 BSR at 80 %, T = 1024, binary32 result)
     T = B * S
-    w2 = layers[0].l2.upload(et)
-    ntile = len(layers[0].l2.col_idx)
+    w2s = [l.l2.upload(et) for l in layers]
+    ntile = len(layers[0].l2.col_idx)  # the same count in every layer: int(9216 * (1 - 0.8))
     flops = 2.0 * 256 * ntile * T  # algorithmic: 2 * 16*16 * surviving tiles * token rows
-    ksec = time_ffn_down_kernel(et, w2, T)
+    ksec = time_ffn_down_kernel(et, w2s, T)
     achieved = flops / ksec / 1e12
-    roofline = {"bound": "mfma", "kernel": "bsr16_linear_kernel<1,true,NONE> FFN down-projection 768x3072 @80%, T=1024",
+    traffic, traffic_note = traffic_from_profile()
+    roofline = {"bound": "mfma", "kernel": DOMINANT_KERNEL,
                 "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 5), "us_per_launch": round(ksec * 1e6, 3),
-                "flop_per_launch": flops, "traffic": round(FFN_DOWN_TRAFFIC_BYTES)}
-    # The same launch against the other roof: algorithmic bytes 2T(in+out) + 516 ntile + 4(out/16+1) + 2 out.
-    # At 109 flop per byte the shape sits below the ridge of the machine (312 flop/B), i.e. on the HBM roof.
-    alg_bytes = 2.0 * T * (FF + H) + 516.0 * ntile + 4.0 * (H // 16 + 1) + 2.0 * H
+                "flop_per_launch": flops, "traffic": None if traffic is None else round(traffic),
+                "traffic_source": traffic_note}
+    # The same launch against the other roof: algorithmic bytes 2 T in + 4 T out (binary32 result)
+    # + 516 ntile + 4(out/16+1) + 2 out.  At 93 flop per byte the shape sits below the ridge of the
+    # machine (312 flop/B), i.e. on the HBM roof.
+    alg_bytes = 2.0 * T * FF + 4.0 * T * H + 516.0 * ntile + 4.0 * (H // 16 + 1) + 2.0 * H
     roofline["hbm_view"] = {"bound": "hbm", "achieved": round(alg_bytes / ksec / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
                             "frac": round(alg_bytes / ksec / 8e12, 5), "bytes_per_launch": alg_bytes}
 
