@@ -22,6 +22,14 @@ inline void linear_vo_forward(const half *Wt, const half *bias, const half *X, h
                              m.seq_len, m.emdim, N, m.nhead, stream));
 }
 
+// The projection key-contiguous and without its bias, [batch][nh][N][S]: the operand layout of the
+// attention kernel that keeps the probabilities on chip (et_mha_vo_otf_f16 adds the bias itself).
+inline void linear_vo_forward_keys(const half *Wt, const half *X, half *out, const Model_t &m, int batch, int N,
+                                   stream_t stream) {
+    etChk(et_linear_vo_keys_f16(reinterpret_cast<const et_f16 *>(Wt), reinterpret_cast<const et_f16 *>(X),
+                                reinterpret_cast<et_f16 *>(out), batch, m.seq_len, m.emdim, N, m.nhead, stream));
+}
+
 // Device copy of W[nh][H][N] turned into [nh][N][H], made once at construction: the GEMM behind
 // the projection reads k-contiguous operands about twice as fast.
 inline DeviceBuffer<half> transposed_heads(const half *W_dev, int nhead, int H, int N) {
@@ -73,6 +81,9 @@ class Linear_VO {
     void forward(half *output, const half *input, et::stream_t stream = nullptr, int batch = 1) {
         et::linear_vo_forward(weight_t.get(), bias.get(), input, output, *model, batch, model->emdim, stream);
     }
+    void forward_keys(half *output, const half *input, et::stream_t stream = nullptr, int batch = 1) {
+        et::linear_vo_forward_keys(weight_t.get(), input, output, *model, batch, model->emdim, stream);
+    }
 
   private:
     static ptr_t checked_transpose(const ptr_t &w, const Model_t &m) {
@@ -100,6 +111,9 @@ class Linear_VO_prune {
     int out_width() const { return (int)weight.col_id->size; }
     void forward(half *output, const half *input, et::stream_t stream = nullptr, int batch = 1) {
         et::linear_vo_forward(weight_t.get(), bias.get(), input, output, *model, batch, out_width(), stream);
+    }
+    void forward_keys(half *output, const half *input, et::stream_t stream = nullptr, int batch = 1) {
+        et::linear_vo_forward_keys(weight_t.get(), input, output, *model, batch, out_width(), stream);
     }
 
   private:

@@ -412,6 +412,26 @@ int et_mha_vo_f16(const et_f16 *Q, const et_f16 *K, int ldq, int ldk,
                   int hd, int N, int out_width, float scale, int flags,
                   et_stream stream);
 
+/* The same attention with the probabilities kept on chip (the reference's
+ * OTF_fused_attn, Fused_attention/Fused_attention.cu:10-116), in two calls.
+ * et_linear_vo_keys_f16 writes the projection key-contiguous and without its
+ * bias, VOt[b][h][n][s] = sum_k Wt[h][n][k] X[b*S+s][k] (Wt as for
+ * et_linear_vo_t_f16): both matrix-core operands of the attention kernel are
+ * then 16-byte loads and nothing is staged through LDS.  et_mha_vo_otf_f16
+ * gives the waves of a workgroup (32 queries x 64 output columns) a head each,
+ * sums softmax_h * VO_h in fp32, adds sum_h bias_vo[h][n] (the probabilities of
+ * a row add up to one; bias_vo [nh][N] or NULL) and bias_o, and writes every
+ * element of out once: no P buffer, no atomics, out need not be cleared.  The
+ * other arguments as et_mha_vo_f16. */
+int et_linear_vo_keys_f16(const et_f16 *Wt, const et_f16 *X, et_f16 *VOt, int B,
+                          int S, int H, int N, int nh, et_stream stream);
+int et_mha_vo_otf_f16(const et_f16 *Q, const et_f16 *K, int ldq, int ldk,
+                      const et_f16 *VOt, const et_f16 *bias_vo, et_f16 *out,
+                      const et_f16 *bias_o, const int32_t *col_scatter,
+                      const et_f16 *mask, const int32_t *lens, int B, int S,
+                      int nh, int hd, int N, int out_width, float scale,
+                      int flags, et_stream stream);
+
 /* ------------------------------------------------------------------------
  * Normalisation and element-wise operators.
  * ------------------------------------------------------------------------ */

@@ -107,6 +107,8 @@ _SIGNATURES = {
     "et_linear_vo_t_f16": (_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp),
     "et_transpose_heads_f16": (_vp, _vp, _i, _i, _i, _vp),
     "et_mha_vo_f16": (_vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp),
+    "et_linear_vo_keys_f16": (_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp),
+    "et_mha_vo_otf_f16": (_vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _vp),
     "et_graph_begin_capture": (_vp,),
     "et_graph_end_capture": (_vp, C.POINTER(_vp)),
     "et_graph_launch": (_vp, _vp),

@@ -259,6 +259,27 @@ int et_linear_vo_t_f16(const et_f16 *Wt, const et_f16 *bias, const et_f16 *X, et
     return launch_gemm(g, B * nh, true, as_stream(stream));
 }
 
+int et_linear_vo_keys_f16(const et_f16 *Wt, const et_f16 *X, et_f16 *VOt, int B, int S, int H_, int N, int nh,
+                          et_stream stream) {
+    ET_REQUIRE(Wt && X && VOt, ET_ERR_INVALID_ARG, "et_linear_vo_keys_f16: NULL pointer");
+    ET_REQUIRE(B >= 0 && S > 0 && H_ > 0 && N > 0 && nh > 0, ET_ERR_INVALID_ARG,
+               "et_linear_vo_keys_f16: B=%d S=%d H=%d N=%d nh=%d", B, S, H_, N, nh);
+    ET_REQUIRE(S % 16 == 0 && H_ % 16 == 0 && N % 16 == 0, ET_ERR_UNSUPPORTED,
+               "et_linear_vo_keys_f16: S=%d H=%d N=%d must be multiples of 16", S, H_, N);
+    ET_REQUIRE((long long)B * nh <= 65535, ET_ERR_UNSUPPORTED, "et_linear_vo_keys_f16: batch*nhead too large");
+    if (B == 0) return ET_OK;
+    // VOt[b][h] (N x S) = Wt[h] (N x H) * X[b]^T (X[b] is S x H): the operands of et_linear_vo_t_f16 exchanged
+    GemmArgs g = gemm_args(H(Wt), H(X), H(VOt), N, S, H_, H_, H_, S);
+    g.batch_inner = nh;
+    g.sAo = 0;
+    g.sAi = (long long)N * H_;
+    g.sBo = (long long)S * H_;
+    g.sBi = 0;
+    g.sCo = (long long)nh * N * S;
+    g.sCi = (long long)N * S;
+    return launch_gemm(g, B * nh, true, as_stream(stream));
+}
+
 int et_mha_vo_f16(const et_f16 *Q, const et_f16 *K, int ldq, int ldk, const et_f16 *VO, et_f16 *P,
                   et_f16 *out, const et_f16 *bias_o, const int32_t *col_scatter, const et_f16 *mask,
                   const int32_t *lens, int B, int S, int nh, int hd, int N, int out_width, float scale,

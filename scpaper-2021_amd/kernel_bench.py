@@ -233,6 +233,13 @@ class Bench:
                                                             None, None, None, None, B, S, nh, hd, N, N, hd ** -0.5, 0,
                                                             self.stream)), launches)
         self.record("mha_vo", f"B{B} S{S} nh{nh} hd{hd} N{N}", us, 2 * B * S * S * nh * (hd + N), "mfma")
+        us = self.time_us(lambda: et.check(lib.et_linear_vo_keys_f16(wt.ptr, x.ptr, vo.ptr, B, S, H, N, nh, self.stream)),
+                          launches)
+        self.record("linear_vo_keys", f"B{B} S{S} H{H} N{N} nh{nh}", us, 2 * B * S * H * N * nh, "mfma")
+        us = self.time_us(lambda: et.check(lib.et_mha_vo_otf_f16(qk.ptr, qk.offset(2 * H), 2 * H, 2 * H, vo.ptr, None,
+                                                                out.ptr, None, None, None, None, B, S, nh, hd, N, N,
+                                                                hd ** -0.5, 0, self.stream)), launches)
+        self.record("mha_vo_otf", f"B{B} S{S} nh{nh} hd{hd} N{N}", us, 2 * B * S * S * nh * (hd + N), "mfma")
 
     def mha_unfused(self, B, S, nh, hd, launches):
         """Scores through memory: batched GEMM, stand-alone softmax, batched GEMM (the comparison line)."""
@@ -347,7 +354,7 @@ def run_scale(b: Bench):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--set", choices=("configs", "scale", "all"), default="all")
+    ap.add_argument("--set", choices=("configs", "scale", "vo", "all"), default="all")
     ap.add_argument("--json", default=None, help="also write the rows as JSON to this file")
     args = ap.parse_args()
     b = Bench()
@@ -355,6 +362,11 @@ def main():
     if args.set in ("configs", "all"):
         print("# shapes of the benchmark configurations")
         run_configs(b)
+    if args.set == "vo":
+        print("# pre-computed-VO attention: probabilities through memory (mha_vo) and on chip (mha_vo_otf)")
+        for B, N in ((1, 768), (4, 384), (8, 768), (16, 768)):
+            b.mha_vo(B, 128, 12, 64, N, 20)
+        b.mha_vo(4, 512, 16, 64, 1024, 10)
     if args.set in ("scale", "all"):
         print("# shapes where launch latency no longer matters")
         run_scale(b)

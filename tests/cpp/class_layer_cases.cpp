@@ -5,6 +5,7 @@
 //                 the model assembly of the reference example (example/main.cu:24-182)
 //   prune_attn    Attention<tile, tile, row_mat, tile, Prune_attn> (attention-aware pruning)
 //   fused_attn    FusedAttention<NOTF_fused_attn> with the W_VO built by et::build_vo_weight
+//   fused_otf     FusedAttention<OTF_fused_attn>: the same attention with the probabilities kept on chip
 //   fused_prune   FusedAttention<NOTF_fused_prune_attn> over a column-pruned W_VO
 //   factories     the gen_* test factories: closed forms of the reference drivers
 //   attn_variants Attention<> with separate Q/K/V projections under the tags OTF_attn_full,
@@ -442,6 +443,7 @@ int main(int argc, char **argv) {
         if (which == "example") return run_example(dir);
         if (which == "prune_attn") return run_prune_attn(dir);
         if (which == "fused_attn") return run_fused<NOTF_fused_attn>(dir);
+        if (which == "fused_otf") return run_fused<OTF_fused_attn>(dir);
         if (which == "fused_prune") return run_fused<NOTF_fused_prune_attn>(dir);
         if (which == "factories") return run_factories(dir);
         if (which == "attn_variants") return run_attn_variants(dir);

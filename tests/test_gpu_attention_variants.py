@@ -49,13 +49,16 @@ def vo_case(seed, H, nh, N_keep=None):
     return dict(Wq=h16(Wq), Wk=h16(Wk), bq=h16(bq), bk=h16(bk), Wvo=h16(Wvo), bvo=h16(bvo), bo=h16(bo))
 
 
-@pytest.mark.parametrize("B,S,H,nh,pruned", [(1, 128, 768, 12, False), (2, 64, 256, 4, False), (2, 64, 256, 4, True)])
+@pytest.mark.parametrize("B,S,H,nh,pruned", [(1, 128, 768, 12, False), (2, 64, 256, 4, False), (2, 64, 256, 4, True),
+                                             (9, 48, 96, 3, True), (2, 272, 256, 2, False), (1, 128, 512, 8, False),
+                                             (8, 128, 768, 12, False)])
 def test_vo_attention(et, B, S, H, nh, pruned):
-    """Linear_VO + probabilities + one GEMM per sequence == the oracle's sum_h P_h VO_h + b_O."""
+    """Linear_VO + probabilities + one GEMM per sequence == the oracle's sum_h P_h VO_h + b_O, and so
+    does the kernel that keeps the probabilities on chip."""
     T, hd = B * S, H // nh
     c = vo_case(7, H, nh)
     x = Hn.randn((T, H), 8)
-    lens = np.array([S, S - 9][:B], np.int32)
+    lens = np.array([S, S - 9, 1, 0, S // 2, S, 17, S - 1, 5][:B], np.int32)
     Wvo, bvo = c["Wvo"], c["bvo"]
     col_id = None
     if pruned:
@@ -92,11 +95,64 @@ def test_vo_attention(et, B, S, H, nh, pruned):
     want = L.fused_vo_attention(Hn.f32(x), Hn.f32(x), Hn.f32(x), Hn.f32(c["Wq"]), Hn.f32(c["bq"]), Hn.f32(c["Wk"]),
                                 Hn.f32(c["bk"]), torch.from_numpy(Wvo_full), torch.from_numpy(bvo_full), Hn.f32(c["bo"]),
                                 nh, B, lens=lens, store=torch.float16).numpy()
-    got = d_out.numpy()
-    assert Hn.max_abs(got, want) <= 6e-3
-    if pruned:
-        dead = np.setdiff1d(np.arange(H), col_id)
-        assert np.array_equal(got[:, dead], np.broadcast_to(c["bo"][dead], (T, len(dead))))
+    # the projection key-contiguous and without bias, for the kernel that keeps the probabilities on chip
+    d_vok = et.DeviceBuffer.empty((B, nh, N, S), np.float16)
+    et.check(et.lib().et_linear_vo_keys_f16(d_wt.ptr, d_x.ptr, d_vok.ptr, B, S, H, N, nh, None))
+    want_vok = (x.astype(np.float32).reshape(B, 1, S, H) @ Wvo.astype(np.float32)[None]).transpose(0, 1, 3, 2)
+    assert Hn.max_abs(d_vok.numpy(), want_vok.astype(np.float16)) <= 4e-3
+    d_otf = et.DeviceBuffer.empty((T, H), np.float16)
+    et.check(et.lib().et_fill_f16(d_otf.ptr, T * H, 0x7E00, None))
+    et.check(et.lib().et_mha_vo_otf_f16(d_q.ptr, d_k.ptr, H, H, d_vok.ptr, up(et, bvo).ptr, d_otf.ptr, up(et, c["bo"]).ptr,
+                                        None if col_id is None else up(et, col_id).ptr, None, up(et, lens).ptr, B, S, nh,
+                                        hd, N, H, 1 / math.sqrt(hd), 0, None))
+    for got in (d_out.numpy(), d_otf.numpy()):
+        assert Hn.max_abs(got, want) <= 6e-3
+        if pruned:
+            dead = np.setdiff1d(np.arange(H), col_id)
+            assert np.array_equal(got[:, dead], np.broadcast_to(c["bo"][dead], (T, len(dead))))
+    # both kernels round the same fp16 probabilities; they differ in the order of the fp32 sums and in
+    # where the projection's bias is added
+    assert Hn.max_abs(d_out.numpy(), d_otf.numpy()) <= 6e-3  # an fp16 ulp at the largest outputs
+
+
+@pytest.mark.parametrize("B,S,H,nh", [(2, 192, 128, 2), (1, 64, 384, 12), (3, 80, 128, 8), (12, 256, 192, 3)])
+@pytest.mark.parametrize("causal,masked", [(True, False), (False, True), (True, True)])
+def test_vo_attention_on_chip_masks(et, causal, masked, B, S, H, nh):
+    """Causal flag and additive mask of the on-chip VO attention against the oracle, in each of the
+    kernel's forms (a wave per head for up to 4, 8 and more heads; the large-grid form)."""
+    T, hd = B * S, H // nh
+    q, k = Hn.randn((T, H), 40), Hn.randn((T, H), 41)
+    vo = (Hn.randn((B, nh, S, H), 42).astype(np.float32) * 0.25).astype(np.float16)
+    bo = Hn.randn((H,), 43)
+    mask = None
+    if masked:
+        mask = (Hn.randn((S, S), 44).astype(np.float32) * 2).astype(np.float16)
+        mask[:, 5] = -np.inf
+    d_out = et.DeviceBuffer.empty((T, H), np.float16)
+    vo_keys = np.ascontiguousarray(vo.transpose(0, 1, 3, 2))  # [B][nh][N][S]
+    et.check(et.lib().et_mha_vo_otf_f16(up(et, q).ptr, up(et, k).ptr, H, H, up(et, vo_keys).ptr, None, d_out.ptr, up(et, bo).ptr,
+                                        None, None if mask is None else up(et, mask).ptr, None, B, S, nh, hd, H, H,
+                                        1 / math.sqrt(hd), et.MHA_CAUSAL if causal else 0, None))
+    # the oracle's attention with V = VO_h gives softmax_h VO_h per head; the heads are summed here
+    want = np.zeros((T, H), np.float32)
+    for h in range(nh):
+        sl = slice(h * hd, (h + 1) * hd)
+        v_h = vo[:, h].reshape(T, H)
+        z = L.mha(Hn.f32(q[:, sl]), Hn.f32(k[:, sl]), Hn.f32(v_h), 1, B, scale=1 / math.sqrt(hd),
+                  mask=None if mask is None else Hn.f32(mask), causal=causal, store=None)
+        want += z.numpy()
+    want += bo.astype(np.float32)
+    assert Hn.max_abs(d_out.numpy(), want) <= 6e-3
+
+
+def test_vo_attention_on_chip_rejects_bad_shapes(et):
+    d = et.DeviceBuffer.empty((64, 64), np.float16)
+    call = lambda **kw: et.lib().et_mha_vo_otf_f16(d.ptr, d.ptr, kw.get("ld", 64), 64, d.ptr, None, d.ptr, None, None, None, None,
+                                                   1, kw.get("S", 16), 1, kw.get("hd", 64), kw.get("N", 64),
+                                                   kw.get("W", 64), 0.125, kw.get("flags", 0), None)
+    assert call() == et.ET_OK
+    for bad in (dict(S=24), dict(hd=40), dict(N=40, W=40), dict(N=32, W=64), dict(ld=32), dict(flags=8)):
+        assert call(**bad) in (et.ET_ERR_INVALID_ARG, et.ET_ERR_UNSUPPORTED), bad
 
 
 @pytest.mark.parametrize("B,S,nh,hd,keep", [(2, 128, 12, 64, 0.75), (1, 48, 4, 32, 0.5), (1, 272, 2, 64, 0.25)])

@@ -95,7 +95,7 @@ def test_prune_attn_class(tmp_path):
     assert Hn.max_abs(np.load(tmp_path / "out.npy"), want) <= 6e-3
 
 
-@pytest.mark.parametrize("case", ["fused_attn", "fused_prune"])
+@pytest.mark.parametrize("case", ["fused_attn", "fused_otf", "fused_prune"])
 def test_fused_attention_class(tmp_path, case):
     """FusedAttention with W_VO built by et::build_vo_weight equals standard attention followed by
     the output projection (the E.T. identity); the pruned form keeps half of the W_VO columns."""
@@ -119,7 +119,7 @@ def test_fused_attention_class(tmp_path, case):
                                 Hn.f32(b["k"]), Wvo16, bvo16, Hn.f32(b["o"]), nh, B, lens=lens, store=st).numpy()
     got = np.load(tmp_path / "out.npy")
     assert Hn.max_abs(got, want) <= 6e-3
-    if case == "fused_attn":  # and the identity with plain attention + output projection
+    if case in ("fused_attn", "fused_otf"):  # and the identity with plain attention + output projection
         q = L.linear(Hn.f32(x), Hn.f32(W["q"]), Hn.f32(b["q"]), store=st)
         k = L.linear(Hn.f32(x), Hn.f32(W["k"]), Hn.f32(b["k"]), store=st)
         v = L.linear(Hn.f32(x), Hn.f32(W["v"]), Hn.f32(b["v"]))
