@@ -10,9 +10,10 @@ in the engine's mixed-precision mode: fp16 matrix-core operands, fp32 accumulati
 fp32 softmax, LayerNorm and residual stream.
 Prints ONE JSON line: sequences/s (value), ms per step, per-layer latency, the
 roofline of the dominant kernel (the tile-sparse FFN down-projection, 768 x 3072 at
-80 %, binary32 result; timed with HIP events on its own stream over launches that
-rotate through the twelve layers' weights and twelve activation buffers, so that no
-launch finds its operands in the L2s) and the CPU oracle timed on the host cores.
+80 %, binary32 result; timed with HIP events on its own stream as it runs in a layer:
+behind the up-projection that writes its input, rotating through the twelve layers'
+weights and twelve sets of activation buffers, as the replay time of [up, down] pairs
+minus that of the up-projections alone) and the CPU oracle timed on the host cores.
 """
 from __future__ import annotations
 
@@ -134,44 +135,64 @@ def time_stack(et, model, d_out, d_in, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
-def time_ffn_down_kernel(et, weights, T, rounds_per_graph=6, replays=8):
+def time_ffn_down_kernel(et, w1s, w2s, T, rounds_per_graph=6, replays=8):
     """Average duration of the layer's longest kernel at the workload's shape — the FFN
     down-projection through the tile-sparse W2 (768 x 3072 at 80 %), T token rows, binary32
-    result as the mixed-precision stack launches it.  One graph holds `rounds_per_graph` rounds
-    over the twelve layers' weights, each launch with an input and an output buffer of its own
-    (12 x 6 MB + 12 x 3 MB), so that — as inside the stack — no launch finds its weights or its
-    activations where the previous launch left them.  Replayed between two HIP events on the
-    launch stream: no host launch latency is in the figure."""
+    result as the mixed-precision stack launches it.  Returns (seconds as in the stack, seconds
+    alone).
+
+    As in the stack: the launch follows the FFN up-projection + GELU that writes its input, so
+    the input arrives the way it does in a layer (written a moment ago by other compute units)
+    and the launch starts behind another kernel's tail.  Two graphs over the twelve layers'
+    weights, each launch with buffers of its own: [up, down] pairs and [up] alone; the
+    difference of their replay times, per launch, is the figure.  Alone: a graph of
+    down-projections only (every launch still on another layer's weights and buffers, nothing
+    warm in L2).  All replays run between two HIP events on the launch stream: no host launch
+    latency is in either figure."""
     import ctypes as C
     lib = et.lib()
     stream = C.c_void_p()
     et.check(lib.et_stream_create(C.byref(stream)))
     rng = np.random.default_rng(0)
-    xs = [et.DeviceBuffer.from_numpy(rng.standard_normal((T, FF), dtype=np.float32).astype(np.float16))
-          for _ in weights]
-    ys = [et.DeviceBuffer.empty((T, H), np.float32) for _ in weights]
+    n = len(w2s)
+    y1s = [et.DeviceBuffer.from_numpy(rng.standard_normal((T, H), dtype=np.float32).astype(np.float16)) for _ in w2s]
+    xs = [et.DeviceBuffer.from_numpy(rng.standard_normal((T, FF), dtype=np.float32).astype(np.float16)) for _ in w2s]
+    ys = [et.DeviceBuffer.empty((T, H), np.float32) for _ in w2s]
 
-    def launch(i):
-        w = weights[i]
+    def up(i):
+        w = w1s[i]
+        et.check(lib.et_linear_bsr16_f16(w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, w.d_bias.ptr,
+                                         y1s[i].ptr, xs[i].ptr, T, H, FF, et.ACT_GELU, stream))
+
+    def down(i):
+        w = w2s[i]
         et.check(lib.et_linear_bsr16_f16_f32out(w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, w.d_bias.ptr,
                                                 xs[i].ptr, ys[i].ptr, T, FF, H, et.ACT_NONE, stream))
 
-    launch(0)  # eager once (one-time kernel setup)
+    def timed_graph(steps):
+        et.check(lib.et_graph_begin_capture(stream))
+        for _ in range(rounds_per_graph):
+            for i in range(n):
+                for step in steps:
+                    step(i)
+        graph = C.c_void_p()
+        et.check(lib.et_graph_end_capture(stream, C.byref(graph)))
+        et.check(lib.et_graph_launch(graph, stream))  # warm
+        et.check(lib.et_stream_sync(stream))
+        with et.Timer(stream) as t:
+            for _ in range(replays):
+                et.check(lib.et_graph_launch(graph, stream))
+        et.check(lib.et_graph_destroy(graph))
+        return t.ms * 1e-3 / (rounds_per_graph * n * replays)
+
+    up(0)  # eager once (one-time kernel setup)
+    down(0)
     et.check(lib.et_stream_sync(stream))
-    et.check(lib.et_graph_begin_capture(stream))
-    for _ in range(rounds_per_graph):
-        for i in range(len(weights)):
-            launch(i)
-    graph = C.c_void_p()
-    et.check(lib.et_graph_end_capture(stream, C.byref(graph)))
-    et.check(lib.et_graph_launch(graph, stream))  # warm
-    et.check(lib.et_stream_sync(stream))
-    with et.Timer(stream) as t:
-        for _ in range(replays):
-            et.check(lib.et_graph_launch(graph, stream))
-    et.check(lib.et_graph_destroy(graph))
+    alone = timed_graph([down])
+    only_up = timed_graph([up])
+    pair = timed_graph([up, down])
     et.check(lib.et_stream_destroy(stream))
-    return t.ms * 1e-3 / (rounds_per_graph * len(weights) * replays)
+    return pair - only_up, alone
 
 
 def oracle_params(layers):
@@ -264,15 +285,17 @@ def main():
 
     # dominant kernel: FFN down-projection (768x3072 BSR at 80 %, T = 1024, binary32 result)
     T = B * S
+    w1s = [l.l1.upload(et) for l in layers]
     w2s = [l.l2.upload(et) for l in layers]
     ntile = len(layers[0].l2.col_idx)  # the same count in every layer: int(9216 * (1 - 0.8))
     flops = 2.0 * 256 * ntile * T  # algorithmic: 2 * 16*16 * surviving tiles * token rows
-    ksec = time_ffn_down_kernel(et, w2s, T)
+    ksec, ksec_alone = time_ffn_down_kernel(et, w1s, w2s, T)
     achieved = flops / ksec / 1e12
     traffic, traffic_note = traffic_from_profile()
     roofline = {"bound": "mfma", "kernel": DOMINANT_KERNEL,
                 "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 5), "us_per_launch": round(ksec * 1e6, 3),
+                "us_per_launch_alone": round(ksec_alone * 1e6, 3),
                 "flop_per_launch": flops, "traffic": None if traffic is None else round(traffic),
                 "traffic_source": traffic_note}
     # The same launch against the other roof: algorithmic bytes 2 T in + 4 T out (binary32 result)

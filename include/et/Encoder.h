@@ -69,8 +69,11 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
     DeviceBuffer<half> temp_linear;  // [rows x dimFF]
     DeviceBuffer<half> temp_attn;    // [rows x emdim]
     DeviceBuffer<half> temp_LN;      // [rows x emdim]
+    // linear2's result has a buffer of its own (and so has its binary32 twin): written into
+    // temp_attn, which the layer has just read, the same launch takes 1.5-2 us longer
+    DeviceBuffer<half> temp_ffn;     // [rows x emdim]
     // binary32 twins of temp_attn and temp_LN, present after enable_mixed()
-    std::unique_ptr<DeviceBuffer<float>> temp_attn32, temp_LN32;
+    std::unique_ptr<DeviceBuffer<float>> temp_attn32, temp_LN32, temp_ffn32;
 
     EncoderLayer(std::unique_ptr<attn_t> _attn, std::unique_ptr<SkipLayerNorm> _LN1,
                  std::unique_ptr<SkipLayerNorm> _LN2, std::unique_ptr<linear1_t> _linear1,
@@ -78,7 +81,7 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
         : attn(std::move(_attn)), LN1(std::move(_LN1)), LN2(std::move(_LN2)), linear1(std::move(_linear1)),
           linear2(std::move(_linear2)), model(std::move(_model)), rows(attn->rows()),
           temp_linear((std::size_t)rows * model->dimFF), temp_attn((std::size_t)rows * model->emdim),
-          temp_LN((std::size_t)rows * model->emdim) {
+          temp_LN((std::size_t)rows * model->emdim), temp_ffn((std::size_t)rows * model->emdim) {
         require(linear1->size == rows && linear2->size == rows,
                 "Encoder: the Linear layers must be built for batch * seq_len rows");
     }
@@ -106,8 +109,8 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
             LN1->forward(temp_LN.get(), temp_attn.get(), src, rows, stream);
             linear1->forward_act(temp_linear.get(), temp_LN.get(), act_code<ACT_OP_t>(), stream);
         }
-        linear2->forward(temp_attn.get(), temp_linear.get(), stream);
-        LN2->forward(out, temp_attn.get(), temp_LN.get(), rows, stream);
+        linear2->forward(temp_ffn.get(), temp_linear.get(), stream);
+        LN2->forward(out, temp_ffn.get(), temp_LN.get(), rows, stream);
     }
 
     // Mixed precision.  The residual stream — the layer input, both projections that feed a
@@ -121,14 +124,15 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
     void enable_mixed() {
         if (!temp_attn32) temp_attn32 = std::make_unique<DeviceBuffer<float>>((std::size_t)rows * model->emdim);
         if (!temp_LN32) temp_LN32 = std::make_unique<DeviceBuffer<float>>((std::size_t)rows * model->emdim);
+        if (!temp_ffn32) temp_ffn32 = std::make_unique<DeviceBuffer<float>>((std::size_t)rows * model->emdim);
     }
     void forward_mixed(float *out32, half *out16, const float *src32, half *src16, stream_t stream = nullptr) {
         require(temp_attn32 && temp_LN32, "Encoder: call enable_mixed() before forward_mixed()");
         attn_forward_f32(temp_attn32->get(), src16, stream);
         LN1->forward_mixed(temp_LN32->get(), temp_LN.get(), temp_attn32->get(), src32, rows, stream);
         linear1->forward_act(temp_linear.get(), temp_LN.get(), act_code<ACT_OP_t>(), stream);
-        linear_forward_f32(*linear2, temp_attn32->get(), temp_linear.get(), temp_attn.get(), stream);
-        LN2->forward_mixed(out32, out16, temp_attn32->get(), temp_LN32->get(), rows, stream);
+        linear_forward_f32(*linear2, temp_ffn32->get(), temp_linear.get(), temp_ffn.get(), stream);
+        LN2->forward_mixed(out32, out16, temp_ffn32->get(), temp_LN32->get(), rows, stream);
     }
 
   private:

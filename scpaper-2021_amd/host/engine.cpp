@@ -61,8 +61,10 @@ struct et_model_s {
     std::shared_ptr<Model_t> model;
     std::vector<HostLayer> host;
     std::vector<std::unique_ptr<ILayer>> layers;
-    std::unique_ptr<et::DeviceBuffer<half>> pp[2];
-    std::unique_ptr<et::DeviceBuffer<float>> pp32[2];  // mixed precision: the residual stream between layers
+    // layer i writes ring slot i % kRing, layer i + 1 reads it; a slot is written again kRing layers on
+    static constexpr int kRing = 4;
+    std::unique_ptr<et::DeviceBuffer<half>> pp[kRing];
+    std::unique_ptr<et::DeviceBuffer<float>> pp32[kRing];  // mixed precision: the residual stream between layers
     std::unique_ptr<et::DeviceBuffer<half>> warm;      // result of the eager pass that precedes a capture
     std::vector<int> lens;   // empty = no padding
     std::vector<half> mask;  // empty = no additive mask
@@ -157,13 +159,14 @@ void check_layer_index(const et_model_s *m, int layer) {
 void run_layers_mixed(et_model_s &m, half *out, half *in, stream_t stream) {
     const int n = (int)m.layers.size();
     const std::size_t elems = (std::size_t)m.rows() * m.desc.emdim;
-    etChk(et_f16_to_f32(m.pp32[1]->get(), et::f16(in), elems, stream));
-    const float *src32 = m.pp32[1]->get();
+    constexpr int R = et_model_s::kRing;
+    etChk(et_f16_to_f32(m.pp32[R - 1]->get(), et::f16(in), elems, stream));
+    const float *src32 = m.pp32[R - 1]->get();
     half *src16 = in;
     for (int i = 0; i < n; i++) {
         const bool last = i == n - 1;
-        float *dst32 = last ? nullptr : m.pp32[i % 2]->get();
-        half *dst16 = last ? out : m.pp[i % 2]->get();
+        float *dst32 = last ? nullptr : m.pp32[i % R]->get();
+        half *dst16 = last ? out : m.pp[i % R]->get();
         m.layers[(size_t)i]->forward_mixed(dst32, dst16, src32, src16, stream);
         src32 = dst32;
         src16 = dst16;
@@ -175,7 +178,7 @@ void run_layers(et_model_s &m, half *out, half *in, stream_t stream) {
     const int n = (int)m.layers.size();
     half *src = in;
     for (int i = 0; i < n; i++) {
-        half *dst = (i == n - 1) ? out : m.pp[i % 2]->get();
+        half *dst = (i == n - 1) ? out : m.pp[i % et_model_s::kRing]->get();
         m.layers[(size_t)i]->forward(dst, src, stream);
         src = dst;
     }
@@ -336,12 +339,10 @@ int et_model_finalize(et_model m) {
             else m->layers.push_back(build_layer_act<base_mat, dense_attn_cfg>(*m, h));
         }
         const size_t act_elems = (size_t)m->rows() * m->desc.emdim;
-        m->pp[0] = std::make_unique<et::DeviceBuffer<half>>(act_elems);
-        m->pp[1] = std::make_unique<et::DeviceBuffer<half>>(act_elems);
+        for (auto &b : m->pp) b = std::make_unique<et::DeviceBuffer<half>>(act_elems);
         m->warm = std::make_unique<et::DeviceBuffer<half>>(act_elems);
         if (m->desc.mixed) {
-            m->pp32[0] = std::make_unique<et::DeviceBuffer<float>>(act_elems);
-            m->pp32[1] = std::make_unique<et::DeviceBuffer<float>>(act_elems);
+            for (auto &b : m->pp32) b = std::make_unique<et::DeviceBuffer<float>>(act_elems);
             for (auto &l : m->layers) l->enable_mixed();
         }
         etChk(et_stream_create(&m->own_stream));
@@ -361,8 +362,8 @@ int et_model_forward_layer(et_model m, int layer, et_f16 *out, const et_f16 *in,
         half *o = reinterpret_cast<half *>(out);
         half *i = reinterpret_cast<half *>(const_cast<et_f16 *>(in));
         if (m->desc.mixed) {  // one layer between binary16 buffers: the residual starts from the binary16 input
-            etChk(et_f16_to_f32(m->pp32[1]->get(), in, (std::size_t)m->rows() * m->desc.emdim, stream));
-            m->layers[(size_t)layer]->forward_mixed(nullptr, o, m->pp32[1]->get(), i, stream);
+            etChk(et_f16_to_f32(m->pp32[0]->get(), in, (std::size_t)m->rows() * m->desc.emdim, stream));
+            m->layers[(size_t)layer]->forward_mixed(nullptr, o, m->pp32[0]->get(), i, stream);
         } else {
             m->layers[(size_t)layer]->forward(o, i, stream);
         }
