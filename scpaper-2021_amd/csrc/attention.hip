@@ -94,6 +94,7 @@ template <int HD> __device__ __forceinline__ constexpr int vt_unit_keys(int kg) 
 // is held to the 168 registers of three resident waves per SIMD; left alone the allocator takes
 // a few more and the third wave is lost, which costs more than the prefetch gains.
 template <int HD, int NW, bool COMPACT, int QT> constexpr bool mha_prefetches() {
+    if (HD == 128 && !COMPACT && NW == 8 && QT == 1) return true;  // 202 registers: two waves per SIMD either way
     return HD <= 64 && !COMPACT && ((NW == 4 && QT == 1) || (NW == 8 && QT == 2));
 }
 template <int HD, int NW, bool COMPACT, int QT> constexpr bool mha_three_waves() {
@@ -912,8 +913,10 @@ static int launch_mha_nw(const MhaArgs &args, hipStream_t stream) {
 // queries and pay once the grid still fills the chip: 8 waves (128 queries) from 256 such
 // workgroups on (2048 keys, 16 x 16 heads: 546 -> 516 us; 128-wide heads 592 -> 570 us), and 8
 // waves with two query tiles each (256 queries; every K and V^T fragment read from LDS feeds two
-// MFMAs) from 512 on (-> 464 us; it needs 214 registers, two waves per SIMD, so 64-wide heads
-// only).  Two tiles on 4 waves lose more to the missing third wave than they save (735 us).
+// MFMAs) from 512 on (-> 464 us; 214 registers, two waves per SIMD).  128-wide heads: the 8-wave
+// form prefetches the next block through registers (565 -> 532 us at 2048 keys, 16 x 8 heads),
+// the two-tile form takes all 256 registers and spills 45, and is still the faster one (503 us).
+// Two tiles on 4 waves lose more to the missing third wave than they save (735 us).
 template <int HD, bool COMPACT>
 static int launch_mha(const MhaArgs &args, int B, hipStream_t stream) {
     (void)B;
@@ -921,6 +924,8 @@ static int launch_mha(const MhaArgs &args, int B, hipStream_t stream) {
     if (!COMPACT) {
         if (HD == 64 && qblocks % 16 == 0 && (long)args.nbh * (qblocks / 16) >= 512)
             return launch_mha_nw<(HD == 64 ? HD : 64), COMPACT, 8, 2>(args, stream);
+        if (HD == 128 && qblocks % 16 == 0 && (long)args.nbh * (qblocks / 16) >= 512)
+            return launch_mha_nw<(HD == 128 ? HD : 128), COMPACT, 8, 2>(args, stream);
         if (HD >= 64 && qblocks % 8 == 0 && (long)args.nbh * (qblocks / 8) >= 256)
             return launch_mha_nw<HD, COMPACT, 8, 1>(args, stream);
     }

@@ -354,7 +354,7 @@ def run_scale(b: Bench):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--set", choices=("configs", "scale", "vo", "all"), default="all")
+    ap.add_argument("--set", choices=("configs", "scale", "vo", "mha", "all"), default="all")
     ap.add_argument("--json", default=None, help="also write the rows as JSON to this file")
     args = ap.parse_args()
     b = Bench()
@@ -362,6 +362,17 @@ def main():
     if args.set in ("configs", "all"):
         print("# shapes of the benchmark configurations")
         run_configs(b)
+    if args.set == "mha":
+        print("# fused attention from the benchmark shape to 2048 keys")
+        rng = np.random.default_rng(1)
+        for B in (1, 8, 16):
+            b.mha(B, 128, 12, 64, 50)
+        b.mha(8, 128, 12, 64, 50, lens=rng.integers(64, 129, 8))
+        b.mha(4, 512, 16, 64, 20)
+        b.mha(64, 512, 16, 64, 10)
+        b.mha(16, 2048, 16, 64, 5)
+        b.mha(16, 2048, 8, 128, 5)
+        b.mha(16, 2048, 32, 32, 5)
     if args.set == "vo":
         print("# pre-computed-VO attention: probabilities through memory (mha_vo) and on chip (mha_vo_otf)")
         for B, N in ((1, 768), (4, 384), (8, 768), (16, 768)):

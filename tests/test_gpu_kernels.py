@@ -586,7 +586,9 @@ def test_mha_large_grid(et, causal, padded):
 @pytest.mark.parametrize("B,S,nh,hd,causal", [(6, 768, 32, 64, False),    # 8 waves x 2 tiles, three query strips, six key blocks
                                               (6, 768, 32, 64, True),
                                               (16, 128, 16, 128, False),  # 8 waves x 1 tile with 128-wide heads
-                                              (4, 384, 24, 128, True)])
+                                              (4, 384, 24, 128, True),
+                                              (32, 256, 16, 128, False),  # 8 waves x 2 tiles with 128-wide heads
+                                              (16, 512, 16, 128, True)])
 def test_mha_large_grid_shapes(et, B, S, nh, hd, causal):
     lens = [S - (37 * b) % (S // 2) for b in range(B)]
     got, want = run_mha(et, B, S, nh, hd, seed=64, lens=lens, causal=causal)
