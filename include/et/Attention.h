@@ -229,9 +229,11 @@ class Attention<_config, std::enable_if_t<!_config::isSingleKernel>> : public et
         if constexpr (std::is_same<OTF_attn_Ofused, typename config::attn_t>::value) {
             static_assert(std::is_same<typename config::WO_t, tile_mat>::value,
                           "the O-fused form needs a tile-sparse output projection");
-            Multihead_atttion_fuseO(mat_q->get(), mat_k->get(), mat_v->get(), nullptr, mat_z->get(),
-                                    linearO->weight.row_ptr.get(), linearO->weight.row_offset.get(),
-                                    linearO->weight.data.get(), linearO->bias.get(), model, out, r);
+            // what Multihead_atttion_fuseO does, with the projection through the Linear object (which
+            // may hold a plan or a dense image of its weight)
+            et::fused_mha(mat_q->get(), mat_k->get(), mat_v->get(), model->kdim, model->kdim, model->vdim,
+                          mat_z->get(), model->vdim, *model, r);
+            linearO->forward(out, mat_z->get(), stream);
         } else {
             Multihead_atttion<typename config::attn_t>(mat_q.get(), mat_k.get(), mat_v.get(), mat_qk.get(),
                                                        nullptr, mat_z.get(), model, r);

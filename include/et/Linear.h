@@ -7,6 +7,7 @@
 // kernel's epilogue, and the row/column-pruned forms gather/scatter inside the
 // GEMM instead of the reference's extra passes.  Nothing blocks the host.
 #pragma once
+#include <algorithm>
 #include <memory>
 #include <type_traits>
 #include <utility>
@@ -134,6 +135,16 @@ template <> class Linear<tile_mat> {
     };
     std::unique_ptr<et_bsr_plan_s, PlanDeleter> plan;
     static bool wants_plan(int in, int rows) { return in >= 128 && (in > 5112 || (in >= 3072 && rows >= 4096)); }
+    // Dense image of the weight, held where the dense GEMM is the faster kernel: a matrix that
+    // keeps most of its tiles (measured at 2048 rows: the tile kernel overtakes the dense one at
+    // 35-50 % sparsity for 768-wide inputs, at 55 % for 3072-wide ones).  Not built when a tile
+    // position occurs twice (the tile kernel adds such tiles up, an image cannot).
+    std::unique_ptr<et::DeviceBuffer<half>> dense;
+    std::unique_ptr<et::DeviceBuffer<half>> dense_out16;  // fp16 result ahead of the widening in forward_f32
+    static bool wants_dense(int in, int out, int ntile) {
+        const double kept = (double)ntile * 256.0 / ((double)in * (double)out);
+        return kept > (in >= 3072 ? 0.45 : 0.50);
+    }
 
     Linear(int _in_size, int _out_size, const tile_mat &w, const half *b, int _size)
         : in_size(_in_size), out_size(_out_size), size(_size), weight(w), bias(b, (std::size_t)_out_size) {
@@ -154,6 +165,11 @@ template <> class Linear<tile_mat> {
         forward_act(output, input, ET_ACT_NONE, stream);
     }
     void forward_act(half *output, const half *input, int act, et::stream_t stream = nullptr) {
+        if (dense) {
+            etChk(et_linear_dense_f16(et::f16(dense->get()), et::f16(bias.get()), et::f16(input), et::f16(output), size,
+                                      (int)in_size, (int)out_size, act, stream));
+            return;
+        }
         if (plan) {
             etChk(et_linear_bsr16_planned_f16(plan.get(), et::f16(bias.get()), et::f16(input), et::f16(output), nullptr,
                                               size, act, stream));
@@ -166,6 +182,12 @@ template <> class Linear<tile_mat> {
     // binary32 result (fp16 operands, fp32 accumulator stored unrounded): what the
     // mixed-precision encoder layer adds to its fp32 residual stream
     void forward_f32(float *output, const half *input, et::stream_t stream = nullptr) {
+        if (dense) {  // the dense GEMM stores fp16: widened afterwards
+            if (!dense_out16) dense_out16 = std::make_unique<et::DeviceBuffer<half>>((std::size_t)size * out_size);
+            forward_act(dense_out16->get(), input, ET_ACT_NONE, stream);
+            etChk(et_f16_to_f32(output, et::f16(dense_out16->get()), (std::size_t)size * out_size, stream));
+            return;
+        }
         if (plan) {
             etChk(et_linear_bsr16_planned_f16(plan.get(), et::f16(bias.get()), et::f16(input), nullptr, output, size,
                                               ET_ACT_NONE, stream));
@@ -194,12 +216,35 @@ template <> class Linear<tile_mat> {
         et::require(weight.blk_row_num * 16 == (int)out_size && weight.blk_col_num * 16 == (int)in_size,
                     "Linear<tile_mat>: weight shape does not match in/out sizes");
         et::require(bias.size == out_size, "Linear<tile_mat>: bias must hold out_size values");
+        if (size > 0 && size % 16 == 0 && wants_dense((int)in_size, (int)out_size, weight.num_blk) &&
+            !names_a_position_twice()) {
+            dense = std::make_unique<et::DeviceBuffer<half>>((std::size_t)in_size * out_size);
+            etChk(et_bsr16_to_dense_f16(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
+                                        et::f16(dense->get()), (int)in_size, (int)out_size, nullptr));
+            etChk(et_device_sync());
+            return;
+        }
         if (size > 0 && size % 16 == 0 && wants_plan((int)in_size, size)) {
             et_bsr_plan p = nullptr;
             etChk(et_bsr16_plan_create(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()), size,
                                        (int)in_size, (int)out_size, 0, 0, 0, &p));
             plan.reset(p);
         }
+    }
+    // true when some block-row lists one column twice, or an index lies outside the matrix (such a
+    // weight stays with the tile kernel, which reports it)
+    bool names_a_position_twice() const {
+        const std::vector<int> rp = weight.row_ptr.to_host(), col = weight.row_offset.to_host();
+        std::vector<char> seen((std::size_t)weight.blk_col_num);
+        for (int r = 0; r + 1 < (int)rp.size(); r++) {
+            if (rp[r] < 0 || rp[r + 1] < rp[r] || rp[r + 1] > (int)col.size()) return true;
+            std::fill(seen.begin(), seen.end(), 0);
+            for (int t = rp[r]; t < rp[r + 1]; t++) {
+                if (col[t] < 0 || col[t] >= weight.blk_col_num || seen[(std::size_t)col[t]]) return true;
+                seen[(std::size_t)col[t]] = 1;
+            }
+        }
+        return false;
     }
 };
 

@@ -310,6 +310,17 @@ int et_vec1x16_to_dense_f16(const int32_t *tile_idx, const int32_t *row_idx,
                             const et_f16 *data, et_f16 *W, int in, int out,
                             et_stream stream);
 
+/* Dense image W[out x in] of a 16x16 BSR weight (device pointers; row_ptr[out/16+1],
+ * col_idx and tiles as for et_linear_bsr16_f16; column-tile indices must be in
+ * range; a position named twice keeps the later tile, so callers with such
+ * weights stay on the tile kernel).  A tile-pruned matrix that keeps most of its
+ * tiles is a dense matrix with holes: Linear<tile_mat> runs the dense GEMM on this
+ * image below 50 % sparsity (55 % for inputs of 3072 and wider), where that is
+ * the faster kernel.  No counterpart in the reference. */
+int et_bsr16_to_dense_f16(const int32_t *row_ptr, const int32_t *col_idx,
+                          const et_f16 *tiles, et_f16 *W, int in, int out,
+                          et_stream stream);
+
 /* Unstructured CSR weight over [out x in] (indices need not be sorted inside a
  * row).  T may be any size; out % 4 == 0.  Replaces Linear<csr_mat>::forward
  * (Linear/cusp.cu:23-82, cusparseSpMM + bias map); no workspace is allocated. */

@@ -98,6 +98,7 @@ _SIGNATURES = {
     "et_fill_rows_bias_f16": (_vp, _vp, _i, _i, _vp),
     "et_linear_vec1x16_f16": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_vec1x16_to_dense_f16": (_vp, _vp, _vp, _vp, _i, _i, _vp),
+    "et_bsr16_to_dense_f16": (_vp, _vp, _vp, _vp, _i, _i, _vp),
     "et_linear_csr_f16": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_mha_compactv_f16": (_vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i,
                             _f, _i, _vp),

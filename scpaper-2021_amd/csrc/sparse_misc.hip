@@ -117,6 +117,21 @@ __global__ __launch_bounds__(256) void vec1x16_expand_kernel(const int32_t *tile
     }
 }
 
+// Dense image of a 16x16 BSR weight: one workgroup per block-row clears its 16 rows of W, then
+// copies the block-row's tiles to their columns (thread t holds element t of every tile).  A
+// position named twice keeps the later tile.
+__global__ __launch_bounds__(256) void bsr16_expand_kernel(const int32_t *row_ptr, const int32_t *col_idx,
+                                                           const _Float16 *tiles, _Float16 *W, int in) {
+    const int rb = blockIdx.x;
+    _Float16 *blk = W + (size_t)rb * 16 * in;
+    const h8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int v = threadIdx.x; v < 2 * in; v += 256) reinterpret_cast<h8 *>(blk)[v] = zero8;  // 16 rows x in / 8 vectors
+    __syncthreads();  // the zeros of other threads are ordered before this thread's tile elements
+    const int lo = row_ptr[rb], hi = row_ptr[rb + 1];
+    const int i = threadIdx.x >> 4, j = threadIdx.x & 15;
+    for (int t = lo; t < hi; t++) blk[(size_t)i * in + col_idx[t] * 16 + j] = tiles[(size_t)t * 256 + threadIdx.x];
+}
+
 // ------------------------------------------------------------------- CSR ----
 struct CsrArgs {
     const int32_t *indptr, *indices;
@@ -214,6 +229,17 @@ int et_vec1x16_to_dense_f16(const int32_t *tile_idx, const int32_t *row_idx, con
     vec1x16_expand_kernel<<<dim3((unsigned)((ncell + 3) / 4)), 256, 0, as_stream(stream)>>>(
         tile_idx, row_idx, H(data), H(W), in, (int)ncell);
     return check_launch("vec1x16_expand_kernel");
+}
+
+int et_bsr16_to_dense_f16(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles, et_f16 *W, int in,
+                          int out, et_stream stream) {
+    ET_REQUIRE(row_ptr && col_idx && tiles && W, ET_ERR_INVALID_ARG, "et_bsr16_to_dense_f16: NULL pointer");
+    ET_REQUIRE(in > 0 && out > 0 && in % 16 == 0 && out % 16 == 0, ET_ERR_UNSUPPORTED,
+               "et_bsr16_to_dense_f16: in=%d out=%d must be positive multiples of 16", in, out);
+    ET_REQUIRE((reinterpret_cast<uintptr_t>(W) & 15) == 0, ET_ERR_UNSUPPORTED,
+               "et_bsr16_to_dense_f16: W must be 16-byte aligned");
+    bsr16_expand_kernel<<<dim3((unsigned)(out / 16)), 256, 0, as_stream(stream)>>>(row_ptr, col_idx, H(tiles), H(W), in);
+    return check_launch("bsr16_expand_kernel");
 }
 
 int et_linear_vec1x16_f16(const int32_t *tile_idx, const int32_t *row_idx, const et_f16 *data,

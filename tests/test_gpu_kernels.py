@@ -170,6 +170,18 @@ def test_linear_bsr16(et, T, inp, out, sp, act):
     assert err <= 4e-3
 
 
+@pytest.mark.parametrize("inp,out,sp", [(256, 128, 0.0), (768, 3072, 0.3), (3072, 768, 0.5), (64, 16, 0.9)])
+def test_bsr16_dense_image(et, inp, out, sp):
+    """The dense image the class multiplies with for weights that keep most of their tiles."""
+    w = Hn.BsrWeight(out, inp, sp, seed=71)
+    d_w = et.DeviceBuffer.empty((out, inp), np.float16)
+    et.check(et.lib().et_fill_f16(d_w.ptr, out * inp, 0x7E00, None))
+    et.check(et.lib().et_bsr16_to_dense_f16(up(et, w.row_ptr).ptr, up(et, w.col_idx).ptr, up(et, w.tiles).ptr, d_w.ptr,
+                                            inp, out, None))
+    want = F.bsr16_to_dense(w.row_ptr, w.col_idx, w.tiles, inp).astype(np.float16)
+    assert np.array_equal(d_w.numpy(), want)
+
+
 @pytest.mark.parametrize("T,inp,out,sp,act", [(1024, 768, 768, 0.8, 0), (1024, 3072, 768, 0.8, 0), (2048, 4096, 1024, 0.9, 0),
                                               (48, 64, 32, 0.3, 2), (64, 6144, 64, 0.5, 1), (4096, 768, 3072, 0.8, 2)])
 def test_linear_bsr16_f32_output(et, T, inp, out, sp, act):
