@@ -206,16 +206,6 @@ int et_norm_from_stats_f16(et_f16 *out, const et_f16 *V, const et_f16 *skip,
                            const et_f16 *beta, int rows, int H, float eps,
                            et_stream stream);
 
-/* Tuning hook: et_linear_bsr16_f16 with an explicit launch geometry — mt in
- * {1,2,4} 16-token blocks per workgroup strip, stage != 0 keeps the strip of X
- * in LDS, threads per workgroup (multiple of 64, <= 512) and block-rows of W per
- * workgroup.  Same result as et_linear_bsr16_f16; no reference counterpart. */
-int et_linear_bsr16_f16_geom(const int32_t *row_ptr, const int32_t *col_idx,
-                             const et_f16 *tiles, const et_f16 *bias,
-                             const et_f16 *X, et_f16 *Y, int T, int in, int out,
-                             int act, int mt, int stage, int threads,
-                             int rows_per_wg, et_stream stream);
-
 /* Dense weight W[out x in] row-major.  Replaces Linear<base_mat>::forward
  * (Linear/Linear.h:53-64) = cuBLAS_mmul (mycublas/cublas.cu:4-22) + bias map. */
 int et_linear_dense_f16(const et_f16 *W, const et_f16 *bias, const et_f16 *X,

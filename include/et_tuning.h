@@ -1,0 +1,29 @@
+/*
+ * et_tuning.h — entry points for tuning experiments.  Not part of the drop-in
+ * boundary (that is et_abi.h): nothing in the class layer calls them and a
+ * binding does not need them.  Exported by the same library.
+ */
+#ifndef ET_TUNING_H
+#define ET_TUNING_H
+
+#include "et_abi.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Tuning hook: et_linear_bsr16_f16 with an explicit launch geometry — mt in
+ * {1,2,4} 16-token blocks per workgroup strip, stage != 0 keeps the strip of X
+ * in LDS, threads per workgroup (multiple of 64, <= 512) and block-rows of W per
+ * workgroup.  Same result as et_linear_bsr16_f16; no reference counterpart. */
+int et_linear_bsr16_f16_geom(const int32_t *row_ptr, const int32_t *col_idx,
+                             const et_f16 *tiles, const et_f16 *bias,
+                             const et_f16 *X, et_f16 *Y, int T, int in, int out,
+                             int act, int mt, int stage, int threads,
+                             int rows_per_wg, et_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* ET_TUNING_H */

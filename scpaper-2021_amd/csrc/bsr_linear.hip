@@ -29,6 +29,7 @@
 // Tile order inside a block-row is free (the sum commutes), as in the
 // reference kernel (Linear/SPMM_tile.cu:277-283).
 #include "common.hip.h"
+#include "../../include/et_tuning.h"
 
 namespace et {
 

@@ -17,7 +17,7 @@ def load_table():
 
 
 def header_declarations():
-    text = (ROOT / "include" / "et_abi.h").read_text()
+    text = "\n".join(h.read_text() for h in sorted((ROOT / "include").glob("*.h")))  # et_abi.h, et_tuning.h
     text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
     text = re.sub(r"//[^\n]*", " ", text)
     decls = {}

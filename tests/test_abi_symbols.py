@@ -1,4 +1,4 @@
-"""The native library loads without a GPU and exports every symbol include/et_abi.h declares."""
+"""The native library loads without a GPU and exports every symbol the headers include/*.h declare."""
 import ctypes
 import re
 from pathlib import Path
@@ -7,7 +7,7 @@ ROOT = Path(__file__).resolve().parent.parent
 
 
 def declared_symbols():
-    text = (ROOT / "include" / "et_abi.h").read_text()
+    text = "\n".join(h.read_text() for h in sorted((ROOT / "include").glob("*.h")))  # et_abi.h, et_tuning.h
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)  # comments cite names that are not declarations
     return sorted(set(re.findall(r"\b(et_[a-z0-9_]+)\s*\(", text)))
 

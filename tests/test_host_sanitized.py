@@ -19,7 +19,7 @@ CLANG = Path("/opt/rocm/lib/llvm/bin/clang++")
 
 
 def abi_functions() -> list[str]:
-    text = (ROOT / "include" / "et_abi.h").read_text()
+    text = "\n".join(h.read_text() for h in sorted((ROOT / "include").glob("*.h")))  # et_abi.h, et_tuning.h
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"^\s*(?:const\s+char\s*\*|int|void)\s*(et_\w+)\s*\(", text, flags=re.M)))
 
