@@ -51,7 +51,8 @@ def vo_case(seed, H, nh, N_keep=None):
 
 @pytest.mark.parametrize("B,S,H,nh,pruned", [(1, 128, 768, 12, False), (2, 64, 256, 4, False), (2, 64, 256, 4, True),
                                              (9, 48, 96, 3, True), (2, 272, 256, 2, False), (1, 128, 512, 8, False),
-                                             (8, 128, 768, 12, False)])
+                                             (8, 128, 768, 12, False), (2, 64, 96, 2, False), (1, 32, 64, 4, True),
+                                             (2, 96, 288, 3, True)])
 def test_vo_attention(et, B, S, H, nh, pruned):
     """Linear_VO + probabilities + one GEMM per sequence == the oracle's sum_h P_h VO_h + b_O, and so
     does the kernel that keeps the probabilities on chip."""
