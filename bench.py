@@ -109,10 +109,11 @@ def build_layers(et):
     return [LayerWeights(et, 100 + i) for i in range(NLAYER)]
 
 
-def build_model(et, layers, use_graph):
+def build_model(et, layers, use_graph, mixed=1):
     # mixed precision: fp16 matrix-core operands, fp32 accumulation, fp32 residual stream / LayerNorm / softmax
+    # (1: SkipLayerNorm folded into the neighbouring projections, 2: launched on its own)
     m = et.Model(H, NH, FF, S, NLAYER, batch=B, act=et.ACT_GELU, eps=1e-5, causal=False, use_graph=use_graph,
-                 mixed=True)
+                 mixed=mixed)
     for i, w in enumerate(layers):
         for which, tw in ((et.W_QKV, w.qkv), (et.W_O, w.o), (et.W_FF1, w.l1), (et.W_FF2, w.l2)):
             m.set_bsr16(i, which, tw.row_ptr, tw.col_idx, tw.tiles, tw.bias)
@@ -264,6 +265,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--eager", action="store_true", help="launch kernel by kernel instead of replaying a graph")
+    ap.add_argument("--separate-ln", action="store_true",
+                    help="SkipLayerNorm as launches of its own (seven launches per layer) instead of folded into the "
+                         "neighbouring projections (five)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain streaming kernel of known size (ReLU over 64 MiB in, 64 MiB out) "
                          "three times, as the reference point for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
@@ -276,7 +280,7 @@ def main():
     et.lib()  # fails loudly if the native library is missing
 
     layers = build_layers(et)
-    model = build_model(et, layers, use_graph=not args.eager)
+    model = build_model(et, layers, use_graph=not args.eager, mixed=2 if args.separate_ln else 1)
     x = np.random.default_rng(4).standard_normal((B * S, H), dtype=np.float32).astype(np.float16)
     d_in = et.DeviceBuffer.from_numpy(x)
     d_out = et.DeviceBuffer.empty((B * S, H), np.float16)

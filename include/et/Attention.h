@@ -135,6 +135,17 @@ template <> struct __matv_helper<Prune_attn> { using type = col_mat; };
 
 namespace et {
 
+// A binary32 sum (projection + bias + residual) that still has to be normalised, as one layer hands
+// it to the next in the split-normalisation form: the sum, its row sums per block-row group, and
+// the SkipLayerNorm parameters to apply.
+struct SplitSum {
+    const float *v = nullptr;
+    const float *stats = nullptr;
+    int groups = 0;
+    const half *gamma = nullptr, *beta = nullptr;
+    float eps = 1e-5f;
+};
+
 // Mask / padding state shared by both Attention forms and FusedAttention.
 class AttnState {
   public:
@@ -289,6 +300,37 @@ class Attention<_config, std::enable_if_t<_config::isSingleKernel>> : public et:
         half *V = K + model->kdim;
         et::fused_mha(Q, K, V, ldm, ldm, ldm, mat_z->get(), model->vdim, *model, run(stream));
         linearO->forward(out, mat_z->get(), stream);
+    }
+
+    // Split normalisation (mixed-precision layer, tile-sparse projections): the QKV projection
+    // normalises the un-normalised result of the previous layer (`in`, or takes x16 when there is
+    // none), the output projection adds the residual — that normalisation again, formed in its
+    // epilogue, or x32 — and leaves the binary32 sum v1 with its row sums.
+    bool split_ok() const {
+        if constexpr (std::is_same<linearQKV_t, Linear<tile_mat>>::value && std::is_same<linearO_t, Linear<tile_mat>>::value)
+            return linearQKV->split_consumer_ok() && linearO->split_producer_ok();
+        else
+            return false;
+    }
+    void forward_split(float *v1, float *stats1, int *groups1, float *fin_in, const et::SplitSum *in, const float *x32,
+                       half *x16, et::stream_t stream = nullptr) {
+        if constexpr (std::is_same<linearQKV_t, Linear<tile_mat>>::value && std::is_same<linearO_t, Linear<tile_mat>>::value) {
+            if (in)
+                linearQKV->forward_norm_f32in(mat_qkv->get(), in->v, in->stats, in->groups, in->gamma, in->beta,
+                                              in->eps, fin_in, nullptr, nullptr, ET_ACT_NONE, stream);
+            else
+                linearQKV->forward(mat_qkv->get(), x16, stream);
+            const int ldm = model->kdim * 2 + model->vdim;
+            half *Q = mat_qkv->get();
+            half *K = Q + model->kdim;
+            half *V = K + model->kdim;
+            et::fused_mha(Q, K, V, ldm, ldm, ldm, mat_z->get(), model->vdim, *model, run(stream));
+            linearO->forward_resid_stats_f32(v1, stats1, groups1, mat_z->get(), in ? in->v : x32, in ? fin_in : nullptr,
+                                             in ? in->gamma : nullptr, in ? in->beta : nullptr, stream);
+        } else {
+            (void)v1; (void)stats1; (void)groups1; (void)fin_in; (void)in; (void)x32; (void)x16; (void)stream;
+            et::require(false, "Attention: the split normalisation needs tile-sparse projections");
+        }
     }
 
     // the same with the output projection stored as binary32 (mixed-precision layer)

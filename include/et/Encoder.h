@@ -135,7 +135,64 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
         LN2->forward_mixed(out32, out16, temp_ffn32->get(), temp_LN32->get(), rows, stream);
     }
 
+    // Split normalisation: five launches per layer, no SkipLayerNorm launch and no normalised
+    // activation in memory.  The layer takes the previous layer's un-normalised result (or, first
+    // layer, the input in both forms) and returns its own; finish_split() normalises the last one.
+    // Same values as forward_mixed up to the rounding of the row statistics (sum and sum of squares
+    // per block-row group, fp32, instead of a two-pass variance).
+    bool split_ok() const {
+        if constexpr (attn_has_split<attn_t>::value && std::is_same_v<linear1_t, Linear<tile_mat>> &&
+                      std::is_same_v<linear2_t, Linear<tile_mat>>)
+            return attn->split_ok() && linear1->split_consumer_ok() && linear2->split_producer_ok();
+        else
+            return false;
+    }
+    void enable_split() {
+        enable_mixed();
+        const std::size_t st = (std::size_t)16 * rows * 2;  // room for 16 block-row groups
+        if (!stats1) stats1 = std::make_unique<DeviceBuffer<float>>(st);
+        if (!stats2) stats2 = std::make_unique<DeviceBuffer<float>>(st);
+        if (!fin_in) fin_in = std::make_unique<DeviceBuffer<float>>((std::size_t)rows * 2);
+        if (!fin1) fin1 = std::make_unique<DeviceBuffer<float>>((std::size_t)rows * 2);
+    }
+    SplitSum forward_split(const SplitSum *in, const float *x32, half *x16, stream_t stream = nullptr) {
+        SplitSum out;
+        if constexpr (attn_has_split<attn_t>::value && std::is_same_v<linear1_t, Linear<tile_mat>> &&
+                      std::is_same_v<linear2_t, Linear<tile_mat>>) {
+            require(stats1 && stats2 && fin_in && fin1, "Encoder: call enable_split() before forward_split()");
+            int g1 = 0, g2 = 0;
+            attn->forward_split(temp_attn32->get(), stats1->get(), &g1, fin_in->get(), in, x32, x16, stream);
+            linear1->forward_norm_f32in(temp_linear.get(), temp_attn32->get(), stats1->get(), g1,
+                                        LN1->gamma(), LN1->beta(), LN1->epsilon(), fin1->get(), nullptr, nullptr,
+                                        act_code<ACT_OP_t>(), stream);
+            linear2->forward_resid_stats_f32(temp_ffn32->get(), stats2->get(), &g2, temp_linear.get(),
+                                             temp_attn32->get(), fin1->get(), LN1->gamma(), LN1->beta(), stream);
+            out.v = temp_ffn32->get();
+            out.stats = stats2->get();
+            out.groups = g2;
+            out.gamma = LN2->gamma();
+            out.beta = LN2->beta();
+            out.eps = LN2->epsilon();
+        } else {
+            (void)in; (void)x32; (void)x16; (void)stream;
+            require(false, "Encoder: the split normalisation needs tile-sparse projections");
+        }
+        return out;
+    }
+    void finish_split(float *out32, half *out16, const SplitSum &s, stream_t stream = nullptr) {
+        etChk(et_norm_from_stats_f32in(out32, f16(out16), s.v, s.stats, s.groups, f16(s.gamma), f16(s.beta), rows,
+                                       model->emdim, s.eps, stream));
+    }
+
   private:
+    std::unique_ptr<DeviceBuffer<float>> stats1, stats2, fin_in, fin1;
+    template <typename A, typename = void> struct attn_has_split : std::false_type {};
+    template <typename A>
+    struct attn_has_split<A, std::void_t<decltype(std::declval<A &>().forward_split(
+                                 static_cast<float *>(nullptr), static_cast<float *>(nullptr), static_cast<int *>(nullptr),
+                                 static_cast<float *>(nullptr), static_cast<const SplitSum *>(nullptr),
+                                 static_cast<const float *>(nullptr), static_cast<half *>(nullptr),
+                                 static_cast<stream_t>(nullptr)))>> : std::true_type {};
     template <typename A, typename = void> struct attn_has_f32 : std::false_type {};
     template <typename A>
     struct attn_has_f32<A, std::void_t<decltype(std::declval<A &>().forward_f32(

@@ -197,6 +197,34 @@ template <> class Linear<tile_mat> {
                                          et::f16(bias.get()), et::f16(input), output, size, (int)in_size,
                                          (int)out_size, ET_ACT_NONE, stream));
     }
+    // The split normalisation of the mixed-precision layer (et_linear_bsr16_resid_stats_f32 /
+    // et_norm_linear_bsr16_f32in): this Linear as the producer of a binary32 sum with its row
+    // sums, or as the consumer that normalises such a sum while it stages its token strip.
+    bool split_producer_ok() const {
+        return !dense && !plan && size > 0 && et_linear_bsr16_resid_stats_f32_supported(size, (int)in_size, (int)out_size) == 1;
+    }
+    bool split_consumer_ok() const {
+        return !dense && !plan && size > 0 && et_norm_linear_bsr16_f32in_supported(size, (int)in_size, (int)out_size) == 1;
+    }
+    // V = input W^T + bias + residual (binary32) and stats[*groups][size][2]; the residual is
+    // `resid` itself, or with resid_fin its normalisation by (resid_fin, resid_gamma, resid_beta)
+    void forward_resid_stats_f32(float *V, float *stats, int *groups, const half *input, const float *resid,
+                                 const float *resid_fin, const half *resid_gamma, const half *resid_beta,
+                                 et::stream_t stream = nullptr) {
+        etChk(et_linear_bsr16_resid_stats_f32(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
+                                              et::f16(bias.get()), et::f16(input), resid, resid_fin, et::f16(resid_gamma),
+                                              et::f16(resid_beta), V, stats, groups, size, (int)in_size, (int)out_size,
+                                              stream));
+    }
+    // output = act(normalised(V) W^T + bias); fin_out, ln32, ln16 optional (null = not wanted)
+    void forward_norm_f32in(half *output, const float *V, const float *stats, int groups, const half *gamma,
+                            const half *beta, float eps, float *fin_out, float *ln32, half *ln16, int act,
+                            et::stream_t stream = nullptr) {
+        etChk(et_norm_linear_bsr16_f32in(V, stats, groups, et::f16(gamma), et::f16(beta), eps, fin_out, ln32, et::f16(ln16),
+                                         weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
+                                         et::f16(bias.get()), et::f16(output), size, (int)in_size, (int)out_size, act,
+                                         stream));
+    }
     // ln_out = ln(src + skip); output = act(ln_out * W^T + bias) in one launch: the
     // SkipLayerNorm -> Linear -> activation sequence of Encoder/Encoder.h:85-89.  LN_t is
     // SkipLayerNorm (gamma(), beta(), epsilon(), width()).

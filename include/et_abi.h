@@ -206,6 +206,51 @@ int et_norm_from_stats_f16(et_f16 *out, const et_f16 *V, const et_f16 *skip,
                            const et_f16 *beta, int rows, int H, float eps,
                            et_stream stream);
 
+/* The same split in the mixed-precision layer, where the residual stream is binary32:
+ *
+ *   et_linear_bsr16_resid_stats_f32   V = X W^T + bias + resid, binary32, unrounded (X
+ *       binary16 [T x in], resid and V binary32 [T x out]), and per token the sum and the
+ *       sum of squares of V over each of *stat_groups block-row groups:
+ *       stats[stat_groups][T][2] (room for 16 groups).  With resid_fin != NULL the residual
+ *       is not read but formed: the normalisation of `resid` (then the V of an earlier
+ *       producer) with the row statistics resid_fin[T][2] (mean, rstd — what the consumer of
+ *       that V left in fin_out) and resid_gamma / resid_beta: the rows the consumer formed
+ *       from the same data, which therefore never have to be stored.
+ *   et_norm_linear_bsr16_f32in        ln = (V - mean) * rstd * gamma + beta from those sums,
+ *       formed while the token strip is staged; Y = act(ln W^T + bias) with ln rounded to
+ *       binary16 as the matrix-core operand.
+ *       Optional results (NULL = not wanted): fin_out
+ *       [T][2] = mean and rstd of every row; ln_out32 / ln_out16 = the normalised rows as
+ *       binary32 / binary16 (each row written by one workgroup).
+ *   et_norm_from_stats_f32in          the normalisation alone (after the last layer).
+ *
+ * A layer then runs QKV (normalising the previous layer's sum), attention, O projection
+ * (+ residual, sums), FFN-up (normalising) and FFN-down (+ residual, sums): five launches,
+ * no SkipLayerNorm launch, and no normalised activation is ever written to memory.  The
+ * *_supported functions return 1 when the shape is taken (the token strip must fit in
+ * LDS).  Encoder/Encoder.h:85-92 with SkipLayerNorm (SkipLayerNorm/SkipLayerNorm.cu:73-82)
+ * folded into its neighbours. */
+int et_linear_bsr16_resid_stats_f32_supported(int T, int in, int out);
+int et_norm_linear_bsr16_f32in_supported(int T, int in, int out);
+int et_linear_bsr16_resid_stats_f32(const int32_t *row_ptr, const int32_t *col_idx,
+                                    const et_f16 *tiles, const et_f16 *bias,
+                                    const et_f16 *X, const float *resid,
+                                    const float *resid_fin, const et_f16 *resid_gamma,
+                                    const et_f16 *resid_beta, float *V, float *stats,
+                                    int *stat_groups, int T, int in, int out,
+                                    et_stream stream);
+int et_norm_linear_bsr16_f32in(const float *V, const float *stats, int stat_groups,
+                               const et_f16 *gamma, const et_f16 *beta, float eps,
+                               float *fin_out, float *ln_out32, et_f16 *ln_out16,
+                               const int32_t *row_ptr,
+                               const int32_t *col_idx, const et_f16 *tiles,
+                               const et_f16 *bias, et_f16 *Y, int T, int in, int out,
+                               int act, et_stream stream);
+int et_norm_from_stats_f32in(float *out32, et_f16 *out16, const float *V,
+                             const float *stats, int stat_groups, const et_f16 *gamma,
+                             const et_f16 *beta, int rows, int H, float eps,
+                             et_stream stream);
+
 /* Dense weight W[out x in] row-major.  Replaces Linear<base_mat>::forward
  * (Linear/Linear.h:53-64) = cuBLAS_mmul (mycublas/cublas.cu:4-22) + bias map. */
 int et_linear_dense_f16(const et_f16 *W, const et_f16 *bias, const et_f16 *X,
@@ -517,10 +562,13 @@ typedef struct et_model_desc {
     float eps;     /* LayerNorm epsilon; <= 0 selects 1e-5                        */
     int causal;    /* != 0: causal mask (the reference's hard-wired one)          */
     int use_graph; /* != 0: replay a captured HIP graph; 0: launch kernel by kernel */
-    int mixed;     /* != 0: mixed precision — the residual stream (layer inputs, the two
+    int mixed;     /* 1 or 2: mixed precision — the residual stream (layer inputs, the two
                     * projections that feed a SkipLayerNorm, both SkipLayerNorm results)
                     * is kept in binary32 inside the stack, binary16 only as matrix-core
                     * operands; input and output of et_model_forward stay binary16.
+                    * 1: SkipLayerNorm is folded into the neighbouring tile-sparse projections
+                    *    where the shapes allow (five launches per layer); 2: it keeps its own
+                    *    launches (seven).
                     * 0: every activation is stored as binary16 (the reference's storage) */
 } et_model_desc;
 

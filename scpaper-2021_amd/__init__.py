@@ -99,6 +99,11 @@ _SIGNATURES = {
     "et_linear_vec1x16_f16": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_vec1x16_to_dense_f16": (_vp, _vp, _vp, _vp, _i, _i, _vp),
     "et_bsr16_to_dense_f16": (_vp, _vp, _vp, _vp, _i, _i, _vp),
+    "et_linear_bsr16_resid_stats_f32_supported": (_i, _i, _i),
+    "et_norm_linear_bsr16_f32in_supported": (_i, _i, _i),
+    "et_linear_bsr16_resid_stats_f32": (_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp),
+    "et_norm_linear_bsr16_f32in": (_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_norm_from_stats_f32in": (_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _f, _vp),
     "et_linear_csr_f16": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_mha_compactv_f16": (_vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i,
                             _f, _i, _vp),

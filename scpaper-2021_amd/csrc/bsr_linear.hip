@@ -62,10 +62,27 @@ struct BsrArgs {
     // binary32 result: when set, act(acc + bias) is stored here unrounded (16 bytes per lane)
     // and Y is not written — the mixed-precision layer keeps its residual stream in fp32
     float *Y32;
+    // binary32 forms of the split normalisation (mixed-precision layer).  RES with kFxRes32: the sum
+    // acc + bias + resid32 is stored unrounded to Y32 and the row sums are taken over it (Y, resid
+    // unused).  NORM with kFxNorm32: the strip comes from X32 (that stored sum; ln_skip unused) and
+    // the normalised rows go to ln_out32 and / or ln_out (either may be null), each row written by
+    // one of the strip's block-row groups.
+    const float *resid32;
+    const float *X32;
+    float *ln_out32;
+    // RES32: when rs_fin is set the residual is not read but formed, as the normalisation of
+    // resid32 with these row statistics and affine vectors (what a consumer launched with
+    // kFxNorm32 formed from the same data): the normalised rows then never have to be stored.
+    const float *rs_fin;  // [T][2]: mean and rstd of every row of resid32, as a consumer left them in fin_out
+    const _Float16 *rs_gamma, *rs_beta;
+    // NORM32: when set, block-row group 0 stores mean and rstd of the rows of its strip here, [T][2]
+    float *fin_out;
 };
 
 constexpr int kFxNorm = 1;
 constexpr int kFxRes = 2;
+constexpr int kFxNorm32 = 4;  // with kFxNorm: binary32 strip
+constexpr int kFxRes32 = 8;   // with kFxRes: binary32 residual and result
 
 constexpr int kXcds = 8;      // accelerator dies, each with a private L2
 constexpr int kLdsPad = 8;    // halfs
@@ -98,7 +115,13 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     static_assert(!(FX & kFxNorm) || (STAGE && !LN), "the NORM prologue writes the strip to LDS");
     constexpr bool NORM = (FX & kFxNorm) != 0;
     constexpr bool RES = (FX & kFxRes) != 0;
-    constexpr int kNB = (LN || NORM) ? kGroupsAheadNorm : kGroupsAhead;  // row groups resident per wave
+    constexpr bool NORM32 = (FX & kFxNorm32) != 0;
+    static_assert(!NORM32 || NORM, "kFxNorm32 qualifies kFxNorm");
+    constexpr bool RES32 = (FX & kFxRes32) != 0;
+    static_assert(!RES32 || RES, "kFxRes32 qualifies kFxRes");
+    // row groups resident per wave: four; two in the kernels whose prologue normalises fp16 strips
+    // (four would spill), three with a binary32 strip or a binary32 residual in flight per group
+    constexpr int kNB = (NORM32 || RES32) ? 3 : (LN || NORM) ? kGroupsAheadNorm : kGroupsAhead;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     _Float16 *xs = reinterpret_cast<_Float16 *>(smem_raw);
 
@@ -145,26 +168,42 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     const int total_vec = STAGE ? rows_here * vec_per_row : 0;
     const h8 *src = reinterpret_cast<const h8 *>(a.X + (size_t)tok0 * a.in);
     h8 sv[kStageU];
-    if (STAGE && !LN) {
+    if (STAGE && !LN && !NORM32) {
         // unconditional loads, index clamped into the strip: a load under a branch gets a
         // basic block of its own and the register allocator's copies there make the wave
         // wait for it on the spot — a full memory round trip before the weight loads go out
 #pragma unroll
         for (int u = 0; u < kStageU; u++) sv[u] = src[min((int)threadIdx.x + u * nthr, total_vec - 1)];
     }
-    const h8 *src_skip = NORM ? reinterpret_cast<const h8 *>(a.ln_skip + (size_t)tok0 * a.in) : nullptr;
-    h8 sk[NORM ? kStageU : 1];
-    if (NORM) {
+    constexpr bool SKIP16 = NORM && !NORM32;  // a binary16 skip strip is added
+    const h8 *src_skip = SKIP16 ? reinterpret_cast<const h8 *>(a.ln_skip + (size_t)tok0 * a.in) : nullptr;
+    h8 sk[SKIP16 ? kStageU : 1];
+    if (SKIP16) {
 #pragma unroll
         for (int u = 0; u < kStageU; u++) sk[u] = src_skip[min((int)threadIdx.x + u * nthr, total_vec - 1)];
+    }
+    // binary32 strip: a strip vector of 8 values is two 16-byte loads
+    const f4 *src32 = NORM32 ? reinterpret_cast<const f4 *>(a.X32 + (size_t)tok0 * a.in) : nullptr;
+    f4 s32[NORM32 ? kStageU : 1][2];
+    if (NORM32) {
+#pragma unroll
+        for (int u = 0; u < kStageU; u++) {
+            const int v = min((int)threadIdx.x + u * nthr, total_vec - 1);
+            s32[u][0] = src32[2 * v];
+            s32[u][1] = src32[2 * v + 1];
+        }
     }
     // NORM: per-row (mean, rstd) and the affine vectors go to LDS behind the strip
     float2 *stat_lds = reinterpret_cast<float2 *>(xs + MT * 16 * lds_ld);
     _Float16 *gam_lds = reinterpret_cast<_Float16 *>(stat_lds + MT * 16);
     _Float16 *bet_lds = gam_lds + a.in;
     if (NORM) {
-        if ((int)threadIdx.x < rows_here)
-            stat_lds[threadIdx.x] = row_stats(a.st_in, a.st_groups, a.T, tok0 + threadIdx.x, a.in, a.ln_eps);
+        if ((int)threadIdx.x < rows_here) {
+            const float2 st = row_stats(a.st_in, a.st_groups, a.T, tok0 + threadIdx.x, a.in, a.ln_eps);
+            stat_lds[threadIdx.x] = st;
+            if (NORM32 && a.fin_out && group == 0)
+                *reinterpret_cast<float2 *>(a.fin_out + 2 * (size_t)(tok0 + threadIdx.x)) = st;
+        }
         for (int c = threadIdx.x; c < vec_per_row; c += nthr) {
             *reinterpret_cast<h8 *>(gam_lds + c * 8) = reinterpret_cast<const h8 *>(a.ln_gamma)[c];
             *reinterpret_cast<h8 *>(bet_lds + c * 8) = reinterpret_cast<const h8 *>(a.ln_beta)[c];
@@ -205,6 +244,23 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     h8 w[kNB][kSlots];
     int col[kNB][kSlots];
     h4 bias_v[kNB];
+    // RES32: the residual of the block-row an item finishes (requested with the item, so that the
+    // epilogue of the row does not wait for it), with the affine values of its four features
+    f4 rsd[RES32 ? kNB : 1][MT];
+    h4 rgm[RES32 ? kNB : 1], rbt[RES32 ? kNB : 1];
+    auto load_resid = [&](int wave_row, f4 (&rs)[MT], h4 &gm, h4 &bt) {
+        const int f0 = (rb_begin + wave + nwave * wave_row) * 16 + g * 4;
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const int tok = min(tok0 + m * 16 + r16, a.T - 1);
+            rs[m] = *reinterpret_cast<const f4 *>(a.resid32 + (size_t)tok * a.out + f0);
+        }
+        gm = bt = h4{0, 0, 0, 0};
+        if (a.rs_fin) {
+            gm = *reinterpret_cast<const h4 *>(a.rs_gamma + f0);
+            bt = *reinterpret_cast<const h4 *>(a.rs_beta + f0);
+        }
+    };
     int g_row[kNB], g_nsl[kNB];  // resident items: wave row index (-1 = none), slots in the item
     bool g_last[kNB];            // item ends its block-row
     int it_row = 0, it_part = 0;
@@ -252,6 +308,7 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
             bias_v[buf] = h4{0, 0, 0, 0};
             if (a.bias)
                 bias_v[buf] = *reinterpret_cast<const h4 *>(a.bias + (rb_begin + wave + nwave * it_row) * 16 + g * 4);
+            if (RES32) load_resid(it_row, rsd[RES32 ? buf : 0], rgm[RES32 ? buf : 0], rbt[RES32 ? buf : 0]);
         }
         if (last) {
             it_row++;
@@ -337,13 +394,39 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
         if (group == 0) *reinterpret_cast<h8 *>(a.ln_out + (size_t)(tok0 + r) * a.in + c * 8) = o;
         return o;
     };
+    // the same from the binary32 strip; row r of the strip is written back by group r mod ngroups
+    auto strip_value32 = [&](f4 lo, f4 hi, int r, int c) {
+        const float2 st = stat_lds[r];
+        const h8 gm = *reinterpret_cast<const h8 *>(gam_lds + c * 8);
+        const h8 bt = *reinterpret_cast<const h8 *>(bet_lds + c * 8);
+        f4 y0, y1;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            y0[e] = norm_value(lo[e], st.x, st.y, (float)gm[e], (float)bt[e]);
+            y1[e] = norm_value(hi[e], st.x, st.y, (float)gm[4 + e], (float)bt[4 + e]);
+        }
+        const h8 o = {(_Float16)y0[0], (_Float16)y0[1], (_Float16)y0[2], (_Float16)y0[3],
+                      (_Float16)y1[0], (_Float16)y1[1], (_Float16)y1[2], (_Float16)y1[3]};
+        if (r % ngroups == group) {
+            const size_t at = (size_t)(tok0 + r) * a.in + c * 8;
+            if (a.ln_out32) {
+                *reinterpret_cast<f4 *>(a.ln_out32 + at) = y0;
+                *reinterpret_cast<f4 *>(a.ln_out32 + at + 4) = y1;
+            }
+            if (a.ln_out) *reinterpret_cast<h8 *>(a.ln_out + at) = o;
+        }
+        return o;
+    };
     if (STAGE && !LN) {
         const int dr = nthr / vec_per_row, dc = nthr - dr * vec_per_row;  // (row, col) step of +nthr
         int r = threadIdx.x / vec_per_row, c = threadIdx.x - r * vec_per_row;
 #pragma unroll
         for (int u = 0; u < kStageU; u++) {
             const int idx = threadIdx.x + u * nthr;
-            if (idx < total_vec) *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) = strip_value(sv[u], sk[NORM ? u : 0], r, c);
+            if (idx < total_vec)
+                *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) =
+                    NORM32 ? strip_value32(s32[NORM32 ? u : 0][0], s32[NORM32 ? u : 0][1], r, c)
+                           : strip_value(sv[u], sk[SKIP16 ? u : 0], r, c);
             r += dr;
             c += dc;
             if (c >= vec_per_row) {
@@ -353,15 +436,26 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
         }
         for (int base = threadIdx.x + kStageU * nthr; base < total_vec; base += nthr * kStageU) {
 #pragma unroll
-            for (int u = 0; u < kStageU; u++) sv[u] = src[min(base + u * nthr, total_vec - 1)];
-            if (NORM) {
+            for (int u = 0; u < kStageU; u++) {
+                const int v = min(base + u * nthr, total_vec - 1);
+                if (NORM32) {
+                    s32[NORM32 ? u : 0][0] = src32[2 * v];
+                    s32[NORM32 ? u : 0][1] = src32[2 * v + 1];
+                } else {
+                    sv[u] = src[v];
+                }
+            }
+            if (SKIP16) {
 #pragma unroll
                 for (int u = 0; u < kStageU; u++) sk[u] = src_skip[min(base + u * nthr, total_vec - 1)];
             }
 #pragma unroll
             for (int u = 0; u < kStageU; u++) {
                 const int idx = base + u * nthr;
-                if (idx < total_vec) *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) = strip_value(sv[u], sk[NORM ? u : 0], r, c);
+                if (idx < total_vec)
+                    *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) =
+                        NORM32 ? strip_value32(s32[NORM32 ? u : 0][0], s32[NORM32 ? u : 0][1], r, c)
+                               : strip_value(sv[u], sk[SKIP16 ? u : 0], r, c);
                 r += dr;
                 c += dc;
                 if (c >= vec_per_row) {
@@ -401,13 +495,35 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     float st1[MT], st2[MT];  // RES: this lane's sums over the values it wrote, per token block
 #pragma unroll
     for (int m = 0; m < MT; m++) st1[m] = st2[m] = 0.0f;
-    auto flush = [&](int wave_row, h4 bv) {
+    // RES32 with a residual that is formed here: mean and rstd of this lane's token of every block
+    float2 tst[RES32 ? MT : 1];
+    if (RES32 && a.rs_fin) {
+#pragma unroll
+        for (int m = 0; m < MT; m++)
+            tst[RES32 ? m : 0] = *reinterpret_cast<const float2 *>(a.rs_fin + 2 * (size_t)min(tok0 + m * 16 + r16, a.T - 1));
+    }
+    auto flush = [&](int wave_row, h4 bv, const f4 (&rs)[MT], h4 gm, h4 bt) {
         const int f0 = (rb_begin + wave + nwave * wave_row) * 16 + g * 4;
 #pragma unroll
         for (int m = 0; m < MT; m++) {
             if (tok_ok[m]) {
                 const int tok = tok0 + m * 16 + r16;
                 h4 o;
+                if (RES32) {  // the binary32 sum itself is the result
+                    f4 v;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        float rv = rs[m][j];
+                        if (a.rs_fin)  // wave-uniform
+                            rv = norm_value(rv, tst[RES32 ? m : 0].x, tst[RES32 ? m : 0].y, (float)gm[j], (float)bt[j]);
+                        v[j] = acc[m][j] + (float)bv[j] + rv;
+                        st1[m] += v[j];
+                        st2[m] = __builtin_fmaf(v[j], v[j], st2[m]);
+                    }
+                    *reinterpret_cast<f4 *>(a.Y32 + (size_t)tok * a.out + f0) = v;
+                    acc[m] = f4{0.f, 0.f, 0.f, 0.f};
+                    continue;
+                }
                 if (RES) {
                     const h4 rv = *reinterpret_cast<const h4 *>(a.resid + (size_t)tok * a.out + f0);
 #pragma unroll
@@ -457,7 +573,7 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
                                 acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[buf][p0 + q], x[q][m], acc[m], 0, 0, 0);
                     }
                 }
-                if (g_last[buf]) flush(g_row[buf], bias_v[buf]);
+                if (g_last[buf]) flush(g_row[buf], bias_v[buf], rsd[RES32 ? buf : 0], rgm[RES32 ? buf : 0], rbt[RES32 ? buf : 0]);
                 issue_item(buf);  // request the item after next into the buffer just drained
             }
         }
@@ -467,7 +583,10 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
         if (lane_read(rp_hi, r) == lane_read(rp_lo, r)) {
             h4 bv = {0, 0, 0, 0};
             if (a.bias) bv = *reinterpret_cast<const h4 *>(a.bias + (rb_begin + wave + nwave * r) * 16 + g * 4);
-            flush(r, bv);
+            f4 rs[MT];
+            h4 gm = {0, 0, 0, 0}, bt = {0, 0, 0, 0};
+            if (RES32) load_resid(r, rs, gm, bt);
+            flush(r, bv, rs, gm, bt);
         }
     }
     if (RES) {
@@ -615,6 +734,36 @@ static BsrPlan plan_bsr_fx(int T, int in, int out, int fx) {
     return p;
 }
 
+// Geometry of the binary32 split-normalisation kernels: that of plan_bsr (one workgroup per
+// compute unit, 32-row strips where a workgroup still gets five block-rows), staged strips only,
+// a RES producer split over at most kMaxStatGroups block-row groups.
+static BsrPlan plan_bsr_fx32(int T, int in, int out, int fx) {
+    const size_t lds_cap = 160 * 1024;
+    const size_t row_bytes = (size_t)(in + kLdsPad) * sizeof(_Float16);
+    const size_t extra = (fx & kFxNorm) ? (size_t)4 * in : 0;  // gamma and beta
+    const int nbr = out / 16;
+    BsrPlan p{};
+    auto fits = [&](int mt, size_t cap) { return mt * 16 * (row_bytes + sizeof(float2)) + extra <= cap; };
+    auto rows_per_wg_for = [&](int mt) {
+        const int strips = (T + mt * 16 - 1) / (mt * 16);
+        int groups = strips >= 256 ? 1 : 256 / strips;
+        if ((fx & kFxRes) && groups > kMaxStatGroups) groups = kMaxStatGroups;
+        return (nbr + groups - 1) / groups;
+    };
+    p.stage = fits(1, lds_cap);
+    p.mt = (T >= 32 && fits(2, lds_cap / 2) && rows_per_wg_for(2) >= 5) ? 2 : 1;
+    int rpw = rows_per_wg_for(p.mt);
+    p.threads = (rpw <= 6 || rpw == 18) ? 384 : 512;
+    const int cap = kMaxWaveRows * (p.threads / 64);
+    if (rpw > cap) rpw = cap;
+    if ((fx & kFxRes) && (nbr + rpw - 1) / rpw > kMaxStatGroups) p.stage = false;
+    p.rows_per_wg = rpw;
+    p.lds = p.mt * 16 * (row_bytes + sizeof(float2)) + extra;
+    const size_t red = (size_t)(p.threads / 64) * p.mt * 16 * sizeof(float2);
+    if ((fx & kFxRes) && p.lds < red) p.lds = red;
+    return p;
+}
+
 template <int MT, bool STAGE, int ACT, int LN = 0, int FX = 0>
 static int launch_bsr_act(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
     auto kernel = bsr16_linear_kernel<MT, STAGE, ACT, LN, FX>;
@@ -676,6 +825,14 @@ static int dispatch_bsr_fx_act(const BsrArgs &args, const BsrPlan &p, hipStream_
 }
 static int dispatch_bsr_norm(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
     return p.mt == 2 ? dispatch_bsr_fx_act<2, kFxNorm>(args, p, stream) : dispatch_bsr_fx_act<1, kFxNorm>(args, p, stream);
+}
+static int dispatch_bsr_norm32(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
+    return p.mt == 2 ? dispatch_bsr_fx_act<2, kFxNorm | kFxNorm32>(args, p, stream)
+                     : dispatch_bsr_fx_act<1, kFxNorm | kFxNorm32>(args, p, stream);
+}
+static int dispatch_bsr_res32(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
+    return p.mt == 2 ? launch_bsr_act<2, true, ET_ACT_NONE, 0, kFxRes | kFxRes32>(args, p, stream)
+                     : launch_bsr_act<1, true, ET_ACT_NONE, 0, kFxRes | kFxRes32>(args, p, stream);
 }
 static int dispatch_bsr_res(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
     return p.mt == 2 ? launch_bsr_act<2, true, ET_ACT_NONE, 0, kFxRes>(args, p, stream)
@@ -873,6 +1030,93 @@ int et_norm_linear_bsr16_f16(const et_f16 *V, const et_f16 *skip, const float *s
                  stats, stat_groups,
                  nullptr, nullptr};
     return dispatch_bsr_norm(args, p, as_stream(stream));
+}
+
+static bool fx32_shape_ok(int T, int in, int out) {
+    return T > 0 && in > 0 && out > 0 && T % 16 == 0 && in % 16 == 0 && out % 16 == 0;
+}
+int et_linear_bsr16_resid_stats_f32_supported(int T, int in, int out) {
+    return fx32_shape_ok(T, in, out) && plan_bsr_fx32(T, in, out, kFxRes).stage ? 1 : 0;
+}
+int et_norm_linear_bsr16_f32in_supported(int T, int in, int out) {
+    return fx32_shape_ok(T, in, out) && plan_bsr_fx32(T, in, out, kFxNorm).stage ? 1 : 0;
+}
+
+int et_linear_bsr16_resid_stats_f32(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles,
+                                    const et_f16 *bias, const et_f16 *X, const float *resid, const float *resid_fin,
+                                    const et_f16 *resid_gamma, const et_f16 *resid_beta, float *V, float *stats,
+                                    int *stat_groups, int T, int in, int out, et_stream stream) {
+    ET_REQUIRE(resid && V && stats && stat_groups, ET_ERR_INVALID_ARG, "et_linear_bsr16_resid_stats_f32: NULL pointer");
+    ET_REQUIRE(resid_fin == nullptr || (resid_gamma && resid_beta), ET_ERR_INVALID_ARG,
+               "et_linear_bsr16_resid_stats_f32: a residual to normalise needs its affine vectors");
+    ET_REQUIRE(V != resid, ET_ERR_INVALID_ARG, "et_linear_bsr16_resid_stats_f32: V must not alias the residual");
+    ET_REQUIRE(((reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(resid)) & 15) == 0, ET_ERR_UNSUPPORTED,
+               "et_linear_bsr16_resid_stats_f32: V and resid must be 16-byte aligned");
+    int s = bsr_check(row_ptr, col_idx, tiles, X, reinterpret_cast<et_f16 *>(V), T, in, out, ET_ACT_NONE);
+    if (s != ET_OK) return s;
+    BsrPlan p = plan_bsr_fx32(T, in, out, kFxRes);
+    ET_REQUIRE(p.stage, ET_ERR_UNSUPPORTED, "et_linear_bsr16_resid_stats_f32: in=%d out=%d outside the staged range", in,
+               out);
+    *stat_groups = (out / 16 + p.rows_per_wg - 1) / p.rows_per_wg;
+    if (T == 0) return ET_OK;
+    BsrArgs args{};
+    args.row_ptr = row_ptr;
+    args.col_idx = col_idx;
+    args.tiles = reinterpret_cast<const _Float16 *>(tiles);
+    args.bias = reinterpret_cast<const _Float16 *>(bias);
+    args.X = reinterpret_cast<const _Float16 *>(X);
+    args.T = T;
+    args.in = in;
+    args.out = out;
+    args.rows_per_wg = p.rows_per_wg;
+    args.act = ET_ACT_NONE;
+    args.st_out = stats;
+    args.Y32 = V;
+    args.resid32 = resid;
+    args.rs_fin = resid_fin;
+    args.rs_gamma = reinterpret_cast<const _Float16 *>(resid_gamma);
+    args.rs_beta = reinterpret_cast<const _Float16 *>(resid_beta);
+    return dispatch_bsr_res32(args, p, as_stream(stream));
+}
+
+int et_norm_linear_bsr16_f32in(const float *V, const float *stats, int stat_groups, const et_f16 *gamma,
+                               const et_f16 *beta, float eps, float *fin_out, float *ln_out32, et_f16 *ln_out16,
+                               const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles, const et_f16 *bias,
+                               et_f16 *Y, int T, int in, int out, int act, et_stream stream) {
+    ET_REQUIRE(V && stats && gamma && beta, ET_ERR_INVALID_ARG, "et_norm_linear_bsr16_f32in: NULL pointer");
+    ET_REQUIRE(stat_groups >= 1 && stat_groups <= kMaxStatGroups, ET_ERR_INVALID_ARG,
+               "et_norm_linear_bsr16_f32in: stat_groups=%d must be in [1, %d]", stat_groups, kMaxStatGroups);
+    ET_REQUIRE(ln_out32 == nullptr || ln_out32 != V, ET_ERR_INVALID_ARG,
+               "et_norm_linear_bsr16_f32in: ln_out32 must not alias V");
+    ET_REQUIRE(((reinterpret_cast<uintptr_t>(V) | reinterpret_cast<uintptr_t>(ln_out32) |
+                 reinterpret_cast<uintptr_t>(ln_out16)) & 15) == 0,
+               ET_ERR_UNSUPPORTED, "et_norm_linear_bsr16_f32in: V and the outputs must be 16-byte aligned");
+    int s = bsr_check(row_ptr, col_idx, tiles, reinterpret_cast<const et_f16 *>(V), Y, T, in, out, act);
+    if (s != ET_OK) return s;
+    BsrPlan p = plan_bsr_fx32(T, in, out, kFxNorm);
+    ET_REQUIRE(p.stage, ET_ERR_UNSUPPORTED, "et_norm_linear_bsr16_f32in: in=%d outside the staged range", in);
+    if (T == 0) return ET_OK;
+    BsrArgs args{};
+    args.row_ptr = row_ptr;
+    args.col_idx = col_idx;
+    args.tiles = reinterpret_cast<const _Float16 *>(tiles);
+    args.bias = reinterpret_cast<const _Float16 *>(bias);
+    args.Y = reinterpret_cast<_Float16 *>(Y);
+    args.T = T;
+    args.in = in;
+    args.out = out;
+    args.rows_per_wg = p.rows_per_wg;
+    args.act = act;
+    args.ln_gamma = reinterpret_cast<const _Float16 *>(gamma);
+    args.ln_beta = reinterpret_cast<const _Float16 *>(beta);
+    args.ln_out = reinterpret_cast<_Float16 *>(ln_out16);
+    args.ln_eps = eps;
+    args.st_in = stats;
+    args.st_groups = stat_groups;
+    args.X32 = V;
+    args.ln_out32 = ln_out32;
+    args.fin_out = fin_out;
+    return dispatch_bsr_norm32(args, p, as_stream(stream));
 }
 
 // Tuning hook: same computation with an explicit launch geometry.  mt in

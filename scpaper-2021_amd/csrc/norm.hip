@@ -222,6 +222,40 @@ __global__ __launch_bounds__(256) void norm_from_stats_kernel(_Float16 *__restri
     }
 }
 
+// the same from a binary32 sum (no skip: the producer added it), binary32 and / or binary16 result
+__global__ __launch_bounds__(256) void norm_from_stats_f32in_kernel(float *__restrict__ out32, _Float16 *__restrict__ out16,
+                                                                    const float *__restrict__ V,
+                                                                    const float *__restrict__ stats, int groups,
+                                                                    const _Float16 *__restrict__ gamma,
+                                                                    const _Float16 *__restrict__ beta, int rows, int H,
+                                                                    float eps) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int row = blockIdx.x * kRowsPerBlock + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float2 st = row_stats(stats, groups, rows, row, H, eps);
+    const int vecs = H >> 3;
+    const f4 *v = reinterpret_cast<const f4 *>(V + (size_t)row * H);
+    for (int c = lane; c < vecs; c += kWave) {
+        const f4 lo = v[2 * c], hi = v[2 * c + 1];
+        const h8 gm = reinterpret_cast<const h8 *>(gamma)[c], bt = reinterpret_cast<const h8 *>(beta)[c];
+        f4 y0, y1;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            y0[e] = norm_value(lo[e], st.x, st.y, (float)gm[e], (float)bt[e]);
+            y1[e] = norm_value(hi[e], st.x, st.y, (float)gm[4 + e], (float)bt[4 + e]);
+        }
+        if (out32) {
+            f4 *o = reinterpret_cast<f4 *>(out32 + (size_t)row * H);
+            o[2 * c] = y0;
+            o[2 * c + 1] = y1;
+        }
+        if (out16)
+            reinterpret_cast<h8 *>(out16 + (size_t)row * H)[c] =
+                h8{(_Float16)y0[0], (_Float16)y0[1], (_Float16)y0[2], (_Float16)y0[3],
+                   (_Float16)y1[0], (_Float16)y1[1], (_Float16)y1[2], (_Float16)y1[3]};
+    }
+}
+
 template <bool SKIP, typename T>
 static int launch_layernorm(T *out, const T *src, const T *skip, const T *gamma, const T *beta, int rows,
                             int H, float eps, hipStream_t stream) {
@@ -329,6 +363,22 @@ int et_norm_from_stats_f16(et_f16 *out, const et_f16 *V, const et_f16 *skip, con
         reinterpret_cast<const _Float16 *>(skip), stats, stat_groups,
         reinterpret_cast<const _Float16 *>(gamma), reinterpret_cast<const _Float16 *>(beta), rows, H, eps);
     return check_launch("norm_from_stats_kernel");
+}
+
+int et_norm_from_stats_f32in(float *out32, et_f16 *out16, const float *V, const float *stats, int stat_groups,
+                             const et_f16 *gamma, const et_f16 *beta, int rows, int H, float eps, et_stream stream) {
+    ET_REQUIRE((out32 || out16) && V && stats && gamma && beta, ET_ERR_INVALID_ARG,
+               "et_norm_from_stats_f32in: NULL pointer");
+    ET_REQUIRE(rows >= 0 && H > 0, ET_ERR_INVALID_ARG, "et_norm_from_stats_f32in: rows=%d H=%d", rows, H);
+    ET_REQUIRE(stat_groups >= 1 && stat_groups <= kMaxStatGroups, ET_ERR_INVALID_ARG,
+               "et_norm_from_stats_f32in: stat_groups=%d must be in [1, %d]", stat_groups, kMaxStatGroups);
+    ET_REQUIRE(H % 8 == 0, ET_ERR_UNSUPPORTED, "et_norm_from_stats_f32in: H=%d must be a multiple of 8", H);
+    if (rows == 0) return ET_OK;
+    norm_from_stats_f32in_kernel<<<(rows + kRowsPerBlock - 1) / kRowsPerBlock, kWave * kRowsPerBlock, 0,
+                                   as_stream(stream)>>>(out32, reinterpret_cast<_Float16 *>(out16), V, stats, stat_groups,
+                                                        reinterpret_cast<const _Float16 *>(gamma),
+                                                        reinterpret_cast<const _Float16 *>(beta), rows, H, eps);
+    return check_launch("norm_from_stats_f32in_kernel");
 }
 
 int et_skip_layernorm_f32(float *out, const float *src, const float *skip, const float *gamma,

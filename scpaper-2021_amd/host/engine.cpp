@@ -20,6 +20,10 @@ struct ILayer {
     virtual void forward(half *out, half *src, stream_t stream) = 0;
     virtual void enable_mixed() = 0;
     virtual void forward_mixed(float *out32, half *out16, const float *src32, half *src16, stream_t stream) = 0;
+    virtual bool split_ok() const = 0;
+    virtual void enable_split() = 0;
+    virtual et::SplitSum forward_split(const et::SplitSum *in, const float *x32, half *x16, stream_t stream) = 0;
+    virtual void finish_split(float *out32, half *out16, const et::SplitSum &s, stream_t stream) = 0;
     virtual et::AttnState &attn() = 0;
 };
 
@@ -30,6 +34,14 @@ template <typename EncoderT> struct LayerOf final : ILayer {
     void enable_mixed() override { enc->enable_mixed(); }
     void forward_mixed(float *out32, half *out16, const float *src32, half *src16, stream_t stream) override {
         enc->forward_mixed(out32, out16, src32, src16, stream);
+    }
+    bool split_ok() const override { return enc->split_ok(); }
+    void enable_split() override { enc->enable_split(); }
+    et::SplitSum forward_split(const et::SplitSum *in, const float *x32, half *x16, stream_t stream) override {
+        return enc->forward_split(in, x32, x16, stream);
+    }
+    void finish_split(float *out32, half *out16, const et::SplitSum &s, stream_t stream) override {
+        enc->finish_split(out32, out16, s, stream);
     }
     et::AttnState &attn() override { return enc->attention(); }
 };
@@ -69,6 +81,7 @@ struct et_model_s {
     std::vector<int> lens;   // empty = no padding
     std::vector<half> mask;  // empty = no additive mask
     bool finalized = false;
+    bool split = false;  // mixed precision with SkipLayerNorm folded into the projections
 
     stream_t own_stream = nullptr;
     et_graph graph = nullptr;
@@ -156,7 +169,20 @@ void check_layer_index(const et_model_s *m, int layer) {
 
 // Mixed precision: the binary16 input is widened once, every layer hands the next one its result
 // in both forms (binary32 residual, binary16 operand), the last one writes binary16 to `out`.
+// The same with SkipLayerNorm folded into the neighbouring projections (five launches per layer):
+// every layer hands the next one its un-normalised binary32 result with its row sums.
+void run_layers_split(et_model_s &m, half *out, half *in, stream_t stream) {
+    const int n = (int)m.layers.size();
+    const std::size_t elems = (std::size_t)m.rows() * m.desc.emdim;
+    etChk(et_f16_to_f32(m.pp32[0]->get(), et::f16(in), elems, stream));
+    et::SplitSum carry;
+    for (int i = 0; i < n; i++)
+        carry = m.layers[(size_t)i]->forward_split(i ? &carry : nullptr, m.pp32[0]->get(), in, stream);
+    m.layers[(size_t)n - 1]->finish_split(nullptr, out, carry, stream);
+}
+
 void run_layers_mixed(et_model_s &m, half *out, half *in, stream_t stream) {
+    if (m.split) return run_layers_split(m, out, in, stream);
     const int n = (int)m.layers.size();
     const std::size_t elems = (std::size_t)m.rows() * m.desc.emdim;
     constexpr int R = et_model_s::kRing;
@@ -344,6 +370,11 @@ int et_model_finalize(et_model m) {
         if (m->desc.mixed) {
             for (auto &b : m->pp32) b = std::make_unique<et::DeviceBuffer<float>>(act_elems);
             for (auto &l : m->layers) l->enable_mixed();
+            // mixed == 1: the engine folds SkipLayerNorm into the projections where every layer can
+            m->split = m->desc.mixed == 1 && !m->layers.empty();
+            for (auto &l : m->layers) m->split = m->split && l->split_ok();
+            if (m->split)
+                for (auto &l : m->layers) l->enable_split();
         }
         etChk(et_stream_create(&m->own_stream));
         apply_attention_state(*m);

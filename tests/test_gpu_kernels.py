@@ -451,6 +451,89 @@ def test_split_layernorm_between_two_tile_linears(et, T, n_in, n_mid, n_out, sp,
     assert np.array_equal(d_ln2.numpy().view(np.uint16), ln.view(np.uint16))
 
 
+@pytest.mark.parametrize("T,n_in,n_mid,n_out,sp,act", [(1024, 768, 768, 3072, 0.8, 2), (1024, 3072, 768, 2304, 0.8, 0),
+                                                     (48, 256, 512, 64, 0.5, 1), (16, 32, 16, 16, 0.0, 0),
+                                                     (2048, 4096, 1024, 4096, 0.9, 2), (272, 160, 208, 800, 0.5, 0)])
+def test_split_layernorm_binary32_between_two_tile_linears(et, T, n_in, n_mid, n_out, sp, act):
+    """The split normalisation of the mixed-precision layer: the producer stores X W^T + b + residual
+    unrounded with its row sums, the consumer normalises that strip while staging it and writes
+    the normalised rows as binary32 and binary16."""
+    import ctypes as C
+    lib = et.lib()
+    w1 = Hn.BsrWeight(n_mid, n_in, sp, seed=41, bias_std=0.05).upload(et)
+    w2 = Hn.BsrWeight(n_out, n_mid, sp, seed=44, bias_std=0.05).upload(et)
+    x = Hn.randn((T, n_in), 47)
+    resid = Hn.randn((T, n_mid), 48, 1.0, np.float32)
+    gamma = (1 + Hn.randn((n_mid,), 49, 0.1, np.float32)).astype(np.float16)
+    beta = Hn.randn((n_mid,), 50, 0.1)
+    d_v = et.DeviceBuffer.empty((T, n_mid), np.float32)
+    d_stats = et.DeviceBuffer.empty((16, T, 2), np.float32)
+    groups = C.c_int(0)
+    assert lib.et_linear_bsr16_resid_stats_f32_supported(T, n_in, n_mid) == 1
+    assert lib.et_norm_linear_bsr16_f32in_supported(T, n_mid, n_out) == 1
+    et.check(lib.et_linear_bsr16_resid_stats_f32(w1.d_row_ptr.ptr, w1.d_col_idx.ptr, w1.d_tiles.ptr, w1.d_bias.ptr,
+                                                 up(et, x).ptr, up(et, resid).ptr, None, None, None, d_v.ptr,
+                                                 d_stats.ptr, C.byref(groups), T, n_in, n_mid, None))
+    G = groups.value
+    assert 1 <= G <= 16
+    v = d_v.numpy()
+    want_v = L.linear(Hn.f32(x), Hn.f32(w1.dense), Hn.f32(w1.bias)).numpy() + resid
+    assert Hn.max_abs(v, want_v) <= 1e-4 * max(1.0, float(np.abs(want_v).max()))
+    st = d_stats.numpy()[:G].astype(np.float64).sum(0)
+    v64 = v.astype(np.float64)
+    assert np.allclose(st[:, 0], v64.sum(1), rtol=1e-5, atol=1e-3)
+    assert np.allclose(st[:, 1], (v64 * v64).sum(1), rtol=1e-5, atol=1e-3)
+
+    d_ln32 = et.DeviceBuffer.empty((T, n_mid), np.float32)
+    d_ln16 = et.DeviceBuffer.empty((T, n_mid), np.float16)
+    d_y = et.DeviceBuffer.empty((T, n_out), np.float16)
+    et.check(lib.et_fill_f16(d_ln16.ptr, T * n_mid, 0x7E00, None))
+    d_g, d_b = up(et, gamma), up(et, beta)
+    d_fin = et.DeviceBuffer.empty((T, 2), np.float32)
+    et.check(lib.et_norm_linear_bsr16_f32in(d_v.ptr, d_stats.ptr, G, d_g.ptr, d_b.ptr, 1e-5, d_fin.ptr, d_ln32.ptr, d_ln16.ptr,
+                                            w2.d_row_ptr.ptr, w2.d_col_idx.ptr, w2.d_tiles.ptr, w2.d_bias.ptr, d_y.ptr,
+                                            T, n_mid, n_out, act, None))
+    ln32, ln16 = d_ln32.numpy(), d_ln16.numpy()
+    fin = d_fin.numpy().astype(np.float64)
+    assert np.allclose(fin[:, 0], v64.mean(1), rtol=1e-5, atol=1e-5)
+    assert np.allclose(fin[:, 1], 1 / np.sqrt(v64.var(1) + 1e-5), rtol=1e-4)
+    want_ln = L.layernorm(torch.from_numpy(v), Hn.f32(gamma), Hn.f32(beta), 1e-5).numpy()
+    assert Hn.max_abs(ln32, want_ln) <= 2e-4 * max(1.0, float(np.abs(want_ln).max()))
+    assert np.array_equal(ln16.view(np.uint16), ln32.astype(np.float16).view(np.uint16))  # one value, two roundings
+    want_y = L.linear(Hn.f32(ln16), Hn.f32(w2.dense), Hn.f32(w2.bias), {0: None, 1: "relu", 2: "gelu"}[act],
+                      torch.float16).numpy()
+    assert Hn.max_abs(d_y.numpy(), want_y) <= 5e-3
+    # without the binary16 copy (what the layer asks for) Y does not change
+    d_y2 = et.DeviceBuffer.empty((T, n_out), np.float16)
+    et.check(lib.et_norm_linear_bsr16_f32in(d_v.ptr, d_stats.ptr, G, d_g.ptr, d_b.ptr, 1e-5, None, d_ln32.ptr, None,
+                                            w2.d_row_ptr.ptr, w2.d_col_idx.ptr, w2.d_tiles.ptr, w2.d_bias.ptr, d_y2.ptr,
+                                            T, n_mid, n_out, act, None))
+    assert np.array_equal(d_y2.numpy().view(np.uint16), d_y.numpy().view(np.uint16))
+    # the stand-alone normalisation from the same sums is bit-identical
+    d_o32 = et.DeviceBuffer.empty((T, n_mid), np.float32)
+    d_o16 = et.DeviceBuffer.empty((T, n_mid), np.float16)
+    et.check(lib.et_norm_from_stats_f32in(d_o32.ptr, d_o16.ptr, d_v.ptr, d_stats.ptr, G, d_g.ptr, d_b.ptr, T, n_mid,
+                                          1e-5, None))
+    assert np.array_equal(d_o32.numpy().view(np.uint32), ln32.view(np.uint32))
+    assert np.array_equal(d_o16.numpy().view(np.uint16), ln16.view(np.uint16))
+    # a second producer whose residual is that normalisation, formed in its epilogue from V and the sums
+    # instead of being read: the same result as with the stored rows
+    w3 = Hn.BsrWeight(n_mid, n_out, sp, seed=45, bias_std=0.05).upload(et)
+    d_v2a, d_v2b = et.DeviceBuffer.empty((T, n_mid), np.float32), et.DeviceBuffer.empty((T, n_mid), np.float32)
+    d_st2a, d_st2b = et.DeviceBuffer.empty((16, T, 2), np.float32), et.DeviceBuffer.empty((16, T, 2), np.float32)
+    g2 = C.c_int(0)
+    common = (w3.d_row_ptr.ptr, w3.d_col_idx.ptr, w3.d_tiles.ptr, w3.d_bias.ptr, d_y.ptr)
+    et.check(lib.et_linear_bsr16_resid_stats_f32(*common, d_ln32.ptr, None, None, None, d_v2a.ptr, d_st2a.ptr,
+                                                 C.byref(g2), T, n_out, n_mid, None))
+    et.check(lib.et_linear_bsr16_resid_stats_f32(*common, d_v.ptr, d_fin.ptr, d_g.ptr, d_b.ptr, d_v2b.ptr,
+                                                 d_st2b.ptr, C.byref(g2), T, n_out, n_mid, None))
+    assert np.array_equal(d_v2a.numpy().view(np.uint32), d_v2b.numpy().view(np.uint32))
+    assert np.array_equal(d_st2a.numpy()[:g2.value].view(np.uint32), d_st2b.numpy()[:g2.value].view(np.uint32))
+    want_v2 = L.linear(Hn.f32(d_y.numpy()), Hn.f32(w3.dense), Hn.f32(w3.bias)).numpy() + want_ln
+    assert Hn.max_abs(d_v2b.numpy(), want_v2) <= 3e-4 * max(1.0, float(np.abs(want_v2).max()))
+
+
+
 def test_split_layernorm_rejects_unsupported(et):
     import ctypes as C
     lib = et.lib()

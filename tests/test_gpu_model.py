@@ -85,20 +85,20 @@ TOL_MIXED_VS_ORACLE = 6e-3   # against the oracle rounding where the engine does
 TOL_F16_DEEP = 5e-2          # all-fp16 storage over 12+ layers: two realisations of the storage noise
 
 
-@pytest.mark.parametrize("seed0,xseed", [(100, 4), (300, 307), (500, 507)])
-def test_bert_base_12_layers_batch8_tile80_attention_aware_mixed(et, seed0, xseed):
+@pytest.mark.parametrize("seed0,xseed,mode", [(100, 4, 1), (300, 307, 1), (500, 507, 1), (100, 4, 2)])
+def test_bert_base_12_layers_batch8_tile80_attention_aware_mixed(et, seed0, xseed, mode):
     """The headline configuration in the engine's mixed-precision mode: 12 layers, B8 S128, 80 %
     tile sparsity, 25 % of the V rows (and the matching O columns) dead in head-aligned groups."""
     H, S, B = 768, 128, 8
     layers = headline_layers(seed0)
     assert len(layers[0].qkv.col_idx) == F.tile_count(3 * H, H, 0.8)
-    m = Hn.build_model(et, layers, S, B, mixed=True)
+    m = Hn.build_model(et, layers, S, B, mixed=mode)
     x = Hn.randn((B * S, H), xseed)
     got = run_model(et, m, x, reps=2)
     want32 = Hn.oracle_stack(x, layers, B, store=None)
     want_mixed = Hn.oracle_stack(x, layers, B, store=torch.float16, resid=torch.float32)
     e32, em = Hn.max_abs(got[0], want32), Hn.max_abs(got[0], want_mixed)
-    print(f"12-layer B8 S128 mixed seed {seed0}: vs fp32 forward {e32:.3e}, vs mixed oracle {em:.3e}")
+    print(f"12-layer B8 S128 mixed (mode {mode}) seed {seed0}: vs fp32 forward {e32:.3e}, vs mixed oracle {em:.3e}")
     assert e32 <= TOL_MIXED_VS_F32 and em <= TOL_MIXED_VS_ORACLE
     assert np.array_equal(got[0], got[1])
 
@@ -164,12 +164,13 @@ def test_bert_large_shape_padded_4_layers_fp16_storage(et):
     assert err <= TOL_F16
 
 
+@pytest.mark.parametrize("mode", [1, 2])  # SkipLayerNorm folded into the projections / launched on its own
 @pytest.mark.parametrize("use_graph", [True, False])
-def test_mixed_small_stack_graph_eager_inplace_and_single_layers(et, use_graph):
+def test_mixed_small_stack_graph_eager_inplace_and_single_layers(et, use_graph, mode):
     H, nh, FF, S, B = 128, 2, 256, 32, 2
     layers = [Hn.LayerWeights(H, nh, FF, 0.5, seed=60 + i) for i in range(3)]
     lens = np.array([20, 32], np.int32)
-    m = Hn.build_model(et, layers, S, B, lens=lens, use_graph=use_graph, mixed=True)
+    m = Hn.build_model(et, layers, S, B, lens=lens, use_graph=use_graph, mixed=mode)
     x = Hn.randn((B * S, H), 98)
     outs = run_model(et, m, x, reps=3)
     want = Hn.oracle_stack(x, layers, B, lens, store=torch.float16, resid=torch.float32)
