@@ -10,7 +10,8 @@ in the engine's mixed-precision mode: fp16 matrix-core operands, fp32 accumulati
 fp32 softmax, LayerNorm and residual stream.
 Prints ONE JSON line: sequences/s (value), ms per step, per-layer latency, the
 roofline of the dominant kernel (the tile-sparse FFN down-projection, 768 x 3072 at
-80 %, binary32 result; timed with HIP events on its own stream as it runs in a layer:
+80 %, with the residual added and the row sums of the binary32 result taken in its
+epilogue; timed with HIP events on its own stream as it runs in a layer:
 behind the up-projection that writes its input, rotating through the twelve layers'
 weights and twelve sets of activation buffers, as the replay time of [up, down] pairs
 minus that of the up-projections alone) and the CPU oracle timed on the host cores.
@@ -42,15 +43,20 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak (vendor figure)
 # counter reads for a streaming kernel of known size.  The summary ends in one machine-readable
 # line, "bench.py reads: {json}", which is all this file takes from it.
 TRAFFIC_PROFILE = ROOT / "profiles" / "encoder_stack_bert_base_b8_s128_hbm_traffic.txt"
-DOMINANT_KERNEL = "bsr16_linear_kernel<1,true,NONE> FFN down-projection 768x3072 @80%, T=1024, binary32 result"
+DOMINANT_KERNEL = ("bsr16_linear_kernel<1,true,NONE,0,RES|RES32> FFN down-projection 768x3072 @80%, T=1024, "
+                   "+ normalised residual, binary32 result, row sums")
+DOMINANT_KERNEL_SEPARATE = "bsr16_linear_kernel<1,true,NONE> FFN down-projection 768x3072 @80%, T=1024, binary32 result"
 
 
-def traffic_from_profile():
-    """(bytes per launch, source note) of the dominant kernel, or (None, reason)."""
+def traffic_from_profile(kernel):
+    """(bytes per launch, source note) of the dominant kernel, or (None, reason).  `kernel` is the
+    instantiation the timed launch runs: counters of another one are not reported."""
     try:
         for line in TRAFFIC_PROFILE.read_text().splitlines():
             if line.startswith("bench.py reads:"):
                 d = json.loads(line.split(":", 1)[1])
+                if d["kernel"] != kernel:
+                    return None, f"{TRAFFIC_PROFILE.name} holds the counters of {d['kernel']}, not of {kernel}"
                 return (d["fetch_kib"] * d["fetch_factor"] + d["write_kib"] * d["write_factor"]) * 1024.0, d["kernel"]
     except (OSError, ValueError, KeyError) as e:
         return None, f"{TRAFFIC_PROFILE.name}: {e}"
@@ -136,11 +142,17 @@ def time_stack(et, model, d_out, d_in, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
-def time_ffn_down_kernel(et, w1s, w2s, T, rounds_per_graph=6, replays=8):
+def time_ffn_down_kernel(et, layers, T, folded, rounds_per_graph=6, replays=8):
     """Average duration of the layer's longest kernel at the workload's shape — the FFN
     down-projection through the tile-sparse W2 (768 x 3072 at 80 %), T token rows, binary32
-    result as the mixed-precision stack launches it.  Returns (seconds as in the stack, seconds
+    result, as the mixed-precision stack launches it.  Returns (seconds as in the stack, seconds
     alone).
+
+    `folded` (the default stack, five launches per layer): the down-projection adds its residual —
+    the normalisation of the O-projection's sum, formed in the epilogue — and leaves the row sums
+    of its result (et_linear_bsr16_resid_stats_f32); the up-projection before it is the launch
+    that normalises that sum while staging it (et_norm_linear_bsr16_f32in).  Otherwise (seven
+    launches): the plain projections with a binary32 result.
 
     As in the stack: the launch follows the FFN up-projection + GELU that writes its input, so
     the input arrives the way it does in a layer (written a moment ago by other compute units)
@@ -155,20 +167,48 @@ def time_ffn_down_kernel(et, w1s, w2s, T, rounds_per_graph=6, replays=8):
     stream = C.c_void_p()
     et.check(lib.et_stream_create(C.byref(stream)))
     rng = np.random.default_rng(0)
-    n = len(w2s)
-    y1s = [et.DeviceBuffer.from_numpy(rng.standard_normal((T, H), dtype=np.float32).astype(np.float16)) for _ in w2s]
-    xs = [et.DeviceBuffer.from_numpy(rng.standard_normal((T, FF), dtype=np.float32).astype(np.float16)) for _ in w2s]
-    ys = [et.DeviceBuffer.empty((T, H), np.float32) for _ in w2s]
+    n = len(layers)
+    D = et.DeviceBuffer
+    f16 = lambda *shape: D.from_numpy(rng.standard_normal(shape, dtype=np.float32).astype(np.float16))
+    f32 = lambda *shape: D.from_numpy(rng.standard_normal(shape, dtype=np.float32))
+    W = lambda w: (w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, w.d_bias.ptr)
+    for l in layers:
+        for w in (l.o, l.l1, l.l2):
+            w.upload(et)
+        l.d_g1, l.d_b1 = D.from_numpy(l.g1), D.from_numpy(l.be1)
+    y1s = [f16(T, H) for _ in layers]        # separate mode: the up-projection's input
+    xs = [f16(T, FF) for _ in layers]        # the down-projection's input
+    ys = [D.empty((T, H), np.float32) for _ in layers]
+    groups = C.c_int(0)
+    if folded:
+        # the O-projection's sum and its row sums, made by the producer itself from random operands
+        zs, x32 = [f16(T, H) for _ in layers], [f32(T, H) for _ in layers]
+        v1 = [D.empty((T, H), np.float32) for _ in layers]
+        st1 = [D.empty((16, T, 2), np.float32) for _ in layers]
+        st2 = [D.empty((16, T, 2), np.float32) for _ in layers]
+        fin1 = [D.empty((T, 2), np.float32) for _ in layers]
+        g1 = C.c_int(0)
+        for i, l in enumerate(layers):
+            et.check(lib.et_linear_bsr16_resid_stats_f32(*W(l.o), zs[i].ptr, x32[i].ptr, None, None, None, v1[i].ptr,
+                                                         st1[i].ptr, C.byref(g1), T, H, H, stream))
 
     def up(i):
-        w = w1s[i]
-        et.check(lib.et_linear_bsr16_f16(w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, w.d_bias.ptr,
-                                         y1s[i].ptr, xs[i].ptr, T, H, FF, et.ACT_GELU, stream))
+        l = layers[i]
+        if folded:
+            et.check(lib.et_norm_linear_bsr16_f32in(v1[i].ptr, st1[i].ptr, g1.value, l.d_g1.ptr, l.d_b1.ptr, 1e-5,
+                                                    fin1[i].ptr, None, None, *W(l.l1), xs[i].ptr, T, H, FF, et.ACT_GELU,
+                                                    stream))
+        else:
+            et.check(lib.et_linear_bsr16_f16(*W(l.l1), y1s[i].ptr, xs[i].ptr, T, H, FF, et.ACT_GELU, stream))
 
     def down(i):
-        w = w2s[i]
-        et.check(lib.et_linear_bsr16_f16_f32out(w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, w.d_bias.ptr,
-                                                xs[i].ptr, ys[i].ptr, T, FF, H, et.ACT_NONE, stream))
+        l = layers[i]
+        if folded:
+            et.check(lib.et_linear_bsr16_resid_stats_f32(*W(l.l2), xs[i].ptr, v1[i].ptr, fin1[i].ptr, l.d_g1.ptr,
+                                                         l.d_b1.ptr, ys[i].ptr, st2[i].ptr, C.byref(groups), T, FF, H,
+                                                         stream))
+        else:
+            et.check(lib.et_linear_bsr16_f16_f32out(*W(l.l2), xs[i].ptr, ys[i].ptr, T, FF, H, et.ACT_NONE, stream))
 
     def timed_graph(steps):
         et.check(lib.et_graph_begin_capture(stream))
@@ -186,7 +226,8 @@ def time_ffn_down_kernel(et, w1s, w2s, T, rounds_per_graph=6, replays=8):
         et.check(lib.et_graph_destroy(graph))
         return t.ms * 1e-3 / (rounds_per_graph * n * replays)
 
-    up(0)  # eager once (one-time kernel setup)
+    for i in range(n):  # eager once: one-time kernel setup, and in folded mode fin1 for the loop of down-projections
+        up(i)
     down(0)
     et.check(lib.et_stream_sync(stream))
     alone = timed_graph([down])
@@ -289,23 +330,27 @@ def main():
 
     # dominant kernel: FFN down-projection (768x3072 BSR at 80 %, T = 1024, binary32 result)
     T = B * S
-    w1s = [l.l1.upload(et) for l in layers]
-    w2s = [l.l2.upload(et) for l in layers]
+    folded = not args.separate_ln
     ntile = len(layers[0].l2.col_idx)  # the same count in every layer: int(9216 * (1 - 0.8))
     flops = 2.0 * 256 * ntile * T  # algorithmic: 2 * 16*16 * surviving tiles * token rows
-    ksec, ksec_alone = time_ffn_down_kernel(et, w1s, w2s, T)
+    ksec, ksec_alone = time_ffn_down_kernel(et, layers, T, folded)
     achieved = flops / ksec / 1e12
-    traffic, traffic_note = traffic_from_profile()
-    roofline = {"bound": "mfma", "kernel": DOMINANT_KERNEL,
+    traffic, traffic_note = traffic_from_profile("bsr16_linear_kernel<1,true,0,0,10>" if folded
+                                                 else "bsr16_linear_kernel<1,true,0,0,0>")
+    roofline = {"bound": "mfma", "kernel": DOMINANT_KERNEL if folded else DOMINANT_KERNEL_SEPARATE,
                 "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 5), "us_per_launch": round(ksec * 1e6, 3),
                 "us_per_launch_alone": round(ksec_alone * 1e6, 3),
                 "flop_per_launch": flops, "traffic": None if traffic is None else round(traffic),
                 "traffic_source": traffic_note}
     # The same launch against the other roof: algorithmic bytes 2 T in + 4 T out (binary32 result)
-    # + 516 ntile + 4(out/16+1) + 2 out.  At 93 flop per byte the shape sits below the ridge of the
-    # machine (312 flop/B), i.e. on the HBM roof.
+    # + 516 ntile + 4(out/16+1) + 2 out, and folded: + 4 T out (the sum whose normalisation is the
+    # residual) + 8 T (its row statistics) + 4 out (gamma, beta) + 8 T groups (row sums written).
+    # At 70-93 flop per byte the shape sits below the ridge of the machine (312 flop/B), i.e. on
+    # the HBM roof.
     alg_bytes = 2.0 * T * FF + 4.0 * T * H + 516.0 * ntile + 4.0 * (H // 16 + 1) + 2.0 * H
+    if folded:
+        alg_bytes += 4.0 * T * H + 8.0 * T + 4.0 * H + 8.0 * T * 4
     roofline["hbm_view"] = {"bound": "hbm", "achieved": round(alg_bytes / ksec / 1e9, 1), "peak": 8000.0, "unit": "GB/s",
                             "frac": round(alg_bytes / ksec / 8e12, 5), "bytes_per_launch": alg_bytes}
 
