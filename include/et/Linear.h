@@ -183,7 +183,6 @@ template <> class Linear<tile_mat> {
     // mixed-precision encoder layer adds to its fp32 residual stream
     void forward_f32(float *output, const half *input, et::stream_t stream = nullptr) {
         if (dense) {  // the dense GEMM stores fp16: widened afterwards
-            if (!dense_out16) dense_out16 = std::make_unique<et::DeviceBuffer<half>>((std::size_t)size * out_size);
             forward_act(dense_out16->get(), input, ET_ACT_NONE, stream);
             etChk(et_f16_to_f32(output, et::f16(dense_out16->get()), (std::size_t)size * out_size, stream));
             return;
@@ -247,6 +246,7 @@ template <> class Linear<tile_mat> {
         if (size > 0 && size % 16 == 0 && wants_dense((int)in_size, (int)out_size, weight.num_blk) &&
             !names_a_position_twice()) {
             dense = std::make_unique<et::DeviceBuffer<half>>((std::size_t)in_size * out_size);
+            dense_out16 = std::make_unique<et::DeviceBuffer<half>>((std::size_t)size * out_size);  // forward allocates nothing
             etChk(et_bsr16_to_dense_f16(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
                                         et::f16(dense->get()), (int)in_size, (int)out_size, nullptr));
             etChk(et_device_sync());

@@ -207,6 +207,20 @@ def test_layer_at_4096_rows_uses_the_streaming_linear(et, mixed):
     assert np.array_equal(got[0], got[1])
 
 
+@pytest.mark.parametrize("mode", [0, 1, 2])
+def test_stack_of_weights_that_keep_most_tiles(et, mode):
+    """20 % tile sparsity: the class multiplies with a dense image of each weight, and the
+    mixed-precision engine keeps SkipLayerNorm as launches of its own (nothing to fold it into)."""
+    H, nh, FF, S, B = 128, 2, 256, 32, 2
+    layers = [Hn.LayerWeights(H, nh, FF, 0.2, seed=80 + i) for i in range(2)]
+    m = Hn.build_model(et, layers, S, B, mixed=mode)
+    x = Hn.randn((B * S, H), 96)
+    got = run_model(et, m, x, reps=2)
+    want = Hn.oracle_stack(x, layers, B, store=torch.float16, resid=torch.float32 if mode else "same")
+    assert Hn.max_abs(got[0], want) <= (4e-3 if mode else TOL_F16)
+    assert np.array_equal(got[0], got[1])
+
+
 def test_in_place_forward_with_graph_all_fp16(et):
     H, nh, FF, S, B = 128, 2, 256, 32, 1
     layers = [Hn.LayerWeights(H, nh, FF, 0.5, seed=70 + i) for i in range(2)]
