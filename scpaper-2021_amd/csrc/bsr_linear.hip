@@ -65,7 +65,7 @@ struct BsrArgs {
     // binary32 forms of the split normalisation (mixed-precision layer).  RES with kFxRes32: the sum
     // acc + bias + resid32 is stored unrounded to Y32 and the row sums are taken over it (Y, resid
     // unused).  NORM with kFxNorm32: the strip comes from X32 (that stored sum; ln_skip unused) and
-    // the normalised rows go to ln_out32 and / or ln_out (either may be null), each row written by
+    // the normalised rows go to ln_out32 and / or ln_out (either may be null), each vector written by
     // one of the strip's block-row groups.
     const float *resid32;
     const float *X32;
@@ -96,6 +96,7 @@ constexpr int kGroupsAhead = 4;
 constexpr int kGroupsAheadNorm = 2;
 constexpr int kStageU = 8;    // 16-byte strip vectors a thread keeps in flight
 constexpr int kMaxWaveRows = 64;  // block-rows one wave can own (one lane each)
+constexpr int kScalarRows = 4;    // up to this many, a wave fetches its row pointers with scalar loads
 
 template <int ACT> __device__ __forceinline__ float act_fixed(float x) {
     if (ACT == ET_ACT_RELU) return x > 0.0f ? x : 0.0f;
@@ -110,7 +111,7 @@ __device__ __forceinline__ int lane_read(int v, int lane) {
 // ACT is a template parameter: the epilogue carries no run-time branch and each
 // fused activation is a separately named kernel in a profile.
 template <int MT, bool STAGE, int ACT, int LN = 0, int FX = 0>
-__global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
+__global__ __launch_bounds__((MT == 1 && (FX & kFxRes32)) ? 768 : 512) void bsr16_linear_kernel(const BsrArgs a) {
     static_assert(!LN || STAGE, "the fused LayerNorm prologue writes the strip to LDS");
     static_assert(!(FX & kFxNorm) || (STAGE && !LN), "the NORM prologue writes the strip to LDS");
     constexpr bool NORM = (FX & kFxNorm) != 0;
@@ -122,6 +123,10 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     // row groups resident per wave: four; two in the kernels whose prologue normalises fp16 strips
     // (four would spill), three with a binary32 strip or a binary32 residual in flight per group
     constexpr int kNB = (NORM32 || RES32) ? 3 : (LN || NORM) ? kGroupsAheadNorm : kGroupsAhead;
+    // 16-byte strip vectors a thread requests before it writes the first to LDS: a 16-row strip of a
+    // 3072-wide input (12 per thread of 512) is requested whole, so that none of it queues behind
+    // the weight requests; binary32 vectors are two loads each
+    constexpr int kSU = (MT == 1 && !LN && !NORM && !RES32) ? 12 : NORM32 ? 6 : kStageU;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     _Float16 *xs = reinterpret_cast<_Float16 *>(smem_raw);
 
@@ -155,10 +160,36 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     // issue order and everything below depends on these few bytes)
     const int nrw = max(0, (rb_end - rb_begin - wave + nwave - 1) / nwave);
     int rp_lo = 0, rp_hi = 0;
-    if (lane < nrw) {
+    // A few rows: scalar loads, kept in scalar registers until the first use.  They do not queue in
+    // the vector memory pipeline behind the strip loads of the other waves of the compute unit.
+    const bool rows_scalar = nrw <= kScalarRows;
+    const auto *rpc = reinterpret_cast<const __attribute__((address_space(4))) int32_t *>(
+        reinterpret_cast<uintptr_t>(a.row_ptr));
+    auto rb_of = [&](int i) { return min(rb_begin + wave + nwave * i, nbr - 1); };
+    const int slo0 = rpc[rb_of(0)], shi0 = rpc[rb_of(0) + 1];
+    const int slo1 = rpc[rb_of(1)], shi1 = rpc[rb_of(1) + 1];
+    const int slo2 = rpc[rb_of(2)], shi2 = rpc[rb_of(2) + 1];
+    const int slo3 = rpc[rb_of(3)], shi3 = rpc[rb_of(3) + 1];
+    static_assert(kScalarRows == 4, "four named pairs");
+    if (!rows_scalar && lane < nrw) {
         const int rb = rb_begin + wave + nwave * lane;
         rp_lo = a.row_ptr[rb];
         rp_hi = a.row_ptr[rb + 1];
+    }
+
+    // ---- NORM: the row sums (wave 0, a token per lane) and the affine vectors are requested ahead
+    // of the strip.  Loads return in order: behind the strip they would keep the waves that
+    // put them into LDS waiting for the whole strip before their weight requests go out.
+    float2 st_part[NORM ? kMaxStatGroups : 1];
+    h8 aff[NORM ? 2 : 1][2];  // gamma and beta vectors threadIdx.x and threadIdx.x + blockDim.x of the row
+    if constexpr (NORM) {
+        if (wave == 0) row_stats_request(st_part, a.st_in, a.st_groups, a.T, min(tok0 + lane, a.T - 1));
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            const int c = min((int)threadIdx.x + k * nthr, (a.in >> 3) - 1);
+            aff[k][0] = reinterpret_cast<const h8 *>(a.ln_gamma)[c];
+            aff[k][1] = reinterpret_cast<const h8 *>(a.ln_beta)[c];
+        }
     }
 
     // ---- strip copy, first batch: loads only.  X[tok0 .. tok0+MT*16) is one
@@ -167,27 +198,27 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     const int rows_here = min(MT * 16, a.T - tok0);
     const int total_vec = STAGE ? rows_here * vec_per_row : 0;
     const h8 *src = reinterpret_cast<const h8 *>(a.X + (size_t)tok0 * a.in);
-    h8 sv[kStageU];
+    h8 sv[kSU];
     if (STAGE && !LN && !NORM32) {
         // unconditional loads, index clamped into the strip: a load under a branch gets a
         // basic block of its own and the register allocator's copies there make the wave
         // wait for it on the spot — a full memory round trip before the weight loads go out
 #pragma unroll
-        for (int u = 0; u < kStageU; u++) sv[u] = src[min((int)threadIdx.x + u * nthr, total_vec - 1)];
+        for (int u = 0; u < kSU; u++) sv[u] = src[min((int)threadIdx.x + u * nthr, total_vec - 1)];
     }
     constexpr bool SKIP16 = NORM && !NORM32;  // a binary16 skip strip is added
     const h8 *src_skip = SKIP16 ? reinterpret_cast<const h8 *>(a.ln_skip + (size_t)tok0 * a.in) : nullptr;
-    h8 sk[SKIP16 ? kStageU : 1];
+    h8 sk[SKIP16 ? kSU : 1];
     if (SKIP16) {
 #pragma unroll
-        for (int u = 0; u < kStageU; u++) sk[u] = src_skip[min((int)threadIdx.x + u * nthr, total_vec - 1)];
+        for (int u = 0; u < kSU; u++) sk[u] = src_skip[min((int)threadIdx.x + u * nthr, total_vec - 1)];
     }
     // binary32 strip: a strip vector of 8 values is two 16-byte loads
     const f4 *src32 = NORM32 ? reinterpret_cast<const f4 *>(a.X32 + (size_t)tok0 * a.in) : nullptr;
-    f4 s32[NORM32 ? kStageU : 1][2];
+    f4 s32[NORM32 ? kSU : 1][2];
     if (NORM32) {
 #pragma unroll
-        for (int u = 0; u < kStageU; u++) {
+        for (int u = 0; u < kSU; u++) {
             const int v = min((int)threadIdx.x + u * nthr, total_vec - 1);
             s32[u][0] = src32[2 * v];
             s32[u][1] = src32[2 * v + 1];
@@ -197,18 +228,6 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     float2 *stat_lds = reinterpret_cast<float2 *>(xs + MT * 16 * lds_ld);
     _Float16 *gam_lds = reinterpret_cast<_Float16 *>(stat_lds + MT * 16);
     _Float16 *bet_lds = gam_lds + a.in;
-    if (NORM) {
-        if ((int)threadIdx.x < rows_here) {
-            const float2 st = row_stats(a.st_in, a.st_groups, a.T, tok0 + threadIdx.x, a.in, a.ln_eps);
-            stat_lds[threadIdx.x] = st;
-            if (NORM32 && a.fin_out && group == 0)
-                *reinterpret_cast<float2 *>(a.fin_out + 2 * (size_t)(tok0 + threadIdx.x)) = st;
-        }
-        for (int c = threadIdx.x; c < vec_per_row; c += nthr) {
-            *reinterpret_cast<h8 *>(gam_lds + c * 8) = reinterpret_cast<const h8 *>(a.ln_gamma)[c];
-            *reinterpret_cast<h8 *>(bet_lds + c * 8) = reinterpret_cast<const h8 *>(a.ln_beta)[c];
-        }
-    }
     // Fused SkipLayerNorm: a wave normalises rows wave, wave+nwave, ... of the strip
     // (at most kLnRows of them); all their loads are issued here, one round trip.
     constexpr int kLnRows = LN ? MT * 16 / 8 : 1;        // rows per wave: LN kernels run 8 waves
@@ -242,7 +261,8 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     // ---- row-group stream of this wave.  An item is up to kSlots slots of one
     // block-row; (it_row, it_part) is the next item to request.
     h8 w[kNB][kSlots];
-    int col[kNB][kSlots];
+    // column indices of an item's 2*kSlots tiles: one load, lane L holds that of tile L % 16
+    int colv[kNB];
     h4 bias_v[kNB];
     // RES32: the residual of the block-row an item finishes (requested with the item, so that the
     // epilogue of the row does not wait for it), with the affine values of its four features
@@ -264,12 +284,16 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
     int g_row[kNB], g_nsl[kNB];  // resident items: wave row index (-1 = none), slots in the item
     bool g_last[kNB];            // item ends its block-row
     int it_row = 0, it_part = 0;
+    if (rows_scalar) {  // the scalar row pointers take their lanes (first use: the wait for them is here)
+        rp_lo = lane == 0 ? slo0 : lane == 1 ? slo1 : lane == 2 ? slo2 : slo3;
+        rp_hi = lane == 0 ? shi0 : lane == 1 ? shi1 : lane == 2 ? shi2 : shi3;
+    }
     // skip rows without tiles (they are written at the end)
     auto skip_empty = [&]() {
         while (it_row < nrw && lane_read(rp_hi, it_row) == lane_read(rp_lo, it_row)) it_row++;
     };
     skip_empty();
-    auto issue_item = [&](int buf) {
+    auto issue_item = [&](int buf) __attribute__((always_inline)) {
         if (it_row >= nrw) {
             g_row[buf] = -1;
             return;
@@ -284,26 +308,24 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
         g_nsl[buf] = nsl;
         g_last[buf] = last;
         const int tf = t0 + 2 * first_slot;  // first tile of the item
-        // per-lane base pointers; slot p adds an immediate p*1024 B / p*8 B
+        // per-lane base pointer; slot p adds an immediate p*1024 B
         const _Float16 *wp = a.tiles + (size_t)(tf + sel) * 256 + r16 * 16 + koff;
-        const int32_t *cp = a.col_idx + tf + sel;
 #pragma unroll
         for (int p = 0; p < kSlots; p++) {
             if (p < nsl) {
                 if (odd_tail && p == nsl - 1) {
-                    // lanes of the missing second tile: zero weights, index of the first tile
+                    // lanes of the missing second tile: zero weights
                     w[buf][p] = zero8;
                     if (sel == 0) w[buf][p] = *reinterpret_cast<const h8 *>(wp + p * 512);
-                    col[buf][p] = a.col_idx[tf + 2 * p];
                 } else {
                     w[buf][p] = *reinterpret_cast<const h8 *>(wp + p * 512);
-                    col[buf][p] = cp[2 * p];
                 }
             } else if (p & 1) {
                 w[buf][p] = zero8;  // partner of the last slot inside a two-slot step
-                col[buf][p] = 0;
             }
         }
+        // tiles past the row (zero weights) take the column of its last tile
+        colv[buf] = a.col_idx[min(tf + r16, t1 - 1)];
         if (last) {  // the item that finishes the row carries its bias
             bias_v[buf] = h4{0, 0, 0, 0};
             if (a.bias)
@@ -318,8 +340,31 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
             it_part++;
         }
     };
+    // Row groups requested before the strip is written; the others follow when the registers of
+    // the strip vectors are free again (only the 12-wave producer, at 170 registers per lane, has any)
+    constexpr int kEarly = (MT == 1 && RES32) ? 2 : kNB;
 #pragma unroll
-    for (int buf = 0; buf < kNB; buf++) issue_item(buf);
+    for (int buf = 0; buf < kEarly; buf++) issue_item(buf);
+
+    // NORM: per-row (mean, rstd) and the affine vectors go to LDS behind the strip
+    if constexpr (NORM) {
+        if (wave == 0) {
+            const float2 st = row_stats_finish(st_part, a.st_groups, a.in, a.ln_eps);
+            if (lane < rows_here) {
+                stat_lds[lane] = st;
+                if (NORM32 && a.fin_out && group == 0)
+                    *reinterpret_cast<float2 *>(a.fin_out + 2 * (size_t)(tok0 + lane)) = st;
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            const int c = threadIdx.x + k * nthr;
+            if (c < vec_per_row) {
+                *reinterpret_cast<h8 *>(gam_lds + c * 8) = aff[k][0];
+                *reinterpret_cast<h8 *>(bet_lds + c * 8) = aff[k][1];
+            }
+        }
+    }
 
     // ---- fused SkipLayerNorm: statistics in fp32 per row (wave64 butterflies), the
     // normalised row goes to LDS as fp16 — the value a separate LayerNorm kernel would
@@ -394,8 +439,13 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
         if (group == 0) *reinterpret_cast<h8 *>(a.ln_out + (size_t)(tok0 + r) * a.in + c * 8) = o;
         return o;
     };
-    // the same from the binary32 strip; row r of the strip is written back by group r mod ngroups
-    auto strip_value32 = [&](f4 lo, f4 hi, int r, int c) {
+    // the same from the binary32 strip; the block-row groups of a strip each write back an equal
+    // run of its vectors (no run at all when neither output is asked for)
+    const bool norm_wr = NORM32 && (a.ln_out32 || a.ln_out);
+    const int own_per = (total_vec + ngroups - 1) / ngroups;
+    const int own_lo = norm_wr ? group * own_per : 0;
+    const int own_hi = norm_wr ? min(total_vec, own_lo + own_per) : 0;
+    auto strip_value32 = [&](f4 lo, f4 hi, int r, int c, int idx) {
         const float2 st = stat_lds[r];
         const h8 gm = *reinterpret_cast<const h8 *>(gam_lds + c * 8);
         const h8 bt = *reinterpret_cast<const h8 *>(bet_lds + c * 8);
@@ -407,7 +457,7 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
         }
         const h8 o = {(_Float16)y0[0], (_Float16)y0[1], (_Float16)y0[2], (_Float16)y0[3],
                       (_Float16)y1[0], (_Float16)y1[1], (_Float16)y1[2], (_Float16)y1[3]};
-        if (r % ngroups == group) {
+        if (idx >= own_lo && idx < own_hi) {
             const size_t at = (size_t)(tok0 + r) * a.in + c * 8;
             if (a.ln_out32) {
                 *reinterpret_cast<f4 *>(a.ln_out32 + at) = y0;
@@ -421,11 +471,11 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
         const int dr = nthr / vec_per_row, dc = nthr - dr * vec_per_row;  // (row, col) step of +nthr
         int r = threadIdx.x / vec_per_row, c = threadIdx.x - r * vec_per_row;
 #pragma unroll
-        for (int u = 0; u < kStageU; u++) {
+        for (int u = 0; u < kSU; u++) {
             const int idx = threadIdx.x + u * nthr;
             if (idx < total_vec)
                 *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) =
-                    NORM32 ? strip_value32(s32[NORM32 ? u : 0][0], s32[NORM32 ? u : 0][1], r, c)
+                    NORM32 ? strip_value32(s32[NORM32 ? u : 0][0], s32[NORM32 ? u : 0][1], r, c, idx)
                            : strip_value(sv[u], sk[SKIP16 ? u : 0], r, c);
             r += dr;
             c += dc;
@@ -434,9 +484,9 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
                 r++;
             }
         }
-        for (int base = threadIdx.x + kStageU * nthr; base < total_vec; base += nthr * kStageU) {
+        for (int base = threadIdx.x + kSU * nthr; base < total_vec; base += nthr * kSU) {
 #pragma unroll
-            for (int u = 0; u < kStageU; u++) {
+            for (int u = 0; u < kSU; u++) {
                 const int v = min(base + u * nthr, total_vec - 1);
                 if (NORM32) {
                     s32[NORM32 ? u : 0][0] = src32[2 * v];
@@ -447,14 +497,14 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
             }
             if (SKIP16) {
 #pragma unroll
-                for (int u = 0; u < kStageU; u++) sk[u] = src_skip[min(base + u * nthr, total_vec - 1)];
+                for (int u = 0; u < kSU; u++) sk[u] = src_skip[min(base + u * nthr, total_vec - 1)];
             }
 #pragma unroll
-            for (int u = 0; u < kStageU; u++) {
+            for (int u = 0; u < kSU; u++) {
                 const int idx = base + u * nthr;
                 if (idx < total_vec)
                     *reinterpret_cast<h8 *>(xs + r * lds_ld + c * 8) =
-                        NORM32 ? strip_value32(s32[NORM32 ? u : 0][0], s32[NORM32 ? u : 0][1], r, c)
+                        NORM32 ? strip_value32(s32[NORM32 ? u : 0][0], s32[NORM32 ? u : 0][1], r, c, idx)
                                : strip_value(sv[u], sk[SKIP16 ? u : 0], r, c);
                 r += dr;
                 c += dc;
@@ -469,6 +519,8 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
             const int rr = idx / vec_per_row, cc = idx - rr * vec_per_row;
             *reinterpret_cast<h8 *>(xs + rr * lds_ld + cc * 8) = zero8;
         }
+#pragma unroll
+        for (int buf = kEarly; buf < kNB; buf++) issue_item(buf);
         __syncthreads();
     }
 
@@ -559,11 +611,17 @@ __global__ __launch_bounds__(512) void bsr16_linear_kernel(const BsrArgs a) {
                 for (int p0 = 0; p0 < kSlots; p0 += 2) {
                     if (p0 < nsl) {  // wave-uniform; slot p0+1 is real or zero-weighted
                         h8 x[2][MT];
+                        int ca[2], cd[2];  // column of a slot's first tile; second minus first
+#pragma unroll
+                        for (int q = 0; q < 2; q++) {
+                            ca[q] = lane_read(colv[buf], 2 * (p0 + q));
+                            cd[q] = lane_read(colv[buf], 2 * (p0 + q) + 1) - ca[q];
+                        }
 #pragma unroll
                         for (int q = 0; q < 2; q++)
 #pragma unroll
                             for (int m = 0; m < MT; m++) {
-                                x[q][m] = *reinterpret_cast<const h8 *>(xrow[m] + col[buf][p0 + q] * 16);
+                                x[q][m] = *reinterpret_cast<const h8 *>(xrow[m] + (ca[q] + sel * cd[q]) * 16);
                                 if (!STAGE && !tok_ok[m]) x[q][m] = zero8;
                             }
 #pragma unroll
@@ -754,6 +812,9 @@ static BsrPlan plan_bsr_fx32(int T, int in, int out, int fx) {
     p.mt = (T >= 32 && fits(2, lds_cap / 2) && rows_per_wg_for(2) >= 5) ? 2 : 1;
     int rpw = rows_per_wg_for(p.mt);
     p.threads = (rpw <= 6 || rpw == 18) ? 384 : 512;
+    // a producer on 16-row strips whose block-rows deal evenly to 12 waves runs 12: with a row or two
+    // per wave, all its weights are requested before the strip has arrived
+    if ((fx & kFxRes) && p.mt == 1 && rpw % 12 == 0 && rpw <= 24) p.threads = 768;
     const int cap = kMaxWaveRows * (p.threads / 64);
     if (rpw > cap) rpw = cap;
     if ((fx & kFxRes) && (nbr + rpw - 1) / rpw > kMaxStatGroups) p.stage = false;

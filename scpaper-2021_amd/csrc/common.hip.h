@@ -122,11 +122,14 @@ constexpr int kMaxStatGroups = 16;  // block-row groups a RES producer may split
 // added in group order (every consumer of the same sums gets the same bits).  All loads are
 // issued before the first addition (index clamped, surplus selected away): a loop with a
 // run-time trip count would wait for each load in turn.
-__device__ __forceinline__ float2 row_stats(const float *st, int groups, int T, int tok, int H, float eps) {
-    float2 p[kMaxStatGroups];
+// The two halves of row_stats: the requests (held in registers, so a kernel can put them ahead of
+// larger loads and use them long after) and the sums.
+__device__ __forceinline__ void row_stats_request(float2 (&p)[kMaxStatGroups], const float *st, int groups, int T, int tok) {
 #pragma unroll
     for (int gi = 0; gi < kMaxStatGroups; gi++)
         p[gi] = *reinterpret_cast<const float2 *>(st + ((size_t)min(gi, groups - 1) * T + tok) * 2);
+}
+__device__ __forceinline__ float2 row_stats_finish(const float2 (&p)[kMaxStatGroups], int groups, int H, float eps) {
     float s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
     for (int gi = 0; gi < kMaxStatGroups; gi++) {
@@ -137,6 +140,11 @@ __device__ __forceinline__ float2 row_stats(const float *st, int groups, int T, 
     const float mean = s1 * inv_h;
     const float var = fmaxf(__builtin_fmaf(-mean, mean, s2 * inv_h), 0.0f);
     return float2{mean, rsqrtf(var + eps)};
+}
+__device__ __forceinline__ float2 row_stats(const float *st, int groups, int T, int tok, int H, float eps) {
+    float2 p[kMaxStatGroups];
+    row_stats_request(p, st, groups, T, tok);
+    return row_stats_finish(p, groups, H, eps);
 }
 
 // one normalised value: the same two roundings wherever it is evaluated
