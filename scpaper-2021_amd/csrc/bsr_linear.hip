@@ -111,7 +111,7 @@ __device__ __forceinline__ int lane_read(int v, int lane) {
 // ACT is a template parameter: the epilogue carries no run-time branch and each
 // fused activation is a separately named kernel in a profile.
 template <int MT, bool STAGE, int ACT, int LN = 0, int FX = 0>
-__global__ __launch_bounds__((MT == 1 && (FX & kFxRes32)) ? 768 : 512) void bsr16_linear_kernel(const BsrArgs a) {
+__global__ __launch_bounds__(((MT == 1 && (FX & kFxRes32)) || (FX & kFxNorm32)) ? 768 : 512) void bsr16_linear_kernel(const BsrArgs a) {
     static_assert(!LN || STAGE, "the fused LayerNorm prologue writes the strip to LDS");
     static_assert(!(FX & kFxNorm) || (STAGE && !LN), "the NORM prologue writes the strip to LDS");
     constexpr bool NORM = (FX & kFxNorm) != 0;
@@ -122,11 +122,11 @@ __global__ __launch_bounds__((MT == 1 && (FX & kFxRes32)) ? 768 : 512) void bsr1
     static_assert(!RES32 || RES, "kFxRes32 qualifies kFxRes");
     // row groups resident per wave: four; two in the kernels whose prologue normalises fp16 strips
     // (four would spill), three with a binary32 strip or a binary32 residual in flight per group
-    constexpr int kNB = (NORM32 || RES32) ? 3 : (LN || NORM) ? kGroupsAheadNorm : kGroupsAhead;
+    constexpr int kNB = NORM32 ? 2 : RES32 ? 3 : (LN || NORM) ? kGroupsAheadNorm : kGroupsAhead;
     // 16-byte strip vectors a thread requests before it writes the first to LDS: a 16-row strip of a
     // 3072-wide input (12 per thread of 512) is requested whole, so that none of it queues behind
     // the weight requests; binary32 vectors are two loads each
-    constexpr int kSU = (MT == 1 && !LN && !NORM && !RES32) ? 12 : NORM32 ? 6 : kStageU;
+    constexpr int kSU = (MT == 1 && !LN && !NORM && !RES32) ? 12 : NORM32 ? 4 : kStageU;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     _Float16 *xs = reinterpret_cast<_Float16 *>(smem_raw);
 
@@ -180,10 +180,18 @@ __global__ __launch_bounds__((MT == 1 && (FX & kFxRes32)) ? 768 : 512) void bsr1
     // ---- NORM: the row sums (wave 0, a token per lane) and the affine vectors are requested ahead
     // of the strip.  Loads return in order: behind the strip they would keep the waves that
     // put them into LDS waiting for the whole strip before their weight requests go out.
-    float2 st_part[NORM ? kMaxStatGroups : 1];
+    static_assert(!NORM || MT <= 2, "a half-wave of tokens");
+    float2 st_part[NORM ? kMaxStatGroups / 2 : 1];  // lanes 0-31: groups 0-7 of token lane; lanes 32-63: groups 8-15
     h8 aff[NORM ? 2 : 1][2];  // gamma and beta vectors threadIdx.x and threadIdx.x + blockDim.x of the row
     if constexpr (NORM) {
-        if (wave == 0) row_stats_request(st_part, a.st_in, a.st_groups, a.T, min(tok0 + lane, a.T - 1));
+        if (wave == 0) {
+            const int tok = min(tok0 + (lane & 31), a.T - 1);
+#pragma unroll
+            for (int k = 0; k < kMaxStatGroups / 2; k++) {
+                const int gi = min((lane >> 5) * (kMaxStatGroups / 2) + k, a.st_groups - 1);
+                st_part[k] = *reinterpret_cast<const float2 *>(a.st_in + ((size_t)gi * a.T + tok) * 2);
+            }
+        }
 #pragma unroll
         for (int k = 0; k < 2; k++) {
             const int c = min((int)threadIdx.x + k * nthr, (a.in >> 3) - 1);
@@ -349,7 +357,18 @@ __global__ __launch_bounds__((MT == 1 && (FX & kFxRes32)) ? 768 : 512) void bsr1
     // NORM: per-row (mean, rstd) and the affine vectors go to LDS behind the strip
     if constexpr (NORM) {
         if (wave == 0) {
-            const float2 st = row_stats_finish(st_part, a.st_groups, a.in, a.ln_eps);
+            float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+            for (int k = 0; k < kMaxStatGroups / 2; k++) {
+                const bool real = (lane >> 5) * (kMaxStatGroups / 2) + k < a.st_groups;
+                s1 += real ? st_part[k].x : 0.0f;
+                s2 += real ? st_part[k].y : 0.0f;
+            }
+            s1 += __shfl_xor(s1, 32, 64);
+            s2 += __shfl_xor(s2, 32, 64);
+            const float inv_h = 1.0f / (float)a.in;
+            const float mean = s1 * inv_h;
+            const float2 st = float2{mean, rsqrtf(fmaxf(__builtin_fmaf(-mean, mean, s2 * inv_h), 0.0f) + a.ln_eps)};
             if (lane < rows_here) {
                 stat_lds[lane] = st;
                 if (NORM32 && a.fin_out && group == 0)
@@ -815,6 +834,9 @@ static BsrPlan plan_bsr_fx32(int T, int in, int out, int fx) {
     // a producer on 16-row strips whose block-rows deal evenly to 12 waves runs 12: with a row or two
     // per wave, all its weights are requested before the strip has arrived
     if ((fx & kFxRes) && p.mt == 1 && rpw % 12 == 0 && rpw <= 24) p.threads = 768;
+    // a consumer runs up to 12 waves of two block-rows: more instruction streams for the
+    // normalisation and a shorter chain of rows per wave
+    if (fx & kFxNorm) p.threads = rpw > 12 ? 768 : 64 * std::max(4, (rpw + 1) / 2);
     const int cap = kMaxWaveRows * (p.threads / 64);
     if (rpw > cap) rpw = cap;
     if ((fx & kFxRes) && (nbr + rpw - 1) / rpw > kMaxStatGroups) p.stage = false;

@@ -119,7 +119,7 @@ __device__ __forceinline__ float apply_act(float x, int act) {
 constexpr int kMaxStatGroups = 16;  // block-row groups a RES producer may split a row over
 
 // mean and reciprocal standard deviation of a row of H values from its partial sums,
-// added in group order (every consumer of the same sums gets the same bits).  All loads are
+// added in a fixed order (every consumer of the same sums gets the same bits).  All loads are
 // issued before the first addition (index clamped, surplus selected away): a loop with a
 // run-time trip count would wait for each load in turn.
 // The two halves of row_stats: the requests (held in registers, so a kernel can put them ahead of
@@ -130,12 +130,18 @@ __device__ __forceinline__ void row_stats_request(float2 (&p)[kMaxStatGroups], c
         p[gi] = *reinterpret_cast<const float2 *>(st + ((size_t)min(gi, groups - 1) * T + tok) * 2);
 }
 __device__ __forceinline__ float2 row_stats_finish(const float2 (&p)[kMaxStatGroups], int groups, int H, float eps) {
-    float s1 = 0.0f, s2 = 0.0f;
+    // two halves in group order, then their sum: the order a consumer that deals the groups to
+    // the two halves of a wave adds in, so that both get the same bits
+    float s1 = 0.0f, s2 = 0.0f, u1 = 0.0f, u2 = 0.0f;
 #pragma unroll
-    for (int gi = 0; gi < kMaxStatGroups; gi++) {
+    for (int gi = 0; gi < kMaxStatGroups / 2; gi++) {
         s1 += gi < groups ? p[gi].x : 0.0f;
         s2 += gi < groups ? p[gi].y : 0.0f;
+        u1 += gi + kMaxStatGroups / 2 < groups ? p[gi + kMaxStatGroups / 2].x : 0.0f;
+        u2 += gi + kMaxStatGroups / 2 < groups ? p[gi + kMaxStatGroups / 2].y : 0.0f;
     }
+    s1 += u1;
+    s2 += u2;
     const float inv_h = 1.0f / (float)H;
     const float mean = s1 * inv_h;
     const float var = fmaxf(__builtin_fmaf(-mean, mean, s2 * inv_h), 0.0f);
