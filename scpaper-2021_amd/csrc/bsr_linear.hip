@@ -836,7 +836,8 @@ static BsrPlan plan_bsr_fx32(int T, int in, int out, int fx) {
     if ((fx & kFxRes) && p.mt == 1 && rpw % 12 == 0 && rpw <= 24) p.threads = 768;
     // a consumer runs up to 12 waves of two block-rows: more instruction streams for the
     // normalisation and a shorter chain of rows per wave
-    if (fx & kFxNorm) p.threads = rpw > 12 ? 768 : 64 * std::max(4, (rpw + 1) / 2);
+    // (at least 6: the affine vectors of a row, in / 8 <= 640 16-byte pieces, are staged by two passes of the workgroup)
+    if (fx & kFxNorm) p.threads = rpw > 12 ? 768 : 64 * std::max(6, (rpw + 1) / 2);
     const int cap = kMaxWaveRows * (p.threads / 64);
     if (rpw > cap) rpw = cap;
     if ((fx & kFxRes) && (nbr + rpw - 1) / rpw > kMaxStatGroups) p.stage = false;
@@ -910,6 +911,9 @@ static int dispatch_bsr_norm(const BsrArgs &args, const BsrPlan &p, hipStream_t 
     return p.mt == 2 ? dispatch_bsr_fx_act<2, kFxNorm>(args, p, stream) : dispatch_bsr_fx_act<1, kFxNorm>(args, p, stream);
 }
 static int dispatch_bsr_norm32(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
+    ET_REQUIRE(args.in / 8 <= 2 * p.threads, ET_ERR_UNSUPPORTED,
+               "tile-sparse Linear: %d inputs need more than two passes of %d threads for the affine vectors", args.in,
+               p.threads);
     return p.mt == 2 ? dispatch_bsr_fx_act<2, kFxNorm | kFxNorm32>(args, p, stream)
                      : dispatch_bsr_fx_act<1, kFxNorm | kFxNorm32>(args, p, stream);
 }

@@ -453,7 +453,8 @@ def test_split_layernorm_between_two_tile_linears(et, T, n_in, n_mid, n_out, sp,
 
 @pytest.mark.parametrize("T,n_in,n_mid,n_out,sp,act", [(1024, 768, 768, 3072, 0.8, 2), (1024, 3072, 768, 2304, 0.8, 0),
                                                      (48, 256, 512, 64, 0.5, 1), (16, 32, 16, 16, 0.0, 0),
-                                                     (2048, 4096, 1024, 4096, 0.9, 2), (272, 160, 208, 800, 0.5, 0)])
+                                                     (2048, 4096, 1024, 4096, 0.9, 2), (272, 160, 208, 800, 0.5, 0),
+                                                     (48, 256, 4224, 64, 0.5, 0)])  # rows wider than two passes of 256 threads
 def test_split_layernorm_binary32_between_two_tile_linears(et, T, n_in, n_mid, n_out, sp, act):
     """The split normalisation of the mixed-precision layer: the producer stores X W^T + b + residual
     unrounded with its row sums, the consumer normalises that strip while staging it and writes
