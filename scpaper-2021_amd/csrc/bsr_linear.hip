@@ -83,6 +83,7 @@ constexpr int kFxNorm = 1;
 constexpr int kFxRes = 2;
 constexpr int kFxNorm32 = 4;  // with kFxNorm: binary32 strip
 constexpr int kFxRes32 = 8;   // with kFxRes: binary32 residual and result
+constexpr int kFxWide = 16;   // plain kernel built for up to 12 waves (170 registers): two row groups in flight
 
 constexpr int kXcds = 8;      // accelerator dies, each with a private L2
 constexpr int kLdsPad = 8;    // halfs
@@ -111,7 +112,7 @@ __device__ __forceinline__ int lane_read(int v, int lane) {
 // ACT is a template parameter: the epilogue carries no run-time branch and each
 // fused activation is a separately named kernel in a profile.
 template <int MT, bool STAGE, int ACT, int LN = 0, int FX = 0>
-__global__ __launch_bounds__(((MT == 1 && (FX & kFxRes32)) || (FX & kFxNorm32)) ? 768 : 512) void bsr16_linear_kernel(const BsrArgs a) {
+__global__ __launch_bounds__(((MT == 1 && (FX & kFxRes32)) || (FX & (kFxNorm32 | kFxWide))) ? 768 : 512) void bsr16_linear_kernel(const BsrArgs a) {
     static_assert(!LN || STAGE, "the fused LayerNorm prologue writes the strip to LDS");
     static_assert(!(FX & kFxNorm) || (STAGE && !LN), "the NORM prologue writes the strip to LDS");
     constexpr bool NORM = (FX & kFxNorm) != 0;
@@ -122,11 +123,13 @@ __global__ __launch_bounds__(((MT == 1 && (FX & kFxRes32)) || (FX & kFxNorm32)) 
     static_assert(!RES32 || RES, "kFxRes32 qualifies kFxRes");
     // row groups resident per wave: four; two in the kernels whose prologue normalises fp16 strips
     // (four would spill), three with a binary32 strip or a binary32 residual in flight per group
-    constexpr int kNB = NORM32 ? 2 : RES32 ? 3 : (LN || NORM) ? kGroupsAheadNorm : kGroupsAhead;
+    constexpr bool WIDE = (FX & kFxWide) != 0;
+    static_assert(!WIDE || (FX == kFxWide && !LN && MT <= 2), "the 12-wave form of the plain kernel");
+    constexpr int kNB = (NORM32 || WIDE) ? 2 : RES32 ? 3 : (LN || NORM) ? kGroupsAheadNorm : kGroupsAhead;
     // 16-byte strip vectors a thread requests before it writes the first to LDS: a 16-row strip of a
     // 3072-wide input (12 per thread of 512) is requested whole, so that none of it queues behind
     // the weight requests; binary32 vectors are two loads each
-    constexpr int kSU = (MT == 1 && !LN && !NORM && !RES32) ? 12 : NORM32 ? 4 : kStageU;
+    constexpr int kSU = WIDE ? 8 : (MT == 1 && !LN && !NORM && !RES32) ? 12 : NORM32 ? 4 : kStageU;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     _Float16 *xs = reinterpret_cast<_Float16 *>(smem_raw);
 
@@ -752,6 +755,12 @@ static BsrPlan plan_bsr(int T, int in, int out) {
     p.stage = true;
     int rpw = rows_per_wg_for(p.mt);
     p.threads = (rpw <= 6 || rpw == 18) ? 384 : 512;
+    // 16-row strips (inputs too wide for 32 rows) with 24 to 48 block-rows per workgroup: 12 waves of
+    // two to four rows instead of 8 waves of three to six, two row groups in flight per wave
+    // (2048 x 3072 -> 768: 13.6 -> 11.6 us, 16384 rows: 103 -> 87 us).  With fewer rows per
+    // workgroup the 8-wave form, which keeps four row groups in flight, is the faster one, and so it
+    // is on 32-row strips.
+    if (p.mt == 1 && rpw >= 24 && rpw <= 48) p.threads = 768;
     const int cap = kMaxWaveRows * (p.threads / 64);
     if (rpw > cap) rpw = cap;
     p.rows_per_wg = rpw;
@@ -870,6 +879,16 @@ static int launch_bsr_act(const BsrArgs &args, const BsrPlan &p, hipStream_t str
 
 template <int MT, bool STAGE>
 static int launch_bsr(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
+    if constexpr (STAGE && MT <= 2) {
+        if (p.threads > 512) {
+            switch (args.act) {
+                case ET_ACT_RELU: return launch_bsr_act<MT, STAGE, ET_ACT_RELU, 0, kFxWide>(args, p, stream);
+                case ET_ACT_GELU: return launch_bsr_act<MT, STAGE, ET_ACT_GELU, 0, kFxWide>(args, p, stream);
+                default: return launch_bsr_act<MT, STAGE, ET_ACT_NONE, 0, kFxWide>(args, p, stream);
+            }
+        }
+    }
+    ET_REQUIRE(p.threads <= 512, ET_ERR_INVALID_ARG, "tile-sparse Linear: %d threads need the 12-wave form", p.threads);
     switch (args.act) {
         case ET_ACT_RELU: return launch_bsr_act<MT, STAGE, ET_ACT_RELU>(args, p, stream);
         case ET_ACT_GELU: return launch_bsr_act<MT, STAGE, ET_ACT_GELU>(args, p, stream);
