@@ -137,13 +137,14 @@ template <> class Linear<tile_mat> {
     static bool wants_plan(int in, int rows) { return in >= 128 && (in > 5112 || (in >= 3072 && rows >= 4096)); }
     // Dense image of the weight, held where the dense GEMM is the faster kernel: a matrix that
     // keeps most of its tiles (measured at 2048 rows: the tile kernel overtakes the dense one at
-    // 35-50 % sparsity for 768-wide inputs, at 55 % for 3072-wide ones).  Not built when a tile
+    // 35-50 % sparsity for 768-wide inputs, at 50 % for 3072-wide ones).  Not built when a tile
     // position occurs twice (the tile kernel adds such tiles up, an image cannot).
     std::unique_ptr<et::DeviceBuffer<half>> dense;
     std::unique_ptr<et::DeviceBuffer<half>> dense_out16;  // fp16 result ahead of the widening in forward_f32
     static bool wants_dense(int in, int out, int ntile) {
         const double kept = (double)ntile * 256.0 / ((double)in * (double)out);
-        return kept > (in >= 3072 ? 0.45 : 0.50);
+        (void)in;
+        return kept > 0.50;
     }
 
     Linear(int _in_size, int _out_size, const tile_mat &w, const half *b, int _size)
