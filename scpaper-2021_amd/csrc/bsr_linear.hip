@@ -97,7 +97,6 @@ constexpr int kGroupsAhead = 4;
 constexpr int kGroupsAheadNorm = 2;
 constexpr int kStageU = 8;    // 16-byte strip vectors a thread keeps in flight
 constexpr int kMaxWaveRows = 64;  // block-rows one wave can own (one lane each)
-constexpr int kScalarRows = 4;    // up to this many, a wave fetches its row pointers with scalar loads
 
 template <int ACT> __device__ __forceinline__ float act_fixed(float x) {
     if (ACT == ET_ACT_RELU) return x > 0.0f ? x : 0.0f;
@@ -126,10 +125,9 @@ __global__ __launch_bounds__(((MT == 1 && (FX & kFxRes32)) || (FX & (kFxNorm32 |
     constexpr bool WIDE = (FX & kFxWide) != 0;
     static_assert(!WIDE || (FX == kFxWide && !LN && MT <= 2), "the 12-wave form of the plain kernel");
     constexpr int kNB = (NORM32 || WIDE) ? 2 : RES32 ? 3 : (LN || NORM) ? kGroupsAheadNorm : kGroupsAhead;
-    // 16-byte strip vectors a thread requests before it writes the first to LDS: a 16-row strip of a
-    // 3072-wide input (12 per thread of 512) is requested whole, so that none of it queues behind
-    // the weight requests; binary32 vectors are two loads each
-    constexpr int kSU = WIDE ? 8 : (MT == 1 && !LN && !NORM && !RES32) ? 12 : NORM32 ? 4 : kStageU;
+    // 16-byte strip vectors a thread requests before it writes the first to LDS; binary32 vectors are
+    // two loads each
+    constexpr int kSU = NORM32 ? 4 : kStageU;
     extern __shared__ __align__(16) unsigned char smem_raw[];
     _Float16 *xs = reinterpret_cast<_Float16 *>(smem_raw);
 
@@ -163,18 +161,7 @@ __global__ __launch_bounds__(((MT == 1 && (FX & kFxRes32)) || (FX & (kFxNorm32 |
     // issue order and everything below depends on these few bytes)
     const int nrw = max(0, (rb_end - rb_begin - wave + nwave - 1) / nwave);
     int rp_lo = 0, rp_hi = 0;
-    // A few rows: scalar loads, kept in scalar registers until the first use.  They do not queue in
-    // the vector memory pipeline behind the strip loads of the other waves of the compute unit.
-    const bool rows_scalar = nrw <= kScalarRows;
-    const auto *rpc = reinterpret_cast<const __attribute__((address_space(4))) int32_t *>(
-        reinterpret_cast<uintptr_t>(a.row_ptr));
-    auto rb_of = [&](int i) { return min(rb_begin + wave + nwave * i, nbr - 1); };
-    const int slo0 = rpc[rb_of(0)], shi0 = rpc[rb_of(0) + 1];
-    const int slo1 = rpc[rb_of(1)], shi1 = rpc[rb_of(1) + 1];
-    const int slo2 = rpc[rb_of(2)], shi2 = rpc[rb_of(2) + 1];
-    const int slo3 = rpc[rb_of(3)], shi3 = rpc[rb_of(3) + 1];
-    static_assert(kScalarRows == 4, "four named pairs");
-    if (!rows_scalar && lane < nrw) {
+    if (lane < nrw) {
         const int rb = rb_begin + wave + nwave * lane;
         rp_lo = a.row_ptr[rb];
         rp_hi = a.row_ptr[rb + 1];
@@ -295,10 +282,6 @@ __global__ __launch_bounds__(((MT == 1 && (FX & kFxRes32)) || (FX & (kFxNorm32 |
     int g_row[kNB], g_nsl[kNB];  // resident items: wave row index (-1 = none), slots in the item
     bool g_last[kNB];            // item ends its block-row
     int it_row = 0, it_part = 0;
-    if (rows_scalar) {  // the scalar row pointers take their lanes (first use: the wait for them is here)
-        rp_lo = lane == 0 ? slo0 : lane == 1 ? slo1 : lane == 2 ? slo2 : slo3;
-        rp_hi = lane == 0 ? shi0 : lane == 1 ? shi1 : lane == 2 ? shi2 : shi3;
-    }
     // skip rows without tiles (they are written at the end)
     auto skip_empty = [&]() {
         while (it_row < nrw && lane_read(rp_hi, it_row) == lane_read(rp_lo, it_row)) it_row++;
