@@ -1210,14 +1210,14 @@ int et_norm_linear_bsr16_f32in(const float *V, const float *stats, int stat_grou
 
 // Tuning hook: same computation with an explicit launch geometry.  mt in
 // {1,2,4}; stage selects the LDS-staged strip; threads a multiple of 64 up to
-// 512.  Not part of the drop-in surface.
+// 768 (above 512: 16- and 32-row strips).  Not part of the drop-in surface.
 int et_linear_bsr16_f16_geom(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles,
                              const et_f16 *bias, const et_f16 *X, et_f16 *Y, int T, int in,
                              int out, int act, int mt, int stage, int threads, int rows_per_wg,
                              et_stream stream) {
     int s = bsr_check(row_ptr, col_idx, tiles, X, Y, T, in, out, act);
     if (s != ET_OK) return s;
-    ET_REQUIRE((mt == 1 || mt == 2 || mt == 4) && threads >= 64 && threads <= 512 &&
+    ET_REQUIRE((mt == 1 || mt == 2 || mt == 4) && threads >= 64 && threads <= 768 &&
                    threads % 64 == 0 && rows_per_wg >= 1,
                ET_ERR_INVALID_ARG, "et_linear_bsr16_f16_geom: mt=%d threads=%d rows_per_wg=%d", mt,
                threads, rows_per_wg);
