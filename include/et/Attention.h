@@ -325,8 +325,12 @@ class Attention<_config, std::enable_if_t<_config::isSingleKernel>> : public et:
             half *K = Q + model->kdim;
             half *V = K + model->kdim;
             et::fused_mha(Q, K, V, ldm, ldm, ldm, mat_z->get(), model->vdim, *model, run(stream));
-            linearO->forward_resid_stats_f32(v1, stats1, groups1, mat_z->get(), in ? in->v : x32, in ? fin_in : nullptr,
-                                             in ? in->gamma : nullptr, in ? in->beta : nullptr, stream);
+            if (!in && !x32)  // first layer, residual = the binary16 input itself
+                linearO->forward_resid16_stats_f32(v1, stats1, groups1, mat_z->get(), x16, stream);
+            else
+                linearO->forward_resid_stats_f32(v1, stats1, groups1, mat_z->get(), in ? in->v : x32,
+                                                 in ? fin_in : nullptr, in ? in->gamma : nullptr, in ? in->beta : nullptr,
+                                                 stream);
         } else {
             (void)v1; (void)stats1; (void)groups1; (void)fin_in; (void)in; (void)x32; (void)x16; (void)stream;
             et::require(false, "Attention: the split normalisation needs tile-sparse projections");

@@ -216,6 +216,13 @@ template <> class Linear<tile_mat> {
                                               et::f16(resid_beta), V, stats, groups, size, (int)in_size, (int)out_size,
                                               stream));
     }
+    // the same with the residual in binary16
+    void forward_resid16_stats_f32(float *V, float *stats, int *groups, const half *input, const half *resid16,
+                                   et::stream_t stream = nullptr) {
+        etChk(et_linear_bsr16_resid16_stats_f32(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
+                                                et::f16(bias.get()), et::f16(input), et::f16(resid16), V, stats, groups,
+                                                size, (int)in_size, (int)out_size, stream));
+    }
     // output = act(normalised(V) W^T + bias); fin_out, ln32, ln16 optional (null = not wanted)
     void forward_norm_f32in(half *output, const float *V, const float *stats, int groups, const half *gamma,
                             const half *beta, float eps, float *fin_out, float *ln32, half *ln16, int act,

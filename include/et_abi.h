@@ -239,6 +239,13 @@ int et_linear_bsr16_resid_stats_f32(const int32_t *row_ptr, const int32_t *col_i
                                     const et_f16 *resid_beta, float *V, float *stats,
                                     int *stat_groups, int T, int in, int out,
                                     et_stream stream);
+/* The producer with its residual in binary16 (the first layer of a stack adds the model's
+ * binary16 input: no widened copy of it is needed); otherwise et_linear_bsr16_resid_stats_f32
+ * with resid_fin NULL. */
+int et_linear_bsr16_resid16_stats_f32(const int32_t *row_ptr, const int32_t *col_idx,
+                                      const et_f16 *tiles, const et_f16 *bias, const et_f16 *X,
+                                      const et_f16 *resid16, float *V, float *stats,
+                                      int *stat_groups, int T, int in, int out, et_stream stream);
 int et_norm_linear_bsr16_f32in(const float *V, const float *stats, int stat_groups,
                                const et_f16 *gamma, const et_f16 *beta, float eps,
                                float *fin_out, float *ln_out32, et_f16 *ln_out16,

@@ -102,6 +102,7 @@ _SIGNATURES = {
     "et_linear_bsr16_resid_stats_f32_supported": (_i, _i, _i),
     "et_norm_linear_bsr16_f32in_supported": (_i, _i, _i),
     "et_linear_bsr16_resid_stats_f32": (_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp),
+    "et_linear_bsr16_resid16_stats_f32": (_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp),
     "et_norm_linear_bsr16_f32in": (_vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_norm_from_stats_f32in": (_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _f, _vp),
     "et_linear_csr_f16": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),

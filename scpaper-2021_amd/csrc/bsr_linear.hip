@@ -68,6 +68,7 @@ struct BsrArgs {
     // the normalised rows go to ln_out32 and / or ln_out (either may be null), each vector written by
     // one of the strip's block-row groups.
     const float *resid32;
+    const _Float16 *resid16;  // RES32: when set, the residual in binary16 (resid32 unused)
     const float *X32;
     float *ln_out32;
     // RES32: when rs_fin is set the residual is not read but formed, as the normalisation of
@@ -271,7 +272,12 @@ __global__ __launch_bounds__(((MT == 1 && (FX & kFxRes32)) || (FX & (kFxNorm32 |
 #pragma unroll
         for (int m = 0; m < MT; m++) {
             const int tok = min(tok0 + m * 16 + r16, a.T - 1);
-            rs[m] = *reinterpret_cast<const f4 *>(a.resid32 + (size_t)tok * a.out + f0);
+            if (a.resid16) {  // wave-uniform
+                const h4 r = *reinterpret_cast<const h4 *>(a.resid16 + (size_t)tok * a.out + f0);
+                rs[m] = f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
+            } else {
+                rs[m] = *reinterpret_cast<const f4 *>(a.resid32 + (size_t)tok * a.out + f0);
+            }
         }
         gm = bt = h4{0, 0, 0, 0};
         if (a.rs_fin) {
@@ -1131,11 +1137,35 @@ int et_norm_linear_bsr16_f32in_supported(int T, int in, int out) {
     return fx32_shape_ok(T, in, out) && plan_bsr_fx32(T, in, out, kFxNorm).stage ? 1 : 0;
 }
 
+static int resid_stats_f32(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles, const et_f16 *bias,
+                           const et_f16 *X, const float *resid, const et_f16 *resid16, const float *resid_fin,
+                           const et_f16 *resid_gamma, const et_f16 *resid_beta, float *V, float *stats, int *stat_groups,
+                           int T, int in, int out, et_stream stream);
+
 int et_linear_bsr16_resid_stats_f32(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles,
                                     const et_f16 *bias, const et_f16 *X, const float *resid, const float *resid_fin,
                                     const et_f16 *resid_gamma, const et_f16 *resid_beta, float *V, float *stats,
                                     int *stat_groups, int T, int in, int out, et_stream stream) {
-    ET_REQUIRE(resid && V && stats && stat_groups, ET_ERR_INVALID_ARG, "et_linear_bsr16_resid_stats_f32: NULL pointer");
+    ET_REQUIRE(resid, ET_ERR_INVALID_ARG, "et_linear_bsr16_resid_stats_f32: NULL pointer");
+    return resid_stats_f32(row_ptr, col_idx, tiles, bias, X, resid, nullptr, resid_fin, resid_gamma, resid_beta, V, stats,
+                           stat_groups, T, in, out, stream);
+}
+
+int et_linear_bsr16_resid16_stats_f32(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles,
+                                      const et_f16 *bias, const et_f16 *X, const et_f16 *resid16, float *V, float *stats,
+                                      int *stat_groups, int T, int in, int out, et_stream stream) {
+    ET_REQUIRE(resid16, ET_ERR_INVALID_ARG, "et_linear_bsr16_resid16_stats_f32: NULL pointer");
+    ET_REQUIRE((reinterpret_cast<uintptr_t>(resid16) & 7) == 0, ET_ERR_UNSUPPORTED,
+               "et_linear_bsr16_resid16_stats_f32: the residual must be 8-byte aligned");
+    return resid_stats_f32(row_ptr, col_idx, tiles, bias, X, nullptr, resid16, nullptr, nullptr, nullptr, V, stats,
+                           stat_groups, T, in, out, stream);
+}
+
+static int resid_stats_f32(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles, const et_f16 *bias,
+                           const et_f16 *X, const float *resid, const et_f16 *resid16, const float *resid_fin,
+                           const et_f16 *resid_gamma, const et_f16 *resid_beta, float *V, float *stats, int *stat_groups,
+                           int T, int in, int out, et_stream stream) {
+    ET_REQUIRE(V && stats && stat_groups, ET_ERR_INVALID_ARG, "et_linear_bsr16_resid_stats_f32: NULL pointer");
     ET_REQUIRE(resid_fin == nullptr || (resid_gamma && resid_beta), ET_ERR_INVALID_ARG,
                "et_linear_bsr16_resid_stats_f32: a residual to normalise needs its affine vectors");
     ET_REQUIRE(V != resid, ET_ERR_INVALID_ARG, "et_linear_bsr16_resid_stats_f32: V must not alias the residual");
@@ -1162,6 +1192,7 @@ int et_linear_bsr16_resid_stats_f32(const int32_t *row_ptr, const int32_t *col_i
     args.st_out = stats;
     args.Y32 = V;
     args.resid32 = resid;
+    args.resid16 = reinterpret_cast<const _Float16 *>(resid16);
     args.rs_fin = resid_fin;
     args.rs_gamma = reinterpret_cast<const _Float16 *>(resid_gamma);
     args.rs_beta = reinterpret_cast<const _Float16 *>(resid_beta);

@@ -173,11 +173,10 @@ void check_layer_index(const et_model_s *m, int layer) {
 // every layer hands the next one its un-normalised binary32 result with its row sums.
 void run_layers_split(et_model_s &m, half *out, half *in, stream_t stream) {
     const int n = (int)m.layers.size();
-    const std::size_t elems = (std::size_t)m.rows() * m.desc.emdim;
-    etChk(et_f16_to_f32(m.pp32[0]->get(), et::f16(in), elems, stream));
+    // the first layer adds the binary16 input as its residual: no widened copy
     et::SplitSum carry;
     for (int i = 0; i < n; i++)
-        carry = m.layers[(size_t)i]->forward_split(i ? &carry : nullptr, m.pp32[0]->get(), in, stream);
+        carry = m.layers[(size_t)i]->forward_split(i ? &carry : nullptr, nullptr, in, stream);
     m.layers[(size_t)n - 1]->finish_split(nullptr, out, carry, stream);
 }
 

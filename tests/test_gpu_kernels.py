@@ -529,6 +529,16 @@ def test_split_layernorm_binary32_between_two_tile_linears(et, T, n_in, n_mid, n
     et.check(lib.et_linear_bsr16_resid_stats_f32(*common, d_v.ptr, d_fin.ptr, d_g.ptr, d_b.ptr, d_v2b.ptr,
                                                  d_st2b.ptr, C.byref(g2), T, n_out, n_mid, None))
     assert np.array_equal(d_v2a.numpy().view(np.uint32), d_v2b.numpy().view(np.uint32))
+    # a binary16 residual (the first layer of a stack adds the model's input): the same bits as with its widened copy
+    r16 = Hn.randn((T, n_mid), 46)
+    d_v2c, d_v2d = et.DeviceBuffer.empty((T, n_mid), np.float32), et.DeviceBuffer.empty((T, n_mid), np.float32)
+    d_st2c, d_st2d = et.DeviceBuffer.empty((16, T, 2), np.float32), et.DeviceBuffer.empty((16, T, 2), np.float32)
+    et.check(lib.et_linear_bsr16_resid_stats_f32(*common, et.DeviceBuffer.from_numpy(r16.astype(np.float32)).ptr, None, None,
+                                                 None, d_v2c.ptr, d_st2c.ptr, C.byref(g2), T, n_out, n_mid, None))
+    et.check(lib.et_linear_bsr16_resid16_stats_f32(*common, et.DeviceBuffer.from_numpy(r16).ptr, d_v2d.ptr, d_st2d.ptr,
+                                                   C.byref(g2), T, n_out, n_mid, None))
+    assert np.array_equal(d_v2c.numpy().view(np.uint32), d_v2d.numpy().view(np.uint32))
+    assert np.array_equal(d_st2c.numpy()[: g2.value].view(np.uint32), d_st2d.numpy()[: g2.value].view(np.uint32))
     assert np.array_equal(d_st2a.numpy()[:g2.value].view(np.uint32), d_st2b.numpy()[:g2.value].view(np.uint32))
     want_v2 = L.linear(Hn.f32(d_y.numpy()), Hn.f32(w3.dense), Hn.f32(w3.bias)).numpy() + want_ln
     assert Hn.max_abs(d_v2b.numpy(), want_v2) <= 3e-4 * max(1.0, float(np.abs(want_v2).max()))
