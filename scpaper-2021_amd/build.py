@@ -28,7 +28,10 @@ HIPCC = os.environ.get("HIPCC") or shutil.which("hipcc") or "/opt/rocm/bin/hipcc
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-I", str(ROOT / "include"), "-Wall", "-Wno-unused-function"]
 # Packed-fp32 code generation is switched off for device code.
 DEVICE = [f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-          "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument"]
+          "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument",
+          "-Rpass-analysis=kernel-resource-usage"]  # registers and scratch of every kernel, kept in RESOURCES
+RESOURCES = LIBDIR / "kernel_resources.txt"
+_resource_lines: list[str] = []
 
 
 def sources() -> list[Path]:
@@ -47,7 +50,29 @@ def _compile(src: Path) -> Path:
     # hipcc's host pass does not know the packed-fp32 feature name; that
     # warning is expected and dropped here.
     noise = ("is not a recognized feature for this target", "'-packed-fp32-ops'")
-    err = "\n".join(l for l in res.stderr.splitlines() if not any(n in l for n in noise))
+    lines = [l for l in res.stderr.splitlines() if not any(n in l for n in noise)]
+    # "file:line:col: remark: Function Name: f [-Rpass-analysis=...]", then "remark:     VGPRs: n [...]" lines,
+    # each followed by two lines of source context
+    name = None
+    kept = []
+    skip_context = 0
+    for l in lines:
+        if "remark:" in l and "[-Rpass-analysis=kernel-resource-usage]" in l:
+            text = l.split("remark:", 1)[1].replace("[-Rpass-analysis=kernel-resource-usage]", "").strip()
+            if text.startswith("Function Name:"):
+                name = text.split(":", 1)[1].strip()
+                _resource_lines.append(f"{src.name} {name}")
+            elif name and text.split(":")[0] in ("TotalSGPRs", "VGPRs", "ScratchSize [bytes/lane]", "Occupancy [waves/SIMD]",
+                                                  "LDS Size [bytes/block]"):
+                _resource_lines[-1] += " | " + text
+            skip_context = 2
+            continue
+        if skip_context and ("|" in l):
+            skip_context -= 1
+            continue
+        skip_context = 0
+        kept.append(l)
+    err = "\n".join(kept)
     if res.returncode != 0:
         raise RuntimeError(f"compile failed: {' '.join(cmd)}\n{err}")
     if err.strip():
@@ -59,6 +84,7 @@ def build_all(jobs: int | None = None, verbose: bool = True) -> Path:
     """Compile every source for gfx950 and link the shared library."""
     BUILD.mkdir(exist_ok=True)
     LIBDIR.mkdir(exist_ok=True)
+    _resource_lines.clear()
     srcs = sources()
     jobs = jobs or min(8, len(srcs))
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
@@ -69,6 +95,7 @@ def build_all(jobs: int | None = None, verbose: bool = True) -> Path:
     if res.returncode != 0:
         raise RuntimeError(f"link failed: {' '.join(cmd)}\n{res.stderr}")
     os.replace(tmp, LIB)
+    RESOURCES.write_text("\n".join(sorted(_resource_lines)) + "\n")
     if verbose:
         print(f"built {LIB} from {len(srcs)} sources")
     build_programs(verbose)

@@ -84,6 +84,8 @@ constexpr int kFxNorm = 1;
 constexpr int kFxRes = 2;
 constexpr int kFxNorm32 = 4;  // with kFxNorm: binary32 strip
 constexpr int kFxRes32 = 8;   // with kFxRes: binary32 residual and result
+constexpr int kFxRes16 = 32;  // with kFxRes32: the residual is read as binary16 (a kernel of its own, so that the
+                              // 12-wave producer, at 168 registers, carries no second path)
 constexpr int kFxWide = 16;   // plain kernel built for up to 12 waves (170 registers): two row groups in flight
 
 constexpr int kXcds = 8;      // accelerator dies, each with a private L2
@@ -112,7 +114,7 @@ __device__ __forceinline__ int lane_read(int v, int lane) {
 // ACT is a template parameter: the epilogue carries no run-time branch and each
 // fused activation is a separately named kernel in a profile.
 template <int MT, bool STAGE, int ACT, int LN = 0, int FX = 0>
-__global__ __launch_bounds__(((MT == 1 && (FX & kFxRes32)) || (FX & (kFxNorm32 | kFxWide))) ? 768 : 512) void bsr16_linear_kernel(const BsrArgs a) {
+__global__ __launch_bounds__(((MT == 1 && (FX & kFxRes32) && !(FX & kFxRes16)) || (FX & (kFxNorm32 | kFxWide))) ? 768 : 512) void bsr16_linear_kernel(const BsrArgs a) {
     static_assert(!LN || STAGE, "the fused LayerNorm prologue writes the strip to LDS");
     static_assert(!(FX & kFxNorm) || (STAGE && !LN), "the NORM prologue writes the strip to LDS");
     constexpr bool NORM = (FX & kFxNorm) != 0;
@@ -272,7 +274,7 @@ __global__ __launch_bounds__(((MT == 1 && (FX & kFxRes32)) || (FX & (kFxNorm32 |
 #pragma unroll
         for (int m = 0; m < MT; m++) {
             const int tok = min(tok0 + m * 16 + r16, a.T - 1);
-            if (a.resid16) {  // wave-uniform
+            if constexpr ((FX & kFxRes16) != 0) {
                 const h4 r = *reinterpret_cast<const h4 *>(a.resid16 + (size_t)tok * a.out + f0);
                 rs[m] = f4{(float)r[0], (float)r[1], (float)r[2], (float)r[3]};
             } else {
@@ -926,6 +928,11 @@ static int dispatch_bsr_norm32(const BsrArgs &args, const BsrPlan &p, hipStream_
                      : dispatch_bsr_fx_act<1, kFxNorm | kFxNorm32>(args, p, stream);
 }
 static int dispatch_bsr_res32(const BsrArgs &args, const BsrPlan &p, hipStream_t stream) {
+    if (args.resid16) {  // 8 waves at most: this kernel is not built for the 12-wave launch
+        ET_REQUIRE(p.threads <= 512, ET_ERR_INVALID_ARG, "tile-sparse Linear: the binary16-residual producer runs at most 8 waves");
+        return p.mt == 2 ? launch_bsr_act<2, true, ET_ACT_NONE, 0, kFxRes | kFxRes32 | kFxRes16>(args, p, stream)
+                         : launch_bsr_act<1, true, ET_ACT_NONE, 0, kFxRes | kFxRes32 | kFxRes16>(args, p, stream);
+    }
     return p.mt == 2 ? launch_bsr_act<2, true, ET_ACT_NONE, 0, kFxRes | kFxRes32>(args, p, stream)
                      : launch_bsr_act<1, true, ET_ACT_NONE, 0, kFxRes | kFxRes32>(args, p, stream);
 }
@@ -1176,6 +1183,7 @@ static int resid_stats_f32(const int32_t *row_ptr, const int32_t *col_idx, const
     BsrPlan p = plan_bsr_fx32(T, in, out, kFxRes);
     ET_REQUIRE(p.stage, ET_ERR_UNSUPPORTED, "et_linear_bsr16_resid_stats_f32: in=%d out=%d outside the staged range", in,
                out);
+    if (resid16 && p.threads > 512) p.threads = 512;
     *stat_groups = (out / 16 + p.rows_per_wg - 1) / p.rows_per_wg;
     if (T == 0) return ET_OK;
     BsrArgs args{};
