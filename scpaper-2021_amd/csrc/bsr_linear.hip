@@ -124,7 +124,9 @@ __global__ __launch_bounds__(((MT == 1 && (FX & kFxRes32) && !(FX & kFxRes16)) |
     constexpr bool RES32 = (FX & kFxRes32) != 0;
     static_assert(!RES32 || RES, "kFxRes32 qualifies kFxRes");
     // row groups resident per wave: four; two in the kernels whose prologue normalises fp16 strips
-    // (four would spill), three with a binary32 strip or a binary32 residual in flight per group
+    // (four would spill) and in the forms built for 12 waves of at most two to four block-rows (the
+    // consumer of a binary32 strip, the wide plain kernel); three with a binary32 residual in flight
+    // per group
     constexpr bool WIDE = (FX & kFxWide) != 0;
     static_assert(!WIDE || (FX == kFxWide && !LN && MT <= 2), "the 12-wave form of the plain kernel");
     constexpr int kNB = (NORM32 || WIDE) ? 2 : RES32 ? 3 : (LN || NORM) ? kGroupsAheadNorm : kGroupsAhead;
