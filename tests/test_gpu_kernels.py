@@ -559,7 +559,8 @@ def test_split_layernorm_rejects_unsupported(et):
 
 
 @pytest.mark.parametrize("mt,stage,threads,rpw", [(1, 1, 256, 4), (2, 1, 128, 3), (4, 1, 512, 8),
-                                                  (4, 0, 256, 5), (1, 0, 64, 1), (2, 0, 512, 48)])
+                                                  (4, 0, 256, 5), (1, 0, 64, 1), (2, 0, 512, 48),
+                                                  (1, 1, 768, 24), (2, 1, 768, 48), (1, 1, 640, 7), (2, 1, 576, 10)])  # the 12-wave form
 def test_linear_bsr16_every_geometry(et, mt, stage, threads, rpw):
     """Each launch geometry of the kernel gives the same result, including a token count that
     is not a multiple of the strip."""
@@ -572,6 +573,17 @@ def test_linear_bsr16_every_geometry(et, mt, stage, threads, rpw):
                                                None))
     want = L.linear(Hn.f32(x), Hn.f32(w.dense), Hn.f32(w.bias), "gelu", torch.float16)
     assert Hn.max_abs(d_y.numpy(), want.numpy()) <= 4e-3
+
+
+def test_linear_bsr16_geometry_limits(et):
+    """64-row strips have no 12-wave form, and no geometry runs more than 12 waves: refused, not launched."""
+    w = Hn.BsrWeight(768, 768, 0.8, seed=41).upload(et)
+    d = et.DeviceBuffer.empty((64, 768), np.float16)
+    call = lambda mt, threads: et.lib().et_linear_bsr16_f16_geom(w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr,
+                                                               w.d_bias.ptr, d.ptr, d.ptr, 64, 768, 768, 0, mt, 1, threads,
+                                                               8, None)
+    assert call(4, 768) == et.ET_ERR_INVALID_ARG
+    assert call(1, 832) == et.ET_ERR_INVALID_ARG
 
 
 # ---------------------------------------------------------------- attention --
