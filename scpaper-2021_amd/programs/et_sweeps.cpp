@@ -91,21 +91,41 @@ static int run_seqlen() {
 }
 
 // ---- test/Table2 ----------------------------------------------------------------
-template <typename encoder_t> static double time_layers(std::vector<std::unique_ptr<encoder_t>> &model, model_para_t para) {
+struct layer_times {
+    double eager;     // launches issued one by one, as the reference's driver does
+    double replayed;  // the same launches recorded once in a graph and replayed
+};
+
+template <typename encoder_t>
+static layer_times time_layers(std::vector<std::unique_ptr<encoder_t>> &model, model_para_t para) {
     et::DeviceBuffer<half> IN((std::size_t)para->emdim * para->seq_len, static_cast<half>(0.2f));
     et::DeviceBuffer<half> OUT((std::size_t)para->emdim * para->seq_len);
     for (auto &layer : model) layer->forward(OUT.get(), IN.get());
     etChk(et_device_sync());
-    return wtime_new(
+    layer_times t;
+    t.eager = wtime_new(
         50,
         [&]() {
             for (auto &layer : model) layer->forward(OUT.get(), IN.get());
         },
         []() { etChk(et_device_sync()); });
+    et_stream stream = nullptr;
+    et_graph graph = nullptr;
+    etChk(et_stream_create(&stream));
+    etChk(et_graph_begin_capture(stream));
+    for (auto &layer : model) layer->forward(OUT.get(), IN.get(), stream);
+    etChk(et_graph_end_capture(stream, &graph));
+    etChk(et_graph_launch(graph, stream));
+    etChk(et_stream_sync(stream));
+    t.replayed = wtime_new(
+        50, [&]() { etChk(et_graph_launch(graph, stream)); }, [&]() { etChk(et_stream_sync(stream)); });
+    etChk(et_graph_destroy(graph));
+    etChk(et_stream_destroy(stream));
+    return t;
 }
 
 // every matrix of the layer pruned in tiles at one sparsity (template.hpp:13-52)
-static double test_uniform_tile(model_para_t para, float sparsity, int nlayer) {
+static layer_times test_uniform_tile(model_para_t para, float sparsity, int nlayer) {
     using mat_t = tile_mat;
     using attn_config = Attention_config<mat_t, mat_t, mat_t, mat_t, OTF_attn_full, true, false>;
     using encoder_config = Encoder_config<attn_config, mat_t, mat_t, GELU_OP>;
@@ -123,7 +143,7 @@ static double test_uniform_tile(model_para_t para, float sparsity, int nlayer) {
 }
 
 // attention-aware: W_V row-pruned, compact V, the rest tile-pruned (template.hpp:78-118)
-static double test_prune_attn(model_para_t para, float sparsity, int nlayer) {
+static layer_times test_prune_attn(model_para_t para, float sparsity, int nlayer) {
     using attn_config = Attention_config<tile_mat, tile_mat, row_mat, tile_mat, Prune_attn, false, true>;
     using encoder_config = Encoder_config<attn_config, tile_mat, tile_mat, GELU_OP>;
     std::vector<std::unique_ptr<Encoder<encoder_config>>> model((std::size_t)nlayer);
@@ -147,13 +167,18 @@ static int run_table2(int nlayer, const std::vector<float> &sparsities) {
     std::printf("# %d encoder layers, seq 128, hidden 768, FFN 3072; columns: sparsity", nlayer);
     for (float sp : sparsities) std::printf(" %.2f", sp);
     std::printf("; ms per forward of all layers\n");
-    std::vector<double> tile, aware;
+    std::vector<double> tile, aware, tile_graph, aware_graph;
     for (float sp : sparsities) {
-        tile.push_back(test_uniform_tile(para, sp, nlayer) / 1000);
-        aware.push_back(test_prune_attn(para, sp, nlayer) / 1000);
+        const layer_times t = test_uniform_tile(para, sp, nlayer), a = test_prune_attn(para, sp, nlayer);
+        tile.push_back(t.eager / 1000);
+        aware.push_back(a.eager / 1000);
+        tile_graph.push_back(t.replayed / 1000);
+        aware_graph.push_back(a.replayed / 1000);
     }
     print_series("tile", tile);
     print_series("aware", aware);
+    print_series("tile_graph", tile_graph);
+    print_series("aware_graph", aware_graph);
     return 0;
 }
 
