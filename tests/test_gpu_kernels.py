@@ -170,6 +170,43 @@ def test_linear_bsr16(et, T, inp, out, sp, act):
     assert err <= 4e-3
 
 
+def _random_bsr_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        T = 16 * int(rng.integers(1, 25))
+        inp = 16 * int(rng.integers(1, 65)) if rng.random() < 0.8 else 16 * int(rng.integers(192, 340))
+        out = 16 * int(rng.integers(1, 65)) if rng.random() < 0.8 else 16 * int(rng.integers(100, 200))
+        sp = float(rng.choice([0.0, 0.3, 0.5, 0.8, 0.9, 0.97, 1.0]))
+        cases.append((T, inp, out, sp, int(rng.integers(0, 3)), int(rng.integers(1, 1 << 30))))
+    return cases
+
+
+@pytest.mark.parametrize("T,inp,out,sp,act,seed", _random_bsr_cases(32, 20211114))
+def test_linear_bsr16_random_shapes(et, T, inp, out, sp, act, seed):
+    """Seeded random shapes (every launch plan the shape picks: strips of 16, 32 or 64 rows, staged or not, 6, 8
+    or 12 waves), binary16 and binary32 result against the oracle."""
+    w = Hn.BsrWeight(out, inp, sp, seed=seed, bias_std=0.1).upload(et)
+    x = Hn.randn((T, inp), seed ^ 0x5a5a)
+    d_x = up(et, x)
+    d_y, d_y32 = et.DeviceBuffer.empty((T, out), np.float16), et.DeviceBuffer.empty((T, out), np.float32)
+    w.forward(et, d_x, d_y, T, act)
+    et.check(et.lib().et_linear_bsr16_f16_f32out(w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, w.d_bias.ptr, d_x.ptr,
+                                                d_y32.ptr, T, inp, out, act, None))
+    et.sync()
+    name = {0: None, 1: "relu", 2: "gelu"}[act]
+    want = L.linear(Hn.f32(x), Hn.f32(w.dense), Hn.f32(w.bias), name, torch.float32).numpy()
+    scale = max(1.0, float(np.abs(want).max()))
+    assert Hn.max_abs(d_y32.numpy(), want) <= 2e-4 * scale  # accumulation order only
+    assert Hn.max_abs(d_y.numpy(), want) <= 1.5e-3 * scale  # one binary16 rounding of the result on top
+    a, b = d_y32.numpy().astype(np.float16), d_y.numpy()
+    if act != 2:
+        assert np.array_equal(a, b)
+    else:  # the two instantiations of the tanh-GELU epilogue may differ in the last binary32 bit
+        ulp = np.spacing(np.maximum(np.abs(a), np.abs(b)).astype(np.float16)).astype(np.float32)
+        assert np.all(np.abs(a.astype(np.float32) - b.astype(np.float32)) <= ulp)
+
+
 @pytest.mark.parametrize("inp,out,sp", [(256, 128, 0.0), (768, 3072, 0.3), (3072, 768, 0.5), (64, 16, 0.9)])
 def test_bsr16_dense_image(et, inp, out, sp):
     """The dense image the class multiplies with for weights that keep most of their tiles."""
@@ -451,10 +488,18 @@ def test_split_layernorm_between_two_tile_linears(et, T, n_in, n_mid, n_out, sp,
     assert np.array_equal(d_ln2.numpy().view(np.uint16), ln.view(np.uint16))
 
 
+def _random_split_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    return [(16 * int(rng.integers(1, 21)), 16 * int(rng.integers(1, 49)), 16 * int(rng.integers(1, 129)),
+             16 * int(rng.integers(1, 65)), float(rng.choice([0.0, 0.5, 0.8, 0.9, 0.97])), int(rng.integers(0, 3)))
+            for _ in range(n)]
+
+
 @pytest.mark.parametrize("T,n_in,n_mid,n_out,sp,act", [(1024, 768, 768, 3072, 0.8, 2), (1024, 3072, 768, 2304, 0.8, 0),
                                                      (48, 256, 512, 64, 0.5, 1), (16, 32, 16, 16, 0.0, 0),
                                                      (2048, 4096, 1024, 4096, 0.9, 2), (272, 160, 208, 800, 0.5, 0),
-                                                     (48, 256, 4224, 64, 0.5, 0)])  # rows wider than two passes of 256 threads
+                                                     (48, 256, 4224, 64, 0.5, 0)]  # rows wider than two passes of 256 threads
+                         + _random_split_cases(16, 20211115))
 def test_split_layernorm_binary32_between_two_tile_linears(et, T, n_in, n_mid, n_out, sp, act):
     """The split normalisation of the mixed-precision layer: the producer stores X W^T + b + residual
     unrounded with its row sums, the consumer normalises that strip while staging it and writes
@@ -679,6 +724,34 @@ def test_mha_head_sizes_between_template_sizes(et, B, S, nh, hd, causal):
     got, want = run_mha(et, B, S, nh, hd, seed=70, lens=lens, causal=causal)
     assert Hn.max_abs(got, want) <= 2e-3
     got, want = run_mha(et, B, S, nh, hd, seed=71, single_buffer=True)
+    assert Hn.max_abs(got, want) <= 2e-3
+
+
+def _random_mha_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        S = 16 * int(rng.integers(1, 41))
+        B, nh, hd = int(rng.integers(1, 7)), int(rng.integers(1, 9)), 16 * int(rng.integers(1, 9))
+        kind = int(rng.integers(0, 4))  # 0 plain, 1 right padding, 2 causal, 3 additive mask with padding
+        cases.append((B, S, nh, hd, kind, int(rng.integers(1, 1 << 30))))
+    return cases
+
+
+@pytest.mark.parametrize("B,S,nh,hd,kind,seed", _random_mha_cases(24, 20211116))
+def test_mha_random_shapes(et, B, S, nh, hd, kind, seed):
+    """Seeded random shapes: every head size from 16 to 128, 1 to 40 query tiles, plain, padded, causal and
+    additively masked, separate and interleaved Q/K/V buffers."""
+    rng = np.random.default_rng(seed)
+    lens = rng.integers(0, S + 1, B).astype(np.int32) if kind in (1, 3) else None
+    # the mask is binary16 data: the oracle gets the same rounded values the kernel reads
+    mask = (rng.standard_normal((S, S)) * 2.0).astype(np.float16).astype(np.float32) if kind == 3 else None
+    got, want = run_mha(et, B, S, nh, hd, seed=seed & 0xFFFF, lens=lens, causal=kind == 2, mask=mask,
+                        single_buffer=bool(seed & 1))
+    if lens is not None:  # rows past a sequence's length are padding: not compared
+        for b in range(B):
+            got[b * S + lens[b]:(b + 1) * S] = 0
+            want[b * S + lens[b]:(b + 1) * S] = 0
     assert Hn.max_abs(got, want) <= 2e-3
 
 
