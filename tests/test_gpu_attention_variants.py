@@ -146,6 +146,49 @@ def test_vo_attention_on_chip_masks(et, causal, masked, B, S, H, nh):
     assert Hn.max_abs(d_out.numpy(), want) <= 6e-3
 
 
+def _random_vo_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        nh, hd = int(rng.integers(1, 13)), 16 * int(rng.integers(1, 9))
+        cases.append((int(rng.integers(1, 5)), 16 * int(rng.integers(1, 21)), nh, hd, 16 * int(rng.integers(1, 25)),
+                      int(rng.integers(0, 4)), int(rng.integers(1, 1 << 30))))
+    return cases
+
+
+@pytest.mark.parametrize("B,S,nh,hd,N,kind,seed", _random_vo_cases(20, 20211118))
+def test_vo_attention_on_chip_random_shapes(et, B, S, nh, hd, N, kind, seed):
+    """Seeded random shapes of the on-chip VO attention (any number of heads up to 12, head sizes 16 to 128,
+    output widths that leave a partial column slice): plain, padded, causal, additively masked with padding."""
+    rng = np.random.default_rng(seed)
+    T, H = B * S, nh * hd
+    q, k = Hn.randn((T, H), seed & 0xFFF), Hn.randn((T, H), (seed & 0xFFF) + 1)
+    vo = (Hn.randn((B, nh, S, N), 42).astype(np.float32) * 0.25).astype(np.float16)
+    bvo, bo = Hn.randn((nh, N), 45, 0.1), Hn.randn((N,), 43)
+    lens = rng.integers(0, S + 1, B).astype(np.int32) if kind in (1, 3) else None
+    mask = (rng.standard_normal((S, S)) * 2).astype(np.float16) if kind == 3 else None
+    d_out = et.DeviceBuffer.empty((T, N), np.float16)
+    vo_keys = np.ascontiguousarray(vo.transpose(0, 1, 3, 2))  # [B][nh][N][S]
+    et.check(et.lib().et_mha_vo_otf_f16(up(et, q).ptr, up(et, k).ptr, H, H, up(et, vo_keys).ptr, up(et, bvo).ptr, d_out.ptr,
+                                        up(et, bo).ptr, None, None if mask is None else up(et, mask).ptr,
+                                        None if lens is None else up(et, lens).ptr, B, S, nh, hd, N, N,
+                                        1 / math.sqrt(hd), et.MHA_CAUSAL if kind == 2 else 0, None))
+    want = np.zeros((T, N), np.float32)
+    for h in range(nh):
+        sl = slice(h * hd, (h + 1) * hd)
+        v_h = (vo[:, h].astype(np.float32) + bvo[h].astype(np.float32)).reshape(T, N)
+        z = L.mha(Hn.f32(q[:, sl]), Hn.f32(k[:, sl]), torch.from_numpy(v_h), 1, B, scale=1 / math.sqrt(hd),
+                  mask=None if mask is None else Hn.f32(mask), lens=lens, causal=kind == 2, store=None)
+        want += z.numpy()
+    want += bo.astype(np.float32)
+    got = d_out.numpy().astype(np.float32)
+    if lens is not None:  # rows past a sequence's length are padding: not compared
+        for b in range(B):
+            got[b * S + lens[b]:(b + 1) * S] = 0
+            want[b * S + lens[b]:(b + 1) * S] = 0
+    assert Hn.max_abs(got, want) <= 6e-3 * max(1.0, float(np.abs(want).max()) / 4)
+
+
 def test_vo_attention_on_chip_rejects_bad_shapes(et):
     d = et.DeviceBuffer.empty((64, 64), np.float16)
     call = lambda **kw: et.lib().et_mha_vo_otf_f16(d.ptr, d.ptr, kw.get("ld", 64), 64, d.ptr, None, d.ptr, None, None, None, None,
@@ -176,6 +219,43 @@ def test_compact_v_attention(et, B, S, nh, hd, keep):
     v_full[:, col_id] = vc
     want = L.mha(Hn.f32(q), Hn.f32(k), Hn.f32(v_full), nh, B, lens=lens, store=torch.float16).numpy()
     got = d_z.numpy()
+    assert Hn.max_abs(got, want) <= 2e-3
+    dead = np.setdiff1d(np.arange(H), col_id)
+    assert np.all(got[:, dead] == 0)
+
+
+def _random_compact_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    return [(int(rng.integers(1, 5)), 16 * int(rng.integers(1, 25)), int(rng.integers(1, 13)), 16 * int(rng.integers(1, 9)),
+             float(rng.choice([0.25, 0.5, 0.75, 0.9])), bool(rng.integers(0, 2)), int(rng.integers(1, 1 << 30)))
+            for _ in range(n)]
+
+
+@pytest.mark.parametrize("B,S,nh,hd,keep,causal,seed", _random_compact_cases(20, 20211119))
+def test_compact_v_attention_random_shapes(et, B, S, nh, hd, keep, causal, seed):
+    """Seeded random shapes of the compact-V attention: surviving columns of every count per head (none, a
+    few, runs that do and do not start on multiples of 8), right padding, causal or not."""
+    rng = np.random.default_rng(seed)
+    H, T = nh * hd, B * S
+    q, k = Hn.randn((T, H), seed & 0xFFF), Hn.randn((T, H), (seed & 0xFFF) + 1)
+    col_id = F.gen_row_ids(H, 1 - keep, seed=seed)
+    hp = F.head_ptr(col_id, len(col_id), nh, H)
+    vc = Hn.randn((T, max(len(col_id), 1)), 33)[:, :len(col_id)]
+    vc = np.ascontiguousarray(vc)
+    lens = rng.integers(0, S + 1, B).astype(np.int32)
+    d_z = et.DeviceBuffer.empty((T, H), np.float16)
+    et.check(et.lib().et_fill_f16(d_z.ptr, T * H, 0x7E00, None))
+    et.check(et.lib().et_mha_compactv_f16(up(et, q).ptr, up(et, k).ptr, up(et, vc).ptr, H, H, len(col_id),
+                                          up(et, col_id).ptr, up(et, hp).ptr, len(col_id), d_z.ptr, H, None,
+                                          up(et, lens).ptr, B, S, nh, hd, hd, 1 / math.sqrt(hd),
+                                          et.MHA_CAUSAL if causal else 0, None))
+    v_full = np.zeros((T, H), np.float16)
+    v_full[:, col_id] = vc
+    want = L.mha(Hn.f32(q), Hn.f32(k), Hn.f32(v_full), nh, B, lens=lens, causal=causal, store=torch.float16).numpy()
+    got = d_z.numpy()
+    for b in range(B):  # rows past a sequence's length are padding: not compared
+        got[b * S + lens[b]:(b + 1) * S] = 0
+        want[b * S + lens[b]:(b + 1) * S] = 0
     assert Hn.max_abs(got, want) <= 2e-3
     dead = np.setdiff1d(np.arange(H), col_id)
     assert np.all(got[:, dead] == 0)

@@ -35,6 +35,48 @@ def test_linear_dense(et, T, inp, out, act):
     assert Hn.max_abs(d_y.numpy(), want) <= 4e-3
 
 
+def _random_dense_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        big = rng.random() < 0.3  # some shapes large enough for the 128- and 256-wide tiles
+        T = 16 * int(rng.integers(1, 200 if big else 40))
+        inp = 16 * int(rng.integers(1, 100))
+        out = 16 * int(rng.integers(1, 200 if big else 60))
+        cases.append((T, inp, out, int(rng.integers(0, 3)), int(rng.integers(1, 1 << 30))))
+    return cases
+
+
+@pytest.mark.parametrize("T,inp,out,act,seed", _random_dense_cases(32, 20211117))
+def test_linear_dense_random_shapes(et, T, inp, out, act, seed):
+    """Seeded random shapes, multiples of 16 only: whichever GEMM form and tile the shape picks (one 16x16 tile per
+    workgroup, 64x64, the direct-to-LDS tiles, full or ragged edges), and the row- and column-pruned Linears on
+    top of the same GEMM with a random half of the features."""
+    W, b, x = Hn.randn((out, inp), seed & 0xFFFF, 0.02), Hn.randn((out,), 2, 0.1), Hn.randn((T, inp), 3)
+    d_W, d_b, d_x = up(et, W), up(et, b), up(et, x)
+    d_y = et.DeviceBuffer.empty((T, out), np.float16)
+    et.linear_dense(d_W, d_b, d_x, d_y, T, inp, out, act)
+    want = L.linear(Hn.f32(x), Hn.f32(W), Hn.f32(b), ACT[act], torch.float16).numpy()
+    assert Hn.max_abs(d_y.numpy(), want) <= 4e-3
+    lib = et.lib()
+    row_id = F.gen_row_ids(out, 0.5, seed=seed)
+    if len(row_id):
+        rows = np.ascontiguousarray(W[row_id])
+        et.check(lib.et_fill_f16(d_y.ptr, T * out, 0x7E00, None))
+        et.check(lib.et_linear_rowpruned_f16(up(et, rows).ptr, up(et, row_id).ptr, len(row_id), d_b.ptr, d_x.ptr,
+                                             d_y.ptr, T, inp, out, act, None))
+        want_r = L.linear_rowpruned(Hn.f32(x), Hn.f32(rows), row_id, out, Hn.f32(b), ACT[act], torch.float16).numpy()
+        assert Hn.max_abs(d_y.numpy(), want_r) <= 4e-3
+    col_id = F.gen_col_ids(inp, 0.5, seed=seed + 1)
+    if len(col_id):
+        cols = np.ascontiguousarray(W[:, col_id])
+        et.check(lib.et_fill_f16(d_y.ptr, T * out, 0x7E00, None))
+        et.check(lib.et_linear_colpruned_f16(up(et, cols).ptr, up(et, col_id).ptr, len(col_id), d_b.ptr, d_x.ptr,
+                                             d_y.ptr, T, inp, out, act, None))
+        want_c = L.linear_colpruned(Hn.f32(x), Hn.f32(cols), col_id, Hn.f32(b), ACT[act], torch.float16).numpy()
+        assert Hn.max_abs(d_y.numpy(), want_c) <= 4e-3
+
+
 @pytest.mark.parametrize("T,inp,out", [(4096, 128, 4096), (512, 768, 768)])
 def test_linear_dense_without_bias(et, T, inp, out):
     W, x = Hn.randn((out, inp), 21, 0.02), Hn.randn((T, inp), 22)
