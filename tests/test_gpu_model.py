@@ -193,6 +193,40 @@ def test_mixed_small_stack_graph_eager_inplace_and_single_layers(et, use_graph, 
     assert Hn.max_abs(bufs[1].numpy(np.float16, (B * S, H)), ref.numpy()) <= 4e-3
 
 
+def _random_stack_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        nh = int(rng.integers(1, 9))
+        hd = 16 * int(rng.integers(1, 5))
+        cases.append((nh * hd, nh, 16 * int(rng.integers(2, 49)), 16 * int(rng.integers(1, 13)), int(rng.integers(1, 6)),
+                      int(rng.integers(1, 4)), float(rng.choice([0.3, 0.6, 0.8, 0.9])), int(rng.integers(0, 3)),
+                      bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), int(rng.integers(1, 1 << 20))))
+    return cases
+
+
+@pytest.mark.parametrize("H,nh,FF,S,B,nlayer,sp,mode,padded,causal,seed", _random_stack_cases(18, 20211120))
+def test_random_stacks(et, H, nh, FF, S, B, nlayer, sp, mode, padded, causal, seed):
+    """Seeded random encoder stacks through the model handle: hidden sizes 16 to 512, 1 to 8 heads of 16 to 64,
+    1 to 3 layers, every precision mode (all binary16 storage, binary32 residual stream with SkipLayerNorm folded
+    or launched), tile sparsities on both sides of the dense-image threshold, right padding, causal attention."""
+    layers = [Hn.LayerWeights(H, nh, FF, sp, seed=seed + i) for i in range(nlayer)]
+    rng = np.random.default_rng(seed)
+    lens = rng.integers(1, S + 1, B).astype(np.int32) if padded else None
+    m = Hn.build_model(et, layers, S, B, lens=lens, causal=causal, mixed=mode)
+    x = Hn.randn((B * S, H), seed ^ 0x77)
+    got = run_model(et, m, x, reps=2)
+    want = Hn.oracle_stack(x, layers, B, lens, causal=causal, store=torch.float16,
+                           resid=torch.float32 if mode else "same")
+    a, b = got[0].astype(np.float32), want.astype(np.float32)
+    if lens is not None:  # rows past a sequence's length are padding: not compared
+        for i in range(B):
+            a[i * S + lens[i]:(i + 1) * S] = 0
+            b[i * S + lens[i]:(i + 1) * S] = 0
+    assert Hn.max_abs(a, b) <= (4e-3 if mode else TOL_F16)
+    assert np.array_equal(got[0], got[1])
+
+
 @pytest.mark.parametrize("mixed", [False, True])
 def test_layer_at_4096_rows_uses_the_streaming_linear(et, mixed):
     """32 sequences of 128 tokens: the FFN down-projection (3072 inputs, 4096 token rows) runs on the
