@@ -573,15 +573,38 @@ constexpr int kVoCols = 64;  // output columns of a workgroup
 // wave.  One head per wave and QT = 1 is the latency form (12 waves for BERT-base: every head's
 // chain of load, scores, softmax and product runs at once); fewer waves with QT = 2 reuse each
 // fragment for two query tiles and halve the operand traffic per query.
-template <int HD, int KBLK, bool MASKED, int NW, int QT, bool PF>
+// VC: output columns of a workgroup, 64 or 32
+template <int HD, int KBLK, bool MASKED, int NW, int QT, bool PF, int VC>
 __global__ __launch_bounds__(64 * NW) void mha_vo_otf_kernel(const MhaVoArgs a) {
     constexpr int KS = HD / 32;        // K=32 MFMA steps over the head dimension
-    constexpr int DB = kVoCols / 16;   // 16-wide blocks of the output columns
+    constexpr int DB = VC / 16;   // 16-wide blocks of the output columns
     constexpr int NKB = KBLK / 16;     // score tiles of a key block
     constexpr int kStripQ = 16 * QT;
     constexpr int kTiles = QT * DB;
     __shared__ float red[NW][kTiles][4][64];
     __shared__ int alive[kStripQ];
+    // Fragments through LDS (heads of 64 and 128).  A fragment load straight from memory touches 16
+    // rows with 64 bytes each: half a cache line per row, and the memory pipeline of a CU passes such
+    // an instruction at the cost of 16 whole lines (a wave per head, all heads at once, spent 6.5 us of
+    // a 15 us launch waiting for K that way).  Instead a load instruction takes whole rows — 8 rows of
+    // 128 bytes or 4 of 256 — and the wave turns 32 keys (K) or 16 columns (VO^T) at a time into
+    // fragments through a piece of LDS of its own: written as loaded, read back in fragment order, the
+    // 16-byte chunks of a row XOR-swizzled so that both directions spread over all banks.  One wave's
+    // LDS instructions execute in order, so the piece is reused without a barrier.
+    // (The large-grid forms, which prefetch the next block's fragments while they multiply, keep the
+    // direct fragment loads: there the chip is full, the loads hide behind arithmetic and the LDS
+    // round trip only costs — 40.3 against 37.9 us at eight sequences.)
+    constexpr bool kStaged = HD >= 64 && !PF;
+    constexpr int kCPR = HD / 8;                   // 16-byte chunks of a K row
+    constexpr int kRPI = 64 / kCPR;                // K rows per load instruction
+    constexpr int kNI = kStaged ? KBLK / kRPI : 1; // load instructions per key block
+    constexpr int kPI = 32 / kRPI;                 // ... per 32-key piece
+    constexpr int kCPV = KBLK / 8;                 // 16-byte chunks of a VO^T row inside a key block
+    constexpr int kRPV = 64 / kCPV;                // VO^T rows per load instruction
+    constexpr int kNIV = kStaged ? VC / kRPV : 1;
+    constexpr int kPIV = 16 / kRPV;                // ... per 16-column piece
+    constexpr int kPieceHalfs = kStaged ? (32 * HD > 16 * KBLK ? 32 * HD : 16 * KBLK) : 8;
+    __shared__ __align__(16) _Float16 piece_lds[NW][kPieceHalfs];
 
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
@@ -591,7 +614,7 @@ __global__ __launch_bounds__(64 * NW) void mha_vo_otf_kernel(const MhaVoArgs a) 
     // workgroup id -> (sequence, column slice, query strip): the strips of one (sequence, slice)
     // read the same VO^T rows and get ids that land on one XCD
     const int qstrips = (S + kStripQ - 1) / kStripQ;
-    const int nslices = (a.N + kVoCols - 1) / kVoCols;
+    const int nslices = (a.N + VC - 1) / VC;
     const int xcd = blockIdx.x % kXcds, k_in_xcd = blockIdx.x / kXcds;
     const int unit = xcd + kXcds * (k_in_xcd / qstrips);
     if (unit >= a.B * nslices) return;  // padding of the last round (whole workgroup)
@@ -609,8 +632,8 @@ __global__ __launch_bounds__(64 * NW) void mha_vo_otf_kernel(const MhaVoArgs a) 
     if (a.lens) klimit = min(S, max(a.lens[b], 0));
     if (a.causal) klimit = min(klimit, (qstrip + 1) * kStripQ);
     const int hd = a.hd;
-    const int n0 = slice * kVoCols;
-    const int nlive = min(kVoCols, a.N - n0);  // live columns of the slice (a multiple of 16)
+    const int n0 = slice * VC;
+    const int nlive = min(VC, a.N - n0);  // live columns of the slice (a multiple of 16)
     const int nblocks = (klimit + KBLK - 1) / KBLK;
 
     // No load below is followed by a select in its own basic block: the compiler would wait for
@@ -633,7 +656,7 @@ __global__ __launch_bounds__(64 * NW) void mha_vo_otf_kernel(const MhaVoArgs a) 
 #pragma unroll
     for (int d = 0; d < DB; d++) vrow[d] = (unsigned)(16 * d < nlive ? 16 * d + r16 : 0) * (unsigned)S;
 
-    h8 qf[QT][KS], qn[QT][KS];
+    h8 qf[QT][KS], qn[PF ? QT : 1][PF ? KS : 1];  // qn: the next head's Q, requested while this head is multiplied
     h8 kf[NKB][KS];
     // Q fragments: B operand, lane supplies Q[q][32ks + 8g .. +7]
     auto load_q = [&](int h) {
@@ -641,17 +664,53 @@ __global__ __launch_bounds__(64 * NW) void mha_vo_otf_kernel(const MhaVoArgs a) 
 #pragma unroll
         for (int t = 0; t < QT; t++)
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) qn[t][ks] = *reinterpret_cast<const h8 *>(qh + qoff[t][ks]);
+            for (int ks = 0; ks < KS; ks++) {
+                if constexpr (PF) qn[t][ks] = *reinterpret_cast<const h8 *>(qh + qoff[t][ks]);
+                else qf[t][ks] = *reinterpret_cast<const h8 *>(qh + qoff[t][ks]);  // taken into use at once
+            }
     };
     auto take_q = [&]() {
 #pragma unroll
         for (int t = 0; t < QT; t++)
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) qf[t][ks] = (q_ok[t] && col_ok[ks]) ? qn[t][ks] : zero8;
+            for (int ks = 0; ks < KS; ks++) qf[t][ks] = (q_ok[t] && col_ok[ks]) ? (PF ? qn[PF ? t : 0][PF ? ks : 0] : qf[t][ks]) : zero8;
     };
     // K fragments: A operand of tile kb, row r16 of the tile is key 32(kb/2) + 8(r16/4) + 4(kb%2) + r16%4
+    h8 kraw[kNI];
+    _Float16 *piece = piece_lds[wave];
+    const int k_row = lane / kCPR, k_chunk = lane % kCPR;       // staged form: this lane's place in a load instruction
+    const unsigned k_col = k_chunk * 8 < hd ? k_chunk * 8 : 0;  // (columns past the head meet zeros of Q)
+    // Places in the piece, in halfs.  A row's 16-byte chunks are XORed with three bits that differ
+    // over the 16 rows of a score tile: key & 3, and bit 3 of the key (inside the piece).  For the
+    // writer bit 3 depends on the instruction only, for the reader on nothing but the lane, so two
+    // bases each and compile-time offsets address everything (registers are what this form lacks).
+    int kw[2], kr[2];
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        kw[p] = (k_row * kCPR + (k_chunk ^ ((k_row & 3) | (p << 2)))) * 8;
+        const int key = 8 * (r16 >> 2) + (r16 & 3);  // first tile of the piece; the second is 4 keys on
+        kr[p] = (key * kCPR + ((4 * p + g) ^ ((r16 & 3) | (((r16 >> 2) & 1) << 2)))) * 8;
+    }
+    static_assert(!kStaged || kRPI == 4 || kRPI == 8, "rows per instruction");
+    // VO^T: a row's chunks are XORed with row & 7 (the 16 rows of a piece are the 16 lanes of a fragment read)
+    const int v_row = lane / kCPV, v_chunk = lane % kCPV;
+    int vw[2], vr[2];
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        vw[p] = (v_row * kCPV + (v_chunk ^ ((v_row + 4 * p) & 7))) * 8;
+        vr[p] = (r16 * kCPV + ((4 * p + g) ^ (r16 & 7))) * 8;
+    }
+    static_assert(!kStaged || kRPV == 4 || kRPV == 8, "rows per instruction");
     auto load_k = [&](int h, int k0) {
         const _Float16 *kh = k_seq + h * hd;
+        if constexpr (kStaged) {
+#pragma unroll
+            for (int i = 0; i < kNI; i++) {
+                const int key = min(k0 + i * kRPI + k_row, klimit - 1);
+                kraw[i] = *reinterpret_cast<const h8 *>(kh + ((unsigned)key * (unsigned)a.ldk + k_col));
+            }
+            return;
+        }
 #pragma unroll
         for (int kb = 0; kb < NKB; kb++) {
             const int key = min(k0 + 32 * (kb >> 1) + 8 * (r16 >> 2) + 4 * (kb & 1) + (r16 & 3), klimit - 1);
@@ -668,7 +727,17 @@ __global__ __launch_bounds__(64 * NW) void mha_vo_otf_kernel(const MhaVoArgs a) 
         load_k(h, 0);
         take_q();
     }
-    f4 acc[QT][DB];  // sum over this wave's heads of the normalised products
+    // The sum over this wave's heads of the normalised products: in registers, or (the forms with a wave
+    // per head, which have none to spare) in the wave's rows of `red`, which the reduction at the end
+    // reads anyway.
+    constexpr bool kAccLds = !PF;
+    f4 acc[kAccLds ? 1 : QT][kAccLds ? 1 : DB];
+    if constexpr (!kAccLds) {
+#pragma unroll
+        for (int t = 0; t < QT; t++)
+#pragma unroll
+            for (int d = 0; d < DB; d++) acc[t][d] = f4{0.f, 0.f, 0.f, 0.f};
+    }
     f4 o[QT][DB];
     float m_run[QT], l_part[QT];
 #pragma unroll
@@ -678,7 +747,6 @@ __global__ __launch_bounds__(64 * NW) void mha_vo_otf_kernel(const MhaVoArgs a) 
 #pragma unroll
         for (int d = 0; d < DB; d++) {
             o[t][d] = f4{0.f, 0.f, 0.f, 0.f};
-            acc[t][d] = f4{0.f, 0.f, 0.f, 0.f};
         }
     }
     bool first_head = true;
@@ -694,8 +762,19 @@ __global__ __launch_bounds__(64 * NW) void mha_vo_otf_kernel(const MhaVoArgs a) 
         }
         // ---- VO^T fragments of this block: lane supplies VOt[n0 + 16d + r16][k0 + 32 s2 + 8g .. +7]
         h8 vf[NKB / 2][DB];
+        h8 vraw[kNIV];
         auto load_v = [&]() {
             const _Float16 *vo_h = a.VOt + ((size_t)(b * a.nh + h) * a.N + n0) * S;
+            if constexpr (kStaged) {
+                const int key = k0 + (lane % kCPV) * 8;
+                const unsigned kc = key < klimit ? key : 0;
+#pragma unroll
+                for (int i = 0; i < kNIV; i++) {
+                    const int n = i * kRPV + lane / kCPV;  // column of the slice = row of VO^T
+                    vraw[i] = *reinterpret_cast<const h8 *>(vo_h + ((unsigned)(n < nlive ? n : 0) * (unsigned)S + kc));
+                }
+                return;
+            }
 #pragma unroll
             for (int s2 = 0; s2 < NKB / 2; s2++) {
                 const int key = k0 + 32 * s2 + 8 * g;
@@ -720,15 +799,42 @@ __global__ __launch_bounds__(64 * NW) void mha_vo_otf_kernel(const MhaVoArgs a) 
         }
         // ---- scores S^T = K Q^T
         f4 sc[QT][NKB];
+        if constexpr (kStaged) {
+            // the rows loaded by load_k become fragments 32 keys (two score tiles) at a time and are
+            // multiplied at once, so that only two tiles' fragments are held in registers
 #pragma unroll
-        for (int kb = 0; kb < NKB; kb++)
+            for (int s2 = 0; s2 < KBLK / 32; s2++) {
 #pragma unroll
-            for (int t = 0; t < QT; t++) {
-                sc[t][kb] = f4{0.f, 0.f, 0.f, 0.f};
+                for (int j = 0; j < kPI; j++)  // rows j * kRPI + k_row of the piece
+                    *reinterpret_cast<h8 *>(piece + kw[((j * kRPI) >> 3) & 1] + j * kRPI * kCPR * 8) = kraw[s2 * kPI + j];
 #pragma unroll
-                for (int ks = 0; ks < KS; ks++)
-                    sc[t][kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kb][ks], qf[t][ks], sc[t][kb], 0, 0, 0);
+                for (int t2 = 0; t2 < 2; t2++) {
+                    const int kb = 2 * s2 + t2;
+                    h8 kfr[KS];
+#pragma unroll
+                    for (int ks = 0; ks < KS; ks++)  // row 8 (r16 / 4) + 4 t2 + r16 % 4, chunk 4 ks + g
+                        kfr[ks] = *reinterpret_cast<const h8 *>(piece + kr[ks & 1] + (4 * t2 * kCPR + 8 * (ks >> 1)) * 8);
+#pragma unroll
+                    for (int t = 0; t < QT; t++) {
+                        sc[t][kb] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int ks = 0; ks < KS; ks++)
+                            sc[t][kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kfr[ks], qf[t][ks], sc[t][kb], 0, 0, 0);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);  // pieces one after the other: fragments of one piece in registers at a time
             }
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < NKB; kb++)
+#pragma unroll
+                for (int t = 0; t < QT; t++) {
+                    sc[t][kb] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int ks = 0; ks < KS; ks++)
+                        sc[t][kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kb][ks], qf[t][ks], sc[t][kb], 0, 0, 0);
+                }
+        }
         // ---- request the next (head, block) of this wave
         int h_next = h, blk_next = blk + 1;
         if (blk_next == nblocks) {
@@ -788,14 +894,36 @@ __global__ __launch_bounds__(64 * NW) void mha_vo_otf_kernel(const MhaVoArgs a) 
                 }
         }
         // ---- O^T += VO^T P^T
+        if constexpr (kStaged) {
+            // the rows loaded by load_v become fragments 16 columns at a time and are multiplied at once
 #pragma unroll
-        for (int s2 = 0; s2 < NKB / 2; s2++) {
-            if (k0 + 32 * s2 >= klimit) continue;  // wave-uniform
+            for (int d = 0; d < DB; d++) {
 #pragma unroll
-            for (int d = 0; d < DB; d++)
+                for (int j = 0; j < kPIV; j++)  // rows j * kRPV + v_row of the piece
+                    *reinterpret_cast<h8 *>(piece + vw[(j * kRPV >> 2) & 1] + j * kRPV * kCPV * 8) = vraw[d * kPIV + j];
+                h8 vfr[NKB / 2];
 #pragma unroll
-                for (int t = 0; t < QT; t++)
-                    o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[s2][d], pf[t][s2], o[t][d], 0, 0, 0);
+                for (int s2 = 0; s2 < NKB / 2; s2++)  // row r16, chunk 4 s2 + g
+                    vfr[s2] = *reinterpret_cast<const h8 *>(piece + vr[s2 & 1] + 8 * (s2 >> 1) * 8);
+#pragma unroll
+                for (int s2 = 0; s2 < NKB / 2; s2++) {
+                    if (k0 + 32 * s2 >= klimit) continue;  // wave-uniform
+#pragma unroll
+                    for (int t = 0; t < QT; t++)
+                        o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vfr[s2], pf[t][s2], o[t][d], 0, 0, 0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+#pragma unroll
+            for (int s2 = 0; s2 < NKB / 2; s2++) {
+                if (k0 + 32 * s2 >= klimit) continue;  // wave-uniform
+#pragma unroll
+                for (int d = 0; d < DB; d++)
+#pragma unroll
+                    for (int t = 0; t < QT; t++)
+                        o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[s2][d], pf[t][s2], o[t][d], 0, 0, 0);
+            }
         }
         // ---- the head is done: add its normalised product, start the next head
         if (blk_next == 0) {
@@ -803,10 +931,23 @@ __global__ __launch_bounds__(64 * NW) void mha_vo_otf_kernel(const MhaVoArgs a) 
             for (int t = 0; t < QT; t++) {
                 const float l = rows_sum(l_part[t]);
                 const float inv = l > 0.0f ? 1.0f / l : 0.0f;
-                if (first_head && wave == 0 && g == 0) alive[t * 16 + r16] = l > 0.0f;
+                if (first_head && wave == 0 && g == 0) {
+                    int at = t * 16 + r16;
+                    asm volatile("" : "+v"(at));  // formed here: hoisted out of the loop, the address is a register spilled
+                    alive[at] = l > 0.0f;
+                }
 #pragma unroll
                 for (int d = 0; d < DB; d++) {
-                    acc[t][d] += o[t][d] * inv;
+                    if constexpr (kAccLds) {
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            float v = o[t][d][j] * inv;
+                            if (!first_head) v += red[wave][t * DB + d][j][lane];
+                            red[wave][t * DB + d][j][lane] = v;
+                        }
+                    } else {
+                        acc[kAccLds ? 0 : t][kAccLds ? 0 : d] += o[t][d] * inv;
+                    }
                     o[t][d] = f4{0.f, 0.f, 0.f, 0.f};
                 }
                 m_run[t] = -INFINITY;
@@ -822,12 +963,21 @@ __global__ __launch_bounds__(64 * NW) void mha_vo_otf_kernel(const MhaVoArgs a) 
     if (nblocks == 0 && threadIdx.x < kStripQ) alive[threadIdx.x] = 0;
 
     // ---- add the waves' sums; wave w finishes the tiles w, w + NW, ...
+    if constexpr (kAccLds) {
+        if (first_head) {  // a wave without a head of its own (wave-uniform)
 #pragma unroll
-    for (int t = 0; t < QT; t++)
+            for (int tile = 0; tile < kTiles; tile++)
 #pragma unroll
-        for (int d = 0; d < DB; d++)
+                for (int j = 0; j < 4; j++) red[wave][tile][j][lane] = 0.0f;
+        }
+    } else {
 #pragma unroll
-            for (int j = 0; j < 4; j++) red[wave][t * DB + d][j][lane] = acc[t][d][j];
+        for (int t = 0; t < QT; t++)
+#pragma unroll
+            for (int d = 0; d < DB; d++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) red[wave][t * DB + d][j][lane] = acc[kAccLds ? 0 : t][kAccLds ? 0 : d][j];
+    }
     __syncthreads();
     for (int tile = wave; tile < kTiles; tile += NW) {
         const int t = tile / DB, d = tile - t * DB;
@@ -866,27 +1016,30 @@ __global__ __launch_bounds__(64 * NW) void mha_vo_otf_kernel(const MhaVoArgs a) 
     }
 }
 
-template <int HD, int KBLK, int NW, int QT, bool PF>
+template <int HD, int KBLK, int NW, int QT, bool PF, int VC = kVoCols>
 static int launch_mha_vo_otf_form(const MhaVoArgs &args, hipStream_t stream) {
     constexpr int kStripQ = 16 * QT;
-    const int qstrips = (args.S + kStripQ - 1) / kStripQ, nslices = (args.N + kVoCols - 1) / kVoCols;
+    const int qstrips = (args.S + kStripQ - 1) / kStripQ, nslices = (args.N + VC - 1) / VC;
     const long long rounds = ((long long)args.B * nslices + kXcds - 1) / kXcds;
     const dim3 grid((unsigned)(rounds * kXcds * qstrips));
-    if (args.mask) mha_vo_otf_kernel<HD, KBLK, true, NW, QT, PF><<<grid, 64 * NW, 0, stream>>>(args);
-    else mha_vo_otf_kernel<HD, KBLK, false, NW, QT, PF><<<grid, 64 * NW, 0, stream>>>(args);
+    if (args.mask) mha_vo_otf_kernel<HD, KBLK, true, NW, QT, PF, VC><<<grid, 64 * NW, 0, stream>>>(args);
+    else mha_vo_otf_kernel<HD, KBLK, false, NW, QT, PF, VC><<<grid, 64 * NW, 0, stream>>>(args);
     return check_launch("mha_vo_otf_kernel");
 }
 
 // A workgroup reads the K of all heads and its VO^T slice of all heads (392 KB at 128 keys, 12 heads
-// of 64), and a CU takes in about 32 KB per memory round trip: that, not arithmetic, sets the
-// time of a small grid, and a wave per head (no wave walks several heads) is the fastest form
-// while the grid is a few hundred workgroups.  Beyond that the chip is full either way and the
-// form that reuses each fragment for two query tiles moves half the bytes per query.
+// of 64, 64 columns), and a CU takes in 60 to 80 GB/s: that, not arithmetic, sets the time of a small
+// grid, and a wave per head (no wave walks several heads) is the fastest form while the grid is a few
+// hundred workgroups; a grid that leaves more than half of the CUs idle gives each workgroup 32
+// columns instead of 64 (three quarters of the bytes per CU on twice the CUs).  Beyond that the chip
+// is full either way and the form that reuses each fragment for two query tiles moves half the
+// bytes per query.
 template <int HD, int KBLK> static int launch_mha_vo_otf(const MhaVoArgs &args, hipStream_t stream) {
     const long long small_grid = (long long)args.B * ((args.N + kVoCols - 1) / kVoCols) * ((args.S + 15) / 16);
     if (small_grid > 512) return launch_mha_vo_otf_form<HD, KBLK, 4, 2, true>(args, stream);
     if (args.nh <= 4) return launch_mha_vo_otf_form<HD, KBLK, 4, 1, true>(args, stream);
     if (args.nh <= 8) return launch_mha_vo_otf_form<HD, KBLK, 8, 1, false>(args, stream);
+    if (small_grid <= 128) return launch_mha_vo_otf_form<HD, KBLK, 12, 1, false, 32>(args, stream);
     return launch_mha_vo_otf_form<HD, KBLK, 12, 1, false>(args, stream);
 }
 
