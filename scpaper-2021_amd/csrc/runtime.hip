@@ -5,6 +5,11 @@
 #include <new>
 #include <string.h>
 
+#include <algorithm>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
 #include "common.hip.h"
 
 namespace et {
@@ -97,15 +102,60 @@ int et_device_info(char *name, int cap, int *num_cu, int *lds_bytes) {
     return ET_OK;
 }
 
+// Device memory comes from slabs of 64 MiB.  Where the driver puts separate allocations of a few
+// MiB each (a model makes a hundred of them) decides how they are mapped — translation fragments,
+// memory channels — and the same encoder stack measured anything between 41.4 and 43.6 us per
+// layer from one process start to the next, with the same kernels on the same inputs.  Inside a
+// slab every buffer sits at a fixed distance from its neighbours and shares the slab's large
+// pages.  A slab goes back to the driver when the last buffer cut from it has been freed and a
+// newer slab has taken its place; requests of more than a quarter of a slab get an allocation of
+// their own.
+namespace {
+constexpr size_t kSlabBytes = 64u << 20;
+constexpr size_t kSlabAlign = 4096;
+struct Slab {
+    char *base = nullptr;
+    size_t used = 0;
+    size_t live = 0;  // buffers cut from this slab and not yet freed
+};
+std::mutex g_pool_mu;
+std::vector<Slab *> g_slabs;                       // the last one is the one being cut
+std::unordered_map<void *, Slab *> g_owner;       // buffer -> its slab (nullptr: an allocation of its own)
+}  // namespace
+
 int et_malloc(void **ptr, size_t bytes) {
     ET_REQUIRE(ptr != nullptr, ET_ERR_INVALID_ARG, "et_malloc: ptr is NULL");
     *ptr = nullptr;
     if (bytes == 0) bytes = 16;  // a valid, distinct pointer even for empty buffers
     void *p = nullptr;
-    ET_HIP(hipMalloc(&p, bytes));
+    Slab *slab = nullptr;
+    if (bytes <= kSlabBytes / 4) {
+        std::lock_guard<std::mutex> lk(g_pool_mu);
+        const size_t need = (bytes + kSlabAlign - 1) / kSlabAlign * kSlabAlign;
+        if (g_slabs.empty() || g_slabs.back()->used + need > kSlabBytes) {
+            if (!g_slabs.empty() && g_slabs.back()->live == 0) {  // nothing left in it: cut it again
+                g_slabs.back()->used = 0;
+            } else {
+                void *base = nullptr;
+                ET_HIP(hipMalloc(&base, kSlabBytes));
+                Slab *fresh = new Slab;
+                fresh->base = static_cast<char *>(base);
+                g_slabs.push_back(fresh);
+            }
+        }
+        slab = g_slabs.back();
+        p = slab->base + slab->used;
+        slab->used += need;
+        slab->live++;
+        g_owner[p] = slab;
+    } else {
+        ET_HIP(hipMalloc(&p, bytes));
+        std::lock_guard<std::mutex> lk(g_pool_mu);
+        g_owner[p] = nullptr;
+    }
     int s = check_hip(hipMemset(p, 0, bytes), "hipMemset");
     if (s != ET_OK) {
-        (void)hipFree(p);
+        (void)et_free(p);
         return s;
     }
     *ptr = p;
@@ -114,7 +164,25 @@ int et_malloc(void **ptr, size_t bytes) {
 
 int et_free(void *ptr) {
     if (!ptr) return ET_OK;
-    ET_HIP(hipFree(ptr));
+    void *release = nullptr;
+    {
+        std::lock_guard<std::mutex> lk(g_pool_mu);
+        auto it = g_owner.find(ptr);
+        Slab *slab = it != g_owner.end() ? it->second : nullptr;  // memory from elsewhere goes to the driver as before
+        if (it != g_owner.end()) g_owner.erase(it);
+        if (!slab) {
+            release = ptr;
+        } else if (--slab->live == 0) {
+            if (slab == g_slabs.back()) {
+                slab->used = 0;  // empty again: cut from its start
+            } else {
+                release = slab->base;
+                g_slabs.erase(std::find(g_slabs.begin(), g_slabs.end(), slab));
+                delete slab;
+            }
+        }
+    }
+    if (release) ET_HIP(hipFree(release));
     return ET_OK;
 }
 
