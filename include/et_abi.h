@@ -62,6 +62,18 @@ int et_device_info(char *name, int cap, int *num_cu, int *lds_bytes);
  * ------------------------------------------------------------------------ */
 int et_malloc(void **ptr, size_t bytes);              /* zero-filled, like CUDA_ptr(size) */
 int et_free(void *ptr);                               /* NULL is accepted */
+/* Placement.  et_malloc cuts buffers from 64 MiB slabs (4 KiB granules), so that
+ * buffers allocated one after the other lie next to one another whatever the
+ * driver's allocator holds at the time; a request above 16 MiB gets an
+ * allocation of its own.  Between et_pool_private_begin and
+ * et_pool_private_end the calling thread's et_malloc calls are served from
+ * slabs of their own, the first buffer lead_bytes (a multiple of 4096, at most
+ * 32 MiB) into the first slab: a model built inside such a scope has the same
+ * layout in every process, and its speed does not depend on what was allocated
+ * before it (et_model_finalize opens one).  Scopes do not nest.  No reference
+ * counterpart (lib/CUDA_ptr.hpp:18-31 calls cudaMalloc per buffer). */
+int et_pool_private_begin(size_t lead_bytes);
+int et_pool_private_end(void);
 int et_memset(void *ptr, int byte, size_t bytes, et_stream stream);
 int et_memcpy_h2d(void *dst, const void *src_host, size_t bytes);
 int et_memcpy_d2h(void *dst_host, const void *src, size_t bytes);

@@ -44,6 +44,8 @@ _SIGNATURES = {
     "et_device_info": (C.c_char_p, _i, C.POINTER(_i), C.POINTER(_i)),
     "et_malloc": (C.POINTER(_vp), _sz),
     "et_free": (_vp,),
+    "et_pool_private_begin": (_sz,),
+    "et_pool_private_end": (),
     "et_memset": (_vp, _i, _sz, _vp),
     "et_memcpy_h2d": (_vp, _vp, _sz),
     "et_memcpy_d2h": (_vp, _vp, _sz),

@@ -116,12 +116,49 @@ constexpr size_t kSlabAlign = 4096;
 struct Slab {
     char *base = nullptr;
     size_t used = 0;
-    size_t live = 0;  // buffers cut from this slab and not yet freed
+    size_t live = 0;      // buffers cut from this slab and not yet freed
+    size_t lead = 0;      // where cutting starts (a private scope may ask for a distance from the slab's start)
+    bool current = true;  // still the slab its list cuts from
 };
 std::mutex g_pool_mu;
 std::vector<Slab *> g_slabs;                       // the last one is the one being cut
 std::unordered_map<void *, Slab *> g_owner;       // buffer -> its slab (nullptr: an allocation of its own)
+// A private scope (et_pool_private_begin): the calling thread cuts from slabs of its own.
+struct PrivateScope {
+    std::vector<Slab *> slabs;
+    size_t lead = 0;
+};
+thread_local PrivateScope *t_scope = nullptr;
 }  // namespace
+
+int et_pool_private_begin(size_t lead_bytes) {
+    ET_REQUIRE(t_scope == nullptr, ET_ERR_INVALID_ARG, "et_pool_private_begin: a private scope is already open on this thread");
+    ET_REQUIRE(lead_bytes % kSlabAlign == 0 && lead_bytes <= kSlabBytes / 2, ET_ERR_INVALID_ARG,
+               "et_pool_private_begin: lead_bytes=%zu must be a multiple of %zu, at most %zu", lead_bytes, kSlabAlign,
+               kSlabBytes / 2);
+    t_scope = new PrivateScope;
+    t_scope->lead = lead_bytes;
+    return ET_OK;
+}
+
+int et_pool_private_end(void) {
+    ET_REQUIRE(t_scope != nullptr, ET_ERR_INVALID_ARG, "et_pool_private_end: no private scope is open on this thread");
+    std::vector<void *> release;
+    {
+        std::lock_guard<std::mutex> lk(g_pool_mu);
+        for (Slab *slab : t_scope->slabs) {  // nothing cuts from them any more: each goes when its last buffer does
+            slab->current = false;
+            if (slab->live == 0) {
+                release.push_back(slab->base);
+                delete slab;
+            }
+        }
+    }
+    delete t_scope;
+    t_scope = nullptr;
+    for (void *p : release) ET_HIP(hipFree(p));
+    return ET_OK;
+}
 
 int et_malloc(void **ptr, size_t bytes) {
     ET_REQUIRE(ptr != nullptr, ET_ERR_INVALID_ARG, "et_malloc: ptr is NULL");
@@ -132,18 +169,21 @@ int et_malloc(void **ptr, size_t bytes) {
     if (bytes <= kSlabBytes / 4) {
         std::lock_guard<std::mutex> lk(g_pool_mu);
         const size_t need = (bytes + kSlabAlign - 1) / kSlabAlign * kSlabAlign;
-        if (g_slabs.empty() || g_slabs.back()->used + need > kSlabBytes) {
-            if (!g_slabs.empty() && g_slabs.back()->live == 0) {  // nothing left in it: cut it again
-                g_slabs.back()->used = 0;
+        std::vector<Slab *> &slabs = t_scope ? t_scope->slabs : g_slabs;
+        if (slabs.empty() || slabs.back()->used + need > kSlabBytes) {
+            if (!slabs.empty() && slabs.back()->live == 0) {  // nothing left in it: cut it again
+                slabs.back()->used = slabs.back()->lead;
             } else {
                 void *base = nullptr;
                 ET_HIP(hipMalloc(&base, kSlabBytes));
                 Slab *fresh = new Slab;
                 fresh->base = static_cast<char *>(base);
-                g_slabs.push_back(fresh);
+                fresh->lead = fresh->used = (t_scope && slabs.empty()) ? t_scope->lead : 0;
+                if (!slabs.empty()) slabs.back()->current = false;
+                slabs.push_back(fresh);
             }
         }
-        slab = g_slabs.back();
+        slab = slabs.back();
         p = slab->base + slab->used;
         slab->used += need;
         slab->live++;
@@ -173,11 +213,16 @@ int et_free(void *ptr) {
         if (!slab) {
             release = ptr;
         } else if (--slab->live == 0) {
-            if (slab == g_slabs.back()) {
-                slab->used = 0;  // empty again: cut from its start
+            if (slab->current) {
+                slab->used = slab->lead;  // empty again: cut from its start
             } else {
                 release = slab->base;
-                g_slabs.erase(std::find(g_slabs.begin(), g_slabs.end(), slab));
+                auto at = std::find(g_slabs.begin(), g_slabs.end(), slab);
+                if (at != g_slabs.end()) g_slabs.erase(at);
+                if (t_scope) {
+                    auto mine = std::find(t_scope->slabs.begin(), t_scope->slabs.end(), slab);
+                    if (mine != t_scope->slabs.end()) t_scope->slabs.erase(mine);
+                }
                 delete slab;
             }
         }

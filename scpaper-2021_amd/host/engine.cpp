@@ -351,6 +351,11 @@ int et_model_finalize(et_model m) {
     return guarded([&]() -> int {
         et::require(m != nullptr, "et_model_finalize: NULL handle");
         et::require(!m->finalized, "et_model_finalize: already finalized");
+        // every device buffer of the model comes from slabs of the model's own, at fixed places in them
+        struct PoolScope {
+            PoolScope() { etChk(et_pool_private_begin(0)); }
+            ~PoolScope() { (void)et_pool_private_end(); }
+        } pool_scope;
         for (int i = 0; i < m->desc.nlayer; i++) {
             const HostLayer &h = m->host[(size_t)i];
             const HostMatrix::Kind kind = h.w[0].kind;

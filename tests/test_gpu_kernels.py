@@ -49,6 +49,36 @@ def test_fill_convert_roundtrip(et):
 
 # ---------------------------------------------------------------- norms ------
 
+def test_device_memory_comes_from_slabs_and_private_scopes(et):
+    """Buffers allocated one after the other lie next to one another (4 KiB granules of a 64 MiB slab), a
+    request above a quarter of a slab gets an allocation of its own, a private scope cuts from slabs of its
+    own starting at the distance asked for, memory is zero-filled, and everything can be freed in any order."""
+    import ctypes as C
+    lib = et.lib()
+    def alloc(n):
+        p = C.c_void_p()
+        et.check(lib.et_malloc(C.byref(p), n))
+        return p.value
+    a, b, c = alloc(100), alloc(5000), alloc(1 << 20)
+    assert b - a == 4096 and c - b == 8192
+    big = alloc(17 << 20)
+    d = alloc(64)
+    assert d - c == 1 << 20 and not (a <= big < a + (64 << 20))
+    et.check(lib.et_pool_private_begin(3 * 4096))
+    p1, p2 = alloc(64), alloc(64)
+    assert lib.et_pool_private_begin(0) == et.ET_ERR_INVALID_ARG  # scopes do not nest
+    et.check(lib.et_pool_private_end())
+    assert lib.et_pool_private_end() == et.ET_ERR_INVALID_ARG
+    assert lib.et_pool_private_begin(100) == et.ET_ERR_INVALID_ARG   # not a multiple of 4096
+    e = alloc(64)
+    assert p2 - p1 == 4096 and p1 % (2 << 20) == 3 * 4096 and abs(p1 - a) >= (32 << 20) and e - d == 4096
+    host = np.empty(5000, np.uint8)
+    et.check(lib.et_memcpy_d2h(host.ctypes.data, b, 5000))
+    assert not host.any()
+    for p in (c, p1, a, big, e, b, p2, d):
+        et.check(lib.et_free(p))
+
+
 @pytest.mark.parametrize("rows,H", [(1024, 768), (2048, 1024), (128, 800), (7, 64), (33, 2048), (5, 4100)])
 def test_skip_layernorm(et, rows, H):
     src, skip = Hn.randn((rows, H), 1), Hn.randn((rows, H), 2)
