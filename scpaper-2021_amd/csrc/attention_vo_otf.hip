@@ -12,9 +12,11 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 // On-the-fly attention over a pre-computed VO projection (Fused_attention/Fused_attention.cu:10-116):
 //     out[q][n] = sum_h softmax_h(q, :) . (VO_h[:, n] + b_VO,h[n]) + b_O[n]
-// The probabilities never leave the chip, and neither operand of the two products passes through
-// LDS: the projection is handed over key-contiguous, VOt[b][h][n][key], so that a lane's 8 values
-// of a VO^T fragment are one 16-byte load, and a K fragment is a 16-byte load of one K row.  The
+// The probabilities never leave the chip, and no operand of the two products is staged for more
+// than one wave: the projection is handed over key-contiguous, VOt[b][h][n][key], so that a lane's
+// 8 values of a VO^T fragment are one 16-byte load, and a K fragment is a 16-byte load of one K row
+// (the forms with a wave per head load whole rows instead and turn them into fragments through a
+// wave-private piece of LDS, see kStaged).  The
 // rows of a score tile are dealt to the keys so that the 8 probabilities a lane holds after the
 // softmax (rows 4g..4g+3 of two tiles) are the keys 8g..8g+7 of a 32-key group, the order the
 // VO^T fragment has in memory.
