@@ -171,52 +171,80 @@ __global__ __launch_bounds__(256) void gemm_f16_kernel(const GemmArgs g) {
 // Small results with a long K (one sequence through a pruned or dense Linear: 128 x 80 x 768):
 // the tiled kernels would run a handful of workgroups, each stepping through K stage by stage —
 // 12 dependent round trips for K = 768.  Here a workgroup owns one 16x16 tile of the result and
-// its four waves split K between them; a wave requests all its fragments of up to STEPS K-steps
-// of 32 straight from global memory (L2) before the first product, so the whole kernel is one
-// or two memory round trips plus an LDS reduction of three partial tiles.  B is [N x K]
-// (transposed form), no A-column gather; rows 16-byte aligned.  Every tile reads its 16 rows of
-// A and of B in full, so this only pays while the tiles are few (used up to 1024 of them where
-// the 64x64 tiling has fewer than 64 workgroups; 128 x 768 -> 80 / 384 / 768: 7.1 -> 3.9 / 4.0 /
-// 5.3 us, 256 x 768 -> 768: 7.5 -> 6.8, 128 x 3072 -> 768: 18.6 -> 14.6).  STEPS = 6 when that
-// covers a wave's share of K: fragments requested for steps a wave does not have cost as much
-// as real ones (with 12 where 6 were live the first three shapes took 5.6 / 5.8 / 8.4 us).
+// its four waves split K between them; a wave requests all the rows of up to STEPS pieces of 64
+// k-values before the first product, so the whole kernel is one or two memory round trips plus an
+// LDS reduction of three partial tiles.  B is [N x K] (transposed form), no A-column gather; rows
+// 16-byte aligned.  Every tile reads its 16 rows of A and of B in full, so this only pays while
+// the tiles are few (used up to 1024 of them where the 64x64 tiling has fewer than 64 workgroups;
+// 128 x 768 -> 80 / 384 / 768: 7.1 us tiled, 3.9 / 4.0 / 5.3 with fragments loaded straight from
+// memory, 3.0 / 3.0 / 3.6 with whole rows; 256 x 768 -> 768: 7.5 -> 6.8 -> 4.4; 128 x 3072 -> 768:
+// 18.6 -> 14.6 -> 7.7).  STEPS = 3 when that covers a wave's share of K: rows requested for
+// pieces a wave does not have cost as much as real ones.
 template <int STEPS>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs g) {
-    constexpr int kSkinnySteps = STEPS;
+    // STEPS = pieces of 64 k-values (two MFMAs) a wave requests per round.  A wave loads whole rows
+    // of its share — 8 rows x 128 bytes per instruction, the four lanes of a quad inside one cache
+    // line — and turns each piece into fragments through 4 KB of LDS of its own (written as
+    // loaded, read back in fragment order, 16-byte chunks XOR-swizzled by the row): a fragment
+    // load straight from memory puts a quad of lanes on four rows and costs the memory pipeline
+    // four times as much.  One wave's LDS instructions execute in order, so the piece is reused
+    // without a barrier.
+    constexpr int kPieces = STEPS;
     __shared__ f4 part[3][64];
+    __shared__ __align__(16) _Float16 piece_lds[4][2][16 * 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, grp = lane >> 4;
+    const int row8 = lane >> 3, ch = lane & 7;  // place of this lane in a whole-row load
     const int ntn = g.N >> 4;
     const int tm = blockIdx.x / ntn, tn = blockIdx.x - tm * ntn;
     const long long zo = blockIdx.z / g.batch_inner, zi = blockIdx.z % g.batch_inner;
-    const _Float16 *A = g.A + zo * g.sAo + zi * g.sAi + (size_t)(tm * 16 + r16) * g.lda;  // this lane's token row
-    const _Float16 *B = g.B + zo * g.sBo + zi * g.sBi + (size_t)(tn * 16 + r16) * g.ldb;  // ... and feature row
+    const _Float16 *A = g.A + zo * g.sAo + zi * g.sAi + (size_t)(tm * 16 + row8) * g.lda;  // token rows row8 and row8 + 8
+    const _Float16 *B = g.B + zo * g.sBo + zi * g.sBi + (size_t)(tn * 16 + row8) * g.ldb;  // feature rows likewise
     _Float16 *Cm = g.C + zo * g.sCo + zi * g.sCi;
     const _Float16 *bias = g.bias ? g.bias + zo * g.sBias_o + zi * g.sBias_i : nullptr;
     const h8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-
-    // K-steps of this wave: [s_begin, s_end) of ceil(K / 32), a quarter each
-    const int nsteps = (g.K + 31) >> 5;
-    const int per = (nsteps + 3) >> 2;
-    const int s_begin = wave * per, s_end = min(nsteps, s_begin + per);
-    f4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int s0 = s_begin; s0 < s_end; s0 += kSkinnySteps) {
-        // unconditional loads from clamped addresses; values past K or past this wave's share
-        // are selected away (a load under a branch would be waited for on the spot)
-        h8 fa[kSkinnySteps], fb[kSkinnySteps];
+    _Float16 *pa = piece_lds[wave][0], *pb = piece_lds[wave][1];
+    // places in a piece, in halfs: row * 64 + (chunk ^ (row & 7)) * 8
+    const int w_at = row8 * 64 + ((ch ^ row8) * 8);  // rows row8 (+ 8 rows = + 512 halfs, same swizzle)
+    int r_at[2];
 #pragma unroll
-        for (int i = 0; i < kSkinnySteps; i++) {
-            const int k = (s0 + i) * 32 + 8 * grp;
-            const int kc = min(k, g.K - 8);
-            fa[i] = *reinterpret_cast<const h8 *>(A + kc);
-            fb[i] = *reinterpret_cast<const h8 *>(B + kc);
+    for (int s2 = 0; s2 < 2; s2++) r_at[s2] = r16 * 64 + (((4 * s2 + grp) ^ (r16 & 7)) * 8);
+
+    // pieces of this wave: [p_begin, p_end) of ceil(K / 64), a quarter each
+    const int npieces = (g.K + 63) >> 6;
+    const int per = (npieces + 3) >> 2;
+    const int p_begin = wave * per, p_end = min(npieces, p_begin + per);
+    f4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int p0 = p_begin; p0 < p_end; p0 += kPieces) {
+        // unconditional loads from clamped addresses; values past K or past this wave's share
+        // become zeros on their way into LDS (a load under a branch would be waited for on the spot)
+        h8 ra[kPieces][2], rb[kPieces][2];
+#pragma unroll
+        for (int i = 0; i < kPieces; i++) {
+            const int kc = min((p0 + i) * 64 + 8 * ch, g.K - 8);
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                ra[i][h] = *reinterpret_cast<const h8 *>(A + (size_t)(8 * h) * g.lda + kc);
+                rb[i][h] = *reinterpret_cast<const h8 *>(B + (size_t)(8 * h) * g.ldb + kc);
+            }
         }
 #pragma unroll
-        for (int i = 0; i < kSkinnySteps; i++) {
-            const int k = (s0 + i) * 32 + 8 * grp;
-            const bool live = s0 + i < s_end && k < g.K;
-            // features are the A operand: the lane ends with four consecutive features of its token
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(live ? fb[i] : zero8, live ? fa[i] : zero8, acc, 0, 0, 0);
+        for (int i = 0; i < kPieces; i++) {
+            if (p0 + i < p_end) {  // wave-uniform
+                const bool live = (p0 + i) * 64 + 8 * ch < g.K;
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    *reinterpret_cast<h8 *>(pa + w_at + h * 512) = live ? ra[i][h] : zero8;
+                    *reinterpret_cast<h8 *>(pb + w_at + h * 512) = live ? rb[i][h] : zero8;
+                }
+#pragma unroll
+                for (int s2 = 0; s2 < 2; s2++) {
+                    const h8 fa = *reinterpret_cast<const h8 *>(pa + r_at[s2]);
+                    const h8 fb = *reinterpret_cast<const h8 *>(pb + r_at[s2]);
+                    // features are the A operand: the lane ends with four consecutive features of its token
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb, fa, acc, 0, 0, 0);
+                }
+            }
         }
     }
     if (wave > 0) part[wave - 1][lane] = acc;
@@ -321,8 +349,8 @@ static int launch_gemm_tile(const GemmArgs &g, int batch, bool trans_b, hipStrea
 int launch_gemm(const GemmArgs &g, int batch, bool trans_b, hipStream_t stream) {
     if (gemm_skinny_applies(g, batch, trans_b)) {
         const dim3 grid((unsigned)((g.M / 16) * (g.N / 16)), 1, (unsigned)batch);
-        if (g.K <= 6 * 4 * 32) gemm_skinny_kernel<6><<<grid, 256, 0, stream>>>(g);  // at most 6 K-steps per wave
-        else gemm_skinny_kernel<12><<<grid, 256, 0, stream>>>(g);
+        if (g.K <= 3 * 4 * 64) gemm_skinny_kernel<3><<<grid, 256, 0, stream>>>(g);  // at most 3 pieces of 64 per wave
+        else gemm_skinny_kernel<6><<<grid, 256, 0, stream>>>(g);
         return check_launch("gemm_skinny_kernel");
     }
     if (gemm_dma_applies(g, batch, trans_b)) return launch_gemm_dma(g, batch, trans_b, stream);
