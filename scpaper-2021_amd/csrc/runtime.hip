@@ -204,6 +204,9 @@ int et_malloc(void **ptr, size_t bytes) {
 
 int et_free(void *ptr) {
     if (!ptr) return ET_OK;
+    // hipFree waits for the device before it releases memory; a buffer cut from a slab is handed out
+    // again without the driver, so the wait is made here: work still running on the buffer ends first
+    ET_HIP(hipDeviceSynchronize());
     void *release = nullptr;
     {
         std::lock_guard<std::mutex> lk(g_pool_mu);
