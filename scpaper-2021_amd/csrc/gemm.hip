@@ -392,6 +392,36 @@ __global__ __launch_bounds__(256) void gather_cols_kernel(_Float16 *__restrict__
     }
 }
 
+// The same through LDS: a workgroup stages R whole rows of X with 16-byte loads (a quad of lanes
+// inside one cache line), then every lane picks its 8 columns out of LDS.  The 2-byte reads of the
+// kernel above go to memory one by one, each quad of lanes on up to four cache lines of a row
+// that the other waves are picking from at the same time.  R * in halfs of dynamic LDS.
+__global__ __launch_bounds__(256) void gather_cols_staged_kernel(_Float16 *__restrict__ dst,
+                                                                 const _Float16 *__restrict__ X,
+                                                                 const int32_t *__restrict__ col_id, int T,
+                                                                 int in, int nnz, int R) {
+    extern __shared__ __align__(16) unsigned char gather_smem[];
+    _Float16 *rows = reinterpret_cast<_Float16 *>(gather_smem);
+    const int per_row = nnz >> 3, chunks = in >> 3;
+    for (int r0 = blockIdx.x * R; r0 < T; r0 += gridDim.x * R) {
+        const int nrow = min(R, T - r0);
+        for (int i = threadIdx.x; i < nrow * chunks; i += 256)  // rows r0 .. r0 + nrow are contiguous in X
+            reinterpret_cast<h8 *>(rows)[i] = reinterpret_cast<const h8 *>(X + (size_t)r0 * in)[i];
+        __syncthreads();
+        for (int v = threadIdx.x; v < nrow * per_row; v += 256) {
+            const int r = v / per_row, c = (v - r * per_row) * 8;
+            const int4 i0 = *reinterpret_cast<const int4 *>(col_id + c);
+            const int4 i1 = *reinterpret_cast<const int4 *>(col_id + c + 4);
+            const _Float16 *row = rows + r * in;
+            h8 o;
+            o[0] = row[i0.x]; o[1] = row[i0.y]; o[2] = row[i0.z]; o[3] = row[i0.w];
+            o[4] = row[i1.x]; o[5] = row[i1.y]; o[6] = row[i1.z]; o[7] = row[i1.w];
+            *reinterpret_cast<h8 *>(dst + (size_t)(r0 + r) * nnz + c) = o;
+        }
+        __syncthreads();
+    }
+}
+
 }  // namespace et
 
 
@@ -561,6 +591,14 @@ int et_gather_cols_f16(et_f16 *dst, const et_f16 *X, const int32_t *col_id, int 
     if (total == 0) return ET_OK;
     size_t blocks = (total + 255) / 256;
     if (blocks > 4096) blocks = 4096;
+    if (in % 8 == 0 && in <= 16384 && (reinterpret_cast<uintptr_t>(X) & 15) == 0) {
+        // about 16 KB of rows a workgroup, so that several of them share a CU whatever the row length
+        const int rows = std::max(1, std::min(8, 8192 / in));
+        const unsigned groups = (unsigned)std::min<size_t>(((size_t)T + rows - 1) / rows, 2048);
+        gather_cols_staged_kernel<<<groups, 256, (size_t)rows * in * sizeof(_Float16), as_stream(stream)>>>(
+            H(dst), H(X), col_id, T, in, nnz_col, rows);
+        return check_launch("gather_cols_staged_kernel");
+    }
     gather_cols_kernel<<<(unsigned)blocks, 256, 0, as_stream(stream)>>>(H(dst), H(X), col_id, T, in, nnz_col);
     return check_launch("gather_cols_kernel");
 }

@@ -177,6 +177,21 @@ def test_linear_colpruned(et, T, inp, out, sp, act):
     assert Hn.max_abs(d_y2.numpy(), want) <= 4e-3
 
 
+@pytest.mark.parametrize("T,inp,sp", [(2048, 768, 0.0), (2051, 768, 0.5), (1, 16, 0.0), (7, 3072, 0.9), (300, 8192, 0.5),
+                                      (13, 1040, 0.3),
+                                      # rows too long for the staged form: the lane-per-chunk kernel
+                                      (5, 16400, 0.5), (64, 32768, 0.9)])
+def test_gather_cols_is_exact(et, T, inp, sp):
+    """Both column gathers (rows staged in LDS, and one chunk of eight a lane straight from memory)
+    copy X[:, col_id] bit for bit, whatever the number of rows a workgroup ends on."""
+    col_id = F.gen_col_ids(inp, sp, seed=T + inp)
+    col_id = col_id[:len(col_id) // 8 * 8]
+    x = Hn.randn((T, inp), 21)
+    d_ws = et.DeviceBuffer.empty((T, len(col_id)), np.float16)
+    et.check(et.lib().et_gather_cols_f16(d_ws.ptr, up(et, x).ptr, up(et, col_id).ptr, T, inp, len(col_id), None))
+    assert np.array_equal(d_ws.numpy(), x[:, col_id])
+
+
 @pytest.mark.parametrize("T,inp,out,sp,act", [(2048, 768, 768, 0.8, 0), (128, 768, 3072, 0.5, 2), (16, 32, 16, 0.0, 0),
                                               (80, 3072, 64, 0.9, 1)])
 def test_linear_vec1x16(et, T, inp, out, sp, act):
