@@ -273,7 +273,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const GemmArgs g) {
     }
 }
 
-// The small-result kernel applies when the 64x64 tiling would leave most of the chip idle.
+// The small-result kernel applies when the 64x64 tiling would leave most of the chip idle.  Up to
+// 2048 tiles of 16 x 16 it beats the 64 x 64 tiles (512 x 768 -> 768: 6.1 against 7.3 us; 128 x 768
+// -> 2304: 5.4 against 7.0), from about 2300 on it loses (256 x 768 -> 2304: 8.0 against 7.4).
 static bool gemm_skinny_applies(const GemmArgs &g, int batch, bool trans_b) {
     const auto misaligned = [](const void *p, int a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; };
     if (!trans_b || g.a_gather || batch < 1 || batch > 65535) return false;
@@ -283,7 +285,7 @@ static bool gemm_skinny_applies(const GemmArgs &g, int batch, bool trans_b) {
     if (batch > 1 && (((g.sAo | g.sAi | g.sBo | g.sBi) & 7) || ((g.sCo | g.sCi) & 3))) return false;
     const long long tiles64 = (long long)((g.M + 63) / 64) * ((g.N + 63) / 64) * batch;
     const long long tiles16 = (long long)(g.M / 16) * (g.N / 16);
-    return tiles64 < 64 && tiles16 <= 1024;
+    return tiles64 < 128 && tiles16 <= 2048;
 }
 
 // C[r][c] = act(bias[c]) for the columns a row-pruned weight does not produce.

@@ -26,7 +26,9 @@ up = Hn.up
                                            (1008, 720, 400, 2), (80, 96, 2064, 1), (2032, 176, 48, 0),
                                            # few 64x64 tiles and a long K: one 16x16 tile per workgroup, K split over
                                            # its waves (K a multiple of 32, of 16 only, more than one round of loads)
-                                           (128, 768, 768, 2), (16, 272, 16, 0), (128, 3072, 80, 1), (32, 6160, 48, 0)])
+                                           (128, 768, 768, 2), (16, 272, 16, 0), (128, 3072, 80, 1), (32, 6160, 48, 0),
+                                           # the largest results that kernel takes: 2048 tiles of 16 x 16
+                                           (512, 768, 1024, 2), (128, 768, 2304, 0), (448, 784, 720, 1)])
 def test_linear_dense(et, T, inp, out, act):
     W, b, x = Hn.randn((out, inp), 1, 0.02), Hn.randn((out,), 2, 0.1), Hn.randn((T, inp), 3)
     d_y = et.DeviceBuffer.empty((T, out), np.float16)
