@@ -316,7 +316,16 @@ static bool pick_dma_tile(const GemmArgs &g, int batch, bool trans_b, DmaTile *o
         // 64 x 64 tiles with the edges clamped and masked; large ragged problems are left to the
         // 128 x 128 tiles of the register-staged kernel
         const long long w = (long long)((g.M + 63) / 64) * ((g.N + 63) / 64) * batch;
-        if (g.M % 16 || g.N % 16 || g.K % 16 || w > 1536) return false;
+        if (g.M % 16 || g.N % 16 || g.K % 16) return false;
+        if (batch == 1 && trans_b) {
+            // enough workgroups for the larger tiles, as for whole tiles below (a row- or column-pruned
+            // Linear keeps any multiple of 16 features: 2048 x 768 -> 2928 26.7 -> 21.4 us with 128 x 64 tiles)
+            const long long m128 = (g.M + 127) / 128;
+            if ((long long)((g.M + 255) / 256) * ((g.N + 255) / 256) >= 1024) { *out = {4, 4, 2, true}; return true; }
+            if (m128 * ((g.N + 127) / 128) >= 512) { *out = {2, 2, 2, true}; return true; }
+            if (m128 * ((g.N + 63) / 64) >= 512) { *out = {2, 1, 2, true}; return true; }
+        }
+        if (w > 1536) return false;
         // Batched problems and B stored k-major run on this instantiation too, where they are
         // bound by the latency of a long K loop in few workgroups (the stacked VO product of the
         // pre-computed-VO attention: 32 -> 22 us); gathering the k-major fragments with 2-byte LDS
@@ -385,6 +394,9 @@ int launch_gemm_dma(const GemmArgs &g, int batch, bool trans_b, hipStream_t stre
         if (!trans_b)
             return t.nbuf == 3 ? launch_dma_tile<1, 1, 3, true, true>(g, batch, stream)
                                : launch_dma_tile<1, 1, 2, true, true>(g, batch, stream);
+        if (t.tmw == 4) return launch_dma_tile<4, 4, 2, true>(g, batch, stream);
+        if (t.tmw == 2) return t.tnw == 2 ? launch_dma_tile<2, 2, 2, true>(g, batch, stream)
+                                          : launch_dma_tile<2, 1, 2, true>(g, batch, stream);
         return t.nbuf == 3 ? launch_dma_tile<1, 1, 3, true>(g, batch, stream)
                            : launch_dma_tile<1, 1, 2, true>(g, batch, stream);
     }

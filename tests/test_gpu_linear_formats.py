@@ -28,7 +28,9 @@ up = Hn.up
                                            # its waves (K a multiple of 32, of 16 only, more than one round of loads)
                                            (128, 768, 768, 2), (16, 272, 16, 0), (128, 3072, 80, 1), (32, 6160, 48, 0),
                                            # the largest results that kernel takes: 2048 tiles of 16 x 16
-                                           (512, 768, 1024, 2), (128, 768, 2304, 0), (448, 784, 720, 1)])
+                                           (512, 768, 1024, 2), (128, 768, 2304, 0), (448, 784, 720, 1),
+                                           # edges of 16 with enough work for the 128 x 64 and 128 x 128 tiles
+                                           (2048, 768, 2928, 2), (2000, 720, 2096, 1), (4080, 208, 4112, 0), (8176, 80, 8208, 1)])
 def test_linear_dense(et, T, inp, out, act):
     W, b, x = Hn.randn((out, inp), 1, 0.02), Hn.randn((out,), 2, 0.1), Hn.randn((T, inp), 3)
     d_y = et.DeviceBuffer.empty((T, out), np.float16)
@@ -135,7 +137,8 @@ def test_gemm_rejects_bad_args(et):
                                               (2048, 3072, 768, 0.5, 0), (64, 64, 100 * 16, 0.9, 1),
                                               (8192, 128, 4096, 0.5, 2),  # the 256 x 256-tile kernel
                                               (2048, 720, 784, 0.45, 1),  # 432 surviving rows: a ragged tile edge
-                                              (128, 768, 768, 0.9, 2)])  # one sequence: the small-result kernel, scattered
+                                              (128, 768, 768, 0.9, 2),  # one sequence: the small-result kernel, scattered
+                                              (2048, 768, 3072, 0.05, 2)])  # 2928 surviving rows: ragged 128 x 64 tiles, scattered
 def test_linear_rowpruned(et, T, inp, out, sp, act):
     row_id = F.gen_row_ids(out, sp, seed=8)
     rows, b, x = Hn.randn((len(row_id), inp), 9, 0.02), Hn.randn((out,), 10, 0.1), Hn.randn((T, inp), 11)
