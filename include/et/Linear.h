@@ -52,6 +52,19 @@ template <> class Linear<base_mat> {
     }
 };
 
+namespace et {
+namespace detail {
+// ids (on the device) are exactly 0, 1, ..., n - 1: read back once, at construction
+inline bool is_identity(const et::DeviceBuffer<int> &ids, int n) {
+    if ((long long)ids.size != n) return false;
+    const std::vector<int> host = ids.to_host();
+    for (int i = 0; i < n; i++)
+        if (host[(std::size_t)i] != i) return false;
+    return true;
+}
+}  // namespace detail
+}  // namespace et
+
 // output-feature pruning — Linear/Linear.h:69-86, Linear/SPMM_row.cu:48-95
 template <> class Linear<row_mat> {
   public:
@@ -60,17 +73,27 @@ template <> class Linear<row_mat> {
     row_mat weight;
     et::DeviceBuffer<half> bias;
     int size;
+    bool nothing_pruned = false;  // every row kept, in order: the weight is a plain dense one
 
     Linear(int _in_size, int _out_size, const row_mat &w, const half *b, int _size)
-        : in_size(_in_size), out_size(_out_size), weight(w), bias(b, (std::size_t)_out_size), size(_size) {}
+        : in_size(_in_size), out_size(_out_size), weight(w), bias(b, (std::size_t)_out_size), size(_size) {
+        nothing_pruned = et::detail::is_identity(*weight.row_id, _out_size);
+    }
     Linear(int _in_size, int _out_size, row_mat &&w, const half *b, int _size)
         : in_size(_in_size), out_size(_out_size), weight(std::move(w)), bias(b, (std::size_t)_out_size),
-          size(_size) {}
+          size(_size) {
+        nothing_pruned = et::detail::is_identity(*weight.row_id, _out_size);
+    }
     // full-width output: pruned features carry their bias alone
     void forward(half *output, const half *input, et::stream_t stream = nullptr) const {
         forward_act(output, input, ET_ACT_NONE, stream);
     }
     void forward_act(half *output, const half *input, int act, et::stream_t stream = nullptr) const {
+        if (nothing_pruned) {  // no fill pass, no scattered stores
+            etChk(et_linear_dense_f16(et::f16(weight.rows->get()), et::f16(bias.get()), et::f16(input),
+                                      et::f16(output), size, (int)in_size, (int)out_size, act, stream));
+            return;
+        }
         etChk(et_linear_rowpruned_f16(et::f16(weight.rows->get()), weight.row_id->get(), weight.nnz_row(),
                                       et::f16(bias.get()), et::f16(input), et::f16(output), size,
                                       (int)in_size, (int)out_size, act, stream));
