@@ -312,6 +312,25 @@ class Attention<_config, std::enable_if_t<_config::isSingleKernel>> : public et:
         else
             return false;
     }
+    void prepare_split(int nwave = 0) {
+        if constexpr (std::is_same<linearQKV_t, Linear<tile_mat>>::value && std::is_same<linearO_t, Linear<tile_mat>>::value) {
+            linearQKV->prepare_split_consumer(nwave);
+            linearO->prepare_split_producer(nwave);
+        }
+    }
+    // The pieces a caller needs to run this attention as part of a chain launch (et_encoder_chain_f32):
+    // the two projections, the buffers between them, and the attention kernel on its own.
+    linearQKV_t &qkv_linear() { return *linearQKV; }
+    linearO_t &o_linear() { return *linearO; }
+    half *qkv_buffer() { return mat_qkv->get(); }
+    half *z_buffer() { return mat_z->get(); }
+    void core(et::stream_t stream = nullptr) {
+        const int ldm = model->kdim * 2 + model->vdim;
+        half *Q = mat_qkv->get();
+        half *K = Q + model->kdim;
+        half *V = K + model->kdim;
+        et::fused_mha(Q, K, V, ldm, ldm, ldm, mat_z->get(), model->vdim, *model, run(stream));
+    }
     void forward_split(float *v1, float *stats1, int *groups1, float *fin_in, const et::SplitSum *in, const float *x32,
                        half *x16, et::stream_t stream = nullptr) {
         if constexpr (std::is_same<linearQKV_t, Linear<tile_mat>>::value && std::is_same<linearO_t, Linear<tile_mat>>::value) {

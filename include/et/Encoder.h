@@ -55,6 +55,18 @@ template <typename ACT_OP_t> void act(half *data, int size, et::stream_t stream 
 
 namespace et {
 
+// One layer's operands of a chain launch (et_chain_desc takes the projections of this layer and
+// the QKV projection of the next).
+struct ChainParts {
+    et_bsr_pack qkv = nullptr, o = nullptr, up = nullptr, down = nullptr;
+    const half *bias_qkv = nullptr, *bias_o = nullptr, *bias_up = nullptr, *bias_down = nullptr;
+    half *QKV = nullptr, *Z = nullptr, *H = nullptr;
+    float *fin_in = nullptr, *V1 = nullptr, *stats1 = nullptr, *fin1 = nullptr, *V2 = nullptr, *stats2 = nullptr;
+    const half *gamma1 = nullptr, *beta1 = nullptr, *gamma2 = nullptr, *beta2 = nullptr;
+    float eps1 = 1e-5f, eps2 = 1e-5f;
+    int act = ET_ACT_NONE;
+};
+
 // The layer body shared by Encoder and Encoder_fuse.
 template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_OP_t> class EncoderLayer {
   protected:
@@ -154,6 +166,66 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
         if (!stats2) stats2 = std::make_unique<DeviceBuffer<float>>(st);
         if (!fin_in) fin_in = std::make_unique<DeviceBuffer<float>>((std::size_t)rows * 2);
         if (!fin1) fin1 = std::make_unique<DeviceBuffer<float>>((std::size_t)rows * 2);
+        if constexpr (attn_has_split<attn_t>::value && std::is_same_v<linear1_t, Linear<tile_mat>> &&
+                      std::is_same_v<linear2_t, Linear<tile_mat>>) {
+            // packs of 12 waves where the shape has them: what the one-launch chain takes, and as fast as
+            // any other wave count in separate launches
+            attn->prepare_split(kChainWaves);
+            linear1->prepare_split_consumer(kChainWaves);
+            linear2->prepare_split_producer(kChainWaves);
+            attn->prepare_split();
+            linear1->prepare_split_consumer();
+            linear2->prepare_split_producer();
+        }
+    }
+    static constexpr int kChainWaves = 12;
+    // This layer's share of a chain launch (et_encoder_chain_f32): everything between its attention
+    // kernel and the next layer's.  false when the layer's types have no such form.
+    bool chain_parts(ChainParts &p) {
+        if constexpr (attn_has_split<attn_t>::value && std::is_same_v<linear1_t, Linear<tile_mat>> &&
+                      std::is_same_v<linear2_t, Linear<tile_mat>>) {
+            auto &lq = attn->qkv_linear();
+            auto &lo = attn->o_linear();
+            if (!stats1 || !lq.pack_consumer || !lo.pack_producer || !linear1->pack_consumer || !linear2->pack_producer)
+                return false;
+            p.qkv = lq.pack_consumer.get();
+            p.bias_qkv = lq.bias.get();
+            p.QKV = attn->qkv_buffer();
+            p.fin_in = fin_in->get();
+            p.o = lo.pack_producer.get();
+            p.bias_o = lo.bias.get();
+            p.Z = attn->z_buffer();
+            p.V1 = temp_attn32->get();
+            p.stats1 = stats1->get();
+            p.up = linear1->pack_consumer.get();
+            p.bias_up = linear1->bias.get();
+            p.gamma1 = LN1->gamma();
+            p.beta1 = LN1->beta();
+            p.eps1 = LN1->epsilon();
+            p.fin1 = fin1->get();
+            p.H = temp_linear.get();
+            p.act = act_code<ACT_OP_t>();
+            p.down = linear2->pack_producer.get();
+            p.bias_down = linear2->bias.get();
+            p.V2 = temp_ffn32->get();
+            p.stats2 = stats2->get();
+            p.gamma2 = LN2->gamma();
+            p.beta2 = LN2->beta();
+            p.eps2 = LN2->epsilon();
+            return true;
+        } else {
+            (void)p;
+            return false;
+        }
+    }
+    // the first layer's QKV projection of the binary16 input, and the attention kernel alone
+    void chain_qkv_first(half *x16, stream_t stream = nullptr) {
+        if constexpr (attn_has_split<attn_t>::value) attn->qkv_linear().forward(attn->qkv_buffer(), x16, stream);
+        else (void)x16, (void)stream;
+    }
+    void chain_attention(stream_t stream = nullptr) {
+        if constexpr (attn_has_split<attn_t>::value) attn->core(stream);
+        else (void)stream;
     }
     SplitSum forward_split(const SplitSum *in, const float *x32, half *x16, stream_t stream = nullptr) {
         SplitSum out;

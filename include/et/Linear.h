@@ -8,6 +8,7 @@
 // GEMM instead of the reference's extra passes.  Nothing blocks the host.
 #pragma once
 #include <algorithm>
+#include <cstdlib>
 #include <memory>
 #include <type_traits>
 #include <utility>
@@ -158,6 +159,25 @@ template <> class Linear<tile_mat> {
     };
     std::unique_ptr<et_bsr_plan_s, PlanDeleter> plan;
     static bool wants_plan(int in, int rows) { return in >= 128 && (in > 5112 || (in >= 3072 && rows >= 4096)); }
+    // Copies of the weight in the order one launch of the packed kernel reads it (et_bsr16_pack_create),
+    // held where that kernel applies — up to kPackMaxRows token rows, inputs that are multiples of 128
+    // up to 4096: a launch whose loads are all issued at its start, with no row-pointer round trip.
+    // `pack` serves forward / forward_act / forward_f32; the split normalisation of the
+    // mixed-precision layer builds one more per role on prepare_split_producer / _consumer.
+    struct PackDeleter {
+        void operator()(et_bsr_pack_s *p) const { (void)et_bsr16_pack_destroy(p); }
+    };
+    using pack_ptr = std::unique_ptr<et_bsr_pack_s, PackDeleter>;
+    pack_ptr pack, pack_producer, pack_consumer;
+    static constexpr int kPackMaxRows = 4096;
+    // ET_PACKED=0 in the environment keeps every Linear<tile_mat> on the unpacked kernels (for comparisons)
+    static bool packed_enabled() {
+        static const bool on = [] {
+            const char *e = std::getenv("ET_PACKED");
+            return !(e && e[0] == '0');
+        }();
+        return on;
+    }
     // Dense image of the weight, held where the dense GEMM is the faster kernel: a matrix that
     // keeps most of its tiles (measured at 2048 rows: the tile kernel overtakes the dense one at
     // 35-50 % sparsity for 768-wide inputs, at 50 % for 3072-wide ones).  Not built when a tile
@@ -199,6 +219,11 @@ template <> class Linear<tile_mat> {
                                               size, act, stream));
             return;
         }
+        if (pack) {
+            etChk(et_linear_bsr16_packed_f16(pack.get(), et::f16(bias.get()), et::f16(input), et::f16(output), nullptr,
+                                             size, act, stream));
+            return;
+        }
         etChk(et_linear_bsr16_f16(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
                                   et::f16(bias.get()), et::f16(input), et::f16(output), size, (int)in_size,
                                   (int)out_size, act, stream));
@@ -216,6 +241,11 @@ template <> class Linear<tile_mat> {
                                               ET_ACT_NONE, stream));
             return;
         }
+        if (pack) {
+            etChk(et_linear_bsr16_packed_f16(pack.get(), et::f16(bias.get()), et::f16(input), nullptr, output, size,
+                                             ET_ACT_NONE, stream));
+            return;
+        }
         etChk(et_linear_bsr16_f16_f32out(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
                                          et::f16(bias.get()), et::f16(input), output, size, (int)in_size,
                                          (int)out_size, ET_ACT_NONE, stream));
@@ -229,11 +259,27 @@ template <> class Linear<tile_mat> {
     bool split_consumer_ok() const {
         return !dense && !plan && size > 0 && et_norm_linear_bsr16_f32in_supported(size, (int)in_size, (int)out_size) == 1;
     }
+    // Packs for the two roles (called once, outside any stream capture; a shape the packed kernel does
+    // not take keeps the unpacked one)
+    // (nwave: waves per workgroup the pack is built for, 0 = the builder's choice; the one-launch
+    // chain of the encoder layer takes packs of 12)
+    void prepare_split_producer(int nwave = 0) {
+        if (!pack_producer && !dense && !plan) pack_producer = make_pack(ET_PACK_STATS_PRODUCER, nwave);
+    }
+    void prepare_split_consumer(int nwave = 0) {
+        if (!pack_consumer && !dense && !plan) pack_consumer = make_pack(ET_PACK_NORM_CONSUMER, nwave);
+    }
     // V = input W^T + bias + residual (binary32) and stats[*groups][size][2]; the residual is
     // `resid` itself, or with resid_fin its normalisation by (resid_fin, resid_gamma, resid_beta)
     void forward_resid_stats_f32(float *V, float *stats, int *groups, const half *input, const float *resid,
                                  const float *resid_fin, const half *resid_gamma, const half *resid_beta,
                                  et::stream_t stream = nullptr) {
+        if (pack_producer) {
+            etChk(et_linear_bsr16_packed_resid_stats_f32(pack_producer.get(), et::f16(bias.get()), et::f16(input), resid, nullptr,
+                                                         resid_fin, et::f16(resid_gamma), et::f16(resid_beta), V, stats, groups,
+                                                         size, stream));
+            return;
+        }
         etChk(et_linear_bsr16_resid_stats_f32(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
                                               et::f16(bias.get()), et::f16(input), resid, resid_fin, et::f16(resid_gamma),
                                               et::f16(resid_beta), V, stats, groups, size, (int)in_size, (int)out_size,
@@ -242,6 +288,12 @@ template <> class Linear<tile_mat> {
     // the same with the residual in binary16
     void forward_resid16_stats_f32(float *V, float *stats, int *groups, const half *input, const half *resid16,
                                    et::stream_t stream = nullptr) {
+        if (pack_producer) {
+            etChk(et_linear_bsr16_packed_resid_stats_f32(pack_producer.get(), et::f16(bias.get()), et::f16(input), nullptr,
+                                                         et::f16(resid16), nullptr, nullptr, nullptr, V, stats, groups, size,
+                                                         stream));
+            return;
+        }
         etChk(et_linear_bsr16_resid16_stats_f32(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
                                                 et::f16(bias.get()), et::f16(input), et::f16(resid16), V, stats, groups,
                                                 size, (int)in_size, (int)out_size, stream));
@@ -250,6 +302,11 @@ template <> class Linear<tile_mat> {
     void forward_norm_f32in(half *output, const float *V, const float *stats, int groups, const half *gamma,
                             const half *beta, float eps, float *fin_out, float *ln32, half *ln16, int act,
                             et::stream_t stream = nullptr) {
+        if (pack_consumer && !ln32 && !ln16) {
+            etChk(et_norm_linear_bsr16_packed_f32in(pack_consumer.get(), V, stats, groups, et::f16(gamma), et::f16(beta), eps,
+                                                    fin_out, et::f16(bias.get()), et::f16(output), size, act, stream));
+            return;
+        }
         etChk(et_norm_linear_bsr16_f32in(V, stats, groups, et::f16(gamma), et::f16(beta), eps, fin_out, ln32, et::f16(ln16),
                                          weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
                                          et::f16(bias.get()), et::f16(output), size, (int)in_size, (int)out_size, act,
@@ -288,7 +345,22 @@ template <> class Linear<tile_mat> {
             etChk(et_bsr16_plan_create(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()), size,
                                        (int)in_size, (int)out_size, 0, 0, 0, &p));
             plan.reset(p);
+            return;
         }
+        pack = make_pack(0);
+    }
+    // a pack for this weight and `size` rows, or null where the packed kernel does not apply
+    pack_ptr make_pack(int flags, int nwave = 0) const {
+        pack_ptr made;
+        if (!packed_enabled() || size <= 0 || size % 16 != 0 || size > kPackMaxRows || in_size % 128 != 0 || in_size > 4096)
+            return made;
+        et_bsr_pack p = nullptr;
+        const int s = et_bsr16_pack_create(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()), size,
+                                           (int)in_size, (int)out_size, flags, nwave, &p);
+        if (s == ET_ERR_UNSUPPORTED) return made;  // the unpacked kernel keeps the shape
+        etChk(s);
+        made.reset(p);
+        return made;
     }
     // true when some block-row lists one column twice, or an index lies outside the matrix (such a
     // weight stays with the tile kernel, which reports it)

@@ -158,6 +158,112 @@ int et_linear_bsr16_planned_f16(et_bsr_plan plan, const et_f16 *bias,
                                 const et_f16 *X, et_f16 *Y, float *Y32, int T,
                                 int act, et_stream stream);
 
+/* Tile-sparse Linear through a pack: the launch form for a few hundred to a few
+ * thousand token rows, where a launch is a chain of memory round trips rather
+ * than arithmetic.  et_bsr16_pack_create copies the weight once (device
+ * pointers in the reference layout in; blocking) into the order one launch
+ * geometry for T token rows reads it: per workgroup and wave a fixed number of
+ * two-tile slots, zero-padded, so that every load of a launch is issued when it
+ * starts and none depends on another.  ET_UNSUPPORTED when the shape is outside
+ * that form (in not a multiple of 128 or above 4096, more than 16384 rows, ...):
+ * the caller then uses et_linear_bsr16_f16.  flags: ET_PACK_STATS_PRODUCER keeps
+ * the block-row groups of a strip to the 16 that the row sums of
+ * et_linear_bsr16_packed_resid_stats_f32 allow; ET_PACK_NORM_CONSUMER picks a
+ * workgroup size that deals the binary32 strip of
+ * et_norm_linear_bsr16_packed_f32in evenly (in >= 512).  nwave asks for that
+ * many waves per workgroup (0: chosen with the rest of the geometry; the chain
+ * call below takes packs of 12).  A pack is used with
+ * the T it was built for, or any smaller multiple of 16.  The three calls
+ * compute what et_linear_bsr16_f16 / et_linear_bsr16_f16_f32out,
+ * et_linear_bsr16_resid_stats_f32 / et_linear_bsr16_resid16_stats_f32 (exactly
+ * one of resid and resid16 set) and et_norm_linear_bsr16_f32in (without the
+ * optional normalised outputs) compute, up to the order of the fp32
+ * accumulation.  Replaces Linear<tile_mat>::forward (Linear/SPMM_tile.cu:312-324)
+ * for callers that keep a Linear object. */
+typedef struct et_bsr_pack_s *et_bsr_pack;
+enum et_pack_flags { ET_PACK_NORM_CONSUMER = 1, ET_PACK_STATS_PRODUCER = 2 };
+int et_bsr16_pack_create(const int32_t *row_ptr, const int32_t *col_idx,
+                         const et_f16 *tiles, int T, int in, int out, int flags,
+                         int nwave, et_bsr_pack *pack);
+int et_bsr16_pack_destroy(et_bsr_pack pack);
+/* the geometry a pack was built with: 16-row blocks per token strip, block-row
+ * groups, waves per workgroup, slots per wave, LDS bytes of a workgroup */
+int et_bsr16_pack_info(et_bsr_pack pack, int *mt, int *ngroups, int *nwave,
+                       int *cap, int *lds_bytes);
+int et_linear_bsr16_packed_f16(et_bsr_pack pack, const et_f16 *bias,
+                               const et_f16 *X, et_f16 *Y, float *Y32, int T,
+                               int act, et_stream stream);
+int et_linear_bsr16_packed_resid_stats_f32(et_bsr_pack pack, const et_f16 *bias,
+                                           const et_f16 *X, const float *resid,
+                                           const et_f16 *resid16,
+                                           const float *resid_fin,
+                                           const et_f16 *resid_gamma,
+                                           const et_f16 *resid_beta, float *V,
+                                           float *stats, int *stat_groups, int T,
+                                           et_stream stream);
+int et_norm_linear_bsr16_packed_f32in(et_bsr_pack pack, const float *V,
+                                      const float *stats, int stat_groups,
+                                      const et_f16 *gamma, const et_f16 *beta,
+                                      float eps, float *fin_out,
+                                      const et_f16 *bias, et_f16 *Y, int T,
+                                      int act, et_stream stream);
+
+/* The token-local part of an encoder layer in one launch (mixed-precision layer
+ * with the split SkipLayerNorm, tile-sparse projections through packs of 12 waves):
+ *   V1  = Z W_O^T + b_O + residual                      (binary32, row sums stats1)
+ *   H   = act(LayerNorm1(V1) W_1^T + b_1)               (binary16; fin1 = mean, rstd of V1's rows)
+ *   V2  = H W_2^T + b_2 + LayerNorm1(V1)                (binary32, row sums stats2)
+ *   QKV = LayerNorm2(V2) W_qkv^T + b_qkv                (the NEXT layer's projection; fin2; skipped
+ *                                                        when qkv is NULL)
+ * i.e. et_linear_bsr16_packed_resid_stats_f32, et_norm_linear_bsr16_packed_f32in,
+ * et_linear_bsr16_packed_resid_stats_f32 and et_norm_linear_bsr16_packed_f32in
+ * with the same operands, bit for bit, but with the workgroups of each XCD
+ * meeting at a counter in their L2 between the steps instead of at three kernel
+ * boundaries.  The residual of the first step is resid (binary32; normalised by
+ * resid_fin / resid_gamma / resid_beta when resid_fin is set) or resid16.
+ * sync: ET_CHAIN_SYNC_WORDS words of device memory, 128-byte aligned, ALL ZERO when
+ * the launch starts (et_fill_i32) and used by one launch at a time;
+ * et_encoder_chain_status (blocking) reads back how many workgroups gave up
+ * waiting at a barrier and how many ran on another XCD than the workgroups they
+ * share a counter with —
+ * both 0 in a valid run; otherwise the results are not to be used and the caller
+ * returns to the separate calls.  All workgroups must be resident at once: no
+ * other kernel that itself waits for this one may run beside it.
+ * et_encoder_chain_supported: 1 when the packs form a chain this launch runs
+ * (0: et_last_error says what does not fit).
+ * Replaces the launches between the attention kernels of
+ * Encoder<cfg>::forward (Encoder/Encoder.h:81-96) and the QKV Linear of
+ * Attention<cfg, true>::forward (Attention/Attention.h:246-253). */
+#define ET_CHAIN_SYNC_WORDS 288
+typedef struct et_chain_desc {
+    et_bsr_pack o;
+    const et_f16 *bias_o, *Z;
+    const float *resid;
+    const et_f16 *resid16;
+    const float *resid_fin;
+    const et_f16 *resid_gamma, *resid_beta;
+    float *V1, *stats1;
+    et_bsr_pack up;
+    const et_f16 *bias_up, *gamma1, *beta1;
+    float eps1;
+    float *fin1;
+    et_f16 *H;
+    int act;
+    et_bsr_pack down;
+    const et_f16 *bias_down;
+    float *V2, *stats2;
+    et_bsr_pack qkv;
+    const et_f16 *bias_qkv, *gamma2, *beta2;
+    float eps2;
+    float *fin2;
+    et_f16 *QKV;
+    int T;
+    uint32_t *sync;
+} et_chain_desc;
+int et_encoder_chain_supported(const et_chain_desc *desc);
+int et_encoder_chain_f32(const et_chain_desc *desc, int *stat_groups2, et_stream stream);
+int et_encoder_chain_status(const uint32_t *sync, int *gave_up, int *misplaced);
+
 /* SkipLayerNorm fused into the tile-sparse Linear that consumes it:
  *   ln_out = LayerNorm(src + skip) * gamma + beta      (written, [T x in])
  *   Y      = act(ln_out * W^T + bias)
@@ -581,13 +687,15 @@ typedef struct et_model_desc {
     float eps;     /* LayerNorm epsilon; <= 0 selects 1e-5                        */
     int causal;    /* != 0: causal mask (the reference's hard-wired one)          */
     int use_graph; /* != 0: replay a captured HIP graph; 0: launch kernel by kernel */
-    int mixed;     /* 1 or 2: mixed precision — the residual stream (layer inputs, the two
+    int mixed;     /* 1, 2 or 3: mixed precision — the residual stream (layer inputs, the two
                     * projections that feed a SkipLayerNorm, both SkipLayerNorm results)
                     * is kept in binary32 inside the stack, binary16 only as matrix-core
                     * operands; input and output of et_model_forward stay binary16.
                     * 1: SkipLayerNorm is folded into the neighbouring tile-sparse projections
                     *    where the shapes allow (five launches per layer); 2: it keeps its own
-                    *    launches (seven).
+                    *    launches (seven); 3: as 1, with everything between two attention
+                    *    kernels in one launch (et_encoder_chain_f32: two launches per layer)
+                    *    where the shapes allow and the device runs it as it must, else as 1.
                     * 0: every activation is stored as binary16 (the reference's storage) */
 } et_model_desc;
 
@@ -630,6 +738,11 @@ int et_model_forward(et_model m, et_f16 *out, const et_f16 *in, et_stream stream
 int et_model_forward_layer(et_model m, int layer, et_f16 *out, const et_f16 *in,
                            et_stream stream);
 int et_model_sync(et_model m);
+/* kernel launches per encoder layer of a finalized model in the mode it actually runs
+ * (2: chain launches, 5: SkipLayerNorm folded into the projections, 7: SkipLayerNorm on its own;
+ * 0 before et_model_finalize).  A model asked for mixed = 3 reports 5 once it has gone back to
+ * separate launches. */
+int et_model_launches_per_layer(et_model m, int *launches);
 int et_model_destroy(et_model m);
 
 /* ------------------------------------------------------------------------

@@ -22,6 +22,15 @@ int et_linear_bsr16_f16_geom(const int32_t *row_ptr, const int32_t *col_idx,
                              int act, int mt, int stage, int threads,
                              int rows_per_wg, et_stream stream);
 
+/* Tuning hook: et_bsr16_pack_create with an explicit geometry — mt 16-row blocks
+ * per token strip (1 or 2), block-row groups per strip, waves per workgroup and
+ * slots per wave (4, 8, 12, 16, 20 or 24); 0 picks a value as
+ * et_bsr16_pack_create does.  No reference counterpart. */
+int et_bsr16_pack_create_geom(const int32_t *row_ptr, const int32_t *col_idx,
+                              const et_f16 *tiles, int T, int in, int out,
+                              int flags, int mt, int ngroups, int nwave, int cap,
+                              et_bsr_pack *pack);
+
 #ifdef __cplusplus
 }
 #endif

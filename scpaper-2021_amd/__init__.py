@@ -71,6 +71,16 @@ _SIGNATURES = {
     "et_bsr16_plan_destroy": (_vp,),
     "et_bsr16_plan_info": (_vp, C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)),
     "et_linear_bsr16_planned_f16": (_vp, _vp, _vp, _vp, _vp, _i, _i, _vp),
+    "et_bsr16_pack_create": (_vp, _vp, _vp, _i, _i, _i, _i, _i, C.POINTER(_vp)),
+    "et_bsr16_pack_create_geom": (_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, C.POINTER(_vp)),
+    "et_bsr16_pack_destroy": (_vp,),
+    "et_bsr16_pack_info": (_vp, C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)),
+    "et_linear_bsr16_packed_f16": (_vp, _vp, _vp, _vp, _vp, _i, _i, _vp),
+    "et_linear_bsr16_packed_resid_stats_f32": (_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, C.POINTER(_i), _i, _vp),
+    "et_norm_linear_bsr16_packed_f32in": (_vp, _vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _vp),
+    "et_encoder_chain_supported": (_vp,),
+    "et_encoder_chain_f32": (_vp, C.POINTER(_i), _vp),
+    "et_encoder_chain_status": (_vp, C.POINTER(_i), C.POINTER(_i)),
     "et_linear_bsr16_f16_geom": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp),
     "et_skipln_linear_bsr16_f16": (_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_linear_bsr16_fused_ln_supported": (_i, _i, _i),
@@ -136,6 +146,7 @@ _SIGNATURES = {
     "et_model_forward": (_vp, _vp, _vp, _vp),
     "et_model_forward_layer": (_vp, _i, _vp, _vp, _vp),
     "et_model_sync": (_vp,),
+    "et_model_launches_per_layer": (_vp, C.POINTER(_i)),
     "et_model_destroy": (_vp,),
     "et_fmt_permutation": (C.c_int64, C.c_uint64, _vp),
     "et_fmt_kept_count": (C.c_int64, _f),
@@ -157,6 +168,19 @@ W_QKV, W_O, W_FF1, W_FF2 = 0, 1, 2, 3
 class ModelDesc(C.Structure):
     _fields_ = [("kdim", _i), ("vdim", _i), ("seq_len", _i), ("nhead", _i), ("dimFF", _i), ("emdim", _i),
                 ("nlayer", _i), ("batch", _i), ("act", _i), ("eps", _f), ("causal", _i), ("use_graph", _i), ("mixed", _i)]
+
+
+class ChainDesc(C.Structure):
+    """et_chain_desc of include/et_abi.h"""
+    _fields_ = [("o", _vp), ("bias_o", _vp), ("Z", _vp), ("resid", _vp), ("resid16", _vp), ("resid_fin", _vp),
+                ("resid_gamma", _vp), ("resid_beta", _vp), ("V1", _vp), ("stats1", _vp),
+                ("up", _vp), ("bias_up", _vp), ("gamma1", _vp), ("beta1", _vp), ("eps1", _f), ("fin1", _vp), ("H", _vp),
+                ("act", _i),
+                ("down", _vp), ("bias_down", _vp), ("V2", _vp), ("stats2", _vp),
+                ("qkv", _vp), ("bias_qkv", _vp), ("gamma2", _vp), ("beta2", _vp), ("eps2", _f), ("fin2", _vp), ("QKV", _vp),
+                ("T", _i), ("sync", _vp)]
+
+
 _RESTYPES = {"et_status_string": C.c_char_p, "et_last_error": C.c_char_p}
 
 _lib = None
@@ -389,6 +413,11 @@ class Model:
         beta = np.ascontiguousarray(beta, gamma.dtype)
         fn = lib().et_model_set_norm_f16 if gamma.dtype == np.float16 else lib().et_model_set_norm
         check(fn(self.handle, layer, which, _np_ptr(gamma), _np_ptr(beta)))
+
+    def launches_per_layer(self) -> int:
+        n = _i()
+        check(lib().et_model_launches_per_layer(self.handle, C.byref(n)))
+        return n.value
 
     def set_lens(self, lens):
         lens = None if lens is None else np.ascontiguousarray(lens, np.int32)

@@ -24,6 +24,9 @@ struct ILayer {
     virtual void enable_split() = 0;
     virtual et::SplitSum forward_split(const et::SplitSum *in, const float *x32, half *x16, stream_t stream) = 0;
     virtual void finish_split(float *out32, half *out16, const et::SplitSum &s, stream_t stream) = 0;
+    virtual bool chain_parts(et::ChainParts &p) = 0;
+    virtual void chain_qkv_first(half *x16, stream_t stream) = 0;
+    virtual void chain_attention(stream_t stream) = 0;
     virtual et::AttnState &attn() = 0;
 };
 
@@ -43,6 +46,9 @@ template <typename EncoderT> struct LayerOf final : ILayer {
     void finish_split(float *out32, half *out16, const et::SplitSum &s, stream_t stream) override {
         enc->finish_split(out32, out16, s, stream);
     }
+    bool chain_parts(et::ChainParts &p) override { return enc->chain_parts(p); }
+    void chain_qkv_first(half *x16, stream_t stream) override { enc->chain_qkv_first(x16, stream); }
+    void chain_attention(stream_t stream) override { enc->chain_attention(stream); }
     et::AttnState &attn() override { return enc->attention(); }
 };
 
@@ -82,6 +88,11 @@ struct et_model_s {
     std::vector<half> mask;  // empty = no additive mask
     bool finalized = false;
     bool split = false;  // mixed precision with SkipLayerNorm folded into the projections
+    // split, with everything between two attention kernels in one launch (et_encoder_chain_f32):
+    // one description per layer and the barrier counters of all layers, cleared at the start of a forward
+    bool chain = false;
+    std::vector<et_chain_desc> chain_desc;
+    std::unique_ptr<et::DeviceBuffer<int>> chain_sync;
 
     stream_t own_stream = nullptr;
     et_graph graph = nullptr;
@@ -171,7 +182,105 @@ void check_layer_index(const et_model_s *m, int layer) {
 // in both forms (binary32 residual, binary16 operand), the last one writes binary16 to `out`.
 // The same with SkipLayerNorm folded into the neighbouring projections (five launches per layer):
 // every layer hands the next one its un-normalised binary32 result with its row sums.
+// The descriptions of the chain launches, or false when some layer has no such form.  Layer i's
+// launch holds its output projection and FFN and layer i + 1's QKV projection.
+bool build_chain(et_model_s &m) {
+    const int n = (int)m.layers.size();
+    std::vector<et::ChainParts> parts((size_t)n);
+    for (int i = 0; i < n; i++)
+        if (!m.layers[(size_t)i]->chain_parts(parts[(size_t)i])) return false;
+    m.chain_sync = std::make_unique<et::DeviceBuffer<int>>((size_t)n * ET_CHAIN_SYNC_WORDS);
+    m.chain_desc.assign((size_t)n, et_chain_desc{});
+    for (int i = 0; i < n; i++) {
+        const et::ChainParts &p = parts[(size_t)i];
+        et_chain_desc &d = m.chain_desc[(size_t)i];
+        d.o = p.o;
+        d.bias_o = et::f16(p.bias_o);
+        d.Z = et::f16(p.Z);
+        if (i > 0) {  // the residual is LayerNorm2 of the previous layer's sum, formed from the statistics
+                      // this layer's QKV projection left
+            const et::ChainParts &q = parts[(size_t)i - 1];
+            d.resid = q.V2;
+            d.resid_fin = p.fin_in;
+            d.resid_gamma = et::f16(q.gamma2);
+            d.resid_beta = et::f16(q.beta2);
+        }  // i == 0: resid16 = the model's input, set at run time
+        d.V1 = p.V1;
+        d.stats1 = p.stats1;
+        d.up = p.up;
+        d.bias_up = et::f16(p.bias_up);
+        d.gamma1 = et::f16(p.gamma1);
+        d.beta1 = et::f16(p.beta1);
+        d.eps1 = p.eps1;
+        d.fin1 = p.fin1;
+        d.H = et::f16(p.H);
+        d.act = p.act;
+        d.down = p.down;
+        d.bias_down = et::f16(p.bias_down);
+        d.V2 = p.V2;
+        d.stats2 = p.stats2;
+        if (i + 1 < n) {
+            const et::ChainParts &nx = parts[(size_t)i + 1];
+            d.qkv = nx.qkv;
+            d.bias_qkv = et::f16(nx.bias_qkv);
+            d.gamma2 = et::f16(p.gamma2);
+            d.beta2 = et::f16(p.beta2);
+            d.eps2 = p.eps2;
+            d.fin2 = nx.fin_in;
+            d.QKV = et::f16(nx.QKV);
+        }
+        d.T = m.rows();
+        d.sync = reinterpret_cast<uint32_t *>(m.chain_sync->get()) + (size_t)i * ET_CHAIN_SYNC_WORDS;
+        et_chain_desc probe = d;
+        if (i == 0) probe.resid16 = d.Z;  // any pointer: only the shapes are looked at
+        if (et_encoder_chain_supported(&probe) != 1) return false;
+    }
+    return true;
+}
+
+// Two launches per layer: the attention kernel, and one chain launch for everything up to the next
+// layer's QKV projection.
+void run_layers_chain(et_model_s &m, half *out, half *in, stream_t stream) {
+    const int n = (int)m.layers.size();
+    etChk(et_fill_i32(m.chain_sync->get(), m.chain_sync->size, 0, stream));
+    m.layers[0]->chain_qkv_first(in, stream);
+    et::SplitSum carry;
+    for (int i = 0; i < n; i++) {
+        m.layers[(size_t)i]->chain_attention(stream);
+        et_chain_desc d = m.chain_desc[(size_t)i];
+        if (i == 0) d.resid16 = et::f16(in);
+        int groups2 = 0;
+        etChk(et_encoder_chain_f32(&d, &groups2, stream));
+        carry.v = d.V2;
+        carry.stats = d.stats2;
+        carry.groups = groups2;
+    }
+    // the last layer's sum is normalised by its second LayerNorm
+    et::ChainParts last;
+    (void)m.layers[(size_t)n - 1]->chain_parts(last);
+    carry.gamma = last.gamma2;
+    carry.beta = last.beta2;
+    carry.eps = last.eps2;
+    m.layers[(size_t)n - 1]->finish_split(nullptr, out, carry, stream);
+}
+
+// true when every chain launch of the last forward ran as it must (blocking)
+bool chain_ran_clean(et_model_s &m, std::string &why) {
+    const int n = (int)m.layers.size();
+    for (int i = 0; i < n; i++) {
+        int gave_up = 0, misplaced = 0;
+        etChk(et_encoder_chain_status(m.chain_desc[(size_t)i].sync, &gave_up, &misplaced));
+        if (gave_up || misplaced) {
+            why = "layer " + std::to_string(i) + ": " + std::to_string(gave_up) + " workgroups gave up at a barrier, " +
+                  std::to_string(misplaced) + " ran on another XCD than the rest of their group";
+            return false;
+        }
+    }
+    return true;
+}
+
 void run_layers_split(et_model_s &m, half *out, half *in, stream_t stream) {
+    if (m.chain) return run_layers_chain(m, out, in, stream);
     const int n = (int)m.layers.size();
     // the first layer adds the binary16 input as its residual: no widened copy
     et::SplitSum carry;
@@ -375,10 +484,12 @@ int et_model_finalize(et_model m) {
             for (auto &b : m->pp32) b = std::make_unique<et::DeviceBuffer<float>>(act_elems);
             for (auto &l : m->layers) l->enable_mixed();
             // mixed == 1: the engine folds SkipLayerNorm into the projections where every layer can
-            m->split = m->desc.mixed == 1 && !m->layers.empty();
+            m->split = (m->desc.mixed == 1 || m->desc.mixed == 3) && !m->layers.empty();
             for (auto &l : m->layers) m->split = m->split && l->split_ok();
-            if (m->split)
+            if (m->split) {
                 for (auto &l : m->layers) l->enable_split();
+                m->chain = m->desc.mixed == 3 && build_chain(*m);
+            }
         }
         etChk(et_stream_create(&m->own_stream));
         apply_attention_state(*m);
@@ -425,6 +536,16 @@ int et_model_forward(et_model m, et_f16 *out, const et_f16 *in, et_stream stream
             m->drop_graph();
             run_layers(*m, m->warm->get(), i, s);
             etChk(et_stream_sync(s));
+            std::string why;
+            if (m->chain && !chain_ran_clean(*m, why)) {
+                // a workgroup gave up at a barrier or ran on another XCD than its id says: separate
+                // launches from here on (the eager pass is repeated so that its result is valid too)
+                m->chain = false;
+                et_set_last_error(("et_model_forward: the one-launch chain did not run as it must (" + why +
+                                   "); using separate launches").c_str());
+                run_layers(*m, m->warm->get(), i, s);
+                etChk(et_stream_sync(s));
+            }
             etChk(et_graph_begin_capture(s));
             try {
                 run_layers(*m, o, i, s);
@@ -447,6 +568,14 @@ int et_model_sync(et_model m) {
     return guarded([&]() -> int {
         et::require(m != nullptr, "et_model_sync: NULL handle");
         if (m->own_stream) etChk(et_stream_sync(m->own_stream));
+        return ET_OK;
+    });
+}
+
+int et_model_launches_per_layer(et_model m, int *launches) {
+    return guarded([&]() -> int {
+        et::require(m != nullptr && launches != nullptr, "et_model_launches_per_layer: NULL argument");
+        *launches = !m->finalized ? 0 : m->chain ? 2 : m->split ? 5 : 7;
         return ET_OK;
     });
 }

@@ -85,7 +85,8 @@ TOL_MIXED_VS_ORACLE = 6e-3   # against the oracle rounding where the engine does
 TOL_F16_DEEP = 5e-2          # all-fp16 storage over 12+ layers: two realisations of the storage noise
 
 
-@pytest.mark.parametrize("seed0,xseed,mode", [(100, 4, 1), (300, 307, 1), (500, 507, 1), (100, 4, 2)])
+@pytest.mark.parametrize("seed0,xseed,mode", [(100, 4, 1), (300, 307, 1), (500, 507, 1), (100, 4, 2), (100, 4, 3),
+                                               (300, 307, 3)])
 def test_bert_base_12_layers_batch8_tile80_attention_aware_mixed(et, seed0, xseed, mode):
     """The headline configuration in the engine's mixed-precision mode: 12 layers, B8 S128, 80 %
     tile sparsity, 25 % of the V rows (and the matching O columns) dead in head-aligned groups."""
@@ -117,6 +118,24 @@ def test_bert_base_12_layers_all_fp16_storage(et):
         print(f"{depth}-layer B8 S128 fp16 storage: vs fp16-storage oracle {err:.3e}")
         assert err <= tol
         assert np.array_equal(got[0], got[1])
+
+
+def test_chain_launches_equal_separate_launches(et):
+    """mixed = 3 runs everything between two attention kernels as one launch whose workgroups meet at
+    counters in their XCD's L2 instead of at kernel boundaries: the same arithmetic on the same packs
+    as mixed = 1, so the results agree bit for bit, replay after replay; and the model reports that the
+    chain really ran (two launches per layer)."""
+    H, S, B = 768, 128, 8
+    layers = headline_layers(700)
+    x = Hn.randn((B * S, H), 707)
+    m5 = Hn.build_model(et, layers, S, B, mixed=1)
+    m2 = Hn.build_model(et, layers, S, B, mixed=3)
+    a = run_model(et, m5, x, reps=2)
+    b = run_model(et, m2, x, reps=4)
+    assert m5.launches_per_layer() == 5
+    assert m2.launches_per_layer() == 2, f"the chain was not taken: {et.lib().et_last_error().decode()}"
+    for r in b:
+        assert np.array_equal(r, a[0])
 
 
 def test_bench_workload_mixed_precision(et):
