@@ -593,7 +593,10 @@ int et_mha_vo_f16(const et_f16 *Q, const et_f16 *K, int ldq, int ldk,
  * sums softmax_h * VO_h in fp32, adds sum_h bias_vo[h][n] (the probabilities of
  * a row add up to one; bias_vo [nh][N] or NULL) and bias_o, and writes every
  * element of out once: no P buffer, no atomics, out need not be cleared.  The
- * other arguments as et_mha_vo_f16. */
+ * other arguments as et_mha_vo_f16.  With lens (or a causal strip) the keys
+ * past a sequence's length, up to the next multiple of 8, are still read and
+ * weighted with probabilities that are exactly zero: the rows of X behind them
+ * (and so of VOt) must hold finite values. */
 int et_linear_vo_keys_f16(const et_f16 *Wt, const et_f16 *X, et_f16 *VOt, int B,
                           int S, int H, int N, int nh, et_stream stream);
 int et_mha_vo_otf_f16(const et_f16 *Q, const et_f16 *K, int ldq, int ldk,

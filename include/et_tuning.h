@@ -31,6 +31,17 @@ int et_bsr16_pack_create_geom(const int32_t *row_ptr, const int32_t *col_idx,
                               int flags, int mt, int ngroups, int nwave, int cap,
                               et_bsr_pack *pack);
 
+/* Machine probes (scpaper-2021_amd/kernel_bench.py --set machine): an empty launch of nwg
+ * workgroups (what a kernel boundary costs inside a graph), and a launch in which every
+ * workgroup requests vec_per_thread (4, 8, 16, 32) 16-byte vectors per thread, all before it
+ * uses the first, from a region of src of its own (shared = 0) or from the region of the
+ * first workgroup of its XCD (shared != 0: lines that hit that XCD's L2 after the first
+ * touch): how fast one compute unit takes bytes in.  sink: nwg words.  No reference
+ * counterpart. */
+int et_probe_empty(int nwg, int threads, et_stream stream);
+int et_probe_read(const void *src, size_t src_bytes, int nwg, int threads,
+                  int vec_per_thread, int shared, uint32_t *sink, et_stream stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -81,6 +81,8 @@ _SIGNATURES = {
     "et_encoder_chain_supported": (_vp,),
     "et_encoder_chain_f32": (_vp, C.POINTER(_i), _vp),
     "et_encoder_chain_status": (_vp, C.POINTER(_i), C.POINTER(_i)),
+    "et_probe_empty": (_i, _i, _vp),
+    "et_probe_read": (_vp, _sz, _i, _i, _i, _i, _vp, _vp),
     "et_linear_bsr16_f16_geom": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp),
     "et_skipln_linear_bsr16_f16": (_vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_linear_bsr16_fused_ln_supported": (_i, _i, _i),

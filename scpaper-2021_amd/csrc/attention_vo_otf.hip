@@ -410,7 +410,7 @@ __global__ __launch_bounds__(64 * NW) void mha_vo_otf_kernel(const MhaVoArgs a) 
                 if (first_head && wave == 0 && g == 0) {
                     int at = t * 16 + r16;
                     asm volatile("" : "+v"(at));  // formed here: hoisted out of the loop, the address is a register spilled
-                    alive[at] = l > 0.0f;
+                    alive[at] = l > 0.0f;  // taken from one head: mask and lens are shared by all heads of a query
                 }
 #pragma unroll
                 for (int d = 0; d < DB; d++) {

@@ -142,11 +142,17 @@ __global__ __launch_bounds__(kSNW * 64) void bsr16_stream_kernel(const BsrStream
     const int ahead = a.nbuf - 1;  // chunks in flight beyond the one being multiplied
     for (int c = 0; c < ahead && c < a.nchunk; c++) issue(c, c);
 
-    // tables of this wave and the bias of its rows: requested once, behind the first chunks
+    // tables of this wave (lane L holds those of chunk 64 * block + L; reloaded every 64 chunks) and the
+    // bias of its rows: requested behind the first chunks
     const int32_t *ws = a.wseg + ((size_t)group * a.nchunk * kSNW + wave) * 8;
-    const int lc = min(lane, a.nchunk - 1);
-    const int4 seg_lo = *reinterpret_cast<const int4 *>(ws + (size_t)lc * kSNW * 8);
-    const int seg_n3 = ws[(size_t)lc * kSNW * 8 + 4];
+    auto load_seg = [&](int block, int4 &lo, int &n3) {
+        const int lc = min(block * 64 + lane, a.nchunk - 1);
+        lo = *reinterpret_cast<const int4 *>(ws + (size_t)lc * kSNW * 8);
+        n3 = ws[(size_t)lc * kSNW * 8 + 4];
+    };
+    int4 seg_lo;
+    int seg_n3;
+    load_seg(0, seg_lo, seg_n3);
     h4 bias_v[kSMaxRpw];
 #pragma unroll
     for (int i = 0; i < kSMaxRpw; i++) {
@@ -158,7 +164,7 @@ __global__ __launch_bounds__(kSNW * 64) void bsr16_stream_kernel(const BsrStream
     // also wait for every chunk in flight: take them now, behind the chunks issued so far, so that
     // the waits below see direct-to-LDS loads only
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    const int seg_base_l = seg_lo.x, seg_n0_l = seg_lo.y, seg_n1_l = seg_lo.z, seg_n2_l = seg_lo.w;
+    int seg_base_l = seg_lo.x, seg_n0_l = seg_lo.y, seg_n1_l = seg_lo.z, seg_n2_l = seg_lo.w;
 
     f4 acc[kSMaxRpw][MT];
 #pragma unroll
@@ -176,12 +182,19 @@ __global__ __launch_bounds__(kSNW * 64) void bsr16_stream_kernel(const BsrStream
         wait_vmcnt(max(later, 0) * loads_per_chunk);
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // ... for every wave; buffer b-1 is free
         if (c + ahead < a.nchunk) issue(c + ahead, b == 0 ? a.nbuf - 1 : b - 1);
+        if (c && (c & 63) == 0) {
+            // the next 64 chunks' tables (an ordinary load: it waits for everything in flight, once per 64 chunks)
+            load_seg(c >> 6, seg_lo, seg_n3);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            seg_base_l = seg_lo.x, seg_n0_l = seg_lo.y, seg_n1_l = seg_lo.z, seg_n2_l = seg_lo.w;
+        }
         const _Float16 *xb = xbuf(b) + r16 * KC;
         const _Float16 *wb = wbuf(b) + a_off;
         const int32_t *qb = qbuf(b) + sel;
-        int slot = __builtin_amdgcn_readlane(seg_base_l, c);
-        const int seg_n[4] = {__builtin_amdgcn_readlane(seg_n0_l, c), __builtin_amdgcn_readlane(seg_n1_l, c),
-                              __builtin_amdgcn_readlane(seg_n2_l, c), __builtin_amdgcn_readlane(seg_n3, c)};
+        const int cl = c & 63;  // lane that holds this chunk's tables
+        int slot = __builtin_amdgcn_readlane(seg_base_l, cl);
+        const int seg_n[4] = {__builtin_amdgcn_readlane(seg_n0_l, cl), __builtin_amdgcn_readlane(seg_n1_l, cl),
+                              __builtin_amdgcn_readlane(seg_n2_l, cl), __builtin_amdgcn_readlane(seg_n3, cl)};
         // the wave's slots of this chunk are consecutive; the weights and the column of the next slot
         // are read while the current one is multiplied (one slot past the end is read and dropped)
         h8 w_next = *reinterpret_cast<const h8 *>(wb + slot * 512);

@@ -629,6 +629,8 @@ int et_linear_colpruned_static_f16(const et_f16 *cols, const int32_t *col_id, in
                "et_linear_colpruned_static_f16: T x nnz_col = %d x %d needs %zu bytes of scratch, the built-in "
                "buffer holds %zu; use et_linear_colpruned_ws_f16 with a workspace of your own",
                T, nnz_col, need, kStaticScratchBytes);
+    if (need == 0)  // nothing to gather, so no scratch and no address lookup: bias and activation alone
+        return et_linear_colpruned_f16(cols, col_id, nnz_col, bias, X, Y, T, in, out, act, stream);
     void *ws = nullptr;
     int s = static_scratch(&ws);
     if (s != ET_OK) return s;

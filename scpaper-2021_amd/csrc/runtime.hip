@@ -113,7 +113,9 @@ int et_device_info(char *name, int cap, int *num_cu, int *lds_bytes) {
 namespace {
 constexpr size_t kSlabBytes = 64u << 20;
 constexpr size_t kSlabAlign = 4096;
+struct PrivateScope;
 struct Slab {
+    PrivateScope *owner = nullptr;  // the open private scope whose list holds this slab (nullptr: g_slabs, or none)
     char *base = nullptr;
     size_t used = 0;
     size_t live = 0;      // buffers cut from this slab and not yet freed
@@ -148,6 +150,7 @@ int et_pool_private_end(void) {
         std::lock_guard<std::mutex> lk(g_pool_mu);
         for (Slab *slab : t_scope->slabs) {  // nothing cuts from them any more: each goes when its last buffer does
             slab->current = false;
+            slab->owner = nullptr;
             if (slab->live == 0) {
                 release.push_back(slab->base);
                 delete slab;
@@ -156,8 +159,12 @@ int et_pool_private_end(void) {
     }
     delete t_scope;
     t_scope = nullptr;
-    for (void *p : release) ET_HIP(hipFree(p));
-    return ET_OK;
+    int status = ET_OK;  // every slab is released; the first failure is what the caller hears of
+    for (void *p : release) {
+        const int s = check_hip(hipFree(p), "hipFree");
+        if (status == ET_OK) status = s;
+    }
+    return status;
 }
 
 int et_malloc(void **ptr, size_t bytes) {
@@ -179,6 +186,7 @@ int et_malloc(void **ptr, size_t bytes) {
                 Slab *fresh = new Slab;
                 fresh->base = static_cast<char *>(base);
                 fresh->lead = fresh->used = (t_scope && slabs.empty()) ? t_scope->lead : 0;
+                fresh->owner = t_scope;
                 if (!slabs.empty()) slabs.back()->current = false;
                 slabs.push_back(fresh);
             }
@@ -222,9 +230,10 @@ int et_free(void *ptr) {
                 release = slab->base;
                 auto at = std::find(g_slabs.begin(), g_slabs.end(), slab);
                 if (at != g_slabs.end()) g_slabs.erase(at);
-                if (t_scope) {
-                    auto mine = std::find(t_scope->slabs.begin(), t_scope->slabs.end(), slab);
-                    if (mine != t_scope->slabs.end()) t_scope->slabs.erase(mine);
+                if (slab->owner) {  // a scope that is still open, on this thread or another: its list lets go of the slab
+                    auto &theirs = slab->owner->slabs;
+                    auto mine = std::find(theirs.begin(), theirs.end(), slab);
+                    if (mine != theirs.end()) theirs.erase(mine);
                 }
                 delete slab;
             }

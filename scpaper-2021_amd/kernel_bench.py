@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Per-kernel throughput against the roofline that bounds it, through the C ABI.
 
-    python scpaper-2021_amd/kernel_bench.py [--set configs|scale|all] [--json FILE]
+    python scpaper-2021_amd/kernel_bench.py [--set configs|scale|vo|mha|plan|machine|all] [--json FILE]
 
 `configs` are the shapes of the benchmark configurations (attention block at batch
 1/4/16, the tile/row/column-pruned Linears at 2048 token rows, the BERT-large-shaped
@@ -128,16 +128,80 @@ class Bench:
         self.et.check(fn(n, sparsity, seed, out.ctypes.data, C.byref(count)))
         return out[:count.value].copy()
 
-    def bsr(self, T, n_in, n_out, sparsity, launches):
-        et = self.et
+    def bsr(self, T, n_in, n_out, sparsity, launches, entry="class"):
+        """Tile-sparse Linear.  entry = "class": through the entry point Linear<tile_mat> picks for this shape
+        (include/et/Linear.h: the dense image above half of the tiles, the streaming plan for wide inputs at many
+        rows, a pack up to 4096 rows, else the plain call); "plain" / "plan" / "pack" force one."""
+        et, lib = self.et, self.lib
         row_ptr, col, ntile = self.tile_pattern(n_out, n_in, sparsity, 5)
         d_rp, d_col = self.dev(row_ptr), self.dev(col)
         tiles = self.dev(self.rnd((max(ntile, 1), 256), 0.02))
         bias = self.dev(np.zeros(n_out, np.float16))
         x, y = self.dev(self.rnd((T, n_in))), self.empty((T, n_out))
-        us = self.time_us(lambda: et.linear_bsr16(d_rp, d_col, tiles, bias, x, y, T, n_in, n_out, 0, self.stream),
-                          launches)
-        self.record("linear_bsr16", f"T{T} in{n_in} out{n_out} sparsity {sparsity}", us, 2 * 256 * ntile * T, "mfma")
+        if entry == "class":
+            kept = ntile * 256.0 / (n_in * n_out)
+            if kept > 0.5:
+                entry = "dense image"
+            elif n_in >= 128 and (n_in > 5112 or (n_in >= 3072 and T >= 4096)):
+                entry = "plan"
+            elif T <= 4096 and n_in % 128 == 0 and n_in <= 4096:
+                entry = "pack"
+            else:
+                entry = "plain"
+        handle, destroy = C.c_void_p(), None
+        if entry == "plan":
+            et.check(lib.et_bsr16_plan_create(d_rp.ptr, d_col.ptr, tiles.ptr, T, n_in, n_out, 0, 0, 0, C.byref(handle)))
+            destroy = lib.et_bsr16_plan_destroy
+            fn = lambda: et.check(lib.et_linear_bsr16_planned_f16(handle, bias.ptr, x.ptr, y.ptr, None, T, 0, self.stream))
+        elif entry == "pack":
+            st = lib.et_bsr16_pack_create(d_rp.ptr, d_col.ptr, tiles.ptr, T, n_in, n_out, 0, 0, C.byref(handle))
+            if st == et.ET_ERR_UNSUPPORTED:
+                entry = "plain"
+            else:
+                et.check(st)
+                destroy = lib.et_bsr16_pack_destroy
+                fn = lambda: et.check(lib.et_linear_bsr16_packed_f16(handle, bias.ptr, x.ptr, y.ptr, None, T, 0, self.stream))
+        elif entry == "dense image":
+            w = self.empty((n_out, n_in))
+            et.check(lib.et_bsr16_to_dense_f16(d_rp.ptr, d_col.ptr, tiles.ptr, w.ptr, n_in, n_out, self.stream))
+            fn = lambda: et.check(lib.et_linear_dense_f16(w.ptr, bias.ptr, x.ptr, y.ptr, T, n_in, n_out, 0, self.stream))
+        if entry == "plain":
+            fn = lambda: et.linear_bsr16(d_rp, d_col, tiles, bias, x, y, T, n_in, n_out, 0, self.stream)
+        us = self.time_us(fn, launches)
+        et.check(lib.et_stream_sync(self.stream))
+        if destroy:
+            et.check(destroy(handle))
+        self.record(f"linear_bsr16 ({entry})", f"T{T} in{n_in} out{n_out} sparsity {sparsity}", us, 2 * 256 * ntile * T, "mfma")
+
+    def machine(self):
+        """What a kernel boundary costs and how fast a compute unit takes bytes in (et_probe_*): the two figures
+        that bound a launch of a few hundred kilobytes per compute unit."""
+        et, lib = self.et, self.lib
+        ncu = et.device_info()["num_cu"]
+        us = self.time_us(lambda: et.check(lib.et_probe_empty(ncu, 256, self.stream)), 200)
+        print(f"empty launch of {ncu} workgroups inside a graph: {us:.2f} us per launch (a kernel boundary)", flush=True)
+        self.rows.append({"kernel": "probe_empty", "shape": f"{ncu} workgroups", "us": round(us, 2)})
+        src_bytes = 1 << 30  # above the 256 MB Infinity Cache
+        src = et.DeviceBuffer(src_bytes)
+        sink = et.DeviceBuffer(4 * 4096)
+        for threads, vec in ((256, 16), (512, 16), (768, 16), (768, 32), (1024, 16)):
+            per_wg = threads * vec * 16
+            for shared, what in ((1, "lines shared by the workgroups of an XCD (L2 hits after the first touch)"),
+                                 (0, "lines of its own (first touch: Infinity Cache or HBM)")):
+                # own lines: a different part of the gigabyte for every launch of the graph, so nothing is warm
+                calls = {"n": 0}
+
+                def fn():
+                    off = 0 if shared else (calls["n"] % 8) * ncu * per_wg
+                    calls["n"] += 1
+                    et.check(lib.et_probe_read(src.ptr + off, src_bytes - off, ncu, threads, vec, shared, sink.ptr, self.stream))
+                us = self.time_us(fn, 40)
+                gbs = per_wg / us / 1e3
+                print(f"read probe: {ncu} workgroups x {threads} threads x {vec} x 16 B = {per_wg // 1024} KB per compute unit, {what}: "
+                      f"{us:.2f} us per launch, {gbs:.0f} GB/s per compute unit (launch included), {gbs * ncu / 1e3:.1f} TB/s over the chip",
+                      flush=True)
+                self.rows.append({"kernel": "probe_read", "shape": f"{per_wg // 1024} KB/CU {threads} thr shared={shared}",
+                                  "us": round(us, 2), "gb_s_per_cu": round(gbs, 1)})
 
     def rowcol(self, T, n_in, n_out, sparsity, launches):
         et, lib = self.et, self.lib
@@ -354,7 +418,7 @@ def run_scale(b: Bench):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--set", choices=("configs", "scale", "vo", "mha", "all"), default="all")
+    ap.add_argument("--set", choices=("configs", "scale", "vo", "mha", "plan", "machine", "all"), default="all")
     ap.add_argument("--json", default=None, help="also write the rows as JSON to this file")
     args = ap.parse_args()
     b = Bench()
@@ -378,6 +442,17 @@ def main():
         for B, N in ((1, 768), (4, 384), (8, 768), (16, 768)):
             b.mha_vo(B, 128, 12, 64, N, 20)
         b.mha_vo(4, 512, 16, 64, 1024, 10)
+    if args.set == "plan":
+        print("# tile-sparse Linear: the plain call, the streaming plan and (where it applies) a pack, at the same shapes")
+        for T, n_in, n_out in ((1024, 3072, 768), (2048, 3072, 768), (4096, 3072, 768), (16384, 3072, 768), (16384, 768, 3072),
+                               (2048, 6144, 768)):
+            for entry in ("plain", "plan", "pack"):
+                if entry == "pack" and (T > 4096 or n_in > 4096):
+                    continue
+                b.bsr(T, n_in, n_out, 0.8, 10 if T >= 16384 else 30, entry=entry)
+    if args.set == "machine":
+        print("# machine probes")
+        b.machine()
     if args.set in ("scale", "all"):
         print("# shapes where launch latency no longer matters")
         run_scale(b)

@@ -296,6 +296,8 @@ PLANNED_CASES = [
     (512, 3072, 768, 0.8, 0, (2, 512, 3)),
     (512, 3072, 768, 0.8, 0, (8, 128, 24)),
     (256, 1024, 1024, 0.95, 0, (1, 512, 20)),  # block-rows without tiles in most chunks
+    (64, 8320, 64, 0.5, 0, (1, 128, 4)),       # 65 chunks: the per-chunk tables are reloaded after 64
+    (32, 16512, 32, 0.8, 1, (1, 128, 2)),      # 129 chunks
 ]
 
 

@@ -49,6 +49,45 @@ def test_static_scratch_linear_equals_workspace_form_twice(et):
     assert Hn.max_abs(got, want) <= 4e-3
 
 
+def test_static_scratch_linear_allocates_nothing(et):
+    """Recorded into a HIP graph (stream capture refuses any allocation, and an allocating call would fail the
+    capture) and replayed three times with other work between the replays: every replay gives the eager result;
+    and the device's free memory is the same before and after eager calls."""
+    import ctypes as C
+    lib = et.lib()
+    T, inp, out, act = 256, 768, 384, 1
+    col_id = F.gen_col_ids(inp, 0.5, seed=95)
+    nnz = len(col_id)
+    d_cols, d_id, d_b = up(et, Hn.randn((out, nnz), 96, 0.02)), up(et, col_id), up(et, Hn.randn((out,), 97, 0.1))
+    d_x = up(et, Hn.randn((T, inp), 98))
+    d_eager, d_graph = et.DeviceBuffer.empty((T, out), np.float16), et.DeviceBuffer.empty((T, out), np.float16)
+    stream = C.c_void_p()
+    et.check(lib.et_stream_create(C.byref(stream)))
+    args = (d_cols.ptr, d_id.ptr, nnz, d_b.ptr, d_x.ptr)
+    hip = C.CDLL("libamdhip64.so")
+    free0, free1, total = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    et.check(lib.et_linear_colpruned_static_f16(*args, d_eager.ptr, T, inp, out, act, stream))  # first use: address lookup
+    et.check(lib.et_stream_sync(stream))
+    assert hip.hipMemGetInfo(C.byref(free0), C.byref(total)) == 0
+    for _ in range(3):
+        et.check(lib.et_linear_colpruned_static_f16(*args, d_eager.ptr, T, inp, out, act, stream))
+    et.check(lib.et_stream_sync(stream))
+    assert hip.hipMemGetInfo(C.byref(free1), C.byref(total)) == 0
+    assert free1.value == free0.value
+    want = d_eager.numpy()
+    et.check(lib.et_graph_begin_capture(stream))
+    et.check(lib.et_linear_colpruned_static_f16(*args, d_graph.ptr, T, inp, out, act, stream))
+    graph = C.c_void_p()
+    et.check(lib.et_graph_end_capture(stream, C.byref(graph)))
+    for rep in range(3):
+        et.check(lib.et_fill_f16(d_graph.ptr, T * out, 0x7E00, stream))  # the program's own work between replays
+        et.check(lib.et_graph_launch(graph, stream))
+        et.check(lib.et_stream_sync(stream))
+        assert np.array_equal(d_graph.numpy(), want), f"replay {rep}"
+    et.check(lib.et_graph_destroy(graph))
+    et.check(lib.et_stream_destroy(stream))
+
+
 def test_static_scratch_linear_rejects_what_does_not_fit(et):
     d = et.DeviceBuffer.empty((16,), np.float16)
     # 4096 x 2048 x 2 bytes = 16 MiB > 8 MiB: refused before anything is launched
