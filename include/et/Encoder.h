@@ -4,11 +4,21 @@
 //   f  = act(linear1(y1))       out = SkipLN2(linear2(f), y1)
 // The activation is applied inside linear1's kernel epilogue (on the fp32
 // accumulator) rather than as a separate pass over [rows x dimFF]; act<>() is
-// still provided for callers that use it stand-alone.  forward() issues six or
-// seven launches on one stream, never blocks the host and writes nothing to stdout.
+// still provided for callers that use it stand-alone.  forward() issues six to
+// eight launches on one stream, never blocks the host and writes nothing to stdout.
+//
+// Precision of forward(half *out, half *src), the reference's signature: binary16 where the
+// layer meets its caller and where a value is a matrix-core operand, binary32 for the residual
+// stream inside the layer (both sublayer sums and both normalisations).  Twelve BERT-base layers
+// called one after the other stay within 1e-2 of the binary32 mathematics that way (one binary16
+// rounding per layer boundary, of values up to 8); with the residual stream rounded to binary16
+// after every sublayer, as the reference stores it, they drift to 2e-2 .. 5e-2.  forward_f16() is that all-binary16 form; the environment variable
+// ET_F16_RESIDUAL=1 makes forward() run it.
 #pragma once
+#include <cstdlib>
 #include <memory>
 #include <type_traits>
+#include <utility>
 
 #include "Attention.h"
 #include "Fused_attention.h"
@@ -103,7 +113,35 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
     attn_t &attention() { return *attn; }
     int token_rows() const { return rows; }
 
+    // The reference's entry (Encoder/Encoder.h:81-96).  With the binary32 buffers in place
+    // (prepare_wide_residual(), which the Encoder and Encoder_fuse constructors call) the residual
+    // stream stays binary32 between src and out; without them this is forward_f16().
     void forward(half *out, half *src, stream_t stream = nullptr) {
+        if (!wide) return forward_f16(out, src, stream);
+        if (wide_split) {  // five launches and the closing normalisation
+            const SplitSum s = forward_split(nullptr, nullptr, src, stream);
+            return finish_split(nullptr, out, s, stream);
+        }
+        etChk(et_f16_to_f32(src32->get(), f16(src), (std::size_t)rows * model->emdim, stream));
+        forward_mixed(nullptr, out, src32->get(), src, stream);
+    }
+    // Allocates what forward() needs to keep the residual stream binary32.  Not to be called while a
+    // stream is being captured (it allocates, and tile-sparse layers build their packs).
+    void prepare_wide_residual() {
+        if (wide) return;
+        if (split_ok()) {
+            enable_split();
+            wide_split = true;
+        } else {
+            enable_mixed();
+            src32 = std::make_unique<DeviceBuffer<float>>((std::size_t)rows * model->emdim);
+        }
+        wide = true;
+    }
+    bool wide_residual() const { return wide; }
+
+    // Every activation stored as binary16, the reference's own arithmetic.
+    void forward_f16(half *out, half *src, stream_t stream = nullptr) {
         attn->forward(temp_attn.get(), src, src, src, stream);
         bool fused_ln1 = false;
         if constexpr (std::is_same_v<linear1_t, Linear<tile_mat>>) {
@@ -256,7 +294,16 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
                                        model->emdim, s.eps, stream));
     }
 
+  protected:
+    // what the drop-in classes do at the end of their constructors
+    void prepare_default_precision() {
+        const char *e = std::getenv("ET_F16_RESIDUAL");
+        if (!(e && e[0] == '1')) prepare_wide_residual();
+    }
+
   private:
+    bool wide = false, wide_split = false;
+    std::unique_ptr<DeviceBuffer<float>> src32;
     std::unique_ptr<DeviceBuffer<float>> stats1, stats2, fin_in, fin1;
     template <typename A, typename = void> struct attn_has_split : std::false_type {};
     template <typename A>
@@ -293,7 +340,9 @@ class Encoder : public et::EncoderLayer<Attention<typename _config::attn_config>
                                   Linear<typename _config::linear2_config>, typename _config::act_t>;
 
   public:
-    using base::base;
+    template <typename... Args> explicit Encoder(Args &&...args) : base(std::forward<Args>(args)...) {
+        this->prepare_default_precision();
+    }
 };
 
 // Encoder with the pre-computed-VO attention (Encoder/Encoder.h:99-139): tile-sparse
@@ -304,5 +353,7 @@ class Encoder_fuse
     using base = et::EncoderLayer<FusedAttention<_attn_config>, Linear<tile_mat>, Linear<tile_mat>, GELU_OP>;
 
   public:
-    using base::base;
+    template <typename... Args> explicit Encoder_fuse(Args &&...args) : base(std::forward<Args>(args)...) {
+        this->prepare_default_precision();
+    }
 };

@@ -215,6 +215,7 @@ class LayerConfig:
     store: object = None
     resid: object = "same"  # storage of the residual stream; "same" = as ``store``
     fused_act: bool = True  # activation applied on the fp32 accumulator of linear1
+    boundary: object = None  # storage of a layer's result where it is handed to the next layer (None: as the residual stream)
     extras: dict = field(default_factory=dict)
 
 
@@ -252,5 +253,5 @@ def encoder_layer(x, P: LayerParams, cfg: LayerConfig):
 def encoder_stack(x, layers, cfg: LayerConfig):
     """Layer i feeds layer i+1 (example/main.cu:175-177)."""
     for P in layers:
-        x = encoder_layer(x, P, cfg)
+        x = _store(encoder_layer(x, P, cfg), cfg.boundary)
     return x

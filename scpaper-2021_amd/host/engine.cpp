@@ -33,7 +33,7 @@ struct ILayer {
 template <typename EncoderT> struct LayerOf final : ILayer {
     std::unique_ptr<EncoderT> enc;
     explicit LayerOf(std::unique_ptr<EncoderT> e) : enc(std::move(e)) {}
-    void forward(half *out, half *src, stream_t stream) override { enc->forward(out, src, stream); }
+    void forward(half *out, half *src, stream_t stream) override { enc->forward_f16(out, src, stream); }
     void enable_mixed() override { enc->enable_mixed(); }
     void forward_mixed(float *out32, half *out16, const float *src32, half *src16, stream_t stream) override {
         enc->forward_mixed(out32, out16, src32, src16, stream);
@@ -146,7 +146,9 @@ template <> std::unique_ptr<Linear<base_mat>> make_linear<base_mat>(const HostMa
 
 template <typename MAT, typename attn_cfg, typename ACT>
 std::unique_ptr<ILayer> build_layer(et_model_s &m, const HostLayer &h) {
-    using enc_t = Encoder<Encoder_config<attn_cfg, MAT, MAT, ACT>>;
+    // the layer body of Encoder<Encoder_config<attn_cfg, MAT, MAT, ACT>> without that class's own choice of
+    // precision: the model's `mixed` field decides here which buffers a layer gets
+    using enc_t = et::EncoderLayer<Attention<attn_cfg>, Linear<MAT>, Linear<MAT>, ACT>;
     const int rows = m.rows();
     auto lqkv = make_linear<MAT>(h.w[ET_W_QKV], m.dims(ET_W_QKV), rows);
     auto lo = make_linear<MAT>(h.w[ET_W_O], m.dims(ET_W_O), rows);

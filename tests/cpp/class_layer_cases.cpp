@@ -380,9 +380,12 @@ static int run_encoder_fuse(const std::string &dir) {
     };
     auto enc = build();
     et::DeviceBuffer<half> X(load_half(dir + "/input.npy")), OUT((std::size_t)rows * H);
-    enc->forward(OUT.get(), X.get());
+    enc->forward_f16(OUT.get(), X.get());  // every activation binary16, as the reference stores them
     etChk(et_device_sync());
     save_half(dir + "/out.npy", OUT, (std::size_t)rows, (std::size_t)H);
+    enc->forward(OUT.get(), X.get());  // the drop-in entry: binary32 residual stream inside the layer
+    etChk(et_device_sync());
+    save_half(dir + "/out_forward.npy", OUT, (std::size_t)rows, (std::size_t)H);
     // mixed precision: binary32 residual stream around the same sublayers
     enc->enable_mixed();
     et::DeviceBuffer<float> X32((std::size_t)rows * H), OUT32((std::size_t)rows * H);

@@ -60,7 +60,7 @@ class BsrWeight:
         # write through these arrays, and the digest taken here is compared again at every
         # hand-over to the library (check_tile_pattern), so a change made behind numpy's back
         # cannot go unseen.
-        self.row_ptr, self.col_idx = (isolated(a) for a in self._pattern())
+        self.row_ptr, self.col_idx = self._generate_checked()
         bc = inp // 16
         assert len(self.col_idx) == 0 or (self.col_idx.min() >= 0 and self.col_idx.max() < bc), \
             "pattern generator produced a column tile outside the matrix"
@@ -71,6 +71,26 @@ class BsrWeight:
         self.tiles = randn((n, 256), seed + 1, std)
         self.bias = randn((out,), seed + 2, bias_std) if bias_std else np.zeros(out, np.float16)
         self.dense = F.bsr16_to_dense(self.row_ptr, self.col_idx, self.tiles, inp)  # fp16 values
+
+    def _generate_checked(self):
+        """The generator is deterministic, so two runs must agree; it works in small heap buffers, which is
+        where this process has seen foreign writes (tests/heap_canary.py).  Two isolated copies that differ
+        are written down and the structure is generated again until two consecutive runs agree."""
+        prev = tuple(isolated(a) for a in self._pattern())
+        for attempt in range(4):
+            cur = tuple(isolated(a) for a in self._pattern())
+            if all(np.array_equal(a, b) for a, b in zip(prev, cur)):
+                return cur
+            from tests import heap_canary
+            for name, a, b in zip(("row_ptr", "col_idx"), prev, cur):
+                bad = np.nonzero(a != b)[0]
+                if len(bad):
+                    heap_canary.note(
+                        f"tile pattern {self._pattern_args}: two generations differ in {name} at {bad[:8].tolist()} "
+                        f"(of {len(a)}): {a[bad[:8]].tolist()} against {b[bad[:8]].tolist()}, generation {attempt} and "
+                        f"{attempt + 1}; generated again")
+            prev = cur
+        raise AssertionError(f"tile pattern {self._pattern_args}: no two consecutive generations agree")
 
     def _pattern(self):
         out, inp, sparsity, seed, dead_rows, dead_cols = self._pattern_args
@@ -257,9 +277,12 @@ def build_model(et, layers, S, B, act=2, lens=None, use_graph=True, causal=False
     return m
 
 
-def oracle_stack(x, layers, B, lens=None, act="gelu", causal=False, eps=1e-5, store=torch.float16, resid="same"):
+def oracle_stack(x, layers, B, lens=None, act="gelu", causal=False, eps=1e-5, store=torch.float16, resid="same",
+                 boundary=None):
     """store=None: the fp32 mathematics; store=float16: fp16 at the engine's storage points;
-    store=float16 with resid=float32: the engine's mixed-precision mode."""
+    store=float16 with resid=float32: the engine's mixed-precision mode; with boundary=float16 as well:
+    the class layer's forward(half*, half*), binary32 inside a layer and binary16 between layers."""
     cfg = L.LayerConfig(nh=layers[0].nh, B=B, act=act, eps=eps, causal=causal,
-                        lens=None if lens is None else torch.as_tensor(np.asarray(lens)), store=store, resid=resid)
+                        lens=None if lens is None else torch.as_tensor(np.asarray(lens)), store=store, resid=resid,
+                        boundary=boundary)
     return L.encoder_stack(f32(x), [w.oracle_params() for w in layers], cfg).numpy()

@@ -58,6 +58,41 @@ def test_example_model_from_npz(tmp_path, TEXT):
     assert Hn.max_abs(np.load(tmp_path / "out.npy"), want) <= 2e-2
 
 
+def test_twelve_class_layers_through_forward(tmp_path):
+    """Twelve BERT-base Encoder<> objects (80 % tile sparsity, ReLU) called one after the other through the
+    reference's own signature, forward(half *out, half *src), as example/main.cu:175-177 does: the result of
+    layer 12 stays within the 2e-2 asked of the fp16 path, measured against the fp32 mathematics, because the
+    residual stream is binary32 inside each layer and binary16 only between layers.  Measured 9.7e-3, and the
+    CPU oracle rounding at the same places is 9.7e-3 from the fp32 mathematics too: values reach 7.8, where one
+    binary16 step is 7.8e-3, and every layer boundary rounds once.  (All-binary16 storage: 1.6e-2 on these
+    weights, 2.3e-2 .. 5e-2 on the GELU headline stack.)"""
+    H, nh, FF, S, B, NL, TEXT = 768, 12, 3072, 128, 2, 12, 256
+    layers = [Hn.LayerWeights(H, nh, FF, 0.8, seed=700 + i) for i in range(NL)]
+    dec = Hn.BsrWeight(TEXT, H, 0.8, seed=790, bias_std=0.02)
+    names = []
+    for i, w in enumerate(layers):
+        pre = f"transformer_encoder.layers.{i}."
+        for nm, bw in (("self_attn.in_proj_", w.qkv), ("self_attn.out_proj.", w.o), ("linear1.", w.l1), ("linear2.", w.l2)):
+            F.save_weight_npz(str(tmp_path / (pre + nm)), bw.dense.astype(np.float32), bw.bias.astype(np.float32))
+            names.append(pre + nm + ".npz")
+        for nm, (g, b) in (("norm1.", (w.g1, w.be1)), ("norm2.", (w.g2, w.be2))):
+            F.save_weight_npz(str(tmp_path / (pre + nm)), g.astype(np.float32), b.astype(np.float32))
+            names.append(pre + nm + ".npz")
+    F.save_weight_npz(str(tmp_path / "decoder."), dec.dense.astype(np.float32), dec.bias.astype(np.float32))
+    names.append("decoder..npz")
+    (tmp_path / "weights.txt").write_text("\n".join(names) + "\n")
+    x = Hn.randn((B * S, H), 791)
+    np.save(tmp_path / "input.npy", x.astype(np.float32))
+    np.save(tmp_path / "meta.npy", np.array([H, H, S, nh, FF, H, NL, B, TEXT], np.int32))
+    run_case("example", tmp_path)
+    got = np.load(tmp_path / "hidden.npy")
+    want32 = Hn.oracle_stack(x, layers, B, act="relu", store=None)
+    want = Hn.oracle_stack(x, layers, B, act="relu", store=torch.float16, resid=torch.float32, boundary=torch.float16)
+    e32, eo = Hn.max_abs(got, want32), Hn.max_abs(got, want)
+    print(f"12 class layers through forward(): vs fp32 forward {e32:.3e}, vs the oracle rounding where the classes do {eo:.3e}")
+    assert e32 <= 2e-2 and eo <= 1.6e-2  # the asked bound; two binary16 steps at |x| < 8 between two realisations
+
+
 def attention_inputs(tmp_path, H, nh, S, B, seed):
     g = Hn.rng(seed)
     rn = lambda *s: (torch.randn(*s, generator=g) * 0.05).numpy().astype(np.float16)
@@ -195,6 +230,8 @@ def test_encoder_fuse_class(tmp_path):
     m32, m16 = np.load(tmp_path / "out_mixed32.npy"), np.load(tmp_path / "out_mixed16.npy")
     assert Hn.max_abs(m32, want32) <= 1e-2
     assert np.array_equal(m16.astype(np.float16), m32.astype(np.float16))
+    # forward(half*, half*) keeps the residual stream binary32 inside the layer: the mixed form's binary16 result
+    assert np.array_equal(np.load(tmp_path / "out_forward.npy"), m16)
 
 
 def test_raw_file_constructors(tmp_path):
