@@ -169,6 +169,7 @@ template <> class Linear<tile_mat> {
     };
     using pack_ptr = std::unique_ptr<et_bsr_pack_s, PackDeleter>;
     pack_ptr pack, pack_producer, pack_consumer;
+    int producer_nwave = 0, consumer_nwave = 0;  // the wave counts the role packs were asked for (0: the builder's choice)
     static constexpr int kPackMaxRows = 4096;
     // ET_PACKED=0 in the environment keeps every Linear<tile_mat> on the unpacked kernels (for comparisons)
     static bool packed_enabled() {
@@ -264,10 +265,12 @@ template <> class Linear<tile_mat> {
     // (nwave: waves per workgroup the pack is built for, 0 = the builder's choice; the one-launch
     // chain of the encoder layer takes packs of 12)
     void prepare_split_producer(int nwave = 0) {
-        if (!pack_producer && !dense && !plan) pack_producer = make_pack(ET_PACK_STATS_PRODUCER, nwave);
+        if (!pack_producer && !dense && !plan && (pack_producer = make_pack(ET_PACK_STATS_PRODUCER, nwave)))
+            producer_nwave = nwave;
     }
     void prepare_split_consumer(int nwave = 0) {
-        if (!pack_consumer && !dense && !plan) pack_consumer = make_pack(ET_PACK_NORM_CONSUMER, nwave);
+        if (!pack_consumer && !dense && !plan && (pack_consumer = make_pack(ET_PACK_NORM_CONSUMER, nwave)))
+            consumer_nwave = nwave;
     }
     // V = input W^T + bias + residual (binary32) and stats[*groups][size][2]; the residual is
     // `resid` itself, or with resid_fin its normalisation by (resid_fin, resid_gamma, resid_beta)
@@ -324,6 +327,25 @@ template <> class Linear<tile_mat> {
                                          weight.row_offset.get(), et::f16(weight.data.get()),
                                          et::f16(bias.get()), et::f16(output), size, (int)in_size,
                                          (int)out_size, act, stream));
+    }
+
+    // `weight` is public, as in the reference, but what forward() multiplies with may be a copy made from it
+    // when the object was built (the dense image, the streaming plan, the packs): a caller that writes into
+    // weight.data, or replaces the structure, calls refresh() afterwards — outside any stream capture, it
+    // allocates and synchronises — and every copy is made again, the role packs of the split normalisation
+    // included.
+    void refresh() {
+        const bool had_producer = (bool)pack_producer, had_consumer = (bool)pack_consumer;
+        etChk(et_device_sync());  // launches still reading the old copies end first
+        dense.reset();
+        dense_out16.reset();
+        plan.reset();
+        pack.reset();
+        pack_producer.reset();
+        pack_consumer.reset();
+        check();
+        if (had_producer) prepare_split_producer(producer_nwave);
+        if (had_consumer) prepare_split_consumer(consumer_nwave);
     }
 
   private:

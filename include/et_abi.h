@@ -503,8 +503,10 @@ int et_fill_rows_bias_f16(et_f16 *C, const et_f16 *bias, int rows, int cols,
  * mask: optional additive [S x S] binary16 matrix shared by all sequences and
  * heads (-inf removes a key).  lens: optional int32[B]; keys >= lens[b] of
  * sequence b get probability exactly 0 (right padding).  Scores, softmax and
- * both contractions are fp32-accumulated.  S % 16 == 0; hd a multiple of 16 (the
- * reference's own constraint, Fused_attention/test/testfused.cu:22), at most 128.
+ * both contractions are fp32-accumulated.  S % 16 == 0; hd a multiple of 8, at
+ * most 256 (the reference's kernels ask for multiples of 16,
+ * Fused_attention/test/testfused.cu:22, while its example model has 800 / 4 =
+ * 200-wide heads, example/main.cu:24-31: both are taken).
  *
  * Replaces Multihead_atttion<OTF_attn_full> (Attention/Attention.cu:80-95,
  * Attention/OTFkernel_full.h:15-125), the single-buffer form

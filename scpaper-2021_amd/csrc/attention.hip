@@ -33,7 +33,7 @@ struct MhaArgs {
     const int32_t *lens;   // [B] or nullptr
     int ldq, ldk, ldv, ldz;
     int S, nh;
-    int hd;             // head size, a multiple of 16; the kernel template is the next of 32, 64, 128
+    int hd;             // head size, a multiple of 8; the kernel template is the next of 32, 64, 128, 256
     int nbh;            // sequences * heads
     float scale_log2e;  // scale * log2(e)
     int causal;
@@ -401,20 +401,27 @@ __global__ __launch_bounds__(64 * NW)
                 // head size or the surviving columns hold zeros) so that the reads go out together;
                 // a read under a branch is waited for on the spot.  Only compact V skips the
                 // products of dead blocks (wave-uniform).
-                h8 vf[DB];
+                // (at most 8 fragments, 32 registers, at a time: 256-wide heads take two rounds)
+                constexpr int DC = DB < 8 ? DB : 8;
 #pragma unroll
-                for (int d = 0; d < DB; d++) {
-                    const int swz = vt_swizzle<HD>(d);  // a constant once d is unrolled
-                    const h8 vr = *reinterpret_cast<const h8 *>(Vt + (d * 16 + r16) * L::ldvt +
-                                                                 ((s2 * 32) ^ (swz & 32)) + ((swz & 16) ? g8x : g8));
-                    vf[d] = (swz & 4) ? h8{vr[4], vr[5], vr[6], vr[7], vr[0], vr[1], vr[2], vr[3]} : vr;
-                }
+                for (int d0 = 0; d0 < DB; d0 += DC) {
+                    h8 vf[DC];
 #pragma unroll
-                for (int d = 0; d < DB; d++) {
-                    if (COMPACT && d * 16 >= vlive) continue;
+                    for (int dd = 0; dd < DC; dd++) {
+                        const int d = d0 + dd;
+                        const int swz = vt_swizzle<HD>(d);  // a constant once d is unrolled
+                        const h8 vr = *reinterpret_cast<const h8 *>(Vt + (d * 16 + r16) * L::ldvt +
+                                                                     ((s2 * 32) ^ (swz & 32)) + ((swz & 16) ? g8x : g8));
+                        vf[dd] = (swz & 4) ? h8{vr[4], vr[5], vr[6], vr[7], vr[0], vr[1], vr[2], vr[3]} : vr;
+                    }
 #pragma unroll
-                    for (int t = 0; t < QT; t++)
-                        o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[d], pf[t], o[t][d], 0, 0, 0);
+                    for (int dd = 0; dd < DC; dd++) {
+                        const int d = d0 + dd;
+                        if (COMPACT && d * 16 >= vlive) continue;
+#pragma unroll
+                        for (int t = 0; t < QT; t++)
+                            o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[dd], pf[t], o[t][d], 0, 0, 0);
+                    }
                 }
             }
         };
@@ -443,7 +450,8 @@ __global__ __launch_bounds__(64 * NW)
                 h4 out;
 #pragma unroll
                 for (int j = 0; j < 4; j++) out[j] = (_Float16)(o[t][d][j] * inv[t]);
-                *reinterpret_cast<h4 *>(zp + 16 * d) = out;
+                // a head size that is a multiple of 8 only ends inside the last block: lanes past it store nothing
+                if (16 * d + 4 * g < hd) *reinterpret_cast<h4 *>(zp + 16 * d) = out;
             }
         }
     }
@@ -595,8 +603,9 @@ int et_mha_fused_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V, int ldq,
                flags);
     ET_REQUIRE(S % 16 == 0, ET_ERR_UNSUPPORTED, "et_mha_fused_f16: S=%d must be a multiple of 16",
                S);
-    ET_REQUIRE(hd % 16 == 0 && hd <= 128, ET_ERR_UNSUPPORTED,
-               "et_mha_fused_f16: head dim %d must be a multiple of 16, at most 128", hd);
+    // the reference example's 800 / 4 = 200-wide heads (example/main.cu:24-31) are the reason for the 256 form
+    ET_REQUIRE(hd % 8 == 0 && hd <= 256, ET_ERR_UNSUPPORTED,
+               "et_mha_fused_f16: head dim %d must be a multiple of 8, at most 256", hd);
     const int width = nh * hd;
     ET_REQUIRE(ldq >= width && ldk >= width && ldv >= width && ldz >= width, ET_ERR_INVALID_ARG,
                "et_mha_fused_f16: row strides (%d %d %d %d) smaller than nh*hd=%d", ldq, ldk, ldv,
@@ -630,7 +639,12 @@ int et_mha_fused_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V, int ldq,
     args.v_head_ptr = nullptr;
     if (hd <= 32) return launch_mha<32, false>(args, B, as_stream(stream));
     if (hd <= 64) return launch_mha<64, false>(args, B, as_stream(stream));
-    return launch_mha<128, false>(args, B, as_stream(stream));
+    if (hd <= 128) return launch_mha<128, false>(args, B, as_stream(stream));
+    // Heads up to 256 wide: 4 waves share the staging of a 128-key block (137 KB of LDS), each with one
+    // 16-query tile.  One workgroup per compute unit and one wave per SIMD, so a wave has the whole
+    // register file (8 waves at 256 registers spill 68 bytes per lane); a strip shorter than 64 queries
+    // leaves waves without queries, which stage and otherwise idle.
+    return launch_mha_nw<256, false, 4, 1>(args, as_stream(stream));
 }
 
 int et_mha_compactv_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *Vc, int ldq, int ldk, int ldvc,

@@ -275,6 +275,19 @@ static int run_factories(const std::string &dir) {
         et::DeviceBuffer<half> from_host(host8.data(), 8);
         out.push_back(first_value(from_host, 5));                       // 6
     }
+    {
+        // Linear<tile_mat> multiplies with a copy of its weight made at construction; a caller that writes
+        // into weight.data calls refresh().  All tiles set to 2: 32 * tiles_in_block_row + 0.5
+        auto lin = gen_sparse_linear<tile_mat>(128, 256, T, 0.5f);
+        lin->forward(Y.get(), X256.get());
+        etChk(et_device_sync());
+        lin->weight.data.set(static_cast<half>(2.0f));
+        lin->refresh();
+        lin->forward(Y.get(), X256.get());
+        auto rp = lin->weight.row_ptr.to_host();
+        out.push_back(first_value(Y, 0));
+        out.push_back(32.0f * (float)(rp[1] - rp[0]) + 0.5f);
+    }
     etChk(et_device_sync());
     npy_save(dir + "/factories.npy", out.data(), "<f4", 4, {out.size()});
     return 0;

@@ -26,15 +26,9 @@ def run_case(case, d):
     return res
 
 
-@pytest.mark.parametrize("TEXT", [1024, 28800])
-def test_example_model_from_npz(tmp_path, TEXT):
-    """Two ReLU encoder layers + decoder, the reference example's shape family (emdim 800 is not a
-    multiple of the head size the kernels take, so 768 / 4 heads x 192 is not used either): H 512,
-    4 heads x 128, FFN 208, batch 2 x seq 64; the decoder 1024 wide, and 28 800 wide as in the
-    reference example (example/main.cu:29,164)."""
-    H, nh, FF, S, B, NL = 512, 4, 208, 64, 2, 2
-    layers = [Hn.LayerWeights(H, nh, FF, 0.6, seed=70 + i) for i in range(NL)]
-    dec = Hn.BsrWeight(TEXT, H, 0.7, seed=90, bias_std=0.02)
+def write_example_model(tmp_path, layers, dec, x, S, B):
+    """weights.txt + one .npz per weight in the reference example's naming (example/main.cu:40-160)."""
+    H, nh, FF = layers[0].H, layers[0].nh, layers[0].dimFF
     names = []
     for i, w in enumerate(layers):
         pre = f"transformer_encoder.layers.{i}."
@@ -47,9 +41,20 @@ def test_example_model_from_npz(tmp_path, TEXT):
     F.save_weight_npz(str(tmp_path / "decoder."), dec.dense.astype(np.float32), dec.bias.astype(np.float32))
     names.append("decoder..npz")
     (tmp_path / "weights.txt").write_text("\n".join(names) + "\n")
-    x = Hn.randn((B * S, H), 91)
     np.save(tmp_path / "input.npy", x.astype(np.float32))
-    np.save(tmp_path / "meta.npy", np.array([H, H, S, nh, FF, H, NL, B, TEXT], np.int32))
+    np.save(tmp_path / "meta.npy", np.array([H, H, S, nh, FF, H, len(layers), B, dec.out], np.int32))
+
+
+@pytest.mark.parametrize("H,S,TEXT", [(512, 64, 1024), (512, 64, 28800), (800, 128, 28800)])
+def test_example_model_from_npz(tmp_path, H, S, TEXT):
+    """Two ReLU encoder layers + decoder assembled as the reference example does.  H 800, 4 heads x 200,
+    FFN 208, seq 128, decoder 28 800 wide is the example's own Model_t{800, 800, 128, 4, 208, 800, 2}
+    (example/main.cu:24-31,164); H 512, 4 heads x 128 is a smaller member of the family."""
+    nh, FF, B, NL = 4, 208, 2, 2
+    layers = [Hn.LayerWeights(H, nh, FF, 0.6, seed=70 + i) for i in range(NL)]
+    dec = Hn.BsrWeight(TEXT, H, 0.7, seed=90, bias_std=0.02)
+    x = Hn.randn((B * S, H), 91)
+    write_example_model(tmp_path, layers, dec, x, S, B)
     res = run_case("example", tmp_path)
     assert "encoder layer forward" in res.stdout
     hidden = Hn.oracle_stack(x, layers, B, act="relu")
@@ -69,21 +74,8 @@ def test_twelve_class_layers_through_forward(tmp_path):
     H, nh, FF, S, B, NL, TEXT = 768, 12, 3072, 128, 2, 12, 256
     layers = [Hn.LayerWeights(H, nh, FF, 0.8, seed=700 + i) for i in range(NL)]
     dec = Hn.BsrWeight(TEXT, H, 0.8, seed=790, bias_std=0.02)
-    names = []
-    for i, w in enumerate(layers):
-        pre = f"transformer_encoder.layers.{i}."
-        for nm, bw in (("self_attn.in_proj_", w.qkv), ("self_attn.out_proj.", w.o), ("linear1.", w.l1), ("linear2.", w.l2)):
-            F.save_weight_npz(str(tmp_path / (pre + nm)), bw.dense.astype(np.float32), bw.bias.astype(np.float32))
-            names.append(pre + nm + ".npz")
-        for nm, (g, b) in (("norm1.", (w.g1, w.be1)), ("norm2.", (w.g2, w.be2))):
-            F.save_weight_npz(str(tmp_path / (pre + nm)), g.astype(np.float32), b.astype(np.float32))
-            names.append(pre + nm + ".npz")
-    F.save_weight_npz(str(tmp_path / "decoder."), dec.dense.astype(np.float32), dec.bias.astype(np.float32))
-    names.append("decoder..npz")
-    (tmp_path / "weights.txt").write_text("\n".join(names) + "\n")
     x = Hn.randn((B * S, H), 791)
-    np.save(tmp_path / "input.npy", x.astype(np.float32))
-    np.save(tmp_path / "meta.npy", np.array([H, H, S, nh, FF, H, NL, B, TEXT], np.int32))
+    write_example_model(tmp_path, layers, dec, x, S, B)
     run_case("example", tmp_path)
     got = np.load(tmp_path / "hidden.npy")
     want32 = Hn.oracle_stack(x, layers, B, act="relu", store=None)
@@ -175,7 +167,8 @@ def test_factories_closed_forms(tmp_path):
     # Linear<csr_mat>: dense-image path (80 %) and CSR-kernel path (99 %) both equal the CSR kernel called directly
     assert db[:4] == [1.0, 1.0, 1.0, 0.0]
     assert db[4:8] == [3.0, 4.0, 0.0, 1.0]
-    assert db[8:] == [7.0, 6.0]  # DeviceBuffer(ptr, n) from a device pointer and from a host pointer
+    assert db[8:10] == [7.0, 6.0]  # DeviceBuffer(ptr, n) from a device pointer and from a host pointer
+    assert db[10] == db[11] and db[10] > 32.0  # Linear<tile_mat>::refresh() after the caller rewrote weight.data
 
 
 def test_attention_tags_with_separate_projections(tmp_path):

@@ -748,10 +748,13 @@ def test_mha_shapes(et, B, S, nh, hd, causal):
 
 
 @pytest.mark.parametrize("B,S,nh,hd,causal", [(2, 128, 4, 48, False), (1, 64, 3, 16, True), (2, 160, 2, 96, False),
-                                              (1, 128, 5, 80, True), (1, 32, 2, 112, False)])
+                                              (1, 128, 5, 80, True), (1, 32, 2, 112, False),
+                                              (2, 128, 4, 200, False),  # the reference example's heads (example/main.cu:24-31)
+                                              (1, 160, 3, 256, True), (2, 48, 2, 136, False), (1, 64, 5, 40, True),
+                                              (2, 128, 3, 72, False), (1, 272, 2, 168, False)])
 def test_mha_head_sizes_between_template_sizes(et, B, S, nh, hd, causal):
-    """Head sizes that are multiples of 16 but not 32/64/128 (the reference only asks for hd % 16 == 0,
-    Fused_attention/test/testfused.cu:22), with right padding."""
+    """Head sizes that are multiples of 8 but not 32/64/128/256 (the reference's kernels ask for hd % 16 == 0,
+    Fused_attention/test/testfused.cu:22; its example has 200-wide heads), with right padding."""
     lens = [S - 7 * (b + 1) for b in range(B)]
     got, want = run_mha(et, B, S, nh, hd, seed=70, lens=lens, causal=causal)
     assert Hn.max_abs(got, want) <= 2e-3
@@ -868,8 +871,8 @@ def test_mha_rejects_bad_args(et):
     f = et.lib().et_mha_fused_f16
     args = lambda S, hd, ld: (d.ptr, d.ptr, d.ptr, ld, ld, ld, d.ptr, ld, None, None, 1, S, 12, hd, 0.125, 0, None)
     assert f(*args(120, 64, 768)) == et.ET_ERR_UNSUPPORTED   # S % 16
-    assert f(*args(128, 40, 768)) == et.ET_ERR_UNSUPPORTED   # head dim not a multiple of 16
-    assert f(*args(128, 144, 2048)) == et.ET_ERR_UNSUPPORTED  # head dim above 128
+    assert f(*args(128, 44, 768)) == et.ET_ERR_UNSUPPORTED   # head dim not a multiple of 8
+    assert f(*args(128, 264, 4096)) == et.ET_ERR_UNSUPPORTED  # head dim above 256
     assert f(*args(128, 64, 512)) == et.ET_ERR_INVALID_ARG   # stride < nh*hd
     assert f(None, d.ptr, d.ptr, 768, 768, 768, d.ptr, 768, None, None, 1, 128, 12, 64, 0.125, 0, None) == et.ET_ERR_INVALID_ARG
 
