@@ -62,8 +62,8 @@ def _compile(src: Path) -> Path:
             if text.startswith("Function Name:"):
                 name = text.split(":", 1)[1].strip()
                 _resource_lines.append(f"{src.name} {name}")
-            elif name and text.split(":")[0] in ("TotalSGPRs", "VGPRs", "ScratchSize [bytes/lane]", "Occupancy [waves/SIMD]",
-                                                  "LDS Size [bytes/block]"):
+            elif name and text.split(":")[0] in ("TotalSGPRs", "VGPRs", "AGPRs", "ScratchSize [bytes/lane]", "Occupancy [waves/SIMD]",
+                                                  "SGPRs Spill", "VGPRs Spill", "LDS Size [bytes/block]"):
                 _resource_lines[-1] += " | " + text
             skip_context = 2
             continue

@@ -574,7 +574,7 @@ template <int HD, bool COMPACT>
 static int launch_mha(const MhaArgs &args, int B, hipStream_t stream) {
     (void)B;
     const int qblocks = args.S / 16;
-    if (!COMPACT) {
+    if constexpr (!COMPACT) {
         if (HD == 64 && qblocks % 16 == 0 && (long)args.nbh * (qblocks / 16) >= 512)
             return launch_mha_nw<(HD == 64 ? HD : 64), COMPACT, 8, 2>(args, stream);
         if (HD == 128 && qblocks % 16 == 0 && (long)args.nbh * (qblocks / 16) >= 512)

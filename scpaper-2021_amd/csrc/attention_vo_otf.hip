@@ -498,8 +498,13 @@ static int launch_mha_vo_otf_form(const MhaVoArgs &args, hipStream_t stream) {
     const int qstrips = (args.S + kStripQ - 1) / kStripQ, nslices = (args.N + VC - 1) / VC;
     const long long rounds = ((long long)args.B * nslices + kXcds - 1) / kXcds;
     const dim3 grid((unsigned)(rounds * kXcds * qstrips));
-    if (args.mask) mha_vo_otf_kernel<HD, KBLK, true, NW, QT, PF, VC><<<grid, 64 * NW, 0, stream>>>(args);
-    else mha_vo_otf_kernel<HD, KBLK, false, NW, QT, PF, VC><<<grid, 64 * NW, 0, stream>>>(args);
+    if constexpr (NW <= 8) {  // the 12-wave forms have no masked variant (168 registers do not hold it)
+        if (args.mask) {
+            mha_vo_otf_kernel<HD, KBLK, true, NW, QT, PF, VC><<<grid, 64 * NW, 0, stream>>>(args);
+            return check_launch("mha_vo_otf_kernel");
+        }
+    }
+    mha_vo_otf_kernel<HD, KBLK, false, NW, QT, PF, VC><<<grid, 64 * NW, 0, stream>>>(args);
     return check_launch("mha_vo_otf_kernel");
 }
 
@@ -514,7 +519,8 @@ template <int HD, int KBLK> static int launch_mha_vo_otf(const MhaVoArgs &args, 
     const long long small_grid = (long long)args.B * ((args.N + kVoCols - 1) / kVoCols) * ((args.S + 15) / 16);
     if (small_grid > 512) return launch_mha_vo_otf_form<HD, KBLK, 4, 2, true>(args, stream);
     if (args.nh <= 4) return launch_mha_vo_otf_form<HD, KBLK, 4, 1, true>(args, stream);
-    if (args.nh <= 8) return launch_mha_vo_otf_form<HD, KBLK, 8, 1, false>(args, stream);
+    // (an additive mask costs registers: with it the 12-wave forms would spill, 8 waves walk the heads instead)
+    if (args.nh <= 8 || args.mask) return launch_mha_vo_otf_form<HD, KBLK, 8, 1, false>(args, stream);
     if (small_grid <= 128) return launch_mha_vo_otf_form<HD, KBLK, 12, 1, false, 32>(args, stream);
     return launch_mha_vo_otf_form<HD, KBLK, 12, 1, false>(args, stream);
 }

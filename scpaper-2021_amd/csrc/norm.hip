@@ -64,14 +64,21 @@ __global__ __launch_bounds__(kWave *kRowsPerBlock) void layernorm_rows_kernel(
     // basic block of their own, where the compiler waits for each of them in turn.
     const raw_t *g = reinterpret_cast<const raw_t *>(gamma);
     const raw_t *b = reinterpret_cast<const raw_t *>(beta);
-    raw_t rs[NIT], rk[NIT], rg[NIT], rb[NIT];
+    // (Rows of more than 256 bytes per lane — binary32 rows wider than 4096 — would need more registers
+    // than a lane has for that: there gamma and beta are loaded where they are used, a second round trip
+    // that such a row hides behind its own length.)
+    constexpr bool kLateAffine = sizeof(raw_t) * NIT > 256;
+    constexpr int NAFF = kLateAffine ? 1 : NIT;
+    raw_t rs[NIT], rk[SKIP ? NIT : 1], rg[NAFF], rb[NAFF];
 #pragma unroll
     for (int i = 0; i < NIT; i++) {
         const int c = min(lane + kWave * i, chunks - 1);
         rs[i] = s[c];
         if (SKIP) rk[i] = k[c];
-        rg[i] = g[c];
-        rb[i] = b[c];
+        if (!kLateAffine) {
+            rg[i] = g[c];
+            rb[i] = b[c];
+        }
     }
 
     // values past the row are selected away, not branched around: a branch would give the
@@ -114,8 +121,8 @@ __global__ __launch_bounds__(kWave *kRowsPerBlock) void layernorm_rows_kernel(
         const int c = lane + kWave * i;
         if (c < chunks) {
             float gg[4], bb[4], y[4];
-            unpack4(rg[i], gg);
-            unpack4(rb[i], bb);
+            unpack4(kLateAffine ? g[c] : rg[kLateAffine ? 0 : i], gg);
+            unpack4(kLateAffine ? b[c] : rb[kLateAffine ? 0 : i], bb);
 #pragma unroll
             for (int j = 0; j < 4; j++) y[j] = (x[i][j] - mean) * rstd * gg[j] + bb[j];
             o[c] = pack4_as<raw_t>(y);

@@ -58,27 +58,40 @@ def test_no_product_file_imports_the_oracle():
 
 
 def test_hot_path_kernels_keep_their_registers():
-    """The build records registers and scratch of every kernel next to the library.  A kernel of the
-    encoder stack that spills registers to scratch memory pays for it on every launch (the 12-wave forms
-    of the tile-sparse Linear sit at the 168-register limit), so none of them may; the few kernels known
-    to spill (documented where they are launched) are listed, anything else is a regression."""
+    """The build records registers, spills and scratch of every kernel next to the library.  A kernel that
+    spills vector registers to scratch memory pays for it on every launch (the 12-wave forms of the
+    tile-sparse Linear sit at the 168-register limit), so none may, with the one exception named below by its
+    full instantiation.  Scalar registers parked in the lanes of a vector register ("SGPRs Spill") cost a
+    v_readlane each and no memory access; the compiler reserves 36 bytes of scratch for such kernels without
+    ever addressing it, which is why the criterion is the vector spill count and not the scratch size."""
     import re
     from pathlib import Path
     rec = Path(__file__).resolve().parents[1] / "scpaper-2021_amd" / "lib" / "kernel_resources.txt"
     if not rec.exists():
         pytest.skip("no resource record: the library was built by an older build script")
-    known_to_spill = ("mha_fused_kernelILi128ELb0ELi8ELi2E", "mha_fused_kernelILi128ELb1ELi8ELi2E",  # 256 queries x 128 dims
-                      "mha_vo_otf_kernelILi32ELi128ELb1ELi12E", "mha_vo_otf_kernelILi64ELi128ELb1ELi12E",  # masked, 12 waves
-                      "bsr16_stream_kernel", "gemm_f16_dma_kernelILi4ELi4ELi2E", "layernorm_rows_kernelIfLi32E")
+    # 128-wide heads, 8 waves with two query tiles each (256 queries a workgroup), taken from 512 such
+    # workgroups on: all 256 registers and 50 spilled, and still the fastest form measured at 2048 keys,
+    # 16 x 8 heads (503 us against 532 us for the one-tile form, which does not spill)
+    known_to_spill = {"_ZN2et16mha_fused_kernelILi128ELb0ELi8ELi2EEEvNS_7MhaArgsE"}
+    # the dense GEMM's 256 x 256 tile (4 x 4 MFMA tiles per wave, two LDS stages): 256 accumulator registers
+    # and 256 more for addresses and staging are all taken and 8 are spilled; it is the
+    # form that large dense Linears run fastest on (8192 x 4096 -> 4096: 334 us, 33 % of the MFMA peak;
+    # 16384 x 8192 -> 8192: 39 %), chosen only from 256 whole workgroups on
+    known_to_spill |= {f"_ZN2et19gemm_f16_dma_kernelILi4ELi4ELi2ELb{i}ELb{r}ELb0EEEvNS_8GemmArgsE" for i in (0, 1) for r in (0, 1)}
     seen = 0
     for line in rec.read_text().splitlines():
-        m = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
-        if not m:
+        m = re.search(r"VGPRs Spill: (\d+)", line)
+        sc = re.search(r"ScratchSize \[bytes/lane\]: (\d+)", line)
+        if not m or not sc:
             continue
         seen += 1
         name = line.split()[1]
-        if int(m.group(1)) and not any(k in name for k in known_to_spill):
-            raise AssertionError(f"{name} spills {m.group(1)} bytes per lane to scratch")
-        if "bsr16_linear_kernel" in name or "mha_fused_kernelILi64ELb0ELi4ELi1E" in name:
-            assert int(m.group(1)) == 0, line
+        vspill, scratch = int(m.group(1)), int(sc.group(1))
+        if vspill and name not in known_to_spill:
+            raise AssertionError(f"{name} spills {vspill} vector registers ({scratch} bytes of scratch per lane)")
+        if not vspill:  # scratch without vector spills: only the unused reservation that comes with parked scalar registers
+            assert scratch <= 36 and (scratch == 0 or int(re.search(r"SGPRs Spill: (\d+)", line).group(1)) > 0), line
+        if "bsr16_linear_kernel" in name or "bsr16_packed_kernel" in name or "bsr16_chain_kernel" in name or \
+                "mha_fused_kernelILi64ELb0ELi4ELi1E" in name:
+            assert vspill == 0 and scratch == 0, line
     assert seen > 100
