@@ -171,6 +171,16 @@ template <> class Linear<tile_mat> {
     pack_ptr pack, pack_producer, pack_consumer;
     int producer_nwave = 0, consumer_nwave = 0;  // the wave counts the role packs were asked for (0: the builder's choice)
     static constexpr int kPackMaxRows = 4096;
+    // forward / forward_act / forward_f32 take the one-strip pack up to this many rows (measured at 2048 and 4096
+    // rows: the plain call is 5-25 % faster than the pack for 768 -> 3072 and 3072 -> 768, level for the others)
+    static constexpr int kPlainPackMaxRows = 1536;
+    // From kRowLoopMinRows rows on, for inputs up to 1536 wide: the pack of the row-loop kernel (weights resident
+    // in registers, token strips staged two ahead), where its launch fills the chip — at least 256 (strip, group)
+    // pairs.  Measured against the plain call: 16384 x 768 -> 3072 43 against 60 us, -> 2304 32 against 45 us,
+    // -> 768 16 against 20 us; 4096 x 768 -> 3072 15 against 19 us; 2048 x 768 -> 2304 7.9 against 10.5 us.
+    // Serves forward / forward_act (binary16 results); forward_f32 keeps the plain call.
+    pack_ptr pack_loop;
+    static constexpr int kRowLoopMinRows = 2048;
     // ET_PACKED=0 in the environment keeps every Linear<tile_mat> on the unpacked kernels (for comparisons)
     static bool packed_enabled() {
         static const bool on = [] {
@@ -218,6 +228,11 @@ template <> class Linear<tile_mat> {
         if (plan) {
             etChk(et_linear_bsr16_planned_f16(plan.get(), et::f16(bias.get()), et::f16(input), et::f16(output), nullptr,
                                               size, act, stream));
+            return;
+        }
+        if (pack_loop) {
+            etChk(et_linear_bsr16_packed_f16(pack_loop.get(), et::f16(bias.get()), et::f16(input), et::f16(output), nullptr,
+                                             size, act, stream));
             return;
         }
         if (pack) {
@@ -341,6 +356,7 @@ template <> class Linear<tile_mat> {
         dense_out16.reset();
         plan.reset();
         pack.reset();
+        pack_loop.reset();
         pack_producer.reset();
         pack_consumer.reset();
         check();
@@ -369,12 +385,18 @@ template <> class Linear<tile_mat> {
             plan.reset(p);
             return;
         }
-        pack = make_pack(0);
+        if (size <= kPlainPackMaxRows) pack = make_pack(0);
+        if (size >= kRowLoopMinRows && in_size <= 1536) {
+            pack_loop = make_pack(ET_PACK_ROW_LOOP, 0, 1 << 30);
+            int mt = 0, groups = 0;
+            if (pack_loop) etChk(et_bsr16_pack_info(pack_loop.get(), &mt, &groups, nullptr, nullptr, nullptr));
+            if (pack_loop && (long)((size + mt * 16 - 1) / (mt * 16)) * groups < 256) pack_loop.reset();  // the chip would idle
+        }
     }
     // a pack for this weight and `size` rows, or null where the packed kernel does not apply
-    pack_ptr make_pack(int flags, int nwave = 0) const {
+    pack_ptr make_pack(int flags, int nwave = 0, int max_rows = kPackMaxRows) const {
         pack_ptr made;
-        if (!packed_enabled() || size <= 0 || size % 16 != 0 || size > kPackMaxRows || in_size % 128 != 0 || in_size > 4096)
+        if (!packed_enabled() || size <= 0 || size % 16 != 0 || size > max_rows || in_size % 128 != 0 || in_size > 4096)
             return made;
         et_bsr_pack p = nullptr;
         const int s = et_bsr16_pack_create(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()), size,

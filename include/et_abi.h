@@ -178,10 +178,16 @@ int et_linear_bsr16_planned_f16(et_bsr_plan plan, const et_f16 *bias,
  * et_linear_bsr16_resid_stats_f32 / et_linear_bsr16_resid16_stats_f32 (exactly
  * one of resid and resid16 set) and et_norm_linear_bsr16_f32in (without the
  * optional normalised outputs) compute, up to the order of the fp32
- * accumulation.  Replaces Linear<tile_mat>::forward (Linear/SPMM_tile.cu:312-324)
- * for callers that keep a Linear object. */
+ * accumulation.  ET_PACK_ROW_LOOP (alone) builds the pack of the form for many
+ * token rows instead — any number of them, in a multiple of 128 up to 1536:
+ * a workgroup keeps its share of the weight in registers and walks over
+ * token strips staged two ahead, whole block-rows per wave, results stored
+ * straight from the accumulators; such a pack serves
+ * et_linear_bsr16_packed_f16 with a binary16 result only.  Replaces
+ * Linear<tile_mat>::forward (Linear/SPMM_tile.cu:312-324) for callers that keep
+ * a Linear object. */
 typedef struct et_bsr_pack_s *et_bsr_pack;
-enum et_pack_flags { ET_PACK_NORM_CONSUMER = 1, ET_PACK_STATS_PRODUCER = 2 };
+enum et_pack_flags { ET_PACK_NORM_CONSUMER = 1, ET_PACK_STATS_PRODUCER = 2, ET_PACK_ROW_LOOP = 4 };
 int et_bsr16_pack_create(const int32_t *row_ptr, const int32_t *col_idx,
                          const et_f16 *tiles, int T, int in, int out, int flags,
                          int nwave, et_bsr_pack *pack);

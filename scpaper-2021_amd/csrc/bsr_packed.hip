@@ -117,6 +117,33 @@ static int pk_dispatch_norm(const PackArgs &a, const et_bsr_pack_s &p, hipStream
 
 }  // namespace et
 
+namespace et {
+int pack_upload(et_bsr_pack_s &p, const std::vector<uint32_t> &off, const std::vector<int32_t> &tab,
+                const std::vector<int32_t> &order, const et_f16 *tiles) {
+    auto upload = [&](void **dst, const void *src, size_t bytes) -> int {
+        int s = et_malloc(dst, std::max<size_t>(bytes, 16));
+        if (s != ET_OK) return s;
+        if (bytes) ET_HIP(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
+        return ET_OK;
+    };
+    void *d_order = nullptr;
+    int s = upload(&p.poff, off.data(), off.size() * 4);
+    if (s == ET_OK) s = upload(&p.ptab, tab.data(), tab.size() * 4);
+    if (s == ET_OK) s = check_hip(hipMalloc(&d_order, std::max<size_t>(order.size() * 4, 16)), "hipMalloc");
+    if (s == ET_OK) s = check_hip(hipMemcpy(d_order, order.data(), order.size() * 4, hipMemcpyHostToDevice), "hipMemcpy");
+    const size_t nslots = order.size() / 2;
+    if (s == ET_OK) s = et_malloc(&p.pw, std::max<size_t>(nslots * 1024, 16));
+    if (s == ET_OK && nslots) {
+        bsr_pack_gather_kernel<<<(unsigned)nslots, 64>>>(static_cast<_Float16 *>(p.pw), reinterpret_cast<const _Float16 *>(tiles),
+                                                         static_cast<const int32_t *>(d_order), (int)nslots);
+        s = check_launch("bsr_pack_gather_kernel");
+        if (s == ET_OK) s = check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    }
+    (void)hipFree(d_order);
+    return s;
+}
+}  // namespace et
+
 extern "C" {
 
 int et_bsr16_pack_create_geom(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles, int T, int in, int out,
@@ -124,8 +151,9 @@ int et_bsr16_pack_create_geom(const int32_t *row_ptr, const int32_t *col_idx, co
     ET_REQUIRE(pack != nullptr, ET_ERR_INVALID_ARG, "et_bsr16_pack_create: pack is NULL");
     *pack = nullptr;
     ET_REQUIRE(row_ptr && col_idx && tiles, ET_ERR_INVALID_ARG, "et_bsr16_pack_create: NULL pointer");
-    ET_REQUIRE((flags & ~(ET_PACK_NORM_CONSUMER | ET_PACK_STATS_PRODUCER)) == 0, ET_ERR_INVALID_ARG,
-               "et_bsr16_pack_create: flags=%d", flags);
+    ET_REQUIRE((flags & ~(ET_PACK_NORM_CONSUMER | ET_PACK_STATS_PRODUCER | ET_PACK_ROW_LOOP)) == 0 &&
+                   (!(flags & ET_PACK_ROW_LOOP) || flags == ET_PACK_ROW_LOOP),
+               ET_ERR_INVALID_ARG, "et_bsr16_pack_create: flags=%d", flags);
     ET_REQUIRE(T > 0 && in > 0 && out > 0 && T % 16 == 0 && out % 16 == 0, ET_ERR_UNSUPPORTED,
                "et_bsr16_pack_create: T=%d in=%d out=%d must be positive multiples of 16", T, in, out);
     const bool consumer = (flags & ET_PACK_NORM_CONSUMER) != 0, producer = (flags & ET_PACK_STATS_PRODUCER) != 0;
@@ -148,6 +176,11 @@ int et_bsr16_pack_create_geom(const int32_t *row_ptr, const int32_t *col_idx, co
         ET_REQUIRE(ci[(size_t)t] >= 0 && ci[(size_t)t] < bc, ET_ERR_INVALID_ARG,
                    "et_bsr16_pack_create: column-tile index %d of tile %d outside [0, %d)", ci[(size_t)t], t, bc);
 
+    if (flags & ET_PACK_ROW_LOOP) {  // the form for many token rows has a geometry and a builder of its own
+        ET_REQUIRE(mt == 0 && ngroups == 0 && nwave == 0 && cap == 0, ET_ERR_INVALID_ARG,
+                   "et_bsr16_pack_create: a row-loop pack chooses its own geometry");
+        return rowloop_pack_create(rp, ci, tiles, T, in, out, flags, pack);
+    }
     // ---- strips and block-row groups: one workgroup per compute unit where the shape allows it
     if (mt == 0) mt = (T >= 32 && (size_t)32 * in * 2 <= 64 * 1024) ? 2 : 1;
     const int strips = (T + mt * 16 - 1) / (mt * 16);
@@ -321,26 +354,7 @@ int et_bsr16_pack_create_geom(const int32_t *row_ptr, const int32_t *col_idx, co
     p->tab_stride = tab_stride;
     p->flags = flags;
     p->lds = pk_lds_bytes(mt, in, rows_per_wg, nwave);
-    auto upload = [&](void **dst, const void *src, size_t bytes) -> int {
-        int s = et_malloc(dst, std::max<size_t>(bytes, 16));
-        if (s != ET_OK) return s;
-        if (bytes) ET_HIP(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
-        return ET_OK;
-    };
-    void *d_order = nullptr;
-    int s = upload(&p->poff, off.data(), off.size() * 4);
-    if (s == ET_OK) s = upload(&p->ptab, tab.data(), tab.size() * 4);
-    if (s == ET_OK) s = check_hip(hipMalloc(&d_order, std::max<size_t>(order.size() * 4, 16)), "hipMalloc");
-    if (s == ET_OK) s = check_hip(hipMemcpy(d_order, order.data(), order.size() * 4, hipMemcpyHostToDevice), "hipMemcpy");
-    const size_t nslots = order.size() / 2;
-    if (s == ET_OK) s = et_malloc(&p->pw, std::max<size_t>(nslots * 1024, 16));
-    if (s == ET_OK && nslots) {
-        bsr_pack_gather_kernel<<<(unsigned)nslots, 64>>>(static_cast<_Float16 *>(p->pw), reinterpret_cast<const _Float16 *>(tiles),
-                                                         static_cast<const int32_t *>(d_order), (int)nslots);
-        s = check_launch("bsr_pack_gather_kernel");
-        if (s == ET_OK) s = check_hip(hipDeviceSynchronize(), "hipDeviceSynchronize");
-    }
-    (void)hipFree(d_order);
+    const int s = pack_upload(*p, off, tab, order, tiles);
     if (s != ET_OK) {
         delete p;
         return s;
@@ -391,6 +405,11 @@ int et_linear_bsr16_packed_f16(et_bsr_pack pack, const et_f16 *bias, const et_f1
     a.Y = reinterpret_cast<_Float16 *>(Y);
     a.Y32 = Y32;
     a.act = act;
+    if (pack->flags & ET_PACK_ROW_LOOP) {
+        ET_REQUIRE(Y != nullptr && (reinterpret_cast<uintptr_t>(Y) & 15) == 0, ET_ERR_UNSUPPORTED,
+                   "et_linear_bsr16_packed_f16: a row-loop pack stores binary16 results, 16-byte aligned");
+        return rowloop_launch(a, *pack, as_stream(stream));
+    }
     return pk_dispatch_plain<false>(a, *pack, as_stream(stream));
 }
 

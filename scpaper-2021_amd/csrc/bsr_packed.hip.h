@@ -25,6 +25,8 @@
 // direct-to-LDS loads; a binary32 strip that is normalised on the way (the consumer half of the
 // split SkipLayerNorm) passes through registers.
 #pragma once
+#include <vector>
+
 #include "common.hip.h"
 
 namespace et {
@@ -536,6 +538,13 @@ struct et_bsr_pack_s {
 };
 
 namespace et {
+// device copies of a pack's tables and of its weight slabs (slot s = tiles order[2s], order[2s + 1]; negative: zeros)
+int pack_upload(et_bsr_pack_s &p, const std::vector<uint32_t> &off, const std::vector<int32_t> &tab,
+                const std::vector<int32_t> &order, const et_f16 *tiles);
+// the row-loop form (bsr_rowloop.hip): its pack builder, from host copies of the structure, and its launch
+int rowloop_pack_create(const std::vector<int32_t> &row_ptr, const std::vector<int32_t> &col_idx, const et_f16 *tiles, int T, int in,
+                        int out, int flags, et_bsr_pack_s **pack);
+int rowloop_launch(const PackArgs &a, const et_bsr_pack_s &p, hipStream_t stream);
 // kernel arguments of a launch of `p` over T token rows (the operands are filled in by the caller)
 inline PackArgs pk_base_args(const et_bsr_pack_s &p, const et_f16 *bias, int T) {
     PackArgs a{};

@@ -131,20 +131,24 @@ class Bench:
     def bsr(self, T, n_in, n_out, sparsity, launches, entry="class"):
         """Tile-sparse Linear.  entry = "class": through the entry point Linear<tile_mat> picks for this shape
         (include/et/Linear.h: the dense image above half of the tiles, the streaming plan for wide inputs at many
-        rows, a pack up to 4096 rows, else the plain call); "plain" / "plan" / "pack" force one."""
+        rows, the row-loop pack from 2048 rows on for inputs up to 1536 wide where its launch fills the chip, a pack up
+        to 1536 rows, else the plain call); "plain" / "plan" / "pack" / "row loop" force one."""
         et, lib = self.et, self.lib
         row_ptr, col, ntile = self.tile_pattern(n_out, n_in, sparsity, 5)
         d_rp, d_col = self.dev(row_ptr), self.dev(col)
         tiles = self.dev(self.rnd((max(ntile, 1), 256), 0.02))
         bias = self.dev(np.zeros(n_out, np.float16))
         x, y = self.dev(self.rnd((T, n_in))), self.empty((T, n_out))
+        label_class = entry == "class"
         if entry == "class":
             kept = ntile * 256.0 / (n_in * n_out)
             if kept > 0.5:
                 entry = "dense image"
             elif n_in >= 128 and (n_in > 5112 or (n_in >= 3072 and T >= 4096)):
                 entry = "plan"
-            elif T <= 4096 and n_in % 128 == 0 and n_in <= 4096:
+            elif T >= 2048 and n_in % 128 == 0 and n_in <= 1536:
+                entry = "row loop"  # falls back below when its launch would not fill the chip
+            elif T <= 1536 and n_in % 128 == 0 and n_in <= 4096:
                 entry = "pack"
             else:
                 entry = "plain"
@@ -153,9 +157,17 @@ class Bench:
             et.check(lib.et_bsr16_plan_create(d_rp.ptr, d_col.ptr, tiles.ptr, T, n_in, n_out, 0, 0, 0, C.byref(handle)))
             destroy = lib.et_bsr16_plan_destroy
             fn = lambda: et.check(lib.et_linear_bsr16_planned_f16(handle, bias.ptr, x.ptr, y.ptr, None, T, 0, self.stream))
-        elif entry == "pack":
-            st = lib.et_bsr16_pack_create(d_rp.ptr, d_col.ptr, tiles.ptr, T, n_in, n_out, 0, 0, C.byref(handle))
-            if st == et.ET_ERR_UNSUPPORTED:
+        elif entry in ("pack", "row loop"):
+            st = lib.et_bsr16_pack_create(d_rp.ptr, d_col.ptr, tiles.ptr, T, n_in, n_out, 4 if entry == "row loop" else 0, 0,
+                                          C.byref(handle))
+            thin = False
+            if st == 0 and entry == "row loop":
+                mt, groups = C.c_int(), C.c_int()
+                et.check(lib.et_bsr16_pack_info(handle, C.byref(mt), C.byref(groups), None, None, None))
+                thin = -(-T // (16 * mt.value)) * groups.value < 256
+            if st == et.ET_ERR_UNSUPPORTED or (thin and label_class):
+                if st == 0:
+                    et.check(lib.et_bsr16_pack_destroy(handle))
                 entry = "plain"
             else:
                 et.check(st)
@@ -448,6 +460,13 @@ def main():
                                (2048, 6144, 768)):
             for entry in ("plain", "plan", "pack"):
                 if entry == "pack" and (T > 4096 or n_in > 4096):
+                    continue
+                b.bsr(T, n_in, n_out, 0.8, 10 if T >= 16384 else 30, entry=entry)
+        print("# ... and the row-loop pack (weights resident in registers, strips double-buffered) against the plain call and the pack")
+        for T, n_in, n_out in ((1024, 768, 3072), (2048, 768, 3072), (4096, 768, 3072), (16384, 768, 3072), (2048, 768, 768),
+                               (16384, 768, 768), (2048, 768, 2304), (16384, 768, 2304), (16384, 1024, 4096)):
+            for entry in ("plain", "pack", "row loop"):
+                if entry == "pack" and T > 4096:
                     continue
                 b.bsr(T, n_in, n_out, 0.8, 10 if T >= 16384 else 30, entry=entry)
     if args.set == "machine":

@@ -92,6 +92,63 @@ def test_linear_bsr16_packed(et, T, inp, out, sp, act, geom):
         assert Hn.max_abs(d_y.numpy(), want) <= 4e-3
 
 
+ET_PACK_ROW_LOOP = 4
+ROW_LOOP_CASES = [
+    # T, in, out, sparsity, act
+    (2048, 768, 3072, 0.8, 2),     # 32-row strips, several strips per workgroup
+    (4112, 768, 768, 0.8, 0),      # a last strip of 16 rows
+    (16384, 768, 2304, 0.8, 0),    # the large-batch QKV projection
+    (96, 128, 64, 0.5, 1),         # fewer strips than compute units, one group
+    (1024, 1024, 768, 0.9, 1),
+    (528, 1536, 256, 0.8, 2),      # 16-row strips (three 32-row strips of 1536 values do not fit the LDS)
+    (160, 768, 768, 0.97, 0),      # block-rows without tiles
+    (64, 256, 4096, 0.0, 0),       # dense pattern, many groups
+]
+
+
+@pytest.mark.parametrize("T,inp,out,sp,act", ROW_LOOP_CASES)
+def test_linear_bsr16_row_loop(et, T, inp, out, sp, act):
+    """The pack for many token rows (ET_PACK_ROW_LOOP): weights resident in registers, strips double-buffered,
+    results straight from the accumulators — the values of et_linear_bsr16_f16."""
+    lib = et.lib()
+    w = Hn.BsrWeight(out, inp, sp, seed=151, bias_std=0.1).upload(et)
+    x = Hn.randn((T, inp), 152)
+    d_x = up(et, x)
+    with Pack(et, w, T, ET_PACK_ROW_LOOP) as pk:
+        g = pk.info()
+        d_y = et.DeviceBuffer.empty((T, out), np.float16)
+        for rep in range(2):  # the second launch finds the first one's results in place: every element is written again
+            et.check(lib.et_fill_f16(d_y.ptr, T * out, 0x7E00, None))
+            et.check(lib.et_linear_bsr16_packed_f16(pk.h, w.d_bias.ptr, d_x.ptr, d_y.ptr, None, T, act, None))
+        want = L.linear(Hn.f32(x), Hn.f32(w.dense), Hn.f32(w.bias), ACT_NAME[act], torch.float16).numpy()
+        got = d_y.numpy()
+        err = Hn.max_abs(got, want)
+        print(f"row loop T={T} in={inp} out={out} sp={sp} {g}: max-abs {err:.2e}")
+        assert not np.isnan(got.astype(np.float32)).any()
+        assert err <= 4e-3
+        # no bias, fewer rows than the pack was built for (a multiple of 16 that ends inside a 32-row strip)
+        T2 = 16 * max(1, T // 48)
+        d_y2 = et.DeviceBuffer.empty((T2, out), np.float16)
+        et.check(lib.et_linear_bsr16_packed_f16(pk.h, None, d_x.ptr, d_y2.ptr, None, T2, 0, None))
+        want = L.linear(Hn.f32(x[:T2]), Hn.f32(w.dense), None, None, torch.float16).numpy()
+        assert Hn.max_abs(d_y2.numpy(), want) <= 4e-3
+        # a binary32 result is not what this form stores
+        d_y32 = et.DeviceBuffer.empty((16, out), np.float32)
+        assert lib.et_linear_bsr16_packed_f16(pk.h, None, d_x.ptr, None, d_y32.ptr, 16, 0, None) == et.ET_ERR_UNSUPPORTED
+
+
+def test_row_loop_pack_rejects(et):
+    lib = et.lib()
+    w = Hn.BsrWeight(64, 1664, 0.5, seed=153).upload(et)  # in above 1536
+    h = C.c_void_p()
+    args = (w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, 64, w.inp, w.out)
+    assert lib.et_bsr16_pack_create(*args, ET_PACK_ROW_LOOP, 0, C.byref(h)) == et.ET_ERR_UNSUPPORTED
+    w2 = Hn.BsrWeight(64, 256, 0.5, seed=154).upload(et)
+    args = (w2.d_row_ptr.ptr, w2.d_col_idx.ptr, w2.d_tiles.ptr, 64, w2.inp, w2.out)
+    assert lib.et_bsr16_pack_create(*args, ET_PACK_ROW_LOOP | ET_PACK_STATS_PRODUCER, 0, C.byref(h)) == et.ET_ERR_INVALID_ARG
+    assert lib.et_bsr16_pack_create(*args, ET_PACK_ROW_LOOP, 12, C.byref(h)) == et.ET_ERR_INVALID_ARG  # own geometry
+
+
 def test_linear_bsr16_packed_closed_form_and_tile_order(et):
     """All-ones weights and inputs give 16 * tiles-in-row + bias exactly (the closed form of the
     reference's driver, Linear/test/test_tile.cu), whatever the order of the tiles in a row."""
