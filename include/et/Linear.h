@@ -171,9 +171,17 @@ template <> class Linear<tile_mat> {
     pack_ptr pack, pack_producer, pack_consumer;
     int producer_nwave = 0, consumer_nwave = 0;  // the wave counts the role packs were asked for (0: the builder's choice)
     static constexpr int kPackMaxRows = 4096;
-    // forward / forward_act / forward_f32 take the one-strip pack up to this many rows (measured at 2048 and 4096
-    // rows: the plain call is 5-25 % faster than the pack for 768 -> 3072 and 3072 -> 768, level for the others)
-    static constexpr int kPlainPackMaxRows = 1536;
+    // Where a pack pays (measured against the unpacked kernel at 128 .. 1536 rows, 768- and 3072-wide inputs, 80 / 90 /
+    // 95 % sparsity): block-rows of at least 8 tiles on average — below that a wave's fixed run of slots is mostly
+    // padding (768 -> 2304 at 95 %, 128 rows: 8.6 against 3.6 us) — and either a wide input, where the unpacked
+    // kernel's chain of dependent loads is long (3072 -> 768: 0.68 - 0.85 of the unpacked time at any row count), or
+    // at least 256 rows (768-wide at 80 %: 1.12 - 1.37 at 128 rows, 0.89 - 1.01 from 256 on).
+    bool pack_pays() const {
+        return (long)weight.num_blk >= 8L * weight.blk_row_num && (in_size >= 2048 || size >= 256);
+    }
+    // forward / forward_act / forward_f32 take the one-strip pack up to this many rows (at 1536 rows and beyond the
+    // plain call is level or 5-25 % faster)
+    static constexpr int kPlainPackMaxRows = 1024;
     // From kRowLoopMinRows rows on, for inputs up to 1536 wide: the pack of the row-loop kernel (weights resident
     // in registers, token strips staged two ahead), where its launch fills the chip — at least 256 (strip, group)
     // pairs.  Measured against the plain call: 16384 x 768 -> 3072 43 against 60 us, -> 2304 32 against 45 us,
@@ -398,6 +406,7 @@ template <> class Linear<tile_mat> {
         pack_ptr made;
         if (!packed_enabled() || size <= 0 || size % 16 != 0 || size > max_rows || in_size % 128 != 0 || in_size > 4096)
             return made;
+        if (flags != ET_PACK_ROW_LOOP && !pack_pays()) return made;
         et_bsr_pack p = nullptr;
         const int s = et_bsr16_pack_create(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()), size,
                                            (int)in_size, (int)out_size, flags, nwave, &p);

@@ -132,7 +132,7 @@ class Bench:
         """Tile-sparse Linear.  entry = "class": through the entry point Linear<tile_mat> picks for this shape
         (include/et/Linear.h: the dense image above half of the tiles, the streaming plan for wide inputs at many
         rows, the row-loop pack from 2048 rows on for inputs up to 1536 wide where its launch fills the chip, a pack up
-        to 1536 rows, else the plain call); "plain" / "plan" / "pack" / "row loop" force one."""
+        to 1024 rows where block-rows average 8 tiles and the input is wide or the rows are at least 256, else the plain call); "plain" / "plan" / "pack" / "row loop" force one."""
         et, lib = self.et, self.lib
         row_ptr, col, ntile = self.tile_pattern(n_out, n_in, sparsity, 5)
         d_rp, d_col = self.dev(row_ptr), self.dev(col)
@@ -148,7 +148,7 @@ class Bench:
                 entry = "plan"
             elif T >= 2048 and n_in % 128 == 0 and n_in <= 1536:
                 entry = "row loop"  # falls back below when its launch would not fill the chip
-            elif T <= 1536 and n_in % 128 == 0 and n_in <= 4096:
+            elif T <= 1024 and n_in % 128 == 0 and n_in <= 4096 and ntile >= 8 * (n_out // 16) and (n_in >= 2048 or T >= 256):
                 entry = "pack"
             else:
                 entry = "plain"
