@@ -319,6 +319,9 @@ def main():
                          "neighbouring projections (five)")
     ap.add_argument("--chain", action="store_true",
                     help="everything between two attention kernels in one launch (two launches per layer)")
+    ap.add_argument("--fuse-qkv", action="store_true",
+                    help="the QKV projection of every layer after the first inside its attention kernel (four launches "
+                         "per layer)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain streaming kernel of known size (ReLU over 64 MiB in, 64 MiB out) "
                          "three times, as the reference point for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
@@ -331,7 +334,7 @@ def main():
     et.lib()  # fails loudly if the native library is missing
 
     layers = build_layers(et)
-    model = build_model(et, layers, use_graph=not args.eager, mixed=2 if args.separate_ln else 3 if args.chain else 1)
+    model = build_model(et, layers, use_graph=not args.eager, mixed=2 if args.separate_ln else 3 if args.chain else 4 if args.fuse_qkv else 1)
     x = np.random.default_rng(4).standard_normal((B * S, H), dtype=np.float32).astype(np.float16)
     d_in = et.DeviceBuffer.from_numpy(x)
     d_out = et.DeviceBuffer.empty((B * S, H), np.float16)

@@ -279,6 +279,7 @@ class Attention<_config, std::enable_if_t<_config::isSingleKernel>> : public et:
     std::unique_ptr<linearO_t> linearO;
     std::unique_ptr<ptr_t> mat_qkv, mat_z;
     std::shared_ptr<Model_t> model;
+    bool fused_qkv_ = false;
 
   public:
     Attention(std::unique_ptr<linearQKV_t> _linearQKV, std::unique_ptr<linearO_t> _linearO,
@@ -318,6 +319,22 @@ class Attention<_config, std::enable_if_t<_config::isSingleKernel>> : public et:
             linearO->prepare_split_producer(nwave);
         }
     }
+    // The QKV projection inside the attention kernel (one launch instead of two) for the layers whose input is
+    // a previous layer's un-normalised sum: sequences up to 128 tokens, heads of 64, a 768-wide model.
+    // true when forward_split() will run that way.
+    bool prepare_fused_qkv() {
+        if constexpr (std::is_same<linearQKV_t, Linear<tile_mat>>::value) {
+            const int hd = model->kdim / model->nhead;
+            if (model->vdim != model->kdim ||
+                et_norm_qkv_mha_f32in_supported(batch(), model->seq_len, (int)linearQKV->in_size, model->nhead, hd) != 1)
+                return false;
+            fused_qkv_ = linearQKV->prepare_qkv_heads(model->nhead);
+            return fused_qkv_;
+        } else {
+            return false;
+        }
+    }
+    bool fused_qkv() const { return fused_qkv_; }
     // The pieces a caller needs to run this attention as part of a chain launch (et_encoder_chain_f32):
     // the two projections, the buffers between them, and the attention kernel on its own.
     linearQKV_t &qkv_linear() { return *linearQKV; }
@@ -334,16 +351,24 @@ class Attention<_config, std::enable_if_t<_config::isSingleKernel>> : public et:
     void forward_split(float *v1, float *stats1, int *groups1, float *fin_in, const et::SplitSum *in, const float *x32,
                        half *x16, et::stream_t stream = nullptr) {
         if constexpr (std::is_same<linearQKV_t, Linear<tile_mat>>::value && std::is_same<linearO_t, Linear<tile_mat>>::value) {
-            if (in)
-                linearQKV->forward_norm_f32in(mat_qkv->get(), in->v, in->stats, in->groups, in->gamma, in->beta,
-                                              in->eps, fin_in, nullptr, nullptr, ET_ACT_NONE, stream);
-            else
-                linearQKV->forward(mat_qkv->get(), x16, stream);
-            const int ldm = model->kdim * 2 + model->vdim;
-            half *Q = mat_qkv->get();
-            half *K = Q + model->kdim;
-            half *V = K + model->kdim;
-            et::fused_mha(Q, K, V, ldm, ldm, ldm, mat_z->get(), model->vdim, *model, run(stream));
+            if (in && fused_qkv_) {
+                const et::AttnRun r = run(stream);
+                const float scale = r.scale != 0.0f ? r.scale : 1.0f / std::sqrt((float)(model->kdim / model->nhead));
+                linearQKV->forward_norm_qkv_mha(mat_z->get(), model->vdim, in->v, in->stats, in->groups, in->gamma, in->beta,
+                                                in->eps, fin_in, r.mask, r.lens, r.batch, model->seq_len, scale,
+                                                r.causal ? ET_MHA_CAUSAL : 0, stream);
+            } else {
+                if (in)
+                    linearQKV->forward_norm_f32in(mat_qkv->get(), in->v, in->stats, in->groups, in->gamma, in->beta,
+                                                  in->eps, fin_in, nullptr, nullptr, ET_ACT_NONE, stream);
+                else
+                    linearQKV->forward(mat_qkv->get(), x16, stream);
+                const int ldm = model->kdim * 2 + model->vdim;
+                half *Q = mat_qkv->get();
+                half *K = Q + model->kdim;
+                half *V = K + model->kdim;
+                et::fused_mha(Q, K, V, ldm, ldm, ldm, mat_z->get(), model->vdim, *model, run(stream));
+            }
             if (!in && !x32)  // first layer, residual = the binary16 input itself
                 linearO->forward_resid16_stats_f32(v1, stats1, groups1, mat_z->get(), x16, stream);
             else

@@ -216,6 +216,12 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
             linear2->prepare_split_producer();
         }
     }
+    // After enable_split(): the layer's QKV projection moves into its attention kernel (four launches per
+    // layer) whenever its input is a previous layer's sum.  false where the shapes do not allow it.
+    bool enable_fused_qkv() {
+        if constexpr (attn_has_fused_qkv<attn_t>::value) return stats1 && attn->prepare_fused_qkv();
+        else return false;
+    }
     static constexpr int kChainWaves = 12;
     // This layer's share of a chain launch (et_encoder_chain_f32): everything between its attention
     // kernel and the next layer's.  false when the layer's types have no such form.
@@ -312,6 +318,9 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
                                  static_cast<float *>(nullptr), static_cast<const SplitSum *>(nullptr),
                                  static_cast<const float *>(nullptr), static_cast<half *>(nullptr),
                                  static_cast<stream_t>(nullptr)))>> : std::true_type {};
+    template <typename A, typename = void> struct attn_has_fused_qkv : std::false_type {};
+    template <typename A>
+    struct attn_has_fused_qkv<A, std::void_t<decltype(std::declval<A &>().prepare_fused_qkv())>> : std::true_type {};
     template <typename A, typename = void> struct attn_has_f32 : std::false_type {};
     template <typename A>
     struct attn_has_f32<A, std::void_t<decltype(std::declval<A &>().forward_f32(

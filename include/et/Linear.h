@@ -169,6 +169,10 @@ template <> class Linear<tile_mat> {
     };
     using pack_ptr = std::unique_ptr<et_bsr_pack_s, PackDeleter>;
     pack_ptr pack, pack_producer, pack_consumer;
+    // W_qkv ordered head by head for the attention kernel that projects Q, K and V itself
+    // (et_qkv_heads_pack_create); built on prepare_qkv_heads()
+    pack_ptr pack_heads;
+    int heads_nhead = 0;
     int producer_nwave = 0, consumer_nwave = 0;  // the wave counts the role packs were asked for (0: the builder's choice)
     static constexpr int kPackMaxRows = 4096;
     // Where a pack pays (measured against the unpacked kernel at 128 .. 1536 rows, 768- and 3072-wide inputs, 80 / 90 /
@@ -295,6 +299,29 @@ template <> class Linear<tile_mat> {
         if (!pack_consumer && !dense && !plan && (pack_consumer = make_pack(ET_PACK_NORM_CONSUMER, nwave)))
             consumer_nwave = nwave;
     }
+    // This Linear as the QKV projection of `nhead` heads of 64 inside the attention kernel: false (and nothing
+    // built) where that kernel does not take the weight.  Called once, outside any stream capture.
+    bool prepare_qkv_heads(int nhead) {
+        if (pack_heads) return heads_nhead == nhead;
+        if (dense || plan || !packed_enabled() || (long)out_size != 3L * nhead * 64) return false;
+        et_bsr_pack p = nullptr;
+        const int s = et_qkv_heads_pack_create(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
+                                               (int)in_size, nhead, &p);
+        if (s == ET_ERR_UNSUPPORTED) return false;
+        etChk(s);
+        pack_heads.reset(p);
+        heads_nhead = nhead;
+        return true;
+    }
+    // Z = attention over (Q, K, V) = normalised(V32) W^T + bias, in one launch (et_norm_qkv_mha_f32in)
+    void forward_norm_qkv_mha(half *Z, int ldz, const float *V32, const float *stats, int groups, const half *gamma,
+                              const half *beta, float eps, float *fin_out, const half *mask, const int *lens, int batch,
+                              int seq_len, float scale, int flags, et::stream_t stream = nullptr) {
+        et::require((bool)pack_heads, "Linear<tile_mat>: prepare_qkv_heads() was not called or did not apply");
+        etChk(et_norm_qkv_mha_f32in(pack_heads.get(), V32, stats, groups, et::f16(gamma), et::f16(beta), eps, fin_out,
+                                    et::f16(bias.get()), et::f16(Z), ldz, et::f16(mask), lens, batch, seq_len, scale, flags,
+                                    stream));
+    }
     // V = input W^T + bias + residual (binary32) and stats[*groups][size][2]; the residual is
     // `resid` itself, or with resid_fin its normalisation by (resid_fin, resid_gamma, resid_beta)
     void forward_resid_stats_f32(float *V, float *stats, int *groups, const half *input, const float *resid,
@@ -358,7 +385,7 @@ template <> class Linear<tile_mat> {
     // allocates and synchronises — and every copy is made again, the role packs of the split normalisation
     // included.
     void refresh() {
-        const bool had_producer = (bool)pack_producer, had_consumer = (bool)pack_consumer;
+        const bool had_producer = (bool)pack_producer, had_consumer = (bool)pack_consumer, had_heads = (bool)pack_heads;
         etChk(et_device_sync());  // launches still reading the old copies end first
         dense.reset();
         dense_out16.reset();
@@ -367,9 +394,11 @@ template <> class Linear<tile_mat> {
         pack_loop.reset();
         pack_producer.reset();
         pack_consumer.reset();
+        pack_heads.reset();
         check();
         if (had_producer) prepare_split_producer(producer_nwave);
         if (had_consumer) prepare_split_consumer(consumer_nwave);
+        if (had_heads) prepare_qkv_heads(heads_nhead);
     }
 
   private:

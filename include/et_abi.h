@@ -187,7 +187,7 @@ int et_linear_bsr16_planned_f16(et_bsr_plan plan, const et_f16 *bias,
  * Linear<tile_mat>::forward (Linear/SPMM_tile.cu:312-324) for callers that keep
  * a Linear object. */
 typedef struct et_bsr_pack_s *et_bsr_pack;
-enum et_pack_flags { ET_PACK_NORM_CONSUMER = 1, ET_PACK_STATS_PRODUCER = 2, ET_PACK_ROW_LOOP = 4 };
+enum et_pack_flags { ET_PACK_NORM_CONSUMER = 1, ET_PACK_STATS_PRODUCER = 2, ET_PACK_ROW_LOOP = 4, ET_PACK_QKV_HEADS = 8 };
 int et_bsr16_pack_create(const int32_t *row_ptr, const int32_t *col_idx,
                          const et_f16 *tiles, int T, int in, int out, int flags,
                          int nwave, et_bsr_pack *pack);
@@ -540,6 +540,33 @@ int et_mha_compactv_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *Vc,
                         int S, int nh, int hd, int vhd, float scale, int flags,
                         et_stream stream);
 
+/* ---------------------------------------------------------------------------
+ * The QKV projection inside the attention kernel (four launches per layer in
+ * the split-normalisation stack instead of five): one workgroup per (sequence,
+ * head) normalises its sequence's rows of the previous layer's binary32 sum V
+ * with that sum's row statistics (what et_norm_linear_bsr16_f32in does for the
+ * QKV projection), multiplies them with its head's block-rows of the
+ * tile-sparse W_qkv, keeps Q, K and V of the head in LDS and runs the fused
+ * attention of et_mha_fused_f16 on them; fin_out[T][2] receives mean and rstd
+ * of every row (may be NULL).  W_qkv = [Q | K | V] rows as Attention's single
+ * projection holds them (Attention/Attention.h:246-265); et_qkv_heads_pack_create
+ * copies it once into the order the kernel reads (destroy with
+ * et_bsr16_pack_destroy).  Limits, told by et_norm_qkv_mha_f32in_supported:
+ * sequences of a multiple of 16 up to 128 tokens, 768-wide input, heads of 64.
+ * Replaces Attention<cfg, isSingleKernel>::forward up to the O projection
+ * (Attention/Attention_single.cu:10-108).
+ * ------------------------------------------------------------------------ */
+int et_norm_qkv_mha_f32in_supported(int B, int S, int in, int nhead, int hd);
+int et_qkv_heads_pack_create(const int32_t *row_ptr, const int32_t *col_idx,
+                             const et_f16 *tiles, int in, int nhead,
+                             et_bsr_pack *pack);
+int et_norm_qkv_mha_f32in(et_bsr_pack pack, const float *V, const float *stats,
+                          int stat_groups, const et_f16 *gamma,
+                          const et_f16 *beta, float eps, float *fin_out,
+                          const et_f16 *bias_qkv, et_f16 *Z, int ldz,
+                          const et_f16 *mask, const int32_t *lens, int B, int S,
+                          float scale, int flags, et_stream stream);
+
 /* Softmax probabilities written to memory: P[b*S + q][h*S + key] (row stride
  * nh*S), the layout of the reference's __kernel_fused_attention_NOTF
  * (Fused_attention/Fused_attention.cu:118-206).  S <= 512. */
@@ -698,15 +725,20 @@ typedef struct et_model_desc {
     float eps;     /* LayerNorm epsilon; <= 0 selects 1e-5                        */
     int causal;    /* != 0: causal mask (the reference's hard-wired one)          */
     int use_graph; /* != 0: replay a captured HIP graph; 0: launch kernel by kernel */
-    int mixed;     /* 1, 2 or 3: mixed precision — the residual stream (layer inputs, the two
+    int mixed;     /* 1, 2, 3 or 4: mixed precision — the residual stream (layer inputs, the two
                     * projections that feed a SkipLayerNorm, both SkipLayerNorm results)
                     * is kept in binary32 inside the stack, binary16 only as matrix-core
                     * operands; input and output of et_model_forward stay binary16.
                     * 1: SkipLayerNorm is folded into the neighbouring tile-sparse projections
-                    *    where the shapes allow (five launches per layer); 2: it keeps its own
+                    *    where the shapes allow (five launches per layer; four, as under 4, for
+                    *    the batch sizes where that measured faster: 10 to 24 sequences of 48
+                    *    to 128 tokens on 12 heads); 2: it keeps its own
                     *    launches (seven); 3: as 1, with everything between two attention
                     *    kernels in one launch (et_encoder_chain_f32: two launches per layer)
-                    *    where the shapes allow and the device runs it as it must, else as 1.
+                    *    where the shapes allow and the device runs it as it must, else as 1;
+                    *    4: as 1, with the QKV projection of every layer after the first inside
+                    *    its attention kernel (et_norm_qkv_mha_f32in: four launches per layer)
+                    *    where the shapes allow, else as 1.
                     * 0: every activation is stored as binary16 (the reference's storage) */
 } et_model_desc;
 

@@ -20,11 +20,18 @@
 // by the fp32 row sum happens once on the fp32 accumulators.
 #include <math.h>
 
+#include <algorithm>
+#include <new>
+#include <vector>
+
 #include <type_traits>
 
 #include "common.hip.h"
+#include "bsr_packed.hip.h"
 
 namespace et {
+
+#define ET_QM_CONST(T, p) ((const __attribute__((address_space(4))) T *)(p))
 
 struct MhaArgs {
     const _Float16 *Q, *K, *V;
@@ -283,148 +290,7 @@ __global__ __launch_bounds__(64 * NW)
         // no per-16-key branches (the LDS reads of the whole block can be issued ahead of
         // the MFMAs) and the softmax costs one max, one multiply-add, one exp2, half a
         // conversion and half a dot-accumulate per score.
-        auto multiply = [&](auto fast_tag) {
-            constexpr bool FAST = decltype(fast_tag)::value;
-            // ---- scores of the wave's queries against the 128 staged keys
-            f4 sc[QT][kNKB];
-#pragma unroll
-            for (int kb = 0; kb < kNKB; kb++) {
-#pragma unroll
-                for (int t = 0; t < QT; t++) sc[t][kb] = f4{0.f, 0.f, 0.f, 0.f};
-                if (FAST || k0 + kb * 16 < klimit) {  // wave-uniform: skip fully padded key blocks
-                    const _Float16 *kp = Ks + (kb * 16 + r16) * L::ldk + 8 * g;
-#pragma unroll
-                    for (int ks = 0; ks < KS; ks++) {
-                        const h8 kf = *reinterpret_cast<const h8 *>(kp + 32 * ks);
-#pragma unroll
-                        for (int t = 0; t < QT; t++)
-                            sc[t][kb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[t][ks], sc[t][kb], 0, 0, 0);
-                    }
-                }
-            }
-
-            if (FAST && k0 + kKeyBlock > klimit) {  // wave-uniform
-                // The block ends in padded keys: their raw scores become -inf, in place.  Key
-                // 16kb + 4g + j is padded when 16kb + j >= klimit - k0 - 4g (the left side a
-                // constant once unrolled).  (A separate instantiation of this lambda for the
-                // case made the allocator spill in the variants held to 168 registers.)
-                const int lim = klimit - k0 - 4 * g;
-#pragma unroll
-                for (int t = 0; t < QT; t++)
-#pragma unroll
-                    for (int kb = 0; kb < kNKB; kb++)
-#pragma unroll
-                        for (int j = 0; j < 4; j++)
-                            sc[t][kb][j] = (kb * 16 + j >= lim) ? -INFINITY : sc[t][kb][j];
-            }
-            // ---- scale, mask, block max, running max (FAST keeps the raw scores: the scale
-            // is positive there, so the max commutes with it, and it is applied inside the
-            // exponent's multiply-add)
-            float m_use[QT];
-#pragma unroll
-            for (int t = 0; t < QT; t++) {
-                float m_blk = -INFINITY;
-                if (FAST) {
-#pragma unroll
-                    for (int kb = 0; kb < kNKB; kb++)
-#pragma unroll
-                        for (int j = 0; j < 4; j++) m_blk = fmaxf(m_blk, sc[t][kb][j]);
-                    m_blk *= a.scale_log2e;
-                } else {
-#pragma unroll
-                    for (int kb = 0; kb < kNKB; kb++) {
-                        const int key0 = k0 + kb * 16 + 4 * g;
-                        float mk[4] = {0.f, 0.f, 0.f, 0.f};
-                        if (a.mask && q_ok[t] && key0 < S) {
-                            const h4 mv = *reinterpret_cast<const h4 *>(a.mask + (size_t)q[t] * S + key0);
-#pragma unroll
-                            for (int j = 0; j < 4; j++) mk[j] = (float)mv[j] * kLog2e;
-                        }
-#pragma unroll
-                        for (int j = 0; j < 4; j++) {
-                            const int key = key0 + j;
-                            float sv = sc[t][kb][j] * a.scale_log2e + mk[j];
-                            if (key >= klimit || (a.causal && key > q[t])) sv = -INFINITY;
-                            sc[t][kb][j] = sv;
-                            m_blk = fmaxf(m_blk, sv);
-                        }
-                    }
-                }
-                m_blk = rows_max(m_blk);
-
-                const float m_new = fmaxf(m_run[t], m_blk);
-                // all keys so far masked: keep everything at zero without inf - inf
-                m_use[t] = (m_new == -INFINITY) ? 0.0f : m_new;
-                const float alpha = __builtin_amdgcn_exp2f(m_run[t] - m_use[t]);  // m_run = -inf gives 0
-                m_run[t] = m_new;
-                // the running max seldom moves after the first blocks: skip the rescaling of
-                // the accumulators when no lane of the wave needs it
-                if (!__all(alpha == 1.0f)) {
-                    l_part[t] *= alpha;
-#pragma unroll
-                    for (int d = 0; d < DB; d++) o[t][d] *= alpha;
-                }
-            }
-
-            // ---- probabilities (fp32 sum, fp16 operands) and O^T += V^T P^T
-            const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
-            const int g8 = 8 * g, g8x = (8 * g) ^ 16;  // the lane's 8-key chunk of a 32-key group, plain and swizzled
-#pragma unroll
-            for (int s2 = 0; s2 < kNKB / 2; s2++) {
-                if (!FAST && k0 + s2 * 32 >= klimit) continue;  // both key blocks fully padded
-                h8 pf[QT];
-#pragma unroll
-                for (int t = 0; t < QT; t++) {
-                    // the lane's 8 values: keys 4g..4g+3 of score tile 2*s2, then of tile 2*s2+1;
-                    // each fp16 pair is formed once and feeds both the MFMA and the row sum
-#pragma unroll
-                    for (int pr = 0; pr < 4; pr++) {
-                        const int kb = 2 * s2 + (pr >> 1), j = 2 * (pr & 1);
-                        float e0, e1;
-                        if (FAST) {
-                            e0 = sc[t][kb][j] * a.scale_log2e - m_use[t];
-                            e1 = sc[t][kb][j + 1] * a.scale_log2e - m_use[t];
-                        } else {
-                            e0 = sc[t][kb][j] - m_use[t];
-                            e1 = sc[t][kb][j + 1] - m_use[t];
-                        }
-                        // raw v_exp_f32: results below the normal range flush to zero, which
-                        // the conversion to fp16 would do anyway
-                        const h2 hp = {(_Float16)__builtin_amdgcn_exp2f(e0), (_Float16)__builtin_amdgcn_exp2f(e1)};
-                        // the row sum uses the values that enter the MFMA
-                        l_part[t] = __builtin_amdgcn_fdot2(hp, ones, l_part[t], false);
-                        pf[t][2 * pr] = hp[0];
-                        pf[t][2 * pr + 1] = hp[1];
-                    }
-                }
-                // The V^T fragments of the step are read unconditionally (dimension blocks past the
-                // head size or the surviving columns hold zeros) so that the reads go out together;
-                // a read under a branch is waited for on the spot.  Only compact V skips the
-                // products of dead blocks (wave-uniform).
-                // (at most 8 fragments, 32 registers, at a time: 256-wide heads take two rounds)
-                constexpr int DC = DB < 8 ? DB : 8;
-#pragma unroll
-                for (int d0 = 0; d0 < DB; d0 += DC) {
-                    h8 vf[DC];
-#pragma unroll
-                    for (int dd = 0; dd < DC; dd++) {
-                        const int d = d0 + dd;
-                        const int swz = vt_swizzle<HD>(d);  // a constant once d is unrolled
-                        const h8 vr = *reinterpret_cast<const h8 *>(Vt + (d * 16 + r16) * L::ldvt +
-                                                                     ((s2 * 32) ^ (swz & 32)) + ((swz & 16) ? g8x : g8));
-                        vf[dd] = (swz & 4) ? h8{vr[4], vr[5], vr[6], vr[7], vr[0], vr[1], vr[2], vr[3]} : vr;
-                    }
-#pragma unroll
-                    for (int dd = 0; dd < DC; dd++) {
-                        const int d = d0 + dd;
-                        if (COMPACT && d * 16 >= vlive) continue;
-#pragma unroll
-                        for (int t = 0; t < QT; t++)
-                            o[t][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf[dd], pf[t], o[t][d], 0, 0, 0);
-                    }
-                }
-            }
-        };
+#include "attention_core.inc"
         const bool plain = a.mask == nullptr && a.scale_log2e > 0.0f &&
                           (!a.causal || k0 + kKeyBlock <= qstrip * kStripQ + 1);
         if (plain) multiply(std::true_type{});
@@ -587,6 +453,320 @@ static int launch_mha(const MhaArgs &args, int B, hipStream_t stream) {
     return launch_mha_nw<HD, COMPACT, 1, 1>(args, stream);
 }
 
+
+// ---- QKV projection inside the attention kernel --------------------------------------------------------
+// One workgroup per (sequence, head), sequences of at most 128 tokens, heads of 64: the workgroup normalises
+// its sequence's rows of the previous layer's binary32 sum while it stages them (the consumer half of the
+// split SkipLayerNorm, 64 rows at a time), multiplies them with its head's 12 block-rows of the tile-sparse
+// W_qkv (a pack: one block-row per wave, the wave's slots in registers), leaves Q, K and V^T of the head in
+// LDS in the layouts the attention core reads, and runs that core on them.  Q, K and V never exist in memory
+// and the layer has one launch fewer.  The heads of a sequence run on one XCD, so the sum comes from HBM once.
+struct QkvMhaArgs {
+    MhaArgs m;               // Z, ldz, mask, lens, S, nh, hd, nbh, scale_log2e, causal (Q, K, V unused)
+    const _Float16 *pw;      // [nh][12][cap] slots of 1 KiB in lane order (two tiles each, zero slots as padding)
+    const uint32_t *poff;    // [nh][12][cap] byte offsets (column * 32) of a slot's two tiles, 16 bits each
+    const int32_t *pn;       // [nh][12] slots of every block-row
+    const _Float16 *bias;    // [3 * nh * 64] (Q | K | V, as the rows of W_qkv) or nullptr
+    int cap, in, T, B;
+    const float *X32;        // [T][in] the binary32 sum
+    const float *st_in;      // [st_groups][T][2] partial (sum, sum of squares) of every row
+    int st_groups;
+    const _Float16 *gamma, *beta;
+    float eps;
+    float *fin_out;          // [T][2] mean and rstd of every row, written by head 0 (may be null)
+};
+constexpr int kQkvWaves = 12;   // Q, K, V x 4 block-rows of a 64-wide head
+constexpr int kQkvRows = 64;    // token rows staged at a time
+
+// PF of a thread's eight rows of the second 64 are requested before the products of the first 64 (they arrive while the
+// matrix cores work).  NPASS = 1 keeps the wave's slots in registers across both halves; NPASS = 2 or 3 (block-rows of
+// more than 12 slots) fetches them in parts of 8 for every 64 rows.
+template <int CAP, int PF, int NPASS>
+__global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArgs qa) {
+    constexpr int HD = 64, QT = 1;
+    constexpr bool COMPACT = false;
+    using L = MhaLds<HD>;
+    constexpr int KS = HD / 32, DB = HD / 16;
+    constexpr int SU = 8;  // 64 rows / (768 threads / 96 units): the host checks 64 == SU * dr
+    const MhaArgs &a = qa.m;
+    extern __shared__ __align__(256) unsigned char qm_smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r16 = lane & 15, g = lane >> 4, sel = g >> 1, gbit = g & 1;
+    const int S = a.S, in = qa.in;
+    const int stride = in * 2, upr = in >> 3;
+    unsigned char *xs = qm_smem;                                                  // [64][in] binary16, swizzled
+    _Float16 *Qs = reinterpret_cast<_Float16 *>(qm_smem + (size_t)kQkvRows * stride);  // [128][ldk]
+    _Float16 *Ks = Qs + L::k_halfs;                                               // [128][ldk]
+    _Float16 *Vt = Ks + L::k_halfs;                                               // [64][ldvt]
+    float2 *stat = reinterpret_cast<float2 *>(Vt + L::vt_halfs);                 // [128] -mean * rstd and rstd of the sequence's rows
+    _Float16 *gb = reinterpret_cast<_Float16 *>(stat + kKeyBlock);               // gamma | beta
+    float2 *spart = reinterpret_cast<float2 *>(xs);                              // [16][128] partial sums, before xs is written
+
+    const int xcd = blockIdx.x % kXcds, k_in_xcd = blockIdx.x / kXcds;
+    const int b = xcd + kXcds * (k_in_xcd / a.nh), h = k_in_xcd % a.nh;
+    if (b >= qa.B) return;  // padding of the last round (whole workgroup)
+    const size_t row0 = (size_t)b * S;
+    const int nhalf = (S + kQkvRows - 1) / kQkvRows;
+
+    // ---- requests in the order their results are needed (they return in order): the partial row sums, gamma and
+    // beta, the first 64 rows, then the wave's slots
+    // partial sums: thread t takes row t % 128 of groups t / 128, + 6 and + 12
+    const int st_row = threadIdx.x & (kKeyBlock - 1), st_g = threadIdx.x >> 7;
+    float2 ps[3];
+    {
+        const int tok = min(st_row, S - 1);
+#pragma unroll
+        for (int k = 0; k < 3; k++)
+            ps[k] = *reinterpret_cast<const float2 *>(qa.st_in + ((size_t)min(st_g + 6 * k, qa.st_groups - 1) * qa.T + row0 + tok) * 2);
+    }
+    // thread t owns columns 4c .. 4c + 3 and in / 2 + 4c .. + 3, c = t % upr, of staged rows t / upr + u * dr (the host
+    // checks that 768 % upr == 0): the lanes of a request read consecutive 16 bytes
+    const int n_dr = (int)blockDim.x / upr, n_r0 = (int)threadIdx.x / upr, n_c8 = (int)threadIdx.x - n_r0 * upr;
+    h8 gam_in = {}, bet_in = {};
+    if ((int)threadIdx.x < upr) {
+        gam_in = reinterpret_cast<const h8 *>(qa.gamma)[threadIdx.x];
+        bet_in = reinterpret_cast<const h8 *>(qa.beta)[threadIdx.x];
+    }
+    f4 s32[SU][2];
+    // rows [from, to) of the thread's eight in the given half (the thread's place passes through an empty asm: seen as
+    // loop-invariant, the addresses of all sixteen rows are computed up front, 32 registers that spill)
+    auto request_rows = [&](int half, auto from, auto to) {
+        int r0_now = n_r0, c8_now = n_c8;
+        asm volatile("" : "+v"(r0_now), "+v"(c8_now));
+#pragma unroll
+        for (int u = decltype(from)::value; u < decltype(to)::value; u++) {
+            const int tok = min(half * kQkvRows + r0_now + u * n_dr, S - 1);
+            const f4 *p = reinterpret_cast<const f4 *>(qa.X32 + (row0 + tok) * in) + c8_now;
+            s32[u][0] = p[0];
+            s32[u][1] = p[upr];
+        }
+    };
+    using i0 = std::integral_constant<int, 0>;
+    using iPF = std::integral_constant<int, PF>;
+    using iSU = std::integral_constant<int, SU>;
+    // (results return in the order of the requests of the whole compute unit: behind this barrier the few bytes the
+    // statistics wait for are not queued behind other waves' rows)
+    __syncthreads();
+    request_rows(0, i0{}, iSU{});
+
+    // ---- this wave's block-row of W_qkv: part 0 / 1 / 2 = Q / K / V, four block-rows of the head each
+    const int part = wave >> 2, sub = wave & 3;
+    const int rb = part * (a.nh * 4) + 4 * h + sub;  // block-row of W_qkv
+    const size_t slab = (size_t)h * kQkvWaves + wave;
+    const int nsl = ET_QM_CONST(int32_t, qa.pn)[slab];
+    uint32_t offs[CAP];
+    {
+        const auto *op = ET_QM_CONST(uint32_t, qa.poff) + slab * CAP;
+#pragma unroll
+        for (int q4 = 0; q4 < CAP / 4; q4++) {
+            if (4 * q4 < nsl) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) offs[4 * q4 + r] = op[4 * q4 + r];
+            }
+        }
+    }
+    const _Float16 *wp = qa.pw + slab * CAP * 512 + lane * 8;
+    constexpr bool HOLD = NPASS == 1;
+    constexpr int WN = CAP / NPASS;  // slots in registers at a time
+    static_assert(WN % 4 == 0 && WN * NPASS == CAP, "slots are fetched in groups of four");
+    h8 w[WN];
+    // (base and swizzle term pass through an empty asm: seen as loop-invariant, the per-slot addresses and LDS offsets
+    // are computed once in front of the loop, three registers per slot that then spill)
+    auto request_slots = [&](int first) {
+        const _Float16 *wp_now = wp + first * 512;
+        asm volatile("" : "+v"(wp_now));
+#pragma unroll
+        for (int q4 = 0; q4 < WN / 4; q4++) {
+            if (first + 4 * q4 < nsl) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) w[4 * q4 + r] = *reinterpret_cast<const h8 *>(wp_now + (4 * q4 + r) * 512);
+            }
+        }
+    };
+    if constexpr (HOLD) request_slots(0);
+    // bias: Q and K lanes end with features 4g .. 4g + 3 of a token, V lanes with feature r16 of four tokens
+    float bq[4] = {0.f, 0.f, 0.f, 0.f};
+    if (qa.bias) {
+        if (part < 2) {
+            const h4 t = *reinterpret_cast<const h4 *>(qa.bias + rb * 16 + g * 4);
+#pragma unroll
+            for (int e = 0; e < 4; e++) bq[e] = (float)t[e];
+        } else {
+            const float t = (float)qa.bias[rb * 16 + r16];
+#pragma unroll
+            for (int e = 0; e < 4; e++) bq[e] = t;
+        }
+    }
+    const unsigned kx = (unsigned)((gbit ^ r16) & 15) << 4;
+
+    if (nhalf * kQkvRows < kKeyBlock) {
+        // keys that no round stages must hold finite values: their probabilities are exactly zero, and 0 x NaN is not
+        uint4 *z = reinterpret_cast<uint4 *>(Ks);
+        for (int i = threadIdx.x; i < (int)((L::k_halfs + L::vt_halfs) * sizeof(_Float16) / 16); i += blockDim.x)
+            z[i] = uint4{0u, 0u, 0u, 0u};
+    }
+    // ---- mean and rstd of the sequence's rows: the partial sums are added per row in group order through LDS
+#pragma unroll
+    for (int k = 0; k < 3; k++)
+        if (st_g + 6 * k < kMaxStatGroups) spart[(st_g + 6 * k) * kKeyBlock + st_row] = ps[k];
+    if ((int)threadIdx.x < upr) {
+        reinterpret_cast<h8 *>(gb)[threadIdx.x] = gam_in;
+        reinterpret_cast<h8 *>(gb + in)[threadIdx.x] = bet_in;
+    }
+    __syncthreads();
+    if (threadIdx.x < kKeyBlock) {
+        float s1 = 0.0f, s2 = 0.0f;
+        for (int gi = 0; gi < qa.st_groups; gi++) {
+            const float2 pr = spart[gi * kKeyBlock + threadIdx.x];
+            s1 += pr.x;
+            s2 += pr.y;
+        }
+        const float mean = s1 / (float)in;
+        const float2 mine = {mean, rsqrtf(fmaxf(__builtin_fmaf(-mean, mean, s2 / (float)in), 0.0f) + qa.eps)};
+        stat[threadIdx.x] = float2{-mean * mine.y, mine.y};
+        if (qa.fin_out && h == 0 && (int)threadIdx.x < S)
+            *reinterpret_cast<float2 *>(qa.fin_out + 2 * (row0 + threadIdx.x)) = mine;
+    }
+    __syncthreads();  // the statistics are complete and the partial sums read: xs may be written
+
+    for (int half = 0; half < nhalf; half++) {
+        const int tokbase = half * kQkvRows;
+        if (half > 0) request_rows(half, iPF{}, iSU{});  // what was not requested ahead
+        {
+            int r0_now = n_r0, c8_now = n_c8;
+            asm volatile("" : "+v"(r0_now), "+v"(c8_now));
+            const h4 gam0 = reinterpret_cast<const h4 *>(gb)[c8_now], gam1 = reinterpret_cast<const h4 *>(gb)[upr + c8_now];
+            const h4 bet0 = reinterpret_cast<const h4 *>(gb + in)[c8_now], bet1 = reinterpret_cast<const h4 *>(gb + in)[upr + c8_now];
+            const int unit0 = c8_now >> 1, unit1 = (upr + c8_now) >> 1, piece = (c8_now & 1) << 3;  // upr is even
+#pragma unroll
+            for (int u = 0; u < SU; u++) {
+                const int row = r0_now + u * n_dr;
+                const float2 st = stat[tokbase + row];  // rstd and -mean * rstd: two fused multiply-adds per value
+                h4 lo, hi;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    lo[e] = (_Float16)__builtin_fmaf(__builtin_fmaf(s32[u][0][e], st.y, st.x), (float)gam0[e], (float)bet0[e]);
+                    hi[e] = (_Float16)__builtin_fmaf(__builtin_fmaf(s32[u][1][e], st.y, st.x), (float)gam1[e], (float)bet1[e]);
+                }
+                unsigned char *xr = xs + row * stride + piece;
+                *reinterpret_cast<h4 *>(xr + ((unit0 ^ (row & 15)) << 4)) = lo;
+                *reinterpret_cast<h4 *>(xr + ((unit1 ^ (row & 15)) << 4)) = hi;
+                if constexpr (HOLD) {
+                    // the registers of a row go to the same row of the next 64 the moment they are free: the memory
+                    // pipe stays busy through the normalisation and the products
+                    if (u < PF && half + 1 < nhalf) {
+                        const int tok = min(tokbase + kQkvRows + row, S - 1);
+                        const f4 *p = reinterpret_cast<const f4 *>(qa.X32 + (row0 + tok) * in) + c8_now;
+                        s32[u][0] = p[0];
+                        s32[u][1] = p[upr];
+                    }
+                }
+            }
+        }
+        if constexpr (!HOLD) {
+            request_slots(0);  // (after the rows: they and a part of the slots do not fit in registers together)
+            if (half + 1 < nhalf) request_rows(half + 1, i0{}, iPF{});  // in flight during the products
+        }
+        __syncthreads();
+        // ---- the wave's block-row times the four 16-token tiles of the staged rows
+        unsigned kx_now = kx, sel_now = (unsigned)sel << 4;
+        asm volatile("" : "+v"(kx_now), "+v"(sel_now));
+        f4 acc[4];
+#pragma unroll
+        for (int mt = 0; mt < 4; mt++) acc[mt] = f4{0.f, 0.f, 0.f, 0.f};
+        // Q, K: features x tokens (a lane ends with four features of a token); V: tokens x features (a lane ends with
+        // four consecutive tokens of a feature, a piece of a V^T row).  Two loops under one wave-uniform branch: as a
+        // select per product the compiler computes both orientations.
+        auto products = [&](auto swapped, auto first) {
+            constexpr int P0 = decltype(first)::value;
+#pragma unroll
+            for (int p = 0; p < WN; p++) {
+                if ((p & 3) == 0 && P0 + p >= nsl) break;  // wave-uniform: nothing was fetched beyond
+                const unsigned o = ((offs[P0 + p] >> sel_now) & 0xffffu) ^ kx_now;
+#pragma unroll
+                for (int mt = 0; mt < 4; mt++) {
+                    const h8 x = *reinterpret_cast<const h8 *>(xs + (unsigned)((mt * 16 + r16) * stride) + o);
+                    if constexpr (decltype(swapped)::value) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(x, w[p], acc[mt], 0, 0, 0);
+                    else acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[p], x, acc[mt], 0, 0, 0);
+                }
+            }
+        };
+        if (part < 2) products(std::false_type{}, i0{});
+        else products(std::true_type{}, i0{});
+        auto next_part = [&](auto first) {
+            __builtin_amdgcn_sched_barrier(0);  // not above the products that still read the registers' last contents
+            request_slots(decltype(first)::value);
+            if (part < 2) products(std::false_type{}, first);
+            else products(std::true_type{}, first);
+        };
+        if constexpr (NPASS >= 2) next_part(std::integral_constant<int, WN>{});
+        if constexpr (NPASS >= 3) next_part(std::integral_constant<int, 2 * WN>{});
+#pragma unroll
+        for (int mt = 0; mt < 4; mt++) {
+            const h4 v = {(_Float16)(acc[mt][0] + bq[0]), (_Float16)(acc[mt][1] + bq[1]), (_Float16)(acc[mt][2] + bq[2]),
+                          (_Float16)(acc[mt][3] + bq[3])};
+            if (part < 2) {
+                _Float16 *dst = (part == 0 ? Qs : Ks) + (tokbase + mt * 16 + r16) * L::ldk + sub * 16 + 4 * g;
+                *reinterpret_cast<h4 *>(dst) = v;
+            } else {
+                // keys 4kg .. 4kg + 3, kg = 16 half + 4 mt + g, at their place in the V^T row of feature 16 sub + r16
+                const int pos = (32 * (2 * half + (mt >> 1)) + 8 * g + 4 * (mt & 1)) ^ vt_swizzle<HD>(sub);
+                *reinterpret_cast<h4 *>(Vt + (sub * 16 + r16) * L::ldvt + pos) = v;
+            }
+        }
+        if (half + 1 < nhalf) __syncthreads();  // every wave is done with the staged rows
+    }
+    __syncthreads();  // Q, K and V^T of the head are complete
+    if (wave * 16 >= S) return;  // 16 queries per wave: the waves beyond the sequence are done
+
+    // ---- the attention core on the staged head (one key block: S <= 128)
+    int q[QT] = {wave * 16 + r16};
+    bool q_ok[QT] = {q[0] < S};
+    int klimit = S;
+    if (a.lens) klimit = min(S, max(a.lens[b], 0));
+    if (a.causal) klimit = min(klimit, (wave + 1) * 16);
+    const int vlive = HD;
+    h8 qf[QT][KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) qf[0][ks] = *reinterpret_cast<const h8 *>(Qs + (wave * 16 + r16) * L::ldk + 32 * ks + 8 * g);
+    f4 o[QT][DB];
+    float m_run[QT] = {-INFINITY}, l_part[QT] = {0.0f};
+#pragma unroll
+    for (int d = 0; d < DB; d++) o[0][d] = f4{0.f, 0.f, 0.f, 0.f};
+    const int k0 = 0;
+    if (klimit > 0) {
+#include "attention_core.inc"
+        const bool plain = a.mask == nullptr && a.scale_log2e > 0.0f && !a.causal;
+        if (plain) multiply(std::true_type{});
+        else multiply(std::false_type{});
+    }
+    float l = rows_sum(l_part[0]);
+    const float inv = l > 0.0f ? 1.0f / l : 0.0f;
+    if (q_ok[0]) {
+        _Float16 *zp = a.Z + (row0 + q[0]) * a.ldz + h * HD + 4 * g;
+#pragma unroll
+        for (int d = 0; d < DB; d++) {
+            h4 out;
+#pragma unroll
+            for (int j = 0; j < 4; j++) out[j] = (_Float16)(o[0][d][j] * inv);
+            *reinterpret_cast<h4 *>(zp + 16 * d) = out;
+        }
+    }
+}
+
+template <int CAP, int PF, int NPASS> static int launch_qkv_mha(const QkvMhaArgs &qa, size_t lds, hipStream_t stream) {
+    auto kernel = qkv_mha_kernel<CAP, PF, NPASS>;
+    static bool raised = false;  // per instantiation
+    if (!raised) {
+        ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        raised = true;
+    }
+    const int rounds = (qa.B + kXcds - 1) / kXcds;
+    kernel<<<dim3((unsigned)(rounds * kXcds * qa.m.nh)), kQkvWaves * 64, lds, stream>>>(qa);
+    return check_launch("qkv_mha_kernel");
+}
+
 }  // namespace et
 
 using namespace et;
@@ -694,6 +874,122 @@ int et_mha_compactv_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *Vc, int 
     if (hd <= 32) return launch_mha<32, true>(args, B, as_stream(stream));
     if (hd <= 64) return launch_mha<64, true>(args, B, as_stream(stream));
     return launch_mha<128, true>(args, B, as_stream(stream));
+}
+
+
+int et_norm_qkv_mha_f32in_supported(int B, int S, int in, int nhead, int hd) {
+    return B > 0 && S > 0 && S % 16 == 0 && S <= kKeyBlock && in == 768 && nhead > 0 && hd == 64 ? 1 : 0;
+}
+
+int et_qkv_heads_pack_create(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles, int in, int nhead,
+                             et_bsr_pack *pack) {
+    ET_REQUIRE(pack != nullptr, ET_ERR_INVALID_ARG, "et_qkv_heads_pack_create: pack is NULL");
+    *pack = nullptr;
+    ET_REQUIRE(row_ptr && col_idx && tiles, ET_ERR_INVALID_ARG, "et_qkv_heads_pack_create: NULL pointer");
+    ET_REQUIRE(et_norm_qkv_mha_f32in_supported(1, 16, in, nhead, 64) == 1, ET_ERR_UNSUPPORTED,
+               "et_qkv_heads_pack_create: in=%d nhead=%d outside the fused form (768-wide input, heads of 64)", in, nhead);
+    const int nbr = 3 * nhead * 4, bc = in / 16;  // block-rows of W_qkv: Q | K | V, four per head each
+    std::vector<int32_t> rp((size_t)nbr + 1);
+    ET_HIP(hipMemcpy(rp.data(), row_ptr, rp.size() * 4, hipMemcpyDeviceToHost));
+    ET_REQUIRE(rp[0] == 0, ET_ERR_INVALID_ARG, "et_qkv_heads_pack_create: row_ptr must start at 0");
+    for (int r = 0; r < nbr; r++)
+        ET_REQUIRE(rp[(size_t)r + 1] >= rp[(size_t)r], ET_ERR_INVALID_ARG, "et_qkv_heads_pack_create: row_ptr decreases");
+    const int ntile = rp[(size_t)nbr];
+    std::vector<int32_t> ci((size_t)std::max(ntile, 1));
+    if (ntile) ET_HIP(hipMemcpy(ci.data(), col_idx, (size_t)ntile * 4, hipMemcpyDeviceToHost));
+    for (int t = 0; t < ntile; t++)
+        ET_REQUIRE(ci[(size_t)t] >= 0 && ci[(size_t)t] < bc, ET_ERR_INVALID_ARG,
+                   "et_qkv_heads_pack_create: column-tile index %d of tile %d outside [0, %d)", ci[(size_t)t], t, bc);
+    int most = 1;
+    for (int r = 0; r < nbr; r++) most = std::max(most, (rp[(size_t)r + 1] - rp[(size_t)r] + 1) / 2);
+    const int cap = most <= 8 ? 8 : most <= 12 ? 12 : most <= 16 ? 16 : 24;  // the kernel's instantiations
+    ET_REQUIRE(cap <= 24, ET_ERR_UNSUPPORTED, "et_qkv_heads_pack_create: a block-row of %d slots exceeds a wave's 24", most);
+    const size_t nslab = (size_t)nhead * kQkvWaves;
+    std::vector<int32_t> order(nslab * cap * 2, -1), tab(nslab, 0);
+    std::vector<uint32_t> off(nslab * cap, 0);
+    for (int h = 0; h < nhead; h++) {
+        for (int wv = 0; wv < kQkvWaves; wv++) {
+            const int rb = (wv >> 2) * (nhead * 4) + 4 * h + (wv & 3);
+            const size_t slab = (size_t)h * kQkvWaves + wv;
+            int p = 0;
+            for (int t = rp[(size_t)rb]; t < rp[(size_t)rb + 1]; t += 2, p++) {
+                const bool two = t + 1 < rp[(size_t)rb + 1];
+                order[(slab * cap + p) * 2] = t;
+                order[(slab * cap + p) * 2 + 1] = two ? t + 1 : -1;
+                off[slab * cap + p] = (uint32_t)(ci[(size_t)t] * 32) | ((uint32_t)(ci[(size_t)(two ? t + 1 : t)] * 32) << 16);
+            }
+            tab[slab] = p;
+        }
+    }
+    et_bsr_pack_s *p = new (std::nothrow) et_bsr_pack_s;
+    ET_REQUIRE(p != nullptr, ET_ERR_ALLOC, "et_qkv_heads_pack_create: out of host memory");
+    p->in = in;
+    p->out = nbr * 16;
+    p->mt = 4;
+    p->ngroups = nhead;
+    p->nwave = kQkvWaves;
+    p->cap = cap;
+    p->flags = ET_PACK_QKV_HEADS;
+    p->lds = (size_t)kQkvRows * in * 2 + (size_t)(2 * MhaLds<64>::k_halfs + MhaLds<64>::vt_halfs) * sizeof(_Float16) +
+             kKeyBlock * sizeof(float2) + (size_t)in * 4;
+    const int s = pack_upload(*p, off, tab, order, tiles);
+    if (s != ET_OK) {
+        delete p;
+        return s;
+    }
+    *pack = p;
+    return ET_OK;
+}
+
+int et_norm_qkv_mha_f32in(et_bsr_pack pack, const float *V, const float *stats, int stat_groups, const et_f16 *gamma,
+                          const et_f16 *beta, float eps, float *fin_out, const et_f16 *bias_qkv, et_f16 *Z, int ldz,
+                          const et_f16 *mask, const int32_t *lens, int B, int S, float scale, int flags, et_stream stream) {
+    ET_REQUIRE(pack != nullptr && (pack->flags & ET_PACK_QKV_HEADS), ET_ERR_INVALID_ARG,
+               "et_norm_qkv_mha_f32in: needs a pack from et_qkv_heads_pack_create");
+    ET_REQUIRE(V && stats && gamma && beta && Z, ET_ERR_INVALID_ARG, "et_norm_qkv_mha_f32in: NULL pointer");
+    const int nh = pack->ngroups, in = pack->in;
+    ET_REQUIRE(B >= 0 && et_norm_qkv_mha_f32in_supported(std::max(B, 1), S, in, nh, 64) == 1, ET_ERR_UNSUPPORTED,
+               "et_norm_qkv_mha_f32in: B=%d S=%d: sequences of a multiple of 16 up to %d tokens", B, S, kKeyBlock);
+    ET_REQUIRE(stat_groups >= 1 && stat_groups <= kMaxStatGroups, ET_ERR_INVALID_ARG, "et_norm_qkv_mha_f32in: stat_groups=%d",
+               stat_groups);
+    ET_REQUIRE((flags & ~ET_MHA_CAUSAL) == 0, ET_ERR_INVALID_ARG, "et_norm_qkv_mha_f32in: flags=%d", flags);
+    ET_REQUIRE(ldz >= nh * 64 && ldz % 4 == 0 && (reinterpret_cast<uintptr_t>(Z) & 7) == 0 &&
+                   (reinterpret_cast<uintptr_t>(V) & 15) == 0,
+               ET_ERR_UNSUPPORTED, "et_norm_qkv_mha_f32in: Z must be 8-byte and V 16-byte aligned, ldz >= nhead * 64");
+    if (B == 0) return ET_OK;
+    QkvMhaArgs qa{};
+    qa.m.Z = reinterpret_cast<_Float16 *>(Z);
+    qa.m.mask = reinterpret_cast<const _Float16 *>(mask);
+    qa.m.lens = lens;
+    qa.m.ldz = ldz;
+    qa.m.S = S;
+    qa.m.nh = nh;
+    qa.m.hd = 64;
+    qa.m.nbh = B * nh;
+    qa.m.scale_log2e = scale * kLog2e;
+    qa.m.causal = (flags & ET_MHA_CAUSAL) ? 1 : 0;
+    qa.pw = static_cast<const _Float16 *>(pack->pw);
+    qa.poff = static_cast<const uint32_t *>(pack->poff);
+    qa.pn = static_cast<const int32_t *>(pack->ptab);
+    qa.bias = reinterpret_cast<const _Float16 *>(bias_qkv);
+    qa.cap = pack->cap;
+    qa.in = in;
+    qa.T = B * S;
+    qa.B = B;
+    qa.X32 = V;
+    qa.st_in = stats;
+    qa.st_groups = stat_groups;
+    qa.gamma = reinterpret_cast<const _Float16 *>(gamma);
+    qa.beta = reinterpret_cast<const _Float16 *>(beta);
+    qa.eps = eps;
+    qa.fin_out = fin_out;
+    switch (pack->cap) {
+        case 8: return launch_qkv_mha<8, 8, 1>(qa, pack->lds, as_stream(stream));
+        case 12: return launch_qkv_mha<12, 4, 1>(qa, pack->lds, as_stream(stream));
+        case 16: return launch_qkv_mha<16, 4, 2>(qa, pack->lds, as_stream(stream));
+        case 24: return launch_qkv_mha<24, 4, 3>(qa, pack->lds, as_stream(stream));
+        default: return fail(ET_ERR_INVALID_ARG, "et_norm_qkv_mha_f32in: no kernel for %d slots per wave", pack->cap);
+    }
 }
 
 }  // extern "C"

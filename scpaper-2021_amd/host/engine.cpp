@@ -22,6 +22,7 @@ struct ILayer {
     virtual void forward_mixed(float *out32, half *out16, const float *src32, half *src16, stream_t stream) = 0;
     virtual bool split_ok() const = 0;
     virtual void enable_split() = 0;
+    virtual bool enable_fused_qkv() = 0;
     virtual et::SplitSum forward_split(const et::SplitSum *in, const float *x32, half *x16, stream_t stream) = 0;
     virtual void finish_split(float *out32, half *out16, const et::SplitSum &s, stream_t stream) = 0;
     virtual bool chain_parts(et::ChainParts &p) = 0;
@@ -40,6 +41,7 @@ template <typename EncoderT> struct LayerOf final : ILayer {
     }
     bool split_ok() const override { return enc->split_ok(); }
     void enable_split() override { enc->enable_split(); }
+    bool enable_fused_qkv() override { return enc->enable_fused_qkv(); }
     et::SplitSum forward_split(const et::SplitSum *in, const float *x32, half *x16, stream_t stream) override {
         return enc->forward_split(in, x32, x16, stream);
     }
@@ -88,6 +90,7 @@ struct et_model_s {
     std::vector<half> mask;  // empty = no additive mask
     bool finalized = false;
     bool split = false;  // mixed precision with SkipLayerNorm folded into the projections
+    bool fused_qkv = false;  // and the QKV projection of every layer after the first inside its attention kernel
     // split, with everything between two attention kernels in one launch (et_encoder_chain_f32):
     // one description per layer and the barrier counters of all layers, cleared at the start of a forward
     bool chain = false;
@@ -486,11 +489,22 @@ int et_model_finalize(et_model m) {
             for (auto &b : m->pp32) b = std::make_unique<et::DeviceBuffer<float>>(act_elems);
             for (auto &l : m->layers) l->enable_mixed();
             // mixed == 1: the engine folds SkipLayerNorm into the projections where every layer can
-            m->split = (m->desc.mixed == 1 || m->desc.mixed == 3) && !m->layers.empty();
+            m->split = (m->desc.mixed == 1 || m->desc.mixed == 3 || m->desc.mixed == 4) && !m->layers.empty();
             for (auto &l : m->layers) m->split = m->split && l->split_ok();
             if (m->split) {
                 for (auto &l : m->layers) l->enable_split();
                 m->chain = m->desc.mixed == 3 && build_chain(*m);
+                // The QKV projection inside the attention kernel: asked for (mixed == 4), or where it measured faster than
+                // the two launches it replaces — one workgroup per (sequence, head) that reads and normalises its whole
+                // sequence: 12-layer 768-wide stacks at 80 / 90 % sparsity ran 0.89 - 0.97 of the five-launch time with
+                // 144 to 288 such workgroups and sequences of 64 or 128 tokens, the same at 96 and from 384 on, and
+                // 1.04 - 1.11 of it at 48 workgroups or sequences of 32.
+                const long heads = (long)m->desc.batch * m->desc.nhead;
+                const bool pays = heads >= 120 && heads <= 288 && m->desc.seq_len >= 48;
+                if ((m->desc.mixed == 4 || (m->desc.mixed == 1 && pays)) && m->layers.size() > 1) {
+                    m->fused_qkv = true;
+                    for (size_t i = 1; i < m->layers.size(); i++) m->fused_qkv = m->layers[i]->enable_fused_qkv() && m->fused_qkv;
+                }
             }
         }
         etChk(et_stream_create(&m->own_stream));
@@ -577,7 +591,7 @@ int et_model_sync(et_model m) {
 int et_model_launches_per_layer(et_model m, int *launches) {
     return guarded([&]() -> int {
         et::require(m != nullptr && launches != nullptr, "et_model_launches_per_layer: NULL argument");
-        *launches = !m->finalized ? 0 : m->chain ? 2 : m->split ? 5 : 7;
+        *launches = !m->finalized ? 0 : m->chain ? 2 : m->fused_qkv ? 4 : m->split ? 5 : 7;
         return ET_OK;
     });
 }

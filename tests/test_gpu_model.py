@@ -86,7 +86,7 @@ TOL_F16_DEEP = 5e-2          # all-fp16 storage over 12+ layers: two realisation
 
 
 @pytest.mark.parametrize("seed0,xseed,mode", [(100, 4, 1), (300, 307, 1), (500, 507, 1), (100, 4, 2), (100, 4, 3),
-                                               (300, 307, 3)])
+                                               (300, 307, 3), (100, 4, 4), (300, 307, 4)])
 def test_bert_base_12_layers_batch8_tile80_attention_aware_mixed(et, seed0, xseed, mode):
     """The headline configuration in the engine's mixed-precision mode: 12 layers, B8 S128, 80 %
     tile sparsity, 25 % of the V rows (and the matching O columns) dead in head-aligned groups."""
@@ -102,6 +102,58 @@ def test_bert_base_12_layers_batch8_tile80_attention_aware_mixed(et, seed0, xsee
     print(f"12-layer B8 S128 mixed (mode {mode}) seed {seed0}: vs fp32 forward {e32:.3e}, vs mixed oracle {em:.3e}")
     assert e32 <= TOL_MIXED_VS_F32 and em <= TOL_MIXED_VS_ORACLE
     assert np.array_equal(got[0], got[1])
+    if mode == 4:
+        assert m.launches_per_layer() == 4, "the QKV projection did not move into the attention kernel"
+
+
+@pytest.mark.parametrize("S,B,sp,padded,causal", [(128, 3, 0.8, True, False), (48, 5, 0.9, False, True),
+                                                  (64, 9, 0.5, True, True), (16, 1, 0.95, False, False)])
+def test_qkv_inside_attention_stacks(et, S, B, sp, padded, causal):
+    """mixed = 4: the layers after the first project Q, K and V inside their attention kernel (768-wide models with
+    heads of 64, sequences up to 128 tokens): padded, causal, short and odd batch counts, block-rows of few and of
+    many tiles; against the oracle and against the five-launch form (the same arithmetic up to the order of the
+    sums of the row statistics and one fused multiply-add in the normalisation)."""
+    H, nh, FF = 768, 12, 512
+    layers = [Hn.LayerWeights(H, nh, FF, sp, seed=900 + i) for i in range(3)]
+    lens = np.random.default_rng(S * B).integers(S // 2, S + 1, B).astype(np.int32) if padded else None
+    x = Hn.randn((B * S, H), 909)
+    m4 = Hn.build_model(et, layers, S, B, lens=lens, causal=causal, mixed=4)
+    m1 = Hn.build_model(et, layers, S, B, lens=lens, causal=causal, mixed=1)
+    got4, got1 = run_model(et, m4, x, reps=3), run_model(et, m1, x, reps=1)
+    assert m4.launches_per_layer() == 4 and m1.launches_per_layer() == 5
+    want = Hn.oracle_stack(x, layers, B, lens, causal=causal, store=torch.float16, resid=torch.float32)
+    a, b, c = got4[0].astype(np.float32), want.astype(np.float32), got1[0].astype(np.float32)
+    if lens is not None:  # rows past a sequence's length are padding: not compared
+        for i in range(B):
+            for t in (a, b, c):
+                t[i * S + lens[i]:(i + 1) * S] = 0
+    print(f"QKV inside attention S={S} B={B} sparsity {sp}: vs oracle {Hn.max_abs(a, b):.3e}, vs five launches {Hn.max_abs(a, c):.3e}")
+    assert Hn.max_abs(a, b) <= 4e-3 and Hn.max_abs(a, c) <= 4e-3
+    assert np.array_equal(got4[0], got4[1]) and np.array_equal(got4[1], got4[2])
+
+
+def test_qkv_inside_attention_chosen_by_batch(et):
+    """mixed = 1 takes the four-launch form by itself where it measured faster (here 12 sequences of 64 tokens on 12
+    heads) and keeps five launches elsewhere (8 sequences)."""
+    H, nh, FF, S = 768, 12, 512, 64
+    layers = [Hn.LayerWeights(H, nh, FF, 0.8, seed=920 + i) for i in range(2)]
+    for B, launches in ((12, 4), (8, 5)):
+        m = Hn.build_model(et, layers, S, B, mixed=1)
+        assert m.launches_per_layer() == launches
+        x = Hn.randn((B * S, H), 929)
+        got = run_model(et, m, x)[0]
+        want = Hn.oracle_stack(x, layers, B, store=torch.float16, resid=torch.float32)
+        assert Hn.max_abs(got, want) <= 4e-3
+
+
+def test_qkv_inside_attention_falls_back(et):
+    """Shapes the fused kernel does not take (here a 256-wide model) run mixed = 4 exactly as mixed = 1."""
+    H, nh, FF, S, B = 256, 4, 512, 64, 2
+    layers = [Hn.LayerWeights(H, nh, FF, 0.7, seed=940 + i) for i in range(2)]
+    x = Hn.randn((B * S, H), 949)
+    m4, m1 = Hn.build_model(et, layers, S, B, mixed=4), Hn.build_model(et, layers, S, B, mixed=1)
+    assert m4.launches_per_layer() == 5
+    assert np.array_equal(run_model(et, m4, x)[0], run_model(et, m1, x)[0])
 
 
 def test_bert_base_12_layers_all_fp16_storage(et):
