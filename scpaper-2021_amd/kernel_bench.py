@@ -185,6 +185,65 @@ class Bench:
             et.check(destroy(handle))
         self.record(f"linear_bsr16 ({entry})", f"T{T} in{n_in} out{n_out} sparsity {sparsity}", us, 2 * 256 * ntile * T, "mfma")
 
+    def qkv_mha(self, B, S, sparsity, launches, nh=12, hd=64, nset=12):
+        """The consumer QKV projection followed by the fused attention (two launches) against the attention kernel
+        that projects Q, K and V itself (et_norm_qkv_mha_f32in), on the binary32 sum and row statistics a producer
+        leaves; every launch of a graph on another of `nset` weight sets, as the layers of a stack."""
+        et, lib = self.et, self.lib
+        H, T = nh * hd, B * S
+        sets, ntile = [], 0
+        for i in range(nset):
+            row_ptr, col, ntile = self.tile_pattern(3 * H, H, sparsity, 50 + i)
+            d_rp, d_col = self.dev(row_ptr), self.dev(col)
+            tiles = self.dev(self.rnd((max(ntile, 1), 256), 0.02))
+            heads, consumer = C.c_void_p(), C.c_void_p()
+            et.check(lib.et_qkv_heads_pack_create(d_rp.ptr, d_col.ptr, tiles.ptr, H, nh, C.byref(heads)))
+            if lib.et_bsr16_pack_create(d_rp.ptr, d_col.ptr, tiles.ptr, T, H, 3 * H, 1, 0, C.byref(consumer)) != 0:
+                consumer = None
+            sets.append((d_rp, d_col, tiles, heads, consumer))
+        bias = self.dev(np.zeros(3 * H, np.float16))
+        v32 = self.rnd((T, H)).astype(np.float32)
+        groups = 4
+        stats = np.zeros((groups, T, 2), np.float32)
+        for gi in range(groups):
+            blk = v32[:, gi * H // groups:(gi + 1) * H // groups].astype(np.float64)
+            stats[gi, :, 0], stats[gi, :, 1] = blk.sum(1), (blk * blk).sum(1)
+        d_v, d_st = self.dev(v32), self.dev(stats)
+        gamma, beta = self.dev(np.ones(H, np.float16)), self.dev(np.zeros(H, np.float16))
+        fin = et.DeviceBuffer.empty((T, 2), np.float32)
+        z, qkv = self.empty((T, H)), self.empty((T, 3 * H))
+        scale, n = hd ** -0.5, {"i": 0}
+
+        def one_launch():
+            s = sets[n["i"] % nset]
+            n["i"] += 1
+            et.check(lib.et_norm_qkv_mha_f32in(s[3], d_v.ptr, d_st.ptr, groups, gamma.ptr, beta.ptr, 1e-5, fin.ptr, bias.ptr,
+                                               z.ptr, H, None, None, B, S, scale, 0, self.stream))
+
+        def two_launches():
+            s = sets[n["i"] % nset]
+            n["i"] += 1
+            if s[4] is not None:
+                et.check(lib.et_norm_linear_bsr16_packed_f32in(s[4], d_v.ptr, d_st.ptr, groups, gamma.ptr, beta.ptr, 1e-5,
+                                                               fin.ptr, bias.ptr, qkv.ptr, T, 0, self.stream))
+            else:
+                et.check(lib.et_norm_linear_bsr16_f32in(d_v.ptr, d_st.ptr, groups, gamma.ptr, beta.ptr, 1e-5, fin.ptr, None, None,
+                                                        s[0].ptr, s[1].ptr, s[2].ptr, bias.ptr, qkv.ptr, T, H, 3 * H, 0,
+                                                        self.stream))
+            et.check(lib.et_mha_fused_f16(qkv.ptr, qkv.offset(2 * H), qkv.offset(4 * H), 3 * H, 3 * H, 3 * H, z.ptr, H, None,
+                                          None, B, S, nh, hd, scale, 0, self.stream))
+
+        work = 2 * 256 * ntile * T + 4 * B * S * S * hd * nh
+        shape = f"B{B} S{S} nh{nh} hd{hd} sparsity {sparsity}"
+        self.record("norm + QKV + mha (two launches)", shape, self.time_us(two_launches, 4 * nset), work, "mfma")
+        if lib.et_norm_qkv_mha_f32in_supported(B, S, H, nh, hd) == 1:
+            self.record("norm_qkv_mha (one launch)", shape, self.time_us(one_launch, 4 * nset), work, "mfma")
+        et.check(lib.et_stream_sync(self.stream))
+        for s in sets:
+            et.check(lib.et_bsr16_pack_destroy(s[3]))
+            if s[4] is not None:
+                et.check(lib.et_bsr16_pack_destroy(s[4]))
+
     def machine(self):
         """What a kernel boundary costs and how fast a compute unit takes bytes in (et_probe_*): the two figures
         that bound a launch of a few hundred kilobytes per compute unit."""
@@ -430,7 +489,7 @@ def run_scale(b: Bench):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--set", choices=("configs", "scale", "vo", "mha", "plan", "machine", "all"), default="all")
+    ap.add_argument("--set", choices=("configs", "scale", "vo", "mha", "qkv", "plan", "machine", "all"), default="all")
     ap.add_argument("--json", default=None, help="also write the rows as JSON to this file")
     args = ap.parse_args()
     b = Bench()
@@ -449,6 +508,11 @@ def main():
         b.mha(16, 2048, 16, 64, 5)
         b.mha(16, 2048, 8, 128, 5)
         b.mha(16, 2048, 32, 32, 5)
+    if args.set == "qkv":
+        print("# the QKV projection inside the attention kernel against the two launches it replaces (768-wide, 12 heads of 64)")
+        for B, S, sp in ((4, 128, 0.8), (8, 128, 0.8), (8, 128, 0.9), (12, 128, 0.8), (16, 128, 0.8), (16, 128, 0.9), (24, 128, 0.8),
+                         (32, 128, 0.8), (16, 64, 0.8), (32, 64, 0.8), (64, 32, 0.8)):
+            b.qkv_mha(B, S, sp, 48)
     if args.set == "vo":
         print("# pre-computed-VO attention: probabilities through memory (mha_vo) and on chip (mha_vo_otf)")
         for B, N in ((1, 768), (4, 384), (8, 768), (16, 768)):
