@@ -553,6 +553,8 @@ int et_mha_compactv_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *Vc,
  * copies it once into the order the kernel reads (destroy with
  * et_bsr16_pack_destroy).  Limits, told by et_norm_qkv_mha_f32in_supported:
  * sequences of a multiple of 16 up to 128 tokens, 768-wide input, heads of 64.
+ * Rows of V past a sequence's length are projected like the others and their
+ * keys weighted with exactly zero: they must hold finite values.
  * Replaces Attention<cfg, isSingleKernel>::forward up to the O projection
  * (Attention/Attention_single.cu:10-108).
  * ------------------------------------------------------------------------ */

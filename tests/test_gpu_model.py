@@ -154,6 +154,11 @@ def test_qkv_inside_attention_falls_back(et):
     m4, m1 = Hn.build_model(et, layers, S, B, mixed=4), Hn.build_model(et, layers, S, B, mixed=1)
     assert m4.launches_per_layer() == 5
     assert np.array_equal(run_model(et, m4, x)[0], run_model(et, m1, x)[0])
+    # the BERT-large shape (1024 wide, 512 tokens) is outside it as well
+    layers, lens, x, S, B = bert_large_case(2)
+    m4, m1 = Hn.build_model(et, layers, S, B, lens=lens, mixed=4), Hn.build_model(et, layers, S, B, lens=lens, mixed=1)
+    assert m4.launches_per_layer() == 5
+    assert np.array_equal(run_model(et, m4, x)[0], run_model(et, m1, x)[0])
 
 
 def test_bert_base_12_layers_all_fp16_storage(et):

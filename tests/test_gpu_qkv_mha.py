@@ -24,6 +24,10 @@ CASES = [
     (2, 48, 0.5, 1, 2),
     (9, 128, 0.9, 8, 3),
     (1, 16, 0.95, 2, 0),
+    # the attention-block configuration of the benchmark: batch 1 / 4 / 16, 128 tokens, right padding in [64, 128]
+    (1, 128, 0.8, 8, 1),
+    (4, 128, 0.8, 8, 1),
+    (16, 128, 0.8, 8, 1),
 ]
 
 
