@@ -733,8 +733,8 @@ typedef struct et_model_desc {
                     * operands; input and output of et_model_forward stay binary16.
                     * 1: SkipLayerNorm is folded into the neighbouring tile-sparse projections
                     *    where the shapes allow (five launches per layer; four, as under 4, for
-                    *    the batch sizes where that measured faster: 10 to 24 sequences of 48
-                    *    to 128 tokens on 12 heads); 2: it keeps its own
+                    *    the batch sizes where that measured faster: 96 to 400 (sequence, head)
+                    *    pairs, from 120 on for sequences above 64 tokens); 2: it keeps its own
                     *    launches (seven); 3: as 1, with everything between two attention
                     *    kernels in one launch (et_encoder_chain_f32: two launches per layer)
                     *    where the shapes allow and the device runs it as it must, else as 1;

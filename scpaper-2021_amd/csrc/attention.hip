@@ -566,16 +566,19 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
             }
         }
     }
-    const _Float16 *wp = qa.pw + slab * CAP * 512 + lane * 8;
+    const size_t wp_off = slab * CAP * 512 + lane * 8;
     constexpr bool HOLD = NPASS == 1;
     constexpr int WN = CAP / NPASS;  // slots in registers at a time
     static_assert(WN % 4 == 0 && WN * NPASS == CAP, "slots are fetched in groups of four");
     h8 w[WN];
-    // (base and swizzle term pass through an empty asm: seen as loop-invariant, the per-slot addresses and LDS offsets
-    // are computed once in front of the loop, three registers per slot that then spill)
+    // (the slab's offset and the swizzle term pass through an empty asm: seen as loop-invariant, the per-slot addresses
+    // and LDS offsets are computed once in front of the loop, three registers per slot that then spill.  The offset
+    // and not the pointer: a pointer out of an asm has no address space left, and its loads would count as LDS
+    // accesses as well.)
     auto request_slots = [&](int first) {
-        const _Float16 *wp_now = wp + first * 512;
-        asm volatile("" : "+v"(wp_now));
+        size_t off_now = wp_off + (size_t)first * 512;
+        asm volatile("" : "+v"(off_now));
+        const _Float16 *wp_now = qa.pw + off_now;
 #pragma unroll
         for (int q4 = 0; q4 < WN / 4; q4++) {
             if (first + 4 * q4 < nsl) {
@@ -585,18 +588,12 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
         }
     };
     if constexpr (HOLD) request_slots(0);
-    // bias: Q and K lanes end with features 4g .. 4g + 3 of a token, V lanes with feature r16 of four tokens
-    float bq[4] = {0.f, 0.f, 0.f, 0.f};
+    // bias: Q and K lanes end with features 4g .. 4g + 3 of a token, V lanes with feature r16 of four tokens.  Kept as
+    // loaded and widened where it is added: a conversion here would wait for every request above.
+    uint2 bias_bits = {0u, 0u};
     if (qa.bias) {
-        if (part < 2) {
-            const h4 t = *reinterpret_cast<const h4 *>(qa.bias + rb * 16 + g * 4);
-#pragma unroll
-            for (int e = 0; e < 4; e++) bq[e] = (float)t[e];
-        } else {
-            const float t = (float)qa.bias[rb * 16 + r16];
-#pragma unroll
-            for (int e = 0; e < 4; e++) bq[e] = t;
-        }
+        if (part < 2) bias_bits = *reinterpret_cast<const uint2 *>(qa.bias + rb * 16 + g * 4);
+        else bias_bits.x = *reinterpret_cast<const unsigned short *>(qa.bias + rb * 16 + r16);
     }
     const unsigned kx = (unsigned)((gbit ^ r16) & 15) << 4;
 
@@ -702,6 +699,16 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
         };
         if constexpr (NPASS >= 2) next_part(std::integral_constant<int, WN>{});
         if constexpr (NPASS >= 3) next_part(std::integral_constant<int, 2 * WN>{});
+        float bq[4];
+        if (part < 2) {
+            const h4 t = __builtin_bit_cast(h4, bias_bits);
+#pragma unroll
+            for (int e = 0; e < 4; e++) bq[e] = (float)t[e];
+        } else {
+            const float t = (float)__builtin_bit_cast(_Float16, (unsigned short)bias_bits.x);
+#pragma unroll
+            for (int e = 0; e < 4; e++) bq[e] = t;
+        }
 #pragma unroll
         for (int mt = 0; mt < 4; mt++) {
             const h4 v = {(_Float16)(acc[mt][0] + bq[0]), (_Float16)(acc[mt][1] + bq[1]), (_Float16)(acc[mt][2] + bq[2]),

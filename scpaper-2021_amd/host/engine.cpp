@@ -496,11 +496,11 @@ int et_model_finalize(et_model m) {
                 m->chain = m->desc.mixed == 3 && build_chain(*m);
                 // The QKV projection inside the attention kernel: asked for (mixed == 4), or where it measured faster than
                 // the two launches it replaces — one workgroup per (sequence, head) that reads and normalises its whole
-                // sequence: 12-layer 768-wide stacks at 80 / 90 % sparsity ran 0.89 - 0.97 of the five-launch time with
-                // 144 to 288 such workgroups and sequences of 64 or 128 tokens, the same at 96 and from 384 on, and
-                // 1.04 - 1.11 of it at 48 workgroups or sequences of 32.
+                // sequence: 12-layer 768-wide stacks at 80 / 90 / 95 % sparsity ran 0.89 - 0.99 of the five-launch time
+                // with 96 to 384 such workgroups (sequences of 32 to 128 tokens), except 96 of them on sequences of 96 or
+                // 128 tokens (1.00 - 1.01); 1.04 - 1.05 at 72 and below, 1.09 - 1.11 at 768.
                 const long heads = (long)m->desc.batch * m->desc.nhead;
-                const bool pays = heads >= 120 && heads <= 288 && m->desc.seq_len >= 48;
+                const bool pays = heads >= 96 && heads <= 400 && (heads >= 120 || m->desc.seq_len <= 64);
                 if ((m->desc.mixed == 4 || (m->desc.mixed == 1 && pays)) && m->layers.size() > 1) {
                     m->fused_qkv = true;
                     for (size_t i = 1; i < m->layers.size(); i++) m->fused_qkv = m->layers[i]->enable_fused_qkv() && m->fused_qkv;
