@@ -190,7 +190,7 @@ template <> class Linear<tile_mat> {
     // in registers, token strips staged two ahead), where its launch fills the chip — at least 256 (strip, group)
     // pairs.  Measured against the plain call: 16384 x 768 -> 3072 43 against 60 us, -> 2304 32 against 45 us,
     // -> 768 16 against 20 us; 4096 x 768 -> 3072 15 against 19 us; 2048 x 768 -> 2304 7.9 against 10.5 us.
-    // Serves forward / forward_act (binary16 results); forward_f32 keeps the plain call.
+    // Serves forward / forward_act (binary16 results) and forward_f32 (binary32 results).
     pack_ptr pack_loop;
     static constexpr int kRowLoopMinRows = 2048;
     // ET_PACKED=0 in the environment keeps every Linear<tile_mat> on the unpacked kernels (for comparisons)
@@ -267,6 +267,11 @@ template <> class Linear<tile_mat> {
         if (plan) {
             etChk(et_linear_bsr16_planned_f16(plan.get(), et::f16(bias.get()), et::f16(input), nullptr, output, size,
                                               ET_ACT_NONE, stream));
+            return;
+        }
+        if (pack_loop) {
+            etChk(et_linear_bsr16_packed_f16(pack_loop.get(), et::f16(bias.get()), et::f16(input), nullptr, output, size,
+                                             ET_ACT_NONE, stream));
             return;
         }
         if (pack) {

@@ -183,7 +183,7 @@ int et_linear_bsr16_planned_f16(et_bsr_plan plan, const et_f16 *bias,
  * a workgroup keeps its share of the weight in registers and walks over
  * token strips staged two ahead, whole block-rows per wave, results stored
  * straight from the accumulators; such a pack serves
- * et_linear_bsr16_packed_f16 with a binary16 result only.  Replaces
+ * et_linear_bsr16_packed_f16 (binary16 or binary32 result) only.  Replaces
  * Linear<tile_mat>::forward (Linear/SPMM_tile.cu:312-324) for callers that keep
  * a Linear object. */
 typedef struct et_bsr_pack_s *et_bsr_pack;

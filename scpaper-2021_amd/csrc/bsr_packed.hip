@@ -406,8 +406,8 @@ int et_linear_bsr16_packed_f16(et_bsr_pack pack, const et_f16 *bias, const et_f1
     a.Y32 = Y32;
     a.act = act;
     if (pack->flags & ET_PACK_ROW_LOOP) {
-        ET_REQUIRE(Y != nullptr && (reinterpret_cast<uintptr_t>(Y) & 15) == 0, ET_ERR_UNSUPPORTED,
-                   "et_linear_bsr16_packed_f16: a row-loop pack stores binary16 results, 16-byte aligned");
+        ET_REQUIRE((reinterpret_cast<uintptr_t>(Y) & 15) == 0, ET_ERR_UNSUPPORTED,
+                   "et_linear_bsr16_packed_f16: a row-loop pack stores its results 16-byte aligned");
         return rowloop_launch(a, *pack, as_stream(stream));
     }
     return pk_dispatch_plain<false>(a, *pack, as_stream(stream));

@@ -62,7 +62,9 @@ __device__ __forceinline__ void rl_load_to_lds(const void *base, unsigned lane_o
 
 constexpr int kRlBuf = 3;  // strip buffers: the strip being multiplied and the two after it
 
-template <int MT, int CAP>
+// OUT32: the results are stored as binary32 (Y32; the unrounded accumulator plus bias, activated), one 16-byte store
+// per lane and 16-row block instead of packed binary16.
+template <int MT, int CAP, bool OUT32>
 __global__ __launch_bounds__(pk_max_waves(CAP, false) * 64) void bsr16_rowloop_kernel(const PackArgs a) {
     extern __shared__ __align__(256) unsigned char rl_smem[];
     const int lane = threadIdx.x & 63;
@@ -145,7 +147,7 @@ __global__ __launch_bounds__(pk_max_waves(CAP, false) * 64) void bsr16_rowloop_k
 #pragma unroll
     for (int m = 0; m < MT; m++) rowbase[m] = (unsigned)((m * 16 + r16) * stride);
     const int act = a.act;
-    const int spr = MT == 2 ? 1 : MT;  // store instructions per block-row of a whole strip
+    const int spr = OUT32 ? MT : MT == 2 ? 1 : MT;  // store instructions per block-row of a whole strip
 
     int slot = 0, s = s0;
     for (int r = 0; r < rounds; r++, s += step) {
@@ -200,7 +202,14 @@ __global__ __launch_bounds__(pk_max_waves(CAP, false) * 64) void bsr16_rowloop_k
 #pragma unroll
                 for (int m = 0; m < MT; m++)
                     out16[m] = __builtin_bit_cast(uint2, h4{(_Float16)v[m][0], (_Float16)v[m][1], (_Float16)v[m][2], (_Float16)v[m][3]});
-                if (whole) {  // exactly `spr` store instructions, whatever the lanes hold: the waits above count on it
+                if constexpr (OUT32) {
+                    // whole strips: exactly MT store instructions (rows past T exist only in the last strip of all)
+#pragma unroll
+                    for (int m = 0; m < MT; m++) {
+                        const int tok = tok0 + m * 16 + r16;
+                        if (whole || tok < a.T) *reinterpret_cast<f4 *>(a.Y32 + (size_t)tok * a.out + f0) = f4{v[m][0], v[m][1], v[m][2], v[m][3]};
+                    }
+                } else if (whole) {  // exactly `spr` store instructions, whatever the lanes hold: the waits above count on it
                     if constexpr (MT == 2) {
                         // 16-byte stores: an even and the next odd 16-lane row hold features 4g .. 4g + 7 of the same
                         // two tokens; the even row takes both quads of the first token, the odd row those of the second
@@ -226,8 +235,8 @@ __global__ __launch_bounds__(pk_max_waves(CAP, false) * 64) void bsr16_rowloop_k
 
 constexpr size_t kRlLdsBudget = 160 * 1024;
 
-template <int MT, int CAP> static int rl_launch(const PackArgs &a, const et_bsr_pack_s &p, hipStream_t stream) {
-    auto kernel = bsr16_rowloop_kernel<MT, CAP>;
+template <int MT, int CAP, bool OUT32> static int rl_launch(const PackArgs &a, const et_bsr_pack_s &p, hipStream_t stream) {
+    auto kernel = bsr16_rowloop_kernel<MT, CAP, OUT32>;
     if (p.lds > 64 * 1024) {
         static bool raised = false;  // per instantiation
         if (!raised) {
@@ -244,19 +253,20 @@ template <int MT, int CAP> static int rl_launch(const PackArgs &a, const et_bsr_
     return check_launch("bsr16_rowloop_kernel");
 }
 
-template <int MT> static int rl_dispatch_cap(const PackArgs &a, const et_bsr_pack_s &p, hipStream_t stream) {
+template <int MT, bool OUT32> static int rl_dispatch_cap(const PackArgs &a, const et_bsr_pack_s &p, hipStream_t stream) {
     switch (p.cap) {
-        case 8: return rl_launch<MT, 8>(a, p, stream);
-        case 12: return rl_launch<MT, 12>(a, p, stream);
-        case 16: return rl_launch<MT, 16>(a, p, stream);
-        case 20: return rl_launch<MT, 20>(a, p, stream);
-        case 24: return rl_launch<MT, 24>(a, p, stream);
+        case 8: return rl_launch<MT, 8, OUT32>(a, p, stream);
+        case 12: return rl_launch<MT, 12, OUT32>(a, p, stream);
+        case 16: return rl_launch<MT, 16, OUT32>(a, p, stream);
+        case 20: return rl_launch<MT, 20, OUT32>(a, p, stream);
+        case 24: return rl_launch<MT, 24, OUT32>(a, p, stream);
         default: return fail(ET_ERR_INVALID_ARG, "tile-sparse Linear (row loop): no kernel for %d slots per wave", p.cap);
     }
 }
 
 int rowloop_launch(const PackArgs &a, const et_bsr_pack_s &p, hipStream_t stream) {
-    return p.mt == 2 ? rl_dispatch_cap<2>(a, p, stream) : rl_dispatch_cap<1>(a, p, stream);
+    if (a.Y32) return p.mt == 2 ? rl_dispatch_cap<2, true>(a, p, stream) : rl_dispatch_cap<1, true>(a, p, stream);
+    return p.mt == 2 ? rl_dispatch_cap<2, false>(a, p, stream) : rl_dispatch_cap<1, false>(a, p, stream);
 }
 
 // The pack of the row-loop kernel: block-rows cut into `ngroups` contiguous groups of about equally

@@ -403,11 +403,11 @@ class Bench:
                                                                (H // nh) ** -0.5, 0, self.stream)), launches)
         self.record_f32("mha_fused_f32", f"B{B} S{S} nh{nh} hd{H // nh}", us, 4 * B * S * S * H)
 
-    def stack(self, name, H, nh, FF, S, B, nlayer, sparsity, lens, replays=20):
+    def stack(self, name, H, nh, FF, S, B, nlayer, sparsity, lens, replays=20, mixed=0):
         """A whole encoder stack through the model handle (one HIP-graph replay per forward): every
         Linear tile-sparse at `sparsity` with its own seeded pattern, right padding `lens` or None."""
         et = self.et
-        m = et.Model(H, nh, FF, S, nlayer, batch=B, act=et.ACT_GELU, eps=1e-5, causal=False, use_graph=True)
+        m = et.Model(H, nh, FF, S, nlayer, batch=B, act=et.ACT_GELU, eps=1e-5, causal=False, use_graph=True, mixed=mixed)
         flops = 0
         for i in range(nlayer):
             for which, (o, n_in) in ((et.W_QKV, (3 * H, H)), (et.W_O, (H, H)), (et.W_FF1, (FF, H)), (et.W_FF2, (H, FF))):
@@ -431,7 +431,9 @@ class Bench:
             m.forward(y, x)
         m.sync()
         us = (time.perf_counter() - t0) * 1e6 / replays
-        self.record("encoder_stack", f"{name}: {B / us * 1e6:.0f} seq/s, {us / nlayer:.1f} us per layer", us, flops, "mfma")
+        mode = "binary32 residual stream" if mixed else "all activations binary16"
+        self.record("encoder_stack", f"{name}, {mode}, {m.launches_per_layer()} launches per layer: {B / us * 1e6:.0f} seq/s, "
+                                     f"{us / nlayer:.1f} us per layer", us, flops, "mfma")
 
     def record_f32(self, kernel, shape, us, flops):
         achieved, peak = flops / us / 1e6, 157.3

@@ -132,9 +132,19 @@ def test_linear_bsr16_row_loop(et, T, inp, out, sp, act):
         et.check(lib.et_linear_bsr16_packed_f16(pk.h, None, d_x.ptr, d_y2.ptr, None, T2, 0, None))
         want = L.linear(Hn.f32(x[:T2]), Hn.f32(w.dense), None, None, torch.float16).numpy()
         assert Hn.max_abs(d_y2.numpy(), want) <= 4e-3
-        # a binary32 result is not what this form stores
-        d_y32 = et.DeviceBuffer.empty((16, out), np.float32)
-        assert lib.et_linear_bsr16_packed_f16(pk.h, None, d_x.ptr, None, d_y32.ptr, 16, 0, None) == et.ET_ERR_UNSUPPORTED
+        # binary32 results: the accumulator plus bias, activated, unrounded (twice in a row, then a ragged row count)
+        d_y32 = et.DeviceBuffer.empty((T, out), np.float32)
+        want32 = L.linear(Hn.f32(x), Hn.f32(w.dense), Hn.f32(w.bias), ACT_NAME[act], None).numpy()
+        for rep in range(2):
+            et.check(lib.et_memset(d_y32.ptr, 0xFF, T * out * 4, None))  # NaN patterns: every element must be written
+            et.check(lib.et_linear_bsr16_packed_f16(pk.h, w.d_bias.ptr, d_x.ptr, None, d_y32.ptr, T, act, None))
+        got32 = d_y32.numpy()
+        assert not np.isnan(got32).any()
+        assert Hn.max_abs(got32, want32) <= 2e-3
+        d_y32b = et.DeviceBuffer.empty((T2, out), np.float32)
+        et.check(lib.et_memset(d_y32b.ptr, 0xFF, T2 * out * 4, None))
+        et.check(lib.et_linear_bsr16_packed_f16(pk.h, w.d_bias.ptr, d_x.ptr, None, d_y32b.ptr, T2, act, None))
+        assert np.array_equal(d_y32b.numpy(), got32[:T2])
 
 
 def test_row_loop_pack_rejects(et):
