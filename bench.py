@@ -154,7 +154,7 @@ def time_dominant_kernel(et, layers, T, folded, rounds_per_graph=6, replays=8):
     kernel at the workload's shape: the FFN up-projection through the tile-sparse W1 (3072 x 768 at
     80 %) + GELU, T token rows, launched exactly as the stack launches it.
 
-    `folded` (the default stack, five launches per layer): the launch normalises the output
+    `folded` (the default stack, four launches per layer): the launch normalises the output
     projection's binary32 sum V1 with that projection's row sums while it stages its token strip
     (et_norm_linear_bsr16_packed_f32in on a 12-wave pack, as the layer builds it); V1 and the sums are
     made here by the producer itself from random operands.  Otherwise (seven launches): the plain
@@ -319,9 +319,9 @@ def main():
                          "neighbouring projections (five)")
     ap.add_argument("--chain", action="store_true",
                     help="everything between two attention kernels in one launch (two launches per layer)")
-    ap.add_argument("--fuse-qkv", action="store_true",
-                    help="the QKV projection of every layer after the first inside its attention kernel (four launches "
-                         "per layer)")
+    ap.add_argument("--five-launches", action="store_true",
+                    help="the QKV projection as a launch of its own in every layer (five launches per layer) instead of "
+                         "inside the attention kernel (four), which the engine picks for this batch by itself")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain streaming kernel of known size (ReLU over 64 MiB in, 64 MiB out) "
                          "three times, as the reference point for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE")
@@ -334,7 +334,7 @@ def main():
     et.lib()  # fails loudly if the native library is missing
 
     layers = build_layers(et)
-    model = build_model(et, layers, use_graph=not args.eager, mixed=2 if args.separate_ln else 3 if args.chain else 4 if args.fuse_qkv else 1)
+    model = build_model(et, layers, use_graph=not args.eager, mixed=2 if args.separate_ln else 3 if args.chain else 5 if args.five_launches else 1)
     x = np.random.default_rng(4).standard_normal((B * S, H), dtype=np.float32).astype(np.float16)
     d_in = et.DeviceBuffer.from_numpy(x)
     d_out = et.DeviceBuffer.empty((B * S, H), np.float16)

@@ -727,20 +727,20 @@ typedef struct et_model_desc {
     float eps;     /* LayerNorm epsilon; <= 0 selects 1e-5                        */
     int causal;    /* != 0: causal mask (the reference's hard-wired one)          */
     int use_graph; /* != 0: replay a captured HIP graph; 0: launch kernel by kernel */
-    int mixed;     /* 1, 2, 3 or 4: mixed precision — the residual stream (layer inputs, the two
+    int mixed;     /* 1 to 5: mixed precision — the residual stream (layer inputs, the two
                     * projections that feed a SkipLayerNorm, both SkipLayerNorm results)
                     * is kept in binary32 inside the stack, binary16 only as matrix-core
                     * operands; input and output of et_model_forward stay binary16.
                     * 1: SkipLayerNorm is folded into the neighbouring tile-sparse projections
                     *    where the shapes allow (five launches per layer; four, as under 4, for
                     *    the batch sizes where that measured faster: 96 to 400 (sequence, head)
-                    *    pairs, from 120 on for sequences above 64 tokens); 2: it keeps its own
+                    *    pairs); 2: it keeps its own
                     *    launches (seven); 3: as 1, with everything between two attention
                     *    kernels in one launch (et_encoder_chain_f32: two launches per layer)
                     *    where the shapes allow and the device runs it as it must, else as 1;
                     *    4: as 1, with the QKV projection of every layer after the first inside
                     *    its attention kernel (et_norm_qkv_mha_f32in: four launches per layer)
-                    *    where the shapes allow, else as 1.
+                    *    where the shapes allow, else as 1; 5: as 1, always with five launches.
                     * 0: every activation is stored as binary16 (the reference's storage) */
 } et_model_desc;
 

@@ -489,7 +489,7 @@ int et_model_finalize(et_model m) {
             for (auto &b : m->pp32) b = std::make_unique<et::DeviceBuffer<float>>(act_elems);
             for (auto &l : m->layers) l->enable_mixed();
             // mixed == 1: the engine folds SkipLayerNorm into the projections where every layer can
-            m->split = (m->desc.mixed == 1 || m->desc.mixed == 3 || m->desc.mixed == 4) && !m->layers.empty();
+            m->split = (m->desc.mixed == 1 || m->desc.mixed == 3 || m->desc.mixed == 4 || m->desc.mixed == 5) && !m->layers.empty();
             for (auto &l : m->layers) m->split = m->split && l->split_ok();
             if (m->split) {
                 for (auto &l : m->layers) l->enable_split();
@@ -497,10 +497,10 @@ int et_model_finalize(et_model m) {
                 // The QKV projection inside the attention kernel: asked for (mixed == 4), or where it measured faster than
                 // the two launches it replaces — one workgroup per (sequence, head) that reads and normalises its whole
                 // sequence: 12-layer 768-wide stacks at 80 / 90 / 95 % sparsity ran 0.89 - 0.99 of the five-launch time
-                // with 96 to 384 such workgroups (sequences of 32 to 128 tokens), except 96 of them on sequences of 96 or
-                // 128 tokens (1.00 - 1.01); 1.04 - 1.05 at 72 and below, 1.09 - 1.11 at 768.
+                // with 96 to 384 such workgroups (sequences of 32 to 128 tokens) — 96 of them on sequences of 96 or 128
+                // tokens 0.99 - 1.01 —, 1.04 - 1.05 at 72 and below, 1.09 - 1.11 at 768.
                 const long heads = (long)m->desc.batch * m->desc.nhead;
-                const bool pays = heads >= 96 && heads <= 400 && (heads >= 120 || m->desc.seq_len <= 64);
+                const bool pays = heads >= 96 && heads <= 400;
                 if ((m->desc.mixed == 4 || (m->desc.mixed == 1 && pays)) && m->layers.size() > 1) {
                     m->fused_qkv = true;
                     for (size_t i = 1; i < m->layers.size(); i++) m->fused_qkv = m->layers[i]->enable_fused_qkv() && m->fused_qkv;

@@ -86,7 +86,7 @@ TOL_F16_DEEP = 5e-2          # all-fp16 storage over 12+ layers: two realisation
 
 
 @pytest.mark.parametrize("seed0,xseed,mode", [(100, 4, 1), (300, 307, 1), (500, 507, 1), (100, 4, 2), (100, 4, 3),
-                                               (300, 307, 3), (100, 4, 4), (300, 307, 4)])
+                                               (300, 307, 3), (100, 4, 4), (300, 307, 4), (100, 4, 5)])
 def test_bert_base_12_layers_batch8_tile80_attention_aware_mixed(et, seed0, xseed, mode):
     """The headline configuration in the engine's mixed-precision mode: 12 layers, B8 S128, 80 %
     tile sparsity, 25 % of the V rows (and the matching O columns) dead in head-aligned groups."""
@@ -102,12 +102,15 @@ def test_bert_base_12_layers_batch8_tile80_attention_aware_mixed(et, seed0, xsee
     print(f"12-layer B8 S128 mixed (mode {mode}) seed {seed0}: vs fp32 forward {e32:.3e}, vs mixed oracle {em:.3e}")
     assert e32 <= TOL_MIXED_VS_F32 and em <= TOL_MIXED_VS_ORACLE
     assert np.array_equal(got[0], got[1])
-    if mode == 4:
+    if mode in (1, 4):  # at this batch the engine takes the four-launch form by itself as well
         assert m.launches_per_layer() == 4, "the QKV projection did not move into the attention kernel"
+    if mode == 5:
+        assert m.launches_per_layer() == 5
 
 
 @pytest.mark.parametrize("S,B,sp,padded,causal", [(128, 3, 0.8, True, False), (48, 5, 0.9, False, True),
-                                                  (64, 7, 0.5, True, True), (16, 1, 0.95, False, False)])
+                                                  (64, 9, 0.5, True, True), (16, 1, 0.95, False, False),
+                                                  (128, 8, 0.8, True, False)])
 def test_qkv_inside_attention_stacks(et, S, B, sp, padded, causal):
     """mixed = 4: the layers after the first project Q, K and V inside their attention kernel (768-wide models with
     heads of 64, sequences up to 128 tokens): padded, causal, short and odd batch counts, block-rows of few and of
@@ -118,7 +121,7 @@ def test_qkv_inside_attention_stacks(et, S, B, sp, padded, causal):
     lens = np.random.default_rng(S * B).integers(S // 2, S + 1, B).astype(np.int32) if padded else None
     x = Hn.randn((B * S, H), 909)
     m4 = Hn.build_model(et, layers, S, B, lens=lens, causal=causal, mixed=4)
-    m1 = Hn.build_model(et, layers, S, B, lens=lens, causal=causal, mixed=1)
+    m1 = Hn.build_model(et, layers, S, B, lens=lens, causal=causal, mixed=5)
     got4, got1 = run_model(et, m4, x, reps=3), run_model(et, m1, x, reps=1)
     assert m4.launches_per_layer() == 4 and m1.launches_per_layer() == 5
     want = Hn.oracle_stack(x, layers, B, lens, causal=causal, store=torch.float16, resid=torch.float32)
@@ -134,10 +137,10 @@ def test_qkv_inside_attention_stacks(et, S, B, sp, padded, causal):
 
 def test_qkv_inside_attention_chosen_by_batch(et):
     """mixed = 1 takes the four-launch form by itself where it measured faster (here 12 sequences of 64 tokens on 12
-    heads, 8 as well) and keeps five launches elsewhere (4 sequences)."""
+    heads, 8 as well) and keeps five launches elsewhere (4 sequences, 40 sequences)."""
     H, nh, FF, S = 768, 12, 512, 64
     layers = [Hn.LayerWeights(H, nh, FF, 0.8, seed=920 + i) for i in range(2)]
-    for B, launches in ((12, 4), (8, 4), (4, 5)):
+    for B, launches in ((12, 4), (8, 4), (4, 5), (40, 5)):
         m = Hn.build_model(et, layers, S, B, mixed=1)
         assert m.launches_per_layer() == launches
         x = Hn.randn((B * S, H), 929)
@@ -180,12 +183,12 @@ def test_bert_base_12_layers_all_fp16_storage(et):
 def test_chain_launches_equal_separate_launches(et):
     """mixed = 3 runs everything between two attention kernels as one launch whose workgroups meet at
     counters in their XCD's L2 instead of at kernel boundaries: the same arithmetic on the same packs
-    as mixed = 1, so the results agree bit for bit, replay after replay; and the model reports that the
+    as mixed = 5 (five separate launches), so the results agree bit for bit, replay after replay; and the model reports that the
     chain really ran (two launches per layer)."""
     H, S, B = 768, 128, 8
     layers = headline_layers(700)
     x = Hn.randn((B * S, H), 707)
-    m5 = Hn.build_model(et, layers, S, B, mixed=1)
+    m5 = Hn.build_model(et, layers, S, B, mixed=5)
     m2 = Hn.build_model(et, layers, S, B, mixed=3)
     a = run_model(et, m5, x, reps=2)
     b = run_model(et, m2, x, reps=4)
@@ -200,7 +203,7 @@ def test_bench_workload_mixed_precision(et):
     import bench
     layers = bench.build_layers(et)
     m = bench.build_model(et, layers, use_graph=True)
-    assert m.desc.mixed == 1
+    assert m.desc.mixed == 1 and m.launches_per_layer() == 4
     x = np.random.default_rng(4).standard_normal((bench.B * bench.S, bench.H), dtype=np.float32).astype(np.float16)
     got = run_model(et, m, x)[0]
     want32, want_mixed = bench.oracle_forwards(layers, x)
