@@ -322,13 +322,16 @@ class Attention<_config, std::enable_if_t<_config::isSingleKernel>> : public et:
     // The QKV projection inside the attention kernel (one launch instead of two) for the layers whose input is
     // a previous layer's un-normalised sum: sequences up to 128 tokens, heads of 64, a 768-wide model.
     // true when forward_split() will run that way.
-    bool prepare_fused_qkv() {
+    // gamma, beta: the affine vectors of the normalisation whose result this attention will be given (the
+    // previous layer's second SkipLayerNorm), folded into the pack where they are known; forward_split() must then
+    // be given exactly these.
+    bool prepare_fused_qkv(const half *gamma = nullptr, const half *beta = nullptr) {
         if constexpr (std::is_same<linearQKV_t, Linear<tile_mat>>::value) {
             const int hd = model->kdim / model->nhead;
             if (model->vdim != model->kdim ||
                 et_norm_qkv_mha_f32in_supported(batch(), model->seq_len, (int)linearQKV->in_size, model->nhead, hd) != 1)
                 return false;
-            fused_qkv_ = linearQKV->prepare_qkv_heads(model->nhead);
+            fused_qkv_ = linearQKV->prepare_qkv_heads(model->nhead, gamma, beta);
             return fused_qkv_;
         } else {
             return false;

@@ -218,10 +218,15 @@ template <typename attn_t, typename linear1_t, typename linear2_t, typename ACT_
     }
     // After enable_split(): the layer's QKV projection moves into its attention kernel (four launches per
     // layer) whenever its input is a previous layer's sum.  false where the shapes do not allow it.
-    bool enable_fused_qkv() {
-        if constexpr (attn_has_fused_qkv<attn_t>::value) return stats1 && attn->prepare_fused_qkv();
+    // gamma, beta: the previous layer's second normalisation (the one this layer's input carries), folded into
+    // the projection where given.
+    bool enable_fused_qkv(const half *gamma = nullptr, const half *beta = nullptr) {
+        if constexpr (attn_has_fused_qkv<attn_t>::value) return stats1 && attn->prepare_fused_qkv(gamma, beta);
         else return false;
     }
+    // the affine vectors of this layer's second normalisation, as its SplitSum hands them on
+    const half *norm2_gamma() const { return LN2->gamma(); }
+    const half *norm2_beta() const { return LN2->beta(); }
     static constexpr int kChainWaves = 12;
     // This layer's share of a chain launch (et_encoder_chain_f32): everything between its attention
     // kernel and the next layer's.  false when the layer's types have no such form.

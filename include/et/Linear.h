@@ -173,6 +173,7 @@ template <> class Linear<tile_mat> {
     // (et_qkv_heads_pack_create); built on prepare_qkv_heads()
     pack_ptr pack_heads;
     int heads_nhead = 0;
+    const half *heads_gamma = nullptr, *heads_beta = nullptr;  // the normalisation folded into pack_heads (null: none)
     int producer_nwave = 0, consumer_nwave = 0;  // the wave counts the role packs were asked for (0: the builder's choice)
     static constexpr int kPackMaxRows = 4096;
     // Where a pack pays (measured against the unpacked kernel at 128 .. 1536 rows, 768- and 3072-wide inputs, 80 / 90 /
@@ -306,16 +307,25 @@ template <> class Linear<tile_mat> {
     }
     // This Linear as the QKV projection of `nhead` heads of 64 inside the attention kernel: false (and nothing
     // built) where that kernel does not take the weight.  Called once, outside any stream capture.
-    bool prepare_qkv_heads(int nhead) {
-        if (pack_heads) return heads_nhead == nhead;
+    // With gamma and beta (device pointers that stay valid, the affine vectors of the normalisation this projection
+    // will be given) they are folded into the pack: W diag(gamma), bias + W beta.  A caller that rewrites them
+    // calls refresh().
+    bool prepare_qkv_heads(int nhead, const half *gamma = nullptr, const half *beta = nullptr) {
+        if (pack_heads) return heads_nhead == nhead && heads_gamma == gamma && heads_beta == beta;
         if (dense || plan || !packed_enabled() || (long)out_size != 3L * nhead * 64) return false;
         et_bsr_pack p = nullptr;
-        const int s = et_qkv_heads_pack_create(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
-                                               (int)in_size, nhead, &p);
+        const int s = gamma && beta
+                          ? et_qkv_heads_pack_create_folded(weight.row_ptr.get(), weight.row_offset.get(),
+                                                            et::f16(weight.data.get()), et::f16(bias.get()), et::f16(gamma),
+                                                            et::f16(beta), (int)in_size, nhead, &p)
+                          : et_qkv_heads_pack_create(weight.row_ptr.get(), weight.row_offset.get(), et::f16(weight.data.get()),
+                                                     (int)in_size, nhead, &p);
         if (s == ET_ERR_UNSUPPORTED) return false;
         etChk(s);
         pack_heads.reset(p);
         heads_nhead = nhead;
+        heads_gamma = gamma && beta ? gamma : nullptr;
+        heads_beta = gamma && beta ? beta : nullptr;
         return true;
     }
     // Z = attention over (Q, K, V) = normalised(V32) W^T + bias, in one launch (et_norm_qkv_mha_f32in)
@@ -323,6 +333,8 @@ template <> class Linear<tile_mat> {
                               const half *beta, float eps, float *fin_out, const half *mask, const int *lens, int batch,
                               int seq_len, float scale, int flags, et::stream_t stream = nullptr) {
         et::require((bool)pack_heads, "Linear<tile_mat>: prepare_qkv_heads() was not called or did not apply");
+        et::require(heads_gamma == nullptr || (heads_gamma == gamma && heads_beta == beta),
+                    "Linear<tile_mat>: the pack was folded with another normalisation than the one it is given");
         etChk(et_norm_qkv_mha_f32in(pack_heads.get(), V32, stats, groups, et::f16(gamma), et::f16(beta), eps, fin_out,
                                     et::f16(bias.get()), et::f16(Z), ldz, et::f16(mask), lens, batch, seq_len, scale, flags,
                                     stream));
@@ -403,7 +415,7 @@ template <> class Linear<tile_mat> {
         check();
         if (had_producer) prepare_split_producer(producer_nwave);
         if (had_consumer) prepare_split_consumer(consumer_nwave);
-        if (had_heads) prepare_qkv_heads(heads_nhead);
+        if (had_heads) prepare_qkv_heads(heads_nhead, heads_gamma, heads_beta);
     }
 
   private:

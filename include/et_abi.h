@@ -562,6 +562,17 @@ int et_norm_qkv_mha_f32in_supported(int B, int S, int in, int nhead, int hd);
 int et_qkv_heads_pack_create(const int32_t *row_ptr, const int32_t *col_idx,
                              const et_f16 *tiles, int in, int nhead,
                              et_bsr_pack *pack);
+/* The same pack with the affine part of the normalisation folded into the
+ * weight: it holds W_qkv diag(gamma) (binary16) and bias_qkv + W_qkv beta
+ * (binary32), so that the launch normalises a value with one multiply-add,
+ * (v - mean) rstd — the twelve workgroups of a sequence each normalise all of it.
+ * et_norm_qkv_mha_f32in then ignores its gamma, beta and bias_qkv arguments
+ * (they may be NULL); a caller that changes gamma, beta, the bias or the weight
+ * builds the pack again.  bias may be NULL (zeros). */
+int et_qkv_heads_pack_create_folded(const int32_t *row_ptr, const int32_t *col_idx,
+                                    const et_f16 *tiles, const et_f16 *bias,
+                                    const et_f16 *gamma, const et_f16 *beta,
+                                    int in, int nhead, et_bsr_pack *pack);
 int et_norm_qkv_mha_f32in(et_bsr_pack pack, const float *V, const float *stats,
                           int stat_groups, const et_f16 *gamma,
                           const et_f16 *beta, float eps, float *fin_out,

@@ -125,6 +125,7 @@ _SIGNATURES = {
     "et_norm_qkv_mha_f32in_supported": (_i, _i, _i, _i, _i),
     "et_qkv_heads_pack_create": (_vp, _vp, _vp, _i, _i, C.POINTER(_vp)),
     "et_norm_qkv_mha_f32in": (_vp, _vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _f, _i, _vp),
+    "et_qkv_heads_pack_create_folded": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, C.POINTER(_vp)),
     "et_mha_probs_f16": (_vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp),
     "et_mha_unfused_f16": (_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp),
     "et_linear_vo_f16": (_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp),

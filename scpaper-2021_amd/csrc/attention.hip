@@ -21,6 +21,7 @@
 #include <math.h>
 
 #include <algorithm>
+#include <memory>
 #include <new>
 #include <vector>
 
@@ -474,14 +475,18 @@ struct QkvMhaArgs {
     const _Float16 *gamma, *beta;
     float eps;
     float *fin_out;          // [T][2] mean and rstd of every row, written by head 0 (may be null)
+    const float *bias32;     // FOLDED: bias + W beta as binary32 (gamma is inside the slots; gamma, beta, bias unused)
 };
 constexpr int kQkvWaves = 12;   // Q, K, V x 4 block-rows of a 64-wide head
 constexpr int kQkvRows = 64;    // token rows staged at a time
 
 // PF of a thread's eight rows of the second 64 are requested before the products of the first 64 (they arrive while the
-// matrix cores work).  NPASS = 1 keeps the wave's slots in registers across both halves; NPASS = 2 or 3 (block-rows of
-// more than 12 slots) fetches them in parts of 8 for every 64 rows.
-template <int CAP, int PF, int NPASS>
+// matrix cores work).  NPASS = 1 keeps the wave's slots in registers across both halves; NPASS = 2 to 4 (block-rows of
+// more than 12 slots) fetches them in parts of 8 or 4 for every 64 rows.
+// FOLDED: the pack holds W diag(gamma) and bias + W beta, so that a row is normalised with one multiply-add per value,
+// (x - mean) rstd, and the affine part of the normalisation costs nothing (the workgroups of the 12 heads of a sequence
+// each normalise all of it).
+template <int CAP, int PF, int NPASS, bool FOLDED>
 __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArgs qa) {
     constexpr int HD = 64, QT = 1;
     constexpr bool COMPACT = false;
@@ -524,7 +529,7 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
     // checks that 768 % upr == 0): the lanes of a request read consecutive 16 bytes
     const int n_dr = (int)blockDim.x / upr, n_r0 = (int)threadIdx.x / upr, n_c8 = (int)threadIdx.x - n_r0 * upr;
     h8 gam_in = {}, bet_in = {};
-    if ((int)threadIdx.x < upr) {
+    if (!FOLDED && (int)threadIdx.x < upr) {
         gam_in = reinterpret_cast<const h8 *>(qa.gamma)[threadIdx.x];
         bet_in = reinterpret_cast<const h8 *>(qa.beta)[threadIdx.x];
     }
@@ -591,7 +596,11 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
     // bias: Q and K lanes end with features 4g .. 4g + 3 of a token, V lanes with feature r16 of four tokens.  Kept as
     // loaded and widened where it is added: a conversion here would wait for every request above.
     uint2 bias_bits = {0u, 0u};
-    if (qa.bias) {
+    f4 bias_f = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (FOLDED) {
+        if (part < 2) bias_f = *reinterpret_cast<const f4 *>(qa.bias32 + rb * 16 + g * 4);
+        else bias_f[0] = qa.bias32[rb * 16 + r16];
+    } else if (qa.bias) {
         if (part < 2) bias_bits = *reinterpret_cast<const uint2 *>(qa.bias + rb * 16 + g * 4);
         else bias_bits.x = *reinterpret_cast<const unsigned short *>(qa.bias + rb * 16 + r16);
     }
@@ -607,7 +616,7 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
 #pragma unroll
     for (int k = 0; k < 3; k++)
         if (st_g + 6 * k < kMaxStatGroups) spart[(st_g + 6 * k) * kKeyBlock + st_row] = ps[k];
-    if ((int)threadIdx.x < upr) {
+    if (!FOLDED && (int)threadIdx.x < upr) {
         reinterpret_cast<h8 *>(gb)[threadIdx.x] = gam_in;
         reinterpret_cast<h8 *>(gb + in)[threadIdx.x] = bet_in;
     }
@@ -633,8 +642,11 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
         {
             int r0_now = n_r0, c8_now = n_c8;
             asm volatile("" : "+v"(r0_now), "+v"(c8_now));
-            const h4 gam0 = reinterpret_cast<const h4 *>(gb)[c8_now], gam1 = reinterpret_cast<const h4 *>(gb)[upr + c8_now];
-            const h4 bet0 = reinterpret_cast<const h4 *>(gb + in)[c8_now], bet1 = reinterpret_cast<const h4 *>(gb + in)[upr + c8_now];
+            h4 gam0 = {}, gam1 = {}, bet0 = {}, bet1 = {};
+            if constexpr (!FOLDED) {
+                gam0 = reinterpret_cast<const h4 *>(gb)[c8_now], gam1 = reinterpret_cast<const h4 *>(gb)[upr + c8_now];
+                bet0 = reinterpret_cast<const h4 *>(gb + in)[c8_now], bet1 = reinterpret_cast<const h4 *>(gb + in)[upr + c8_now];
+            }
             const int unit0 = c8_now >> 1, unit1 = (upr + c8_now) >> 1, piece = (c8_now & 1) << 3;  // upr is even
 #pragma unroll
             for (int u = 0; u < SU; u++) {
@@ -643,8 +655,13 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
                 h4 lo, hi;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    lo[e] = (_Float16)__builtin_fmaf(__builtin_fmaf(s32[u][0][e], st.y, st.x), (float)gam0[e], (float)bet0[e]);
-                    hi[e] = (_Float16)__builtin_fmaf(__builtin_fmaf(s32[u][1][e], st.y, st.x), (float)gam1[e], (float)bet1[e]);
+                    if constexpr (FOLDED) {
+                        lo[e] = (_Float16)__builtin_fmaf(s32[u][0][e], st.y, st.x);
+                        hi[e] = (_Float16)__builtin_fmaf(s32[u][1][e], st.y, st.x);
+                    } else {
+                        lo[e] = (_Float16)__builtin_fmaf(__builtin_fmaf(s32[u][0][e], st.y, st.x), (float)gam0[e], (float)bet0[e]);
+                        hi[e] = (_Float16)__builtin_fmaf(__builtin_fmaf(s32[u][1][e], st.y, st.x), (float)gam1[e], (float)bet1[e]);
+                    }
                 }
                 unsigned char *xr = xs + row * stride + piece;
                 *reinterpret_cast<h4 *>(xr + ((unit0 ^ (row & 15)) << 4)) = lo;
@@ -699,8 +716,13 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
         };
         if constexpr (NPASS >= 2) next_part(std::integral_constant<int, WN>{});
         if constexpr (NPASS >= 3) next_part(std::integral_constant<int, 2 * WN>{});
+        if constexpr (NPASS >= 4) next_part(std::integral_constant<int, 3 * WN>{});
+        static_assert(NPASS <= 4, "parts of the slots");
         float bq[4];
-        if (part < 2) {
+        if constexpr (FOLDED) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) bq[e] = part < 2 ? bias_f[e] : bias_f[0];
+        } else if (part < 2) {
             const h4 t = __builtin_bit_cast(h4, bias_bits);
 #pragma unroll
             for (int e = 0; e < 4; e++) bq[e] = (float)t[e];
@@ -762,8 +784,8 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
     }
 }
 
-template <int CAP, int PF, int NPASS> static int launch_qkv_mha(const QkvMhaArgs &qa, size_t lds, hipStream_t stream) {
-    auto kernel = qkv_mha_kernel<CAP, PF, NPASS>;
+template <int CAP, int PF, int NPASS, bool FOLDED> static int launch_qkv_mha_f(const QkvMhaArgs &qa, size_t lds, hipStream_t stream) {
+    auto kernel = qkv_mha_kernel<CAP, PF, NPASS, FOLDED>;
     static bool raised = false;  // per instantiation
     if (!raised) {
         ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
@@ -772,6 +794,11 @@ template <int CAP, int PF, int NPASS> static int launch_qkv_mha(const QkvMhaArgs
     const int rounds = (qa.B + kXcds - 1) / kXcds;
     kernel<<<dim3((unsigned)(rounds * kXcds * qa.m.nh)), kQkvWaves * 64, lds, stream>>>(qa);
     return check_launch("qkv_mha_kernel");
+}
+// PFF, NPF: rows requested ahead and parts of the slots in the folded form, whose register needs differ
+template <int CAP, int PF, int NPASS, int PFF = PF, int NPF = NPASS>
+static int launch_qkv_mha(const QkvMhaArgs &qa, size_t lds, hipStream_t stream) {
+    return qa.bias32 ? launch_qkv_mha_f<CAP, PFF, NPF, true>(qa, lds, stream) : launch_qkv_mha_f<CAP, PF, NPASS, false>(qa, lds, stream);
 }
 
 }  // namespace et
@@ -888,8 +915,9 @@ int et_norm_qkv_mha_f32in_supported(int B, int S, int in, int nhead, int hd) {
     return B > 0 && S > 0 && S % 16 == 0 && S <= kKeyBlock && in == 768 && nhead > 0 && hd == 64 ? 1 : 0;
 }
 
-int et_qkv_heads_pack_create(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles, int in, int nhead,
-                             et_bsr_pack *pack) {
+// gamma != nullptr: the pack holds W diag(gamma) and, as binary32, bias + W beta
+static int qkv_heads_pack_build(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles, const et_f16 *bias,
+                                const et_f16 *gamma, const et_f16 *beta, int in, int nhead, et_bsr_pack *pack) {
     ET_REQUIRE(pack != nullptr, ET_ERR_INVALID_ARG, "et_qkv_heads_pack_create: pack is NULL");
     *pack = nullptr;
     ET_REQUIRE(row_ptr && col_idx && tiles, ET_ERR_INVALID_ARG, "et_qkv_heads_pack_create: NULL pointer");
@@ -928,7 +956,7 @@ int et_qkv_heads_pack_create(const int32_t *row_ptr, const int32_t *col_idx, con
             tab[slab] = p;
         }
     }
-    et_bsr_pack_s *p = new (std::nothrow) et_bsr_pack_s;
+    std::unique_ptr<et_bsr_pack_s> p(new (std::nothrow) et_bsr_pack_s);  // freed on every early return
     ET_REQUIRE(p != nullptr, ET_ERR_ALLOC, "et_qkv_heads_pack_create: out of host memory");
     p->in = in;
     p->out = nbr * 16;
@@ -939,13 +967,57 @@ int et_qkv_heads_pack_create(const int32_t *row_ptr, const int32_t *col_idx, con
     p->flags = ET_PACK_QKV_HEADS;
     p->lds = (size_t)kQkvRows * in * 2 + (size_t)(2 * MhaLds<64>::k_halfs + MhaLds<64>::vt_halfs) * sizeof(_Float16) +
              kKeyBlock * sizeof(float2) + (size_t)in * 4;
-    const int s = pack_upload(*p, off, tab, order, tiles);
-    if (s != ET_OK) {
-        delete p;
-        return s;
+    int s = ET_OK;
+    if (gamma) {
+        // W diag(gamma) as binary16 tiles and bias + W beta as binary32, made here from host copies
+        const size_t nvals = (size_t)ntile * 256, nout = (size_t)nbr * 16;
+        std::vector<_Float16> ht(std::max<size_t>(nvals, 1)), hg((size_t)in), hb((size_t)in), hbias(nout);
+        std::vector<float> b32(nout, 0.0f);
+        if (nvals) ET_HIP(hipMemcpy(ht.data(), tiles, nvals * 2, hipMemcpyDeviceToHost));
+        ET_HIP(hipMemcpy(hg.data(), gamma, (size_t)in * 2, hipMemcpyDeviceToHost));
+        ET_HIP(hipMemcpy(hb.data(), beta, (size_t)in * 2, hipMemcpyDeviceToHost));
+        if (bias) {
+            ET_HIP(hipMemcpy(hbias.data(), bias, nout * 2, hipMemcpyDeviceToHost));
+            for (size_t o = 0; o < nout; o++) b32[o] = (float)hbias[o];
+        }
+        for (int rb = 0; rb < nbr; rb++) {
+            for (int t = rp[(size_t)rb]; t < rp[(size_t)rb + 1]; t++) {
+                const size_t c0 = (size_t)ci[(size_t)t] * 16;
+                for (int r = 0; r < 16; r++) {
+                    float dot = 0.0f;
+                    for (int c = 0; c < 16; c++) {
+                        _Float16 &w = ht[(size_t)t * 256 + (size_t)r * 16 + c];  // tile row r = output feature, column c = input
+                        dot += (float)w * (float)hb[c0 + c];
+                        w = (_Float16)((float)w * (float)hg[c0 + c]);
+                    }
+                    b32[(size_t)rb * 16 + r] += dot;
+                }
+            }
+        }
+        void *d_scaled = nullptr;
+        s = check_hip(hipMalloc(&d_scaled, std::max<size_t>(nvals * 2, 16)), "hipMalloc");
+        if (s == ET_OK && nvals) s = check_hip(hipMemcpy(d_scaled, ht.data(), nvals * 2, hipMemcpyHostToDevice), "hipMemcpy");
+        if (s == ET_OK) s = pack_upload(*p, off, tab, order, static_cast<const et_f16 *>(d_scaled));
+        (void)hipFree(d_scaled);
+        if (s == ET_OK) s = et_malloc(&p->bias32, nout * 4);
+        if (s == ET_OK) s = check_hip(hipMemcpy(p->bias32, b32.data(), nout * 4, hipMemcpyHostToDevice), "hipMemcpy");
+    } else {
+        s = pack_upload(*p, off, tab, order, tiles);
     }
-    *pack = p;
+    if (s != ET_OK) return s;
+    *pack = p.release();
     return ET_OK;
+}
+
+int et_qkv_heads_pack_create(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles, int in, int nhead,
+                             et_bsr_pack *pack) {
+    return qkv_heads_pack_build(row_ptr, col_idx, tiles, nullptr, nullptr, nullptr, in, nhead, pack);
+}
+
+int et_qkv_heads_pack_create_folded(const int32_t *row_ptr, const int32_t *col_idx, const et_f16 *tiles, const et_f16 *bias,
+                                    const et_f16 *gamma, const et_f16 *beta, int in, int nhead, et_bsr_pack *pack) {
+    ET_REQUIRE(gamma && beta, ET_ERR_INVALID_ARG, "et_qkv_heads_pack_create_folded: gamma and beta must be set");
+    return qkv_heads_pack_build(row_ptr, col_idx, tiles, bias, gamma, beta, in, nhead, pack);
 }
 
 int et_norm_qkv_mha_f32in(et_bsr_pack pack, const float *V, const float *stats, int stat_groups, const et_f16 *gamma,
@@ -953,7 +1025,8 @@ int et_norm_qkv_mha_f32in(et_bsr_pack pack, const float *V, const float *stats, 
                           const et_f16 *mask, const int32_t *lens, int B, int S, float scale, int flags, et_stream stream) {
     ET_REQUIRE(pack != nullptr && (pack->flags & ET_PACK_QKV_HEADS), ET_ERR_INVALID_ARG,
                "et_norm_qkv_mha_f32in: needs a pack from et_qkv_heads_pack_create");
-    ET_REQUIRE(V && stats && gamma && beta && Z, ET_ERR_INVALID_ARG, "et_norm_qkv_mha_f32in: NULL pointer");
+    const bool folded = pack->bias32 != nullptr;
+    ET_REQUIRE(V && stats && Z && (folded || (gamma && beta)), ET_ERR_INVALID_ARG, "et_norm_qkv_mha_f32in: NULL pointer");
     const int nh = pack->ngroups, in = pack->in;
     ET_REQUIRE(B >= 0 && et_norm_qkv_mha_f32in_supported(std::max(B, 1), S, in, nh, 64) == 1, ET_ERR_UNSUPPORTED,
                "et_norm_qkv_mha_f32in: B=%d S=%d: sequences of a multiple of 16 up to %d tokens", B, S, kKeyBlock);
@@ -990,10 +1063,11 @@ int et_norm_qkv_mha_f32in(et_bsr_pack pack, const float *V, const float *stats, 
     qa.beta = reinterpret_cast<const _Float16 *>(beta);
     qa.eps = eps;
     qa.fin_out = fin_out;
+    qa.bias32 = static_cast<const float *>(pack->bias32);
     switch (pack->cap) {
         case 8: return launch_qkv_mha<8, 8, 1>(qa, pack->lds, as_stream(stream));
-        case 12: return launch_qkv_mha<12, 4, 1>(qa, pack->lds, as_stream(stream));
-        case 16: return launch_qkv_mha<16, 4, 2>(qa, pack->lds, as_stream(stream));
+        case 12: return launch_qkv_mha<12, 4, 1, 8>(qa, pack->lds, as_stream(stream));
+        case 16: return launch_qkv_mha<16, 4, 2, 4, 4>(qa, pack->lds, as_stream(stream));
         case 24: return launch_qkv_mha<24, 4, 3>(qa, pack->lds, as_stream(stream));
         default: return fail(ET_ERR_INVALID_ARG, "et_norm_qkv_mha_f32in: no kernel for %d slots per wave", pack->cap);
     }

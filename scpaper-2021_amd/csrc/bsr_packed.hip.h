@@ -530,10 +530,12 @@ struct et_bsr_pack_s {
     int flags = 0;
     size_t lds = 0;
     void *pw = nullptr, *poff = nullptr, *ptab = nullptr;
+    void *bias32 = nullptr;  // packs with a normalisation's affine part folded in: bias + W beta, binary32
     ~et_bsr_pack_s() {
         (void)et_free(pw);
         (void)et_free(poff);
         (void)et_free(ptab);
+        (void)et_free(bias32);
     }
 };
 

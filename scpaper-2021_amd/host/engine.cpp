@@ -22,7 +22,9 @@ struct ILayer {
     virtual void forward_mixed(float *out32, half *out16, const float *src32, half *src16, stream_t stream) = 0;
     virtual bool split_ok() const = 0;
     virtual void enable_split() = 0;
-    virtual bool enable_fused_qkv() = 0;
+    virtual bool enable_fused_qkv(const half *gamma, const half *beta) = 0;
+    virtual const half *norm2_gamma() const = 0;
+    virtual const half *norm2_beta() const = 0;
     virtual et::SplitSum forward_split(const et::SplitSum *in, const float *x32, half *x16, stream_t stream) = 0;
     virtual void finish_split(float *out32, half *out16, const et::SplitSum &s, stream_t stream) = 0;
     virtual bool chain_parts(et::ChainParts &p) = 0;
@@ -41,7 +43,9 @@ template <typename EncoderT> struct LayerOf final : ILayer {
     }
     bool split_ok() const override { return enc->split_ok(); }
     void enable_split() override { enc->enable_split(); }
-    bool enable_fused_qkv() override { return enc->enable_fused_qkv(); }
+    bool enable_fused_qkv(const half *gamma, const half *beta) override { return enc->enable_fused_qkv(gamma, beta); }
+    const half *norm2_gamma() const override { return enc->norm2_gamma(); }
+    const half *norm2_beta() const override { return enc->norm2_beta(); }
     et::SplitSum forward_split(const et::SplitSum *in, const float *x32, half *x16, stream_t stream) override {
         return enc->forward_split(in, x32, x16, stream);
     }
@@ -503,7 +507,11 @@ int et_model_finalize(et_model m) {
                 const bool pays = heads >= 96 && heads <= 400;
                 if ((m->desc.mixed == 4 || (m->desc.mixed == 1 && pays)) && m->layers.size() > 1) {
                     m->fused_qkv = true;
-                    for (size_t i = 1; i < m->layers.size(); i++) m->fused_qkv = m->layers[i]->enable_fused_qkv() && m->fused_qkv;
+                    // (the affine part of the normalisation a layer is handed — the second one of the layer before —
+                    // goes into its projection's pack)
+                    for (size_t i = 1; i < m->layers.size(); i++)
+                        m->fused_qkv = m->layers[i]->enable_fused_qkv(m->layers[i - 1]->norm2_gamma(), m->layers[i - 1]->norm2_beta()) &&
+                                       m->fused_qkv;
                 }
             }
         }

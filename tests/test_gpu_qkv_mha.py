@@ -31,8 +31,11 @@ CASES = [
 ]
 
 
+@pytest.mark.parametrize("folded", [False, True])
 @pytest.mark.parametrize("B,S,sp,groups,kind", CASES)
-def test_norm_qkv_mha(et, B, S, sp, groups, kind):
+def test_norm_qkv_mha(et, B, S, sp, groups, kind, folded):
+    """folded: the pack holds W diag(gamma) and bias + W beta (et_qkv_heads_pack_create_folded) and the launch is given
+    neither gamma, beta nor the bias."""
     lib = et.lib()
     T = B * S
     w = Hn.BsrWeight(3 * H, H, sp, seed=171, bias_std=0.05).upload(et)
@@ -60,11 +63,16 @@ def test_norm_qkv_mha(et, B, S, sp, groups, kind):
     et.check(lib.et_fill_f16(d_z.ptr, T * H, 0x7E00, None))
     assert lib.et_norm_qkv_mha_f32in_supported(B, S, H, NH, HD) == 1
     pack = C.c_void_p()
-    et.check(lib.et_qkv_heads_pack_create(w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, H, NH, C.byref(pack)))
+    if folded:
+        et.check(lib.et_qkv_heads_pack_create_folded(w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, w.d_bias.ptr, d_g.ptr,
+                                                     d_b.ptr, H, NH, C.byref(pack)))
+    else:
+        et.check(lib.et_qkv_heads_pack_create(w.d_row_ptr.ptr, w.d_col_idx.ptr, w.d_tiles.ptr, H, NH, C.byref(pack)))
     scale = 1.0 / math.sqrt(HD)
     flags = et.MHA_CAUSAL if kind == 2 else 0
     for _ in range(2):
-        et.check(lib.et_norm_qkv_mha_f32in(pack, d_v.ptr, d_st.ptr, groups, d_g.ptr, d_b.ptr, 1e-5, d_fin.ptr, w.d_bias.ptr,
+        et.check(lib.et_norm_qkv_mha_f32in(pack, d_v.ptr, d_st.ptr, groups, None if folded else d_g.ptr,
+                                           None if folded else d_b.ptr, 1e-5, d_fin.ptr, None if folded else w.d_bias.ptr,
                                            d_z.ptr, H, d_mask.ptr if d_mask else None, d_lens.ptr if d_lens else None, B, S,
                                            scale, flags, None))
     et.sync()
@@ -85,7 +93,7 @@ def test_norm_qkv_mha(et, B, S, sp, groups, kind):
                  scale, flags, None)
     et.sync()
     err2 = Hn.max_abs(got, d_z2.numpy())
-    print(f"qkv inside attention B={B} S={S} sp={sp}: vs oracle {err:.2e}, vs the two launches {err2:.2e}")
+    print(f"qkv inside attention{' (folded)' if folded else ''} B={B} S={S} sp={sp}: vs oracle {err:.2e}, vs the two launches {err2:.2e}")
     assert not np.isnan(got.astype(np.float32)).any()
     assert err <= 3e-3 and err2 <= 3e-3
     fin = d_fin.numpy()
