@@ -479,6 +479,7 @@ struct QkvMhaArgs {
 };
 constexpr int kQkvWaves = 12;   // Q, K, V x 4 block-rows of a 64-wide head
 constexpr int kQkvRows = 64;    // token rows staged at a time
+constexpr int kQkvIn = 768;     // input width the kernel is written for: 96 threads per row, 8 rows per pass of 768 threads
 
 // PF of a thread's eight rows of the second 64 are requested before the products of the first 64 (they arrive while the
 // matrix cores work).  NPASS = 1 keeps the wave's slots in registers across both halves; NPASS = 2 to 4 (block-rows of
@@ -498,8 +499,8 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r16 = lane & 15, g = lane >> 4, sel = g >> 1, gbit = g & 1;
-    const int S = a.S, in = qa.in;
-    const int stride = in * 2, upr = in >> 3;
+    constexpr int in = kQkvIn, stride = in * 2, upr = in >> 3;  // compile-time: the addresses below are adds of constants
+    const int S = a.S;
     unsigned char *xs = qm_smem;                                                  // [64][in] binary16, swizzled
     _Float16 *Qs = reinterpret_cast<_Float16 *>(qm_smem + (size_t)kQkvRows * stride);  // [128][ldk]
     _Float16 *Ks = Qs + L::k_halfs;                                               // [128][ldk]
@@ -525,15 +526,18 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
         for (int k = 0; k < 3; k++)
             ps[k] = *reinterpret_cast<const float2 *>(qa.st_in + ((size_t)min(st_g + 6 * k, qa.st_groups - 1) * qa.T + row0 + tok) * 2);
     }
-    // thread t owns columns 4c .. 4c + 3 and in / 2 + 4c .. + 3, c = t % upr, of staged rows t / upr + u * dr (the host
-    // checks that 768 % upr == 0): the lanes of a request read consecutive 16 bytes
-    const int n_dr = (int)blockDim.x / upr, n_r0 = (int)threadIdx.x / upr, n_c8 = (int)threadIdx.x - n_r0 * upr;
+    // thread t owns columns 4c .. 4c + 3 and in / 2 + 4c .. + 3, c = t % upr, of staged rows t / upr + 8 u: the lanes of
+    // a request read consecutive 16 bytes
+    constexpr int n_dr = kQkvWaves * 64 / upr;
+    static_assert(n_dr * upr == kQkvWaves * 64 && SU * n_dr == kQkvRows, "768 threads cover 8 rows of 96 units");
+    const int n_r0 = (int)threadIdx.x / upr, n_c8 = (int)threadIdx.x - n_r0 * upr;
     h8 gam_in = {}, bet_in = {};
     if (!FOLDED && (int)threadIdx.x < upr) {
         gam_in = reinterpret_cast<const h8 *>(qa.gamma)[threadIdx.x];
         bet_in = reinterpret_cast<const h8 *>(qa.beta)[threadIdx.x];
     }
     f4 s32[SU][2];
+    const char *xbase = reinterpret_cast<const char *>(qa.X32 + row0 * in);  // wave-uniform
     // rows [from, to) of the thread's eight in the given half (the thread's place passes through an empty asm: seen as
     // loop-invariant, the addresses of all sixteen rows are computed up front, 32 registers that spill)
     auto request_rows = [&](int half, auto from, auto to) {
@@ -541,10 +545,11 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
         asm volatile("" : "+v"(r0_now), "+v"(c8_now));
 #pragma unroll
         for (int u = decltype(from)::value; u < decltype(to)::value; u++) {
+            // (a wave-uniform base and a 32-bit offset per lane: the sequence's rows are less than 4 GB)
             const int tok = min(half * kQkvRows + r0_now + u * n_dr, S - 1);
-            const f4 *p = reinterpret_cast<const f4 *>(qa.X32 + (row0 + tok) * in) + c8_now;
-            s32[u][0] = p[0];
-            s32[u][1] = p[upr];
+            const unsigned off = (unsigned)tok * (unsigned)(in * 4) + 16u * (unsigned)c8_now;
+            s32[u][0] = *reinterpret_cast<const f4 *>(xbase + off);
+            s32[u][1] = *reinterpret_cast<const f4 *>(xbase + off + 2u * (unsigned)in);
         }
     };
     using i0 = std::integral_constant<int, 0>;
@@ -640,6 +645,8 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
         const int tokbase = half * kQkvRows;
         if (half > 0) request_rows(half, iPF{}, iSU{});  // what was not requested ahead
         {
+            // (the thread's place passes through an empty asm: the offsets made from it below are the same in both
+            // halves, and held across the products they cost the registers that the variants with many slots lack)
             int r0_now = n_r0, c8_now = n_c8;
             asm volatile("" : "+v"(r0_now), "+v"(c8_now));
             h4 gam0 = {}, gam1 = {}, bet0 = {}, bet1 = {};
@@ -647,11 +654,22 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
                 gam0 = reinterpret_cast<const h4 *>(gb)[c8_now], gam1 = reinterpret_cast<const h4 *>(gb)[upr + c8_now];
                 bet0 = reinterpret_cast<const h4 *>(gb + in)[c8_now], bet1 = reinterpret_cast<const h4 *>(gb + in)[upr + c8_now];
             }
-            const int unit0 = c8_now >> 1, unit1 = (upr + c8_now) >> 1, piece = (c8_now & 1) << 3;  // upr is even
+            // Where the thread's two 8-byte pieces of row r0 + 8 u go: the row's swizzle term (row & 15) is r0 for even
+            // u and r0 + 8 for odd u (r0 < 8), so four offsets and a multiple of a constant name all sixteen places.
+            const unsigned unit0 = (unsigned)c8_now >> 1, unit1 = (unsigned)(upr + c8_now) >> 1;  // upr is even
+            const unsigned at0 = (unsigned)r0_now * stride + (((unsigned)c8_now & 1u) << 3);
+            const unsigned wr0[2] = {at0 + ((unit0 ^ (unsigned)r0_now) << 4), at0 + ((unit0 ^ (unsigned)(r0_now + 8)) << 4)};
+            const unsigned wr1[2] = {at0 + ((unit1 ^ (unsigned)r0_now) << 4), at0 + ((unit1 ^ (unsigned)(r0_now + 8)) << 4)};
+            // (the place of the next 64's rows passes through an empty asm: computed per row, two instructions, instead
+            // of eight offsets held from the top of the loop)
+            const int next_row = tokbase + kQkvRows + r0_now;
+            const unsigned next_off = 16u * (unsigned)c8_now;
+            const float2 *strow = stat + tokbase + r0_now;  // -mean * rstd and rstd of the thread's rows, 8 apart
+            float2 st_next = strow[0];
 #pragma unroll
             for (int u = 0; u < SU; u++) {
-                const int row = r0_now + u * n_dr;
-                const float2 st = stat[tokbase + row];  // rstd and -mean * rstd: two fused multiply-adds per value
+                const float2 st = st_next;
+                if (u + 1 < SU) st_next = strow[(u + 1) * n_dr];  // one row ahead: its read is not waited for on the spot
                 h4 lo, hi;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
@@ -663,17 +681,16 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
                         hi[e] = (_Float16)__builtin_fmaf(__builtin_fmaf(s32[u][1][e], st.y, st.x), (float)gam1[e], (float)bet1[e]);
                     }
                 }
-                unsigned char *xr = xs + row * stride + piece;
-                *reinterpret_cast<h4 *>(xr + ((unit0 ^ (row & 15)) << 4)) = lo;
-                *reinterpret_cast<h4 *>(xr + ((unit1 ^ (row & 15)) << 4)) = hi;
+                *reinterpret_cast<h4 *>(xs + wr0[u & 1] + u * n_dr * stride) = lo;
+                *reinterpret_cast<h4 *>(xs + wr1[u & 1] + u * n_dr * stride) = hi;
                 if constexpr (HOLD) {
                     // the registers of a row go to the same row of the next 64 the moment they are free: the memory
                     // pipe stays busy through the normalisation and the products
                     if (u < PF && half + 1 < nhalf) {
-                        const int tok = min(tokbase + kQkvRows + row, S - 1);
-                        const f4 *p = reinterpret_cast<const f4 *>(qa.X32 + (row0 + tok) * in) + c8_now;
-                        s32[u][0] = p[0];
-                        s32[u][1] = p[upr];
+                        const int tok = min(next_row + u * n_dr, S - 1);
+                        const unsigned off = (unsigned)tok * (unsigned)(in * 4) + next_off;
+                        s32[u][0] = *reinterpret_cast<const f4 *>(xbase + off);
+                        s32[u][1] = *reinterpret_cast<const f4 *>(xbase + off + 2u * (unsigned)in);
                     }
                 }
             }
