@@ -555,9 +555,30 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
     using i0 = std::integral_constant<int, 0>;
     using iPF = std::integral_constant<int, PF>;
     using iSU = std::integral_constant<int, SU>;
-    // (results return in the order of the requests of the whole compute unit: behind this barrier the few bytes the
-    // statistics wait for are not queued behind other waves' rows)
+    // ---- mean and rstd of the sequence's rows: the partial sums are added per row in group order through LDS, by the
+    // first two waves, while the others already request their rows.  (Results return in the order of the requests of
+    // the whole compute unit: the few bytes the statistics wait for are requested, and awaited, ahead of all rows.)
+#pragma unroll
+    for (int k = 0; k < 3; k++)
+        if (st_g + 6 * k < kMaxStatGroups) spart[(st_g + 6 * k) * kKeyBlock + st_row] = ps[k];
+    if (!FOLDED && (int)threadIdx.x < upr) {
+        reinterpret_cast<h8 *>(gb)[threadIdx.x] = gam_in;
+        reinterpret_cast<h8 *>(gb + in)[threadIdx.x] = bet_in;
+    }
     __syncthreads();
+    if (threadIdx.x < kKeyBlock) {
+        float s1 = 0.0f, s2 = 0.0f;
+        for (int gi = 0; gi < qa.st_groups; gi++) {
+            const float2 pr = spart[gi * kKeyBlock + threadIdx.x];
+            s1 += pr.x;
+            s2 += pr.y;
+        }
+        const float mean = s1 / (float)in;
+        const float2 mine = {mean, rsqrtf(fmaxf(__builtin_fmaf(-mean, mean, s2 / (float)in), 0.0f) + qa.eps)};
+        stat[threadIdx.x] = float2{-mean * mine.y, mine.y};
+        if (qa.fin_out && h == 0 && (int)threadIdx.x < S)
+            *reinterpret_cast<float2 *>(qa.fin_out + 2 * (row0 + threadIdx.x)) = mine;
+    }
     request_rows(0, i0{}, iSU{});
 
     // ---- this wave's block-row of W_qkv: part 0 / 1 / 2 = Q / K / V, four block-rows of the head each
@@ -616,28 +637,6 @@ __global__ __launch_bounds__(kQkvWaves * 64) void qkv_mha_kernel(const QkvMhaArg
         uint4 *z = reinterpret_cast<uint4 *>(Ks);
         for (int i = threadIdx.x; i < (int)((L::k_halfs + L::vt_halfs) * sizeof(_Float16) / 16); i += blockDim.x)
             z[i] = uint4{0u, 0u, 0u, 0u};
-    }
-    // ---- mean and rstd of the sequence's rows: the partial sums are added per row in group order through LDS
-#pragma unroll
-    for (int k = 0; k < 3; k++)
-        if (st_g + 6 * k < kMaxStatGroups) spart[(st_g + 6 * k) * kKeyBlock + st_row] = ps[k];
-    if (!FOLDED && (int)threadIdx.x < upr) {
-        reinterpret_cast<h8 *>(gb)[threadIdx.x] = gam_in;
-        reinterpret_cast<h8 *>(gb + in)[threadIdx.x] = bet_in;
-    }
-    __syncthreads();
-    if (threadIdx.x < kKeyBlock) {
-        float s1 = 0.0f, s2 = 0.0f;
-        for (int gi = 0; gi < qa.st_groups; gi++) {
-            const float2 pr = spart[gi * kKeyBlock + threadIdx.x];
-            s1 += pr.x;
-            s2 += pr.y;
-        }
-        const float mean = s1 / (float)in;
-        const float2 mine = {mean, rsqrtf(fmaxf(__builtin_fmaf(-mean, mean, s2 / (float)in), 0.0f) + qa.eps)};
-        stat[threadIdx.x] = float2{-mean * mine.y, mine.y};
-        if (qa.fin_out && h == 0 && (int)threadIdx.x < S)
-            *reinterpret_cast<float2 *>(qa.fin_out + 2 * (row0 + threadIdx.x)) = mine;
     }
     __syncthreads();  // the statistics are complete and the partial sums read: xs may be written
 
