@@ -9,11 +9,12 @@
 // flops, one wave per SIMD), is for problems that fill the device with it; smaller problems
 // take smaller tiles (more workgroups, several per compute unit) at the price of more operand
 // traffic from the L2 per flop.  Latencies are covered inside the wave: K advances in stages
-// of 64 through two LDS buffers, the next stage is loaded straight from global memory into
-// the idle buffer while the current one is multiplied (staging through registers and
+// of 64 through two LDS buffers (the 256 x 256 tile: stages of 32 through four, loads three
+// stages ahead), a later stage is loaded straight from global memory into
+// an idle buffer while the current one is multiplied (staging through registers and
 // ds_write costs a third of the rate: the LDS port is then the bound), the fragment reads of
-// the next K slice are issued ahead of the MFMAs that hide them, and the one workgroup barrier
-// of a stage sits before its last K slice.
+// the next K slice and the loads are issued between the MFMAs that hide them, in an order fixed in
+// the source, and the one workgroup barrier of a stage sits before its last K slice.
 //
 // The MFMA A operand is the B matrix (output features) and vice versa, so a lane ends with
 // 4 consecutive features of one row of C per 8-row group of a tile; the epilogue transposes
@@ -25,8 +26,8 @@ namespace et {
 constexpr int kDmaK = 64;                // K per stage: one 128-byte line of every row
 constexpr int kDmaXcds = 8;
 constexpr int kSbM = 4, kSbN = 8;        // tile block one XCD works on at a time
-constexpr size_t dma_lds_bytes(int tmw, int tnw, int nbuf) {  // buffers of (BM + BN) rows of 128 bytes
-    return (size_t)nbuf * 64 * (tmw + tnw) * kDmaK * sizeof(_Float16);
+constexpr size_t dma_lds_bytes(int tmw, int tnw, int nbuf, int ks = kDmaK) {  // buffers of (BM + BN) rows of ks k-values
+    return (size_t)nbuf * 64 * (tmw + tnw) * ks * sizeof(_Float16);
 }
 // s_waitcnt immediate for vmcnt(n) alone on gfx9: vmcnt in bits 3:0 and 15:14, expcnt 6:4 and
 // lgkmcnt 11:8 left at their maxima
@@ -43,9 +44,12 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 // BT: B is stored [K x N] (N contiguous) instead of [N x K]; its stage lies in LDS as loaded, k-major,
 // and a lane gathers the 8 k-values of a fragment with 2-byte reads (64 x 64 tiles only).
 // Problem z = blockIdx.y of a batch uses the operand offsets of GemmArgs.
-template <int TMW, int TNW, int NBUF, bool IDX, bool RAGGED = false, bool BT = false>
+// KS: k-values per stage, 64 or (whole tiles only) 32: half the stage, twice the buffers in the same LDS, so the
+// loads of a stage are issued three stages ahead and spread over two K slices.
+template <int TMW, int TNW, int NBUF, bool IDX, bool RAGGED = false, bool BT = false, int KS = kDmaK>
 __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
-    static_assert(NBUF >= 2 && NBUF <= 4 && (NBUF - 2) * (2 * TMW + 2 * TNW) <= 63, "vmcnt holds 63 loads");
+    static_assert(NBUF >= 2 && NBUF <= 4 && (NBUF - 1) * (2 * TMW + 2 * TNW) * KS / kDmaK <= 63, "vmcnt holds 63 loads");
+    static_assert(KS == kDmaK || (KS == 32 && !RAGGED && !BT), "half stages are written for whole tiles");
     static_assert(!BT || (TMW == 1 && TNW == 1 && RAGGED), "the k-major B stage is written for the 64 x 64 tile");
     GemmArgs g = ga;
     {
@@ -58,11 +62,11 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
     constexpr int BM = 64 * TMW, BN = 64 * TNW;  // workgroup tile
     constexpr int WM = 32 * TMW, WN = 32 * TNW;  // wave block
     extern __shared__ __align__(16) unsigned char dma_smem[];
-    _Float16 *As = reinterpret_cast<_Float16 *>(dma_smem);  // [NBUF][BM][kDmaK], chunks swizzled
-    _Float16 *Bs = As + NBUF * BM * kDmaK;                   // [NBUF][BN][kDmaK]
+    _Float16 *As = reinterpret_cast<_Float16 *>(dma_smem);  // [NBUF][BM][KS], chunks swizzled
+    _Float16 *Bs = As + NBUF * BM * KS;                      // [NBUF][BN][KS]
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: LDS targets of the loads stay scalar
     const int wm = wave >> 1, wn = wave & 1;
     const int l32 = lane & 31, kg = lane >> 5;
     // Workgroup id -> tile, XCD-aware.  Workgroups go to the 8 XCDs round-robin by id and each
@@ -90,7 +94,60 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
     // within the row the lane at position p fetches chunk p ^ swz(row), so that the fragment
     // reads below, 16 rows apart by one chunk column, spread over all banks with no padding.
     const int lrow = lane >> 3, lpos = lane & 7;
+    // Whole tiles (kWhole): a lane's loads differ between stages only by the stage's k0, so a load is a scalar base
+    // that advances by one line per stage plus a 32-bit lane offset computed once; every stage issues its loads
+    // (past the last stage they fetch the last stage again, into a buffer nobody reads any more), which keeps the
+    // loads in the block of the multiplications, where they can be placed between them, and the number of
+    // outstanding loads the same in every stage.
+    constexpr bool kWhole = !RAGGED && !BT;
+    // A stage row holds KS k-values = kLpr 16-byte chunks; one load instruction fills kRpi rows.  The chunk at
+    // position p of row r is chunk p ^ swz(r) of the operand: rows that share their banks (2 rows of 128 bytes,
+    // 4 rows of 64 bytes span all banks) get different chunks at one position.
+    constexpr int kLpr = KS / 8, kRpi = 64 / kLpr;
+    constexpr int kLA = BM / 4 / kRpi, kLB = BN / 4 / kRpi;  // loads per wave and stage
+    auto swz_of = [](int r) { return KS == 64 ? (r >> 1) & 7 : (r >> 2) & 3; };
+    // The instruction's immediate offset is added to the global address and to the LDS address alike: loads
+    // 4j .. 4j + 3 of an operand share one LDS base (M0) and differ in the immediate, 1024 (v % 4), which the
+    // lane's global offset has subtracted again.  One write of M0 per four loads instead of one per load.
+    unsigned offA[kLA], offB[kLB];  // bytes from the tile's first row at k = 0, minus the immediate
+    if (kWhole) {
+        const int lr = lane / kLpr, lp = lane % kLpr;
+#pragma unroll
+        for (int v = 0; v < kLA; v++) {
+            const int r = wave * (BM / 4) + v * kRpi + lr;
+            offA[v] = (unsigned)((r * g.lda + (lp ^ swz_of(r)) * 8) * 2 - (v % 4) * 1024);
+        }
+#pragma unroll
+        for (int v = 0; v < kLB; v++) {
+            const int r = wave * (BN / 4) + v * kRpi + lr;
+            offB[v] = (unsigned)((r * g.ldb + (lp ^ swz_of(r)) * 8) * 2 - (v % 4) * 1024);
+        }
+    }
+    const char *a_tile = reinterpret_cast<const char *>(g.A + (size_t)m0 * g.lda);
+    const char *b_tile = reinterpret_cast<const char *>(g.B + (size_t)n0 * g.ldb);
+    // loads [first, first + count) of a stage's kLA + kLB (whole tiles)
+    auto load_part = [&](int buf, int k0, int first, int count) {
+        const char *ak = a_tile + (size_t)k0 * 2, *bk = b_tile + (size_t)k0 * 2;  // uniform
+        auto four = [&](const char *src, _Float16 *dst, int sub) {  // sub = v % 4 (a constant once unrolled)
+            if (sub == 0) __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(src), ET_LDS_PTR(dst), 16, 0, 0);
+            else if (sub == 1) __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(src), ET_LDS_PTR(dst), 16, 1024, 0);
+            else if (sub == 2) __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(src), ET_LDS_PTR(dst), 16, 2048, 0);
+            else __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(src), ET_LDS_PTR(dst), 16, 3072, 0);
+        };
+#pragma unroll
+        for (int v = 0; v < kLA; v++)
+            if (v >= first && v < first + count)
+                four(ak + offA[v], As + (buf * BM + wave * (BM / 4) + (v / 4) * 4 * kRpi) * KS, v % 4);
+#pragma unroll
+        for (int v = 0; v < kLB; v++)
+            if (kLA + v >= first && kLA + v < first + count)
+                four(bk + offB[v], Bs + (buf * BN + wave * (BN / 4) + (v / 4) * 4 * kRpi) * KS, v % 4);
+    };
     auto load_stage = [&](int buf, int k0) {
+        if constexpr (kWhole) {
+            load_part(buf, k0, 0, kLA + kLB);
+            return;
+        }
 #pragma unroll
         for (int v = 0; v < 2 * TMW; v++) {  // a wave loads a quarter of the rows of each operand
             const int r0 = wave * (BM / 4) + v * 8, r = r0 + lrow;
@@ -140,13 +197,13 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
     // fragments of one 16-wide K slice: the token tiles and feature tiles of the wave's block.
     // Rows WM wm + 32 i + l32: the swizzle term (row >> 1) & 7 depends on the lane only.
     struct Frag { h8 x[TMW], w[TNW]; };
-    const int swz = (l32 >> 1) & 7;
-    const _Float16 *a_rows = As + (wm * WM + l32) * kDmaK, *b_rows = Bs + (wn * WN + l32) * kDmaK;
+    const int swz = swz_of(l32);
+    const _Float16 *a_rows = As + (wm * WM + l32) * KS, *b_rows = Bs + (wn * WN + l32) * KS;
     auto read_frag = [&](Frag &f, int buf, int ks) {
         const int chunk = ((ks * 2 + kg) ^ swz) * 8;
 #pragma unroll
         for (int i = 0; i < TMW; i++)
-            f.x[i] = *reinterpret_cast<const h8 *>(a_rows + buf * BM * kDmaK + chunk + i * 32 * kDmaK);
+            f.x[i] = *reinterpret_cast<const h8 *>(a_rows + buf * BM * KS + chunk + i * 32 * KS);
 #pragma unroll
         for (int j = 0; j < TNW; j++) {
             if (BT) {
@@ -154,7 +211,7 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
 #pragma unroll
                 for (int e = 0; e < 8; e++) f.w[j][e] = col[e * BN];
             } else {
-                f.w[j] = *reinterpret_cast<const h8 *>(b_rows + buf * BN * kDmaK + chunk + j * 32 * kDmaK);
+                f.w[j] = *reinterpret_cast<const h8 *>(b_rows + buf * BN * KS + chunk + j * 32 * KS);
             }
         }
     };
@@ -166,13 +223,13 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f.w[j], f.x[i], acc[i][j], 0, 0, 0);
     };
 
-    const int nstage = RAGGED ? (g.K + kDmaK - 1) / kDmaK : g.K / kDmaK;
+    const int nstage = RAGGED ? (g.K + kDmaK - 1) / kDmaK : g.K / KS;
     // Stage s is multiplied from LDS buffer s % NBUF; the loads of kAhead later stages are in
     // flight meanwhile.  A direct-to-LDS load has landed when vmcnt says so, and vmcnt counts
     // in issue order: "stage s + 1 has landed" is "at most the loads of the stages after it
     // are outstanding".
     constexpr int kAhead = NBUF - 1;
-    constexpr int kStageLoads = 2 * TMW + 2 * TNW;  // per wave
+    constexpr int kStageLoads = kWhole ? kLA + kLB : 2 * TMW + 2 * TNW;  // per wave
     auto wait_stages = [&](int later) {  // wait until at most `later` whole stages are outstanding
         if (later <= 0) __builtin_amdgcn_s_waitcnt(wait_vm(0));
         else if (later == 1) __builtin_amdgcn_s_waitcnt(wait_vm(kStageLoads));
@@ -183,18 +240,71 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
     // included, which is exactly what a deeper pipeline must not do; here this wave's LDS reads
     // are waited for, the barrier is passed, and the compiler moves no memory access across.
     auto lds_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
-    Frag f0, f1;
+    // Order of issue inside one K slice.  The wave's instruction stream is the only thing that feeds the matrix
+    // pipe of its SIMD, so the LDS reads of the next slice go between the MFMAs of the current one instead of in a
+    // run in front of the MFMAs that need them (left alone the scheduler puts every read directly in front of its
+    // first use and the pipe drains while it returns: 2 x 4 of 16 MFMAs apart, then a wait).  Where the slice is not
+    // written out by hand (below), the pattern is given to the scheduler: kNM / kND MFMAs, one LDS read, ...
+    constexpr int kNM = TMW * TNW, kND = TMW + TNW;
+    constexpr int kSlices = KS / 16;                  // K slices (steps) of a stage
+    constexpr int kLoadSteps = KS == 32 ? 2 : 1;      // steps of a stage that issue a share of a later stage's loads
+    constexpr int kStepLoads = kStageLoads / kLoadSteps;
+    auto interleave = [&] {
+        if constexpr (kNM >= kND) {
+            constexpr int per = kNM / kND;  // MFMAs per LDS read
 #pragma unroll
-    for (int p = 0; p < kAhead; p++)
-        if (p < nstage) load_stage(p, p * kDmaK);
-    wait_stages(min(kAhead, nstage) - 1);
+            for (int i = 0; i < kND; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, per, 0);  // MFMA
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);    // LDS read
+            }
+            __builtin_amdgcn_sched_group_barrier(0x008, kNM - per * kND, 0);
+        }
+    };
+    // Whole tiles with at least as many MFMAs as fragments in a K slice: the slice is written out in the order it is
+    // to be issued in, one MFMA at a time with a fence for the scheduler behind it: after every kNM / kND MFMAs
+    // one fragment of the next slice is read from LDS, and `nload` loads of a later stage (from number `first`)
+    // are dealt evenly between the MFMAs (the four waves of a workgroup issue their loads in the same slices, and
+    // a wave whose load waits for the compute unit's one address unit issues no MFMA behind it).
+    constexpr bool kManual = kWhole && kNM >= kND && kNM % kND == 0;
+    static_assert(!kManual || kStepLoads % kNM == 0 || kNM % kStepLoads == 0, "the loads of a slice are dealt evenly to its MFMAs");
+    auto step = [&](const Frag &fm, Frag &fr, int rbuf, int rks, int nload, int lbuf, int k_later, int first) {
+        constexpr int per = kNM / kND;
+        const int chunk = ((rks * 2 + kg) ^ swz) * 8;
+        // more loads than MFMAs: nload / kNM behind every MFMA; fewer: one behind every (kNM / nload)-th
+        const int lpm = nload >= kNM ? nload / kNM : 0;
+        const int every = (nload > 0 && nload < kNM) ? kNM / nload : 1;
+#pragma unroll
+        for (int m = 0; m < kNM; m++) {
+            const int i = m / TNW, j = m % TNW;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fm.w[j], fm.x[i], acc[i][j], 0, 0, 0);
+            if (m % per == per - 1) {
+                const int idx = m / per;
+                if (idx < TMW) fr.x[idx] = *reinterpret_cast<const h8 *>(a_rows + rbuf * BM * KS + chunk + idx * 32 * KS);
+                else fr.w[idx - TMW] = *reinterpret_cast<const h8 *>(b_rows + rbuf * BN * KS + chunk + (idx - TMW) * 32 * KS);
+            }
+            if (lpm > 0) load_part(lbuf, k_later, first + m * lpm, lpm);
+            else if (nload > 0 && m % every == every / 2) load_part(lbuf, k_later, first + m / every, 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    Frag f0, f1;
+    if constexpr (kWhole) {
+#pragma unroll
+        for (int p = 0; p < kAhead; p++) load_stage(p, min(p, nstage - 1) * KS);
+        __builtin_amdgcn_s_waitcnt(wait_vm((kAhead - 1) * kStageLoads));  // stage 0 has landed
+    } else {
+#pragma unroll
+        for (int p = 0; p < kAhead; p++)
+            if (p < nstage) load_stage(p, p * kDmaK);
+        wait_stages(min(kAhead, nstage) - 1);
+    }
     if (RAGGED && nstage == 1 && ktail < kDmaK) zero_tail(0);
     lds_barrier();
     read_frag(f0, 0, 0);
     // One stage, with the matrix pipe fed across the barrier: every K slice is read from LDS
     // while the one before it is multiplied, the first slice of the next stage included, so the
     // barrier of the stage sits before its last slice.  The loads of stage s + kAhead are issued
-    // at the start of stage s into the buffer stage s - 1 was read from (its last readers passed
+    // in stage s into the buffer stage s - 1 was read from (its last readers passed
     // the previous barrier); stage s + 1 is waited for just before the barrier.  The fragment
     // read after the barrier of the last stage touches valid LDS and is never used; the loop
     // has a single exit (a second one in the middle makes the register allocator copy the
@@ -202,20 +312,54 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
     int cur = 0;
     for (int s = 0; s < nstage; s++) {
         const int nxt = cur + 1 == NBUF ? 0 : cur + 1;
-        if (s + kAhead < nstage) load_stage(cur == 0 ? NBUF - 1 : cur - 1, (s + kAhead) * kDmaK);
-        read_frag(f1, cur, 1);
-        multiply(f0);
-        read_frag(f0, cur, 2);
-        multiply(f1);
-        read_frag(f1, cur, 3);
-        multiply(f0);
-        wait_stages(min(kAhead - 1, nstage - 2 - s));
-        if (RAGGED && s + 2 == nstage && ktail < kDmaK) zero_tail(nxt);
-        lds_barrier();
-        read_frag(f0, nxt, 0);
-        multiply(f1);
+        const int prev = cur == 0 ? NBUF - 1 : cur - 1;
+        const int k_later = min(s + kAhead, nstage - 1) * KS;  // whole tiles: past the end, the last stage again
+        if constexpr (kManual) {
+            step(f0, f1, cur, 1, kStepLoads, prev, k_later, 0);
+            if constexpr (kSlices == 4) {
+                step(f1, f0, cur, 2, 0, prev, k_later, 0);
+                step(f0, f1, cur, 3, 0, prev, k_later, 0);
+            }
+            // outstanding at most: the stages after s + 1 as far as they have been issued
+            __builtin_amdgcn_s_waitcnt(wait_vm((kAhead - 2) * kStageLoads + kStepLoads));
+            lds_barrier();
+            step(f1, f0, nxt, 0, kLoadSteps == 2 ? kStepLoads : 0, prev, k_later, kStepLoads);
+        } else {
+            if constexpr (kWhole) {
+                read_frag(f1, cur, 1);
+                load_part(prev, k_later, 0, kStepLoads);
+            } else {
+                if (s + kAhead < nstage) load_stage(prev, (s + kAhead) * kDmaK);
+                read_frag(f1, cur, 1);
+            }
+            multiply(f0);
+            interleave();
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (kSlices == 4) {
+                read_frag(f0, cur, 2);
+                multiply(f1);
+                interleave();
+                __builtin_amdgcn_sched_barrier(0);
+                read_frag(f1, cur, 3);
+                multiply(f0);
+                interleave();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // outstanding at most: the stages after s + 1 as far as they have been issued
+            if constexpr (kWhole) __builtin_amdgcn_s_waitcnt(wait_vm((kAhead - 2) * kStageLoads + kStepLoads));
+            else wait_stages(min(kAhead - 1, nstage - 2 - s));
+            if (RAGGED && s + 2 == nstage && ktail < kDmaK) zero_tail(nxt);
+            lds_barrier();
+            read_frag(f0, nxt, 0);
+            if constexpr (kWhole && kLoadSteps == 2) load_part(prev, k_later, kStepLoads, kStepLoads);
+            multiply(f1);
+            interleave();
+            __builtin_amdgcn_sched_barrier(0);
+        }
         cur = nxt;
     }
+    // the loads issued past the last stage have landed before the staging LDS is written again
+    if constexpr (kWhole) __builtin_amdgcn_s_waitcnt(wait_vm(0));
     __syncthreads();  // the staging LDS becomes the transposition buffer of the epilogue
 
     // Epilogue.  acc[i][j][e] is token WM wm + 32 i + l32, feature WN wn + 32 j + 8 (e / 4) +
@@ -308,7 +452,7 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
 // operand traffic from the L2 per flop but needs enough workgroups to keep every compute unit
 // busy through whole rounds (a 256 x 256 workgroup owns its compute unit; two 128 x 128, three
 // 128 x 64 or five 64 x 64 ones share it and cover each other's prologue and epilogue).
-// 256 x 128 tiles and a fourth LDS buffer were measured and never won.
+// 256 x 128 tiles were measured and never won.
 struct DmaTile { int tmw, tnw, nbuf; bool ragged; };
 static bool pick_dma_tile(const GemmArgs &g, int batch, bool trans_b, DmaTile *out) {
     const bool ragged = g.M % 64 || g.N % 64 || g.K % kDmaK || batch != 1 || !trans_b;
@@ -358,19 +502,20 @@ bool gemm_dma_applies(const GemmArgs &g, int batch, bool trans_b) {
     const auto misaligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) != 0; };
     if (batch < 1 || batch > 65535 || g.a_gather || g.M <= 0) return false;
     if (g.lda % 8 || g.ldb % 8 || g.ldc % 8 || misaligned(g.A) || misaligned(g.B) || misaligned(g.C)) return false;
+    if (g.lda > (1 << 21) || g.ldb > (1 << 21)) return false;  // a tile's rows are addressed with 32-bit byte offsets
     if (batch > 1 && ((g.sAo | g.sAi | g.sBo | g.sBi | g.sCo | g.sCi) & 7)) return false;  // every problem aligned
     return pick_dma_tile(g, batch, trans_b, &t);
 }
 
-template <int TMW, int TNW, int NBUF, bool IDX, bool RAGGED, bool BT = false>
+template <int TMW, int TNW, int NBUF, bool IDX, bool RAGGED, bool BT = false, int KS = kDmaK>
 static int launch_dma_variant(const GemmArgs &g, int batch, hipStream_t stream) {
     constexpr int BM = 64 * TMW, BN = 64 * TNW;
-    constexpr size_t lds = dma_lds_bytes(TMW, TNW, NBUF);
+    constexpr size_t lds = dma_lds_bytes(TMW, TNW, NBUF, KS);
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     const int nsb = ((tiles_m + kSbM - 1) / kSbM) * ((tiles_n + kSbN - 1) / kSbN);
     const int rounds = (nsb + kDmaXcds - 1) / kDmaXcds;
     const dim3 grid((unsigned)(rounds * kDmaXcds * kSbM * kSbN), (unsigned)batch);
-    auto kernel = gemm_f16_dma_kernel<TMW, TNW, NBUF, IDX, RAGGED, BT>;
+    auto kernel = gemm_f16_dma_kernel<TMW, TNW, NBUF, IDX, RAGGED, BT, KS>;
     static bool raised = false;  // more than 64 KB of dynamic LDS needs the attribute, once per kernel
     if (!raised) {
         ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -381,10 +526,10 @@ static int launch_dma_variant(const GemmArgs &g, int batch, hipStream_t stream) 
     return check_launch("gemm_f16_dma_kernel");
 }
 
-template <int TMW, int TNW, int NBUF, bool RAGGED = false, bool BT = false>
+template <int TMW, int TNW, int NBUF, bool RAGGED = false, bool BT = false, int KS = kDmaK>
 static int launch_dma_tile(const GemmArgs &g, int batch, hipStream_t stream) {
-    return (g.c_scatter || g.bias_idx) ? launch_dma_variant<TMW, TNW, NBUF, true, RAGGED, BT>(g, batch, stream)
-                                       : launch_dma_variant<TMW, TNW, NBUF, false, RAGGED, BT>(g, batch, stream);
+    return (g.c_scatter || g.bias_idx) ? launch_dma_variant<TMW, TNW, NBUF, true, RAGGED, BT, KS>(g, batch, stream)
+                                       : launch_dma_variant<TMW, TNW, NBUF, false, RAGGED, BT, KS>(g, batch, stream);
 }
 
 int launch_gemm_dma(const GemmArgs &g, int batch, bool trans_b, hipStream_t stream) {
@@ -401,7 +546,7 @@ int launch_gemm_dma(const GemmArgs &g, int batch, bool trans_b, hipStream_t stre
                            : launch_dma_tile<1, 1, 2, true>(g, batch, stream);
     }
     switch (t.tmw * 100 + t.tnw * 10 + t.nbuf) {
-        case 442: return launch_dma_tile<4, 4, 2>(g, 1, stream);
+        case 442: return launch_dma_tile<4, 4, 4, false, false, 32>(g, 1, stream);  // half stages, four buffers
         case 222: return launch_dma_tile<2, 2, 2>(g, 1, stream);
         case 212: return launch_dma_tile<2, 1, 2>(g, 1, stream);
         case 112: return launch_dma_tile<1, 1, 2>(g, 1, stream);

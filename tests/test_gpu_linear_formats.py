@@ -20,6 +20,8 @@ up = Hn.up
                                            # one shape per tile of the direct-to-LDS kernel: 256x256, 128x128,
                                            # 128x64, 64x64 with three LDS buffers, a single K stage
                                            (4096, 192, 4096, 2), (2048, 128, 4096, 1), (2048, 192, 2304, 0),
+                                           # 256x256 tiles with a single K stage, and with many
+                                           (4096, 64, 4096, 0), (4096, 1024, 4096, 1),
                                            (512, 1536, 768, 2), (256, 64, 256, 0),
                                            # edges that are multiples of 16 only (clamped loads, zeroed K tail,
                                            # masked stores): 16, 32 and 48 k-values in the last stage
