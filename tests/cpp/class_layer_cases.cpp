@@ -289,6 +289,21 @@ static int run_factories(const std::string &dir) {
         out.push_back(32.0f * (float)(rp[1] - rp[0]) + 0.5f);
     }
     etChk(et_device_sync());
+    // Linear<row_mat> picks its form by the share of features that survive: half of them -> a dense image of the
+    // weight; one in sixteen -> the scattering GEMM behind a fill.  Both: live features x.w + b, dead ones b.
+    for (const float sp : {0.5f, 0.9375f}) {
+        auto lin = gen_sparse_linear<row_mat>(512, 256, T, sp);
+        lin->forward(Y.get(), X256.get());
+        auto ids = lin->weight.row_id->to_host();
+        auto y = Y.to_host();
+        int dead = 0;
+        while (std::find(ids.begin(), ids.end(), dead) != ids.end()) dead++;
+        out.push_back(static_cast<float>(y[(std::size_t)ids[0]]));             // 256.5
+        out.push_back(static_cast<float>(y[(std::size_t)dead]));               // 0.5
+        out.push_back(static_cast<float>(y[(std::size_t)(T - 1) * 512 + (std::size_t)ids.back()]));  // 256.5, last row
+        out.push_back((float)ids.size());                                      // 256, 32
+        out.push_back(lin->dense_image ? 1.0f : 0.0f);                         // 1, 0
+    }
     npy_save(dir + "/factories.npy", out.data(), "<f4", 4, {out.size()});
     return 0;
 }

@@ -169,6 +169,9 @@ def test_factories_closed_forms(tmp_path):
     assert db[4:8] == [3.0, 4.0, 0.0, 1.0]
     assert db[8:10] == [7.0, 6.0]  # DeviceBuffer(ptr, n) from a device pointer and from a host pointer
     assert db[10] == db[11] and db[10] > 32.0  # Linear<tile_mat>::refresh() after the caller rewrote weight.data
+    # Linear<row_mat>, 512 features: half kept -> dense image; 1 in 16 kept -> fill + scattering GEMM
+    assert db[12:17] == [256.5, 0.5, 256.5, 256.0, 1.0]
+    assert db[17:22] == [256.5, 0.5, 256.5, 32.0, 0.0]
 
 
 def test_attention_tags_with_separate_projections(tmp_path):
