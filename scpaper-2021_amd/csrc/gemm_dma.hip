@@ -5,8 +5,8 @@
 // MFMA peak is the whole bandwidth of the LDS port, and stages through registers; it tops
 // out near a third of the matrix peak.  Here a workgroup of 4 waves (2 x 2) computes a tile of
 // 64 TMW x 64 TNW and each wave a block of TMW x TNW v_mfma_f32_32x32x16_f16 tiles.  The
-// largest tile, 256 x 256 (a wave: 128 x 128, 256 accumulators in AGPRs, 1 byte of LDS per 64
-// flops, one wave per SIMD), is for problems that fill the device with it; smaller problems
+// largest tile, 256 x 256 (eight waves of 128 x 64, two per SIMD; the RAGGED form four waves of
+// 128 x 128 with 256 accumulators in AGPRs), is for problems that fill the device with it; smaller problems
 // take smaller tiles (more workgroups, several per compute unit) at the price of more operand
 // traffic from the L2 per flop.  Latencies are covered inside the wave: K advances in stages
 // of 64 through two LDS buffers (the 256 x 256 tile: stages of 32 through four, loads three
@@ -26,8 +26,8 @@ namespace et {
 constexpr int kDmaK = 64;                // K per stage: one 128-byte line of every row
 constexpr int kDmaXcds = 8;
 constexpr int kSbM = 4, kSbN = 8;        // tile block one XCD works on at a time
-constexpr size_t dma_lds_bytes(int tmw, int tnw, int nbuf, int ks = kDmaK) {  // buffers of (BM + BN) rows of ks k-values
-    return (size_t)nbuf * 64 * (tmw + tnw) * ks * sizeof(_Float16);
+constexpr size_t dma_lds_bytes(int tmw, int tnw, int nbuf, int ks = kDmaK, int nwn = 2) {  // buffers of (BM + BN) rows of ks k-values
+    return (size_t)nbuf * (64 * tmw + 32 * nwn * tnw) * ks * sizeof(_Float16);
 }
 // s_waitcnt immediate for vmcnt(n) alone on gfx9: vmcnt in bits 3:0 and 15:14, expcnt 6:4 and
 // lgkmcnt 11:8 left at their maxima
@@ -46,8 +46,12 @@ typedef float f16v __attribute__((ext_vector_type(16)));
 // Problem z = blockIdx.y of a batch uses the operand offsets of GemmArgs.
 // KS: k-values per stage, 64 or (whole tiles only) 32: half the stage, twice the buffers in the same LDS, so the
 // loads of a stage are issued three stages ahead and spread over two K slices.
-template <int TMW, int TNW, int NBUF, bool IDX, bool RAGGED = false, bool BT = false, int KS = kDmaK>
-__global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
+// NWN: waves along N, 2 (four waves, one per SIMD) or (whole tiles only) 4: eight waves, two per SIMD, so that a wave
+// held up at a load or at the barrier leaves the matrix pipe to the other.
+template <int TMW, int TNW, int NBUF, bool IDX, bool RAGGED = false, bool BT = false, int KS = kDmaK, int NWN = 2>
+__global__ __launch_bounds__(128 * NWN) void gemm_f16_dma_kernel(const GemmArgs ga) {
+    static_assert(NWN == 2 || (NWN == 4 && !RAGGED && !BT), "eight waves are written for whole tiles");
+    constexpr int kWaves = 2 * NWN;
     static_assert(NBUF >= 2 && NBUF <= 4 && (NBUF - 1) * (2 * TMW + 2 * TNW) * KS / kDmaK <= 63, "vmcnt holds 63 loads");
     static_assert(KS == kDmaK || (KS == 32 && !RAGGED && !BT), "half stages are written for whole tiles");
     static_assert(!BT || (TMW == 1 && TNW == 1 && RAGGED), "the k-major B stage is written for the 64 x 64 tile");
@@ -59,7 +63,7 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
         g.C += zo * g.sCo + zi * g.sCi;
         if (g.bias) g.bias += zo * g.sBias_o + zi * g.sBias_i;
     }
-    constexpr int BM = 64 * TMW, BN = 64 * TNW;  // workgroup tile
+    constexpr int BM = 64 * TMW, BN = 32 * NWN * TNW;  // workgroup tile: 2 x NWN waves
     constexpr int WM = 32 * TMW, WN = 32 * TNW;  // wave block
     extern __shared__ __align__(16) unsigned char dma_smem[];
     _Float16 *As = reinterpret_cast<_Float16 *>(dma_smem);  // [NBUF][BM][KS], chunks swizzled
@@ -67,7 +71,7 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: LDS targets of the loads stay scalar
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / NWN, wn = wave % NWN;
     const int l32 = lane & 31, kg = lane >> 5;
     // Workgroup id -> tile, XCD-aware.  Workgroups go to the 8 XCDs round-robin by id and each
     // XCD runs 32 of them at a time; those 32 are given a 4 x 8 block of tiles (4 panels of A,
@@ -104,7 +108,7 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
     // position p of row r is chunk p ^ swz(r) of the operand: rows that share their banks (2 rows of 128 bytes,
     // 4 rows of 64 bytes span all banks) get different chunks at one position.
     constexpr int kLpr = KS / 8, kRpi = 64 / kLpr;
-    constexpr int kLA = BM / 4 / kRpi, kLB = BN / 4 / kRpi;  // loads per wave and stage
+    constexpr int kLA = BM / kWaves / kRpi, kLB = BN / kWaves / kRpi;  // loads per wave and stage
     auto swz_of = [](int r) { return KS == 64 ? (r >> 1) & 7 : (r >> 2) & 3; };
     // The instruction's immediate offset is added to the global address and to the LDS address alike: loads
     // 4j .. 4j + 3 of an operand share one LDS base (M0) and differ in the immediate, 1024 (v % 4), which the
@@ -114,12 +118,12 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
         const int lr = lane / kLpr, lp = lane % kLpr;
 #pragma unroll
         for (int v = 0; v < kLA; v++) {
-            const int r = wave * (BM / 4) + v * kRpi + lr;
+            const int r = wave * (BM / kWaves) + v * kRpi + lr;
             offA[v] = (unsigned)((r * g.lda + (lp ^ swz_of(r)) * 8) * 2 - (v % 4) * 1024);
         }
 #pragma unroll
         for (int v = 0; v < kLB; v++) {
-            const int r = wave * (BN / 4) + v * kRpi + lr;
+            const int r = wave * (BN / kWaves) + v * kRpi + lr;
             offB[v] = (unsigned)((r * g.ldb + (lp ^ swz_of(r)) * 8) * 2 - (v % 4) * 1024);
         }
     }
@@ -137,11 +141,11 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
 #pragma unroll
         for (int v = 0; v < kLA; v++)
             if (v >= first && v < first + count)
-                four(ak + offA[v], As + (buf * BM + wave * (BM / 4) + (v / 4) * 4 * kRpi) * KS, v % 4);
+                four(ak + offA[v], As + (buf * BM + wave * (BM / kWaves) + (v / 4) * 4 * kRpi) * KS, v % 4);
 #pragma unroll
         for (int v = 0; v < kLB; v++)
             if (kLA + v >= first && kLA + v < first + count)
-                four(bk + offB[v], Bs + (buf * BN + wave * (BN / 4) + (v / 4) * 4 * kRpi) * KS, v % 4);
+                four(bk + offB[v], Bs + (buf * BN + wave * (BN / kWaves) + (v / 4) * 4 * kRpi) * KS, v % 4);
     };
     auto load_stage = [&](int buf, int k0) {
         if constexpr (kWhole) {
@@ -265,10 +269,9 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
     // one fragment of the next slice is read from LDS, and `nload` loads of a later stage (from number `first`)
     // are dealt evenly between the MFMAs (the four waves of a workgroup issue their loads in the same slices, and
     // a wave whose load waits for the compute unit's one address unit issues no MFMA behind it).
-    constexpr bool kManual = kWhole && kNM >= kND && kNM % kND == 0;
+    constexpr bool kManual = kWhole && kNM >= kND;
     static_assert(!kManual || kStepLoads % kNM == 0 || kNM % kStepLoads == 0, "the loads of a slice are dealt evenly to its MFMAs");
     auto step = [&](const Frag &fm, Frag &fr, int rbuf, int rks, int nload, int lbuf, int k_later, int first) {
-        constexpr int per = kNM / kND;
         const int chunk = ((rks * 2 + kg) ^ swz) * 8;
         // more loads than MFMAs: nload / kNM behind every MFMA; fewer: one behind every (kNM / nload)-th
         const int lpm = nload >= kNM ? nload / kNM : 0;
@@ -277,8 +280,9 @@ __global__ __launch_bounds__(256) void gemm_f16_dma_kernel(const GemmArgs ga) {
         for (int m = 0; m < kNM; m++) {
             const int i = m / TNW, j = m % TNW;
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fm.w[j], fm.x[i], acc[i][j], 0, 0, 0);
-            if (m % per == per - 1) {
-                const int idx = m / per;
+            // fragment idx of the next slice behind MFMA (idx kNM) / kND: evenly over the slice
+            const int idx = (m * kND + kNM - 1) / kNM;
+            if (idx < kND && (idx * kNM) / kND == m) {
                 if (idx < TMW) fr.x[idx] = *reinterpret_cast<const h8 *>(a_rows + rbuf * BM * KS + chunk + idx * 32 * KS);
                 else fr.w[idx - TMW] = *reinterpret_cast<const h8 *>(b_rows + rbuf * BN * KS + chunk + (idx - TMW) * 32 * KS);
             }
@@ -507,29 +511,29 @@ bool gemm_dma_applies(const GemmArgs &g, int batch, bool trans_b) {
     return pick_dma_tile(g, batch, trans_b, &t);
 }
 
-template <int TMW, int TNW, int NBUF, bool IDX, bool RAGGED, bool BT = false, int KS = kDmaK>
+template <int TMW, int TNW, int NBUF, bool IDX, bool RAGGED, bool BT = false, int KS = kDmaK, int NWN = 2>
 static int launch_dma_variant(const GemmArgs &g, int batch, hipStream_t stream) {
-    constexpr int BM = 64 * TMW, BN = 64 * TNW;
-    constexpr size_t lds = dma_lds_bytes(TMW, TNW, NBUF, KS);
+    constexpr int BM = 64 * TMW, BN = 32 * NWN * TNW;
+    constexpr size_t lds = dma_lds_bytes(TMW, TNW, NBUF, KS, NWN);
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     const int nsb = ((tiles_m + kSbM - 1) / kSbM) * ((tiles_n + kSbN - 1) / kSbN);
     const int rounds = (nsb + kDmaXcds - 1) / kDmaXcds;
     const dim3 grid((unsigned)(rounds * kDmaXcds * kSbM * kSbN), (unsigned)batch);
-    auto kernel = gemm_f16_dma_kernel<TMW, TNW, NBUF, IDX, RAGGED, BT, KS>;
+    auto kernel = gemm_f16_dma_kernel<TMW, TNW, NBUF, IDX, RAGGED, BT, KS, NWN>;
     static bool raised = false;  // more than 64 KB of dynamic LDS needs the attribute, once per kernel
     if (!raised) {
         ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         raised = true;
     }
-    kernel<<<grid, 256, lds, stream>>>(g);
+    kernel<<<grid, 128 * NWN, lds, stream>>>(g);
     return check_launch("gemm_f16_dma_kernel");
 }
 
-template <int TMW, int TNW, int NBUF, bool RAGGED = false, bool BT = false, int KS = kDmaK>
+template <int TMW, int TNW, int NBUF, bool RAGGED = false, bool BT = false, int KS = kDmaK, int NWN = 2>
 static int launch_dma_tile(const GemmArgs &g, int batch, hipStream_t stream) {
-    return (g.c_scatter || g.bias_idx) ? launch_dma_variant<TMW, TNW, NBUF, true, RAGGED, BT, KS>(g, batch, stream)
-                                       : launch_dma_variant<TMW, TNW, NBUF, false, RAGGED, BT, KS>(g, batch, stream);
+    return (g.c_scatter || g.bias_idx) ? launch_dma_variant<TMW, TNW, NBUF, true, RAGGED, BT, KS, NWN>(g, batch, stream)
+                                       : launch_dma_variant<TMW, TNW, NBUF, false, RAGGED, BT, KS, NWN>(g, batch, stream);
 }
 
 int launch_gemm_dma(const GemmArgs &g, int batch, bool trans_b, hipStream_t stream) {
@@ -546,7 +550,9 @@ int launch_gemm_dma(const GemmArgs &g, int batch, bool trans_b, hipStream_t stre
                            : launch_dma_tile<1, 1, 2, true>(g, batch, stream);
     }
     switch (t.tmw * 100 + t.tnw * 10 + t.nbuf) {
-        case 442: return launch_dma_tile<4, 4, 4, false, false, 32>(g, 1, stream);  // half stages, four buffers
+        // 256 x 256: eight waves of 128 x 64, half stages through four buffers (four waves of 128 x 128 in the same
+        // LDS: 0.5-2 % slower)
+        case 442: return launch_dma_tile<4, 2, 4, false, false, 32, 4>(g, 1, stream);
         case 222: return launch_dma_tile<2, 2, 2>(g, 1, stream);
         case 212: return launch_dma_tile<2, 1, 2>(g, 1, stream);
         case 112: return launch_dma_tile<1, 1, 2>(g, 1, stream);
