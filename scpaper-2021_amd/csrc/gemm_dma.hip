@@ -98,12 +98,15 @@ __global__ __launch_bounds__(128 * NWN) void gemm_f16_dma_kernel(const GemmArgs 
     // within the row the lane at position p fetches chunk p ^ swz(row), so that the fragment
     // reads below, 16 rows apart by one chunk column, spread over all banks with no padding.
     const int lrow = lane >> 3, lpos = lane & 7;
-    // Whole tiles (kWhole): a lane's loads differ between stages only by the stage's k0, so a load is a scalar base
-    // that advances by one line per stage plus a 32-bit lane offset computed once; every stage issues its loads
-    // (past the last stage they fetch the last stage again, into a buffer nobody reads any more), which keeps the
-    // loads in the block of the multiplications, where they can be placed between them, and the number of
-    // outstanding loads the same in every stage.
-    constexpr bool kWhole = !RAGGED && !BT;
+    // K-contiguous operands (kWhole; all but BT): a lane's loads differ between stages only by the stage's k0, so a
+    // load is a scalar base that advances by one line per stage plus a 32-bit lane offset computed once; every stage
+    // issues its loads (past the last stage they fetch the last stage again, into a buffer nobody reads any more),
+    // which keeps the loads in the block of the multiplications, where they can be placed between them, and the
+    // number of outstanding loads the same in every stage.  RAGGED: rows past the end of an operand take the offset
+    // of its last row, and the last stage, when K ends inside it, has offsets of its own: chunks past the end of K
+    // fetch the last chunk of the row instead (and are zeroed in LDS once they have landed).
+    constexpr bool kWhole = !BT;
+    constexpr bool kImm = !RAGGED;  // (a clamped row may have a smaller offset than the immediate it would have to undo)
     // A stage row holds KS k-values = kLpr 16-byte chunks; one load instruction fills kRpi rows.  The chunk at
     // position p of row r is chunk p ^ swz(r) of the operand: rows that share their banks (2 rows of 128 bytes,
     // 4 rows of 64 bytes span all banks) get different chunks at one position.
@@ -114,17 +117,26 @@ __global__ __launch_bounds__(128 * NWN) void gemm_f16_dma_kernel(const GemmArgs 
     // 4j .. 4j + 3 of an operand share one LDS base (M0) and differ in the immediate, 1024 (v % 4), which the
     // lane's global offset has subtracted again.  One write of M0 per four loads instead of one per load.
     unsigned offA[kLA], offB[kLB];  // bytes from the tile's first row at k = 0, minus the immediate
+    unsigned tailA[RAGGED ? kLA : 1], tailB[RAGGED ? kLB : 1];  // the same for a last stage that K ends in
+    const int k_tail0 = (g.K - 1) / KS * KS;   // first k of the last stage
+    const int k_tail = g.K - k_tail0;          // k-values of the last stage, 16 .. KS
     if (kWhole) {
         const int lr = lane / kLpr, lp = lane % kLpr;
 #pragma unroll
         for (int v = 0; v < kLA; v++) {
             const int r = wave * (BM / kWaves) + v * kRpi + lr;
-            offA[v] = (unsigned)((r * g.lda + (lp ^ swz_of(r)) * 8) * 2 - (v % 4) * 1024);
+            const int row = RAGGED ? min(m0 + r, g.M - 1) - m0 : r;
+            const int c8 = (lp ^ swz_of(r)) * 8;
+            offA[v] = (unsigned)((row * g.lda + c8) * 2 - (kImm ? (v % 4) * 1024 : 0));
+            if (RAGGED) tailA[v] = (unsigned)((row * g.lda + min(c8, k_tail - 8)) * 2);
         }
 #pragma unroll
         for (int v = 0; v < kLB; v++) {
             const int r = wave * (BN / kWaves) + v * kRpi + lr;
-            offB[v] = (unsigned)((r * g.ldb + (lp ^ swz_of(r)) * 8) * 2 - (v % 4) * 1024);
+            const int row = RAGGED ? min(n0 + r, g.N - 1) - n0 : r;
+            const int c8 = (lp ^ swz_of(r)) * 8;
+            offB[v] = (unsigned)((row * g.ldb + c8) * 2 - (kImm ? (v % 4) * 1024 : 0));
+            if (RAGGED) tailB[v] = (unsigned)((row * g.ldb + min(c8, k_tail - 8)) * 2);
         }
     }
     const char *a_tile = reinterpret_cast<const char *>(g.A + (size_t)m0 * g.lda);
@@ -138,14 +150,19 @@ __global__ __launch_bounds__(128 * NWN) void gemm_f16_dma_kernel(const GemmArgs 
             else if (sub == 2) __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(src), ET_LDS_PTR(dst), 16, 2048, 0);
             else __builtin_amdgcn_global_load_lds(ET_GLOBAL_PTR(src), ET_LDS_PTR(dst), 16, 3072, 0);
         };
+        const bool tail = RAGGED && k0 == k_tail0 && k_tail < KS;  // uniform
 #pragma unroll
         for (int v = 0; v < kLA; v++)
-            if (v >= first && v < first + count)
-                four(ak + offA[v], As + (buf * BM + wave * (BM / kWaves) + (v / 4) * 4 * kRpi) * KS, v % 4);
+            if (v >= first && v < first + count) {
+                const unsigned off = RAGGED && tail ? tailA[RAGGED ? v : 0] : offA[v];
+                four(ak + off, As + (buf * BM + wave * (BM / kWaves) + (kImm ? (v / 4) * 4 : v) * kRpi) * KS, kImm ? v % 4 : 0);
+            }
 #pragma unroll
         for (int v = 0; v < kLB; v++)
-            if (kLA + v >= first && kLA + v < first + count)
-                four(bk + offB[v], Bs + (buf * BN + wave * (BN / kWaves) + (v / 4) * 4 * kRpi) * KS, v % 4);
+            if (kLA + v >= first && kLA + v < first + count) {
+                const unsigned off = RAGGED && tail ? tailB[RAGGED ? v : 0] : offB[v];
+                four(bk + off, Bs + (buf * BN + wave * (BN / kWaves) + (kImm ? (v / 4) * 4 : v) * kRpi) * KS, kImm ? v % 4 : 0);
+            }
     };
     auto load_stage = [&](int buf, int k0) {
         if constexpr (kWhole) {
@@ -326,6 +343,7 @@ __global__ __launch_bounds__(128 * NWN) void gemm_f16_dma_kernel(const GemmArgs 
             }
             // outstanding at most: the stages after s + 1 as far as they have been issued
             __builtin_amdgcn_s_waitcnt(wait_vm((kAhead - 2) * kStageLoads + kStepLoads));
+            if (RAGGED && s + 2 == nstage && ktail < kDmaK) zero_tail(nxt);
             lds_barrier();
             step(f1, f0, nxt, 0, kLoadSteps == 2 ? kStepLoads : 0, prev, k_later, kStepLoads);
         } else {
