@@ -269,7 +269,8 @@ __global__ __launch_bounds__(128 * NWN) void gemm_f16_dma_kernel(const GemmArgs 
     constexpr int kNM = TMW * TNW, kND = TMW + TNW;
     constexpr int kSlices = KS / 16;                  // K slices (steps) of a stage
     constexpr int kLoadSteps = KS == 32 ? 2 : 1;      // steps of a stage that issue a share of a later stage's loads
-    constexpr int kStepLoads = kStageLoads / kLoadSteps;
+    constexpr int kStepLoads = (kStageLoads + kLoadSteps - 1) / kLoadSteps;  // in the first such step; the rest in the second
+    constexpr int kStepLoads2 = kStageLoads - kStepLoads;
     auto interleave = [&] {
         if constexpr (kNM >= kND) {
             constexpr int per = kNM / kND;  // MFMAs per LDS read
@@ -287,7 +288,8 @@ __global__ __launch_bounds__(128 * NWN) void gemm_f16_dma_kernel(const GemmArgs 
     // are dealt evenly between the MFMAs (the four waves of a workgroup issue their loads in the same slices, and
     // a wave whose load waits for the compute unit's one address unit issues no MFMA behind it).
     constexpr bool kManual = kWhole && kNM >= kND;
-    static_assert(!kManual || kStepLoads % kNM == 0 || kNM % kStepLoads == 0, "the loads of a slice are dealt evenly to its MFMAs");
+    static_assert(!kManual || ((kStepLoads % kNM == 0 || kNM % kStepLoads == 0) && (kLoadSteps == 1 || kStepLoads2 == kStepLoads)),
+                  "the loads of a slice are dealt evenly to its MFMAs");
     auto step = [&](const Frag &fm, Frag &fr, int rbuf, int rks, int nload, int lbuf, int k_later, int first) {
         const int chunk = ((rks * 2 + kg) ^ swz) * 8;
         // more loads than MFMAs: nload / kNM behind every MFMA; fewer: one behind every (kNM / nload)-th
@@ -373,7 +375,7 @@ __global__ __launch_bounds__(128 * NWN) void gemm_f16_dma_kernel(const GemmArgs 
             if (RAGGED && s + 2 == nstage && ktail < kDmaK) zero_tail(nxt);
             lds_barrier();
             read_frag(f0, nxt, 0);
-            if constexpr (kWhole && kLoadSteps == 2) load_part(prev, k_later, kStepLoads, kStepLoads);
+            if constexpr (kWhole && kLoadSteps == 2) load_part(prev, k_later, kStepLoads, kStepLoads2);
             multiply(f1);
             interleave();
             __builtin_amdgcn_sched_barrier(0);
