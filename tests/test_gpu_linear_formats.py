@@ -102,6 +102,29 @@ def test_linear_dense_closed_form_ones(et):
     assert np.all(d_y.numpy().astype(np.float32) == 256.5)
 
 
+# one shape per tile at a depth the oracle cannot afford: 256 x 256 (eight waves, 128 half stages), the same tile with
+# ragged edges and a K tail of 16, 128 x 128, 128 x 64, 64 x 64 with three buffers, and the register-staged kernel's range
+@pytest.mark.parametrize("T,inp,out", [(4096, 4096, 4096), (8176, 4112, 8208), (4096, 4096, 2048), (2048, 6144, 3072),
+                                       (512, 8192, 768), (16384, 768, 3072), (8192, 4080, 4096)])
+def test_linear_dense_deep_k_closed_form(et, T, inp, out):
+    """Small-integer operands with short periods: x[m, k] = (m + k) % 3 - 1, w[n, k] = (n + 2k) % 5 - 2, bias n % 4.
+    Every product and partial sum is an integer below 2^24, so binary32 accumulation is exact in any order and
+    the result depends on (m % 3, n % 5, n % 4) alone: the expected matrix is 15 sums, tiled, rounded once to
+    binary16.  Bit-exact at full size: a stage multiplied from a buffer that was not ready, a tile mapped to the
+    wrong place or a K tail handled wrongly all show."""
+    k = np.arange(inp, dtype=np.int64)
+    x = ((np.arange(T, dtype=np.int64)[:, None] + k[None, :]) % 3 - 1).astype(np.float16)
+    w = ((np.arange(out, dtype=np.int64)[:, None] + 2 * k[None, :]) % 5 - 2).astype(np.float16)
+    bias = (np.arange(out) % 4).astype(np.float16)
+    sums = np.array([[int((((m + k) % 3 - 1) * ((n + 2 * k) % 5 - 2)).sum()) for n in range(5)] for m in range(3)], np.int32)
+    want = sums[np.arange(T)[:, None] % 3, np.arange(out)[None, :] % 5] + (np.arange(out) % 4)[None, :]
+    assert np.abs(want).max() < 2 ** 24
+    d_y = et.DeviceBuffer.empty((T, out), np.float16)
+    et.linear_dense(up(et, w), up(et, bias), up(et, x), d_y, T, inp, out)
+    got = d_y.numpy()
+    assert np.array_equal(got, want.astype(np.float32).astype(np.float16))
+
+
 @pytest.mark.parametrize("trans_b", [True, False])
 @pytest.mark.parametrize("M,N,K,batch", [(128, 64, 128, 12), (256, 768, 1536, 1), (48, 32, 16, 3),
                                          (128, 192, 1040, 3),  # long K in few tiles, 16 k-values in the last stage
