@@ -20,6 +20,9 @@ struct GemmArgs {
     const int32_t *c_scatter; // [N] or nullptr
     const int32_t *bias_idx;  // [N] or nullptr: bias index of result column n (default: the output column)
     int act;
+    // direct-to-LDS kernel only, set by its launcher: tile rows of a group of tiles (x 8 tile columns) that one XCD
+    // works on at a time: 4, 2 or 1
+    int group_rows;
 };
 
 // Launches the MFMA GEMM kernel over batch_outer*batch_inner problems.

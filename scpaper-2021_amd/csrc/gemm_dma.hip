@@ -73,15 +73,37 @@ __global__ __launch_bounds__(128 * NWN) void gemm_f16_dma_kernel(const GemmArgs 
     const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: LDS targets of the loads stay scalar
     const int wm = wave / NWN, wn = wave % NWN;
     const int l32 = lane & 31, kg = lane >> 5;
-    // Workgroup id -> tile, XCD-aware.  Workgroups go to the 8 XCDs round-robin by id and each
-    // XCD runs 32 of them at a time; those 32 are given a 4 x 8 block of tiles (4 panels of A,
-    // 8 of B), so the XCD's L2 serves 12 panels to 32 workgroups instead of up to 64.
+    // Workgroup id -> tile, XCD-aware.  Workgroups go to the 8 XCDs round-robin by id and each XCD runs them in
+    // order; consecutive workgroups of an XCD are given consecutive tiles of an order that walks the result in
+    // blocks of group_rows x 8 tiles (4 x 8: 4 panels of A, 8 of B), so the XCD's L2 serves about 12 panels to 32
+    // workgroups instead of up to 64.  The order counts existing tiles only (a block at the right or lower edge
+    // is narrower or shorter) and the groups are dealt to the XCDs in turn, so every XCD gets the same number of
+    // tiles to within one group; dealing whole 4 x 8 blocks instead gave the XCDs with odd numbers only the
+    // half-empty blocks of a result 12 tiles wide.
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-    const int nsbx = (tiles_n + kSbN - 1) / kSbN;
+    const int sbm = g.group_rows, gsh = sbm == 4 ? 5 : sbm == 2 ? 4 : 3;  // a group: sbm x 8 = 1 << gsh tiles
     const int xcd = blockIdx.x % kDmaXcds, j = blockIdx.x / kDmaXcds;
-    const int gsb = (j / (kSbM * kSbN)) * kDmaXcds + xcd, within = j % (kSbM * kSbN);
-    const int ty = (gsb / nsbx) * kSbM + within / kSbN, tx = (gsb % nsbx) * kSbN + within % kSbN;
-    if (ty >= tiles_m || tx >= tiles_n) return;  // padding of the block grid (whole workgroup)
+    const int t = ((((j >> gsh) * kDmaXcds + xcd)) << gsh) + (j & ((1 << gsh) - 1));
+    if (t >= tiles_m * tiles_n) return;  // padding of the grid (whole workgroup)
+    int ty, tx;
+    {
+        const int per_br = sbm * tiles_n, full_br = tiles_m / sbm;  // tiles of a full block row; such rows
+        const int br = min(t / per_br, full_br);
+        const int rem = t - br * per_br;
+        if (br < full_br && (tiles_n & (kSbN - 1)) == 0) {  // whole blocks only: shifts
+            const int q = rem & ((1 << gsh) - 1);
+            ty = br * sbm + (q >> 3);
+            tx = (rem >> gsh) * kSbN + (q & 7);
+        } else {
+            const int rows = br < full_br ? sbm : tiles_m - full_br * sbm;  // tile rows of this block row
+            const int per_bc = rows * kSbN, full_bc = tiles_n / kSbN;
+            const int bc = min(rem / per_bc, full_bc);
+            const int q = rem - bc * per_bc;
+            const int w = bc < full_bc ? kSbN : tiles_n - full_bc * kSbN;  // tile columns of this block
+            ty = br * sbm + q / w;
+            tx = bc * kSbN + q % w;
+        }
+    }
     const int m0 = ty * BM, n0 = tx * BN;
 
     f16v acc[TMW][TNW];  // [token tile][feature tile]
@@ -536,9 +558,21 @@ static int launch_dma_variant(const GemmArgs &g, int batch, hipStream_t stream) 
     constexpr int BM = 64 * TMW, BN = 32 * NWN * TNW;
     constexpr size_t lds = dma_lds_bytes(TMW, TNW, NBUF, KS, NWN);
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-    const int nsb = ((tiles_m + kSbM - 1) / kSbM) * ((tiles_n + kSbN - 1) / kSbN);
-    const int rounds = (nsb + kDmaXcds - 1) / kDmaXcds;
-    const dim3 grid((unsigned)(rounds * kDmaXcds * kSbM * kSbN), (unsigned)batch);
+    // groups of group_rows x 8 tiles are dealt to the XCDs in turn: the size (32, 16 or 8 tiles) that leaves the
+    // fullest XCD the fewest tiles, the larger on a tie
+    const long long total = (long long)tiles_m * tiles_n;
+    int sbm = kSbM;
+    long long best = -1;
+    for (int cand = kSbM; cand >= 1; cand /= 2) {
+        const long long gsz = (long long)cand * kSbN, ngr = (total + gsz - 1) / gsz;
+        const long long most = (ngr + kDmaXcds - 1) / kDmaXcds * gsz;
+        if (best < 0 || most < best) { best = most; sbm = cand; }
+    }
+    const long long groups = (total + sbm * kSbN - 1) / (sbm * kSbN);
+    const long long rounds = (groups + kDmaXcds - 1) / kDmaXcds;
+    const dim3 grid((unsigned)(rounds * kDmaXcds * sbm * kSbN), (unsigned)batch);
+    GemmArgs ga = g;
+    ga.group_rows = sbm;
     auto kernel = gemm_f16_dma_kernel<TMW, TNW, NBUF, IDX, RAGGED, BT, KS, NWN>;
     static bool raised = false;  // more than 64 KB of dynamic LDS needs the attribute, once per kernel
     if (!raised) {
@@ -546,7 +580,7 @@ static int launch_dma_variant(const GemmArgs &g, int batch, hipStream_t stream) 
                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         raised = true;
     }
-    kernel<<<grid, 128 * NWN, lds, stream>>>(g);
+    kernel<<<grid, 128 * NWN, lds, stream>>>(ga);
     return check_launch("gemm_f16_dma_kernel");
 }
 
