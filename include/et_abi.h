@@ -705,6 +705,38 @@ int et_bias_add_f16(et_f16 *data, const et_f16 *bias, int rows, int cols,
  * ------------------------------------------------------------------------ */
 int et_linear_dense_f32(const float *W, const float *bias, const float *X, float *Y,
                         int T, int in, int out, int act, et_stream stream);
+/* binary32 twins of the Linear layers over the sparse weight containers: the
+ * structure arrays (row_ptr / col_idx, row_id, col_id, tile_idx / row_idx,
+ * indptr / indices) mean what they mean in the _f16 function of the same name;
+ * weights, bias, X and Y are float.  T may be any size.
+ *   et_linear_bsr16_f32             Linear<tile_mat> (Linear/SPMM_tile.cu:312-324); in, out % 16 == 0
+ *   et_linear_rowpruned_f32         Linear<row_mat>  (Linear/SPMM_row.cu:62-75): pruned columns of Y
+ *                                   get act(bias); in % 16 == 0, nnz_row % 4 == 0
+ *   et_linear_rowpruned_compact_f32 its compact-output form (Linear/SPMM_row.cu:78-95)
+ *   et_linear_colpruned_f32         Linear<col_mat>  (Linear/SPMM_col.cu:57-69); the gather happens
+ *                                   while X is staged, no workspace; nnz_col % 16 == 0, out % 4 == 0,
+ *                                   col_id 16-byte aligned
+ *   et_linear_vec1x16_f32           Linear<mat1x16>  (Linear/Linear.h:153-167); in, out % 16 == 0,
+ *                                   at most 16 vectors per (row-set, part) cell
+ *   et_linear_csr_f32               Linear<csr_mat>  (Linear/cusp.cu:23-82); out % 4 == 0 */
+int et_linear_bsr16_f32(const int32_t *row_ptr, const int32_t *col_idx, const float *tiles,
+                        const float *bias, const float *X, float *Y, int T, int in, int out,
+                        int act, et_stream stream);
+int et_linear_rowpruned_f32(const float *rows, const int32_t *row_id, int nnz_row,
+                            const float *bias, const float *X, float *Y, int T, int in,
+                            int out, int act, et_stream stream);
+int et_linear_rowpruned_compact_f32(const float *rows, const int32_t *row_id, int nnz_row,
+                                    const float *bias, const float *X, float *Yc, int T,
+                                    int in, et_stream stream);
+int et_linear_colpruned_f32(const float *cols, const int32_t *col_id, int nnz_col,
+                            const float *bias, const float *X, float *Y, int T, int in,
+                            int out, int act, et_stream stream);
+int et_linear_vec1x16_f32(const int32_t *tile_idx, const int32_t *row_idx, const float *data,
+                          const float *bias, const float *X, float *Y, int T, int in, int out,
+                          int act, et_stream stream);
+int et_linear_csr_f32(const int32_t *indptr, const int32_t *indices, const float *data,
+                      const float *bias, const float *X, float *Y, int T, int in, int out,
+                      int act, et_stream stream);
 int et_mha_fused_f32(const float *Q, const float *K, const float *V, int ldq, int ldk,
                      int ldv, float *Z, int ldz, const float *mask,
                      const int32_t *lens, int B, int S, int nh, int hd, float scale,

@@ -90,6 +90,12 @@ _SIGNATURES = {
     "et_norm_linear_bsr16_f16": (_vp, _vp, _vp, _i, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_norm_from_stats_f16": (_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _f, _vp),
     "et_linear_dense_f32": (_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_linear_bsr16_f32": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_linear_rowpruned_f32": (_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_linear_rowpruned_compact_f32": (_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _vp),
+    "et_linear_colpruned_f32": (_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_linear_vec1x16_f32": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
+    "et_linear_csr_f32": (_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_mha_fused_f32": (_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp),
     "et_skip_layernorm_f32": (_vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp),
     "et_layernorm_f32": (_vp, _vp, _vp, _vp, _i, _i, _f, _vp),

@@ -19,12 +19,24 @@ constexpr int kF32Ld = kF32K + 1;  // LDS row stride in floats (odd: conflict-fr
 // TILE x TILE outputs per workgroup (64 or 32), a wave TILE/2 x TILE/2 of them.  The small
 // tile is for problems that would leave compute units idle with the large one: the fp32 MFMA
 // rate of the waves that run is what bounds a small problem.
-template <int ACT, int TILE>
-__global__ __launch_bounds__(256) void linear_dense_f32_kernel(const float *__restrict__ W,
-                                                               const float *__restrict__ bias,
-                                                               const float *__restrict__ X,
-                                                               float *__restrict__ Y, int T, int in,
-                                                               int out) {
+// The pruned forms run the same kernel.  GATHER (column-pruned weight): W is [out x in] over the
+// surviving input features and feature k of W multiplies X[:, in_id[k]].  OUT (row-pruned weight,
+// W = its surviving rows): kOutScatter stores feature f in column out_id[f] of Y with bias[out_id[f]];
+// kOutCompact stores it in column f with that same bias.  ldx and ldy are the row strides of X and Y.
+constexpr int kOutPlain = 0, kOutScatter = 1, kOutCompact = 2;
+struct LinearF32Args {
+    const float *W, *bias, *X;
+    float *Y;
+    const int32_t *in_id, *out_id;
+    int T, in, out, ldx, ldy;
+};
+template <int ACT, int TILE, bool GATHER, int OUT>
+__global__ __launch_bounds__(256) void linear_dense_f32_kernel(const LinearF32Args a) {
+    const float *__restrict__ W = a.W;
+    const float *__restrict__ bias = a.bias;
+    const float *__restrict__ X = a.X;
+    float *__restrict__ Y = a.Y;
+    const int T = a.T, in = a.in, out = a.out;
     constexpr int WB = TILE / 2;          // wave block
     constexpr int MI = WB / 16;           // 16 x 16 MFMA tiles per wave and dimension
     constexpr int TPR = 256 / TILE;       // staging threads per row
@@ -39,7 +51,7 @@ __global__ __launch_bounds__(256) void linear_dense_f32_kernel(const float *__re
     // staging: thread -> (row, 4 consecutive k at sk, sk + 4 TPR, ...)
     const int srow = threadIdx.x / TPR, sk = (threadIdx.x % TPR) << 2;
     const bool x_ok = tok0 + srow < T, w_ok = f0 + srow < out;
-    const float *xp = X + (size_t)(tok0 + (x_ok ? srow : 0)) * in;
+    const float *xp = X + (size_t)(tok0 + (x_ok ? srow : 0)) * a.ldx;
     const float *wp = W + (size_t)(f0 + (w_ok ? srow : 0)) * in;
     const float4 zero4 = float4{0.0f, 0.0f, 0.0f, 0.0f};
     float4 xv[VPT], wv[VPT];
@@ -50,7 +62,12 @@ __global__ __launch_bounds__(256) void linear_dense_f32_kernel(const float *__re
         for (int j = 0; j < VPT; j++) {
             const int k = k0 + sk + 4 * TPR * j;
             const bool k_ok = k < in;
-            xv[j] = *reinterpret_cast<const float4 *>(xp + (k_ok ? k : 0));
+            if (GATHER) {
+                const int4 id = *reinterpret_cast<const int4 *>(a.in_id + (k_ok ? k : 0));
+                xv[j] = float4{xp[id.x], xp[id.y], xp[id.z], xp[id.w]};
+            } else {
+                xv[j] = *reinterpret_cast<const float4 *>(xp + (k_ok ? k : 0));
+            }
             wv[j] = *reinterpret_cast<const float4 *>(wp + (k_ok ? k : 0));
             if (!(x_ok && k_ok)) xv[j] = zero4;
             if (!(w_ok && k_ok)) wv[j] = zero4;
@@ -100,14 +117,21 @@ __global__ __launch_bounds__(256) void linear_dense_f32_kernel(const float *__re
             if (f >= out) continue;  // out % 4 == 0: a group of 4 is inside or outside
             float4 o;
             float *po = reinterpret_cast<float *>(&o);
+            int col[4];
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                float v = acc[i][j][e] + (bias ? bias[f + e] : 0.0f);
+                col[e] = OUT == kOutPlain ? f + e : a.out_id[f + e];
+                float v = acc[i][j][e] + (bias ? bias[col[e]] : 0.0f);
                 if (ACT == ET_ACT_RELU) v = v > 0.0f ? v : 0.0f;
                 if (ACT == ET_ACT_GELU) v = gelu_tanh(v);
                 po[e] = v;
             }
-            *reinterpret_cast<float4 *>(Y + (size_t)t * out + f) = o;
+            if (OUT == kOutScatter) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) Y[(size_t)t * a.ldy + col[e]] = po[e];
+            } else {
+                *reinterpret_cast<float4 *>(Y + (size_t)t * a.ldy + f) = o;
+            }
         }
     }
 }
@@ -230,11 +254,50 @@ __global__ __launch_bounds__(256) void unary_f32_kernel(float *__restrict__ out,
     }
 }
 
+// Y[r][c] = act(bias[c]) (act(0) without a bias): the value of a pruned output feature.
+__global__ __launch_bounds__(256) void fill_rows_bias_act_f32_kernel(float *__restrict__ Y,
+                                                                     const float *__restrict__ bias, size_t n,
+                                                                     int cols, int act) {
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += step)
+        Y[i] = apply_act(bias ? bias[i % cols] : 0.0f, act);
+}
+
 }  // namespace et
 
 using namespace et;
 
 extern "C" {
+
+// One launch of the Linear kernel in the form (gather, out mode, activation) names.
+static int launch_linear_f32(const LinearF32Args &a, int act, bool gather, int out_mode, hipStream_t st) {
+    // 64 x 64 tiles once they give every compute unit a workgroup, 32 x 32 below that
+    const bool small = (long long)((a.out + 63) / 64) * ((a.T + 63) / 64) < 256;
+    const int tile = small ? 32 : 64;
+    const dim3 grid((a.out + tile - 1) / tile, (a.T + tile - 1) / tile);
+#define ET_F32_FORM(ACTV, G, O)                                                       \
+    {                                                                                 \
+        if (small) linear_dense_f32_kernel<ACTV, 32, G, O><<<grid, 256, 0, st>>>(a);  \
+        else linear_dense_f32_kernel<ACTV, 64, G, O><<<grid, 256, 0, st>>>(a);        \
+    }
+#define ET_F32_LINEAR(ACTV)                                                \
+    {                                                                      \
+        if (gather) ET_F32_FORM(ACTV, true, kOutPlain)                     \
+        else if (out_mode == kOutScatter) ET_F32_FORM(ACTV, false, kOutScatter)  \
+        else if (out_mode == kOutCompact) ET_F32_FORM(ACTV, false, kOutCompact)  \
+        else ET_F32_FORM(ACTV, false, kOutPlain)                           \
+    }
+    switch (act) {
+        case ET_ACT_RELU: ET_F32_LINEAR(ET_ACT_RELU) break;
+        case ET_ACT_GELU: ET_F32_LINEAR(ET_ACT_GELU) break;
+        default: ET_F32_LINEAR(ET_ACT_NONE) break;
+    }
+#undef ET_F32_LINEAR
+#undef ET_F32_FORM
+    return check_launch("linear_dense_f32_kernel");
+}
+
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 int et_linear_dense_f32(const float *W, const float *bias, const float *X, float *Y, int T, int in, int out,
                         int act, et_stream stream) {
@@ -243,26 +306,62 @@ int et_linear_dense_f32(const float *W, const float *bias, const float *X, float
     ET_REQUIRE(act >= ET_ACT_NONE && act <= ET_ACT_GELU, ET_ERR_INVALID_ARG, "et_linear_dense_f32: act=%d", act);
     ET_REQUIRE(in % 16 == 0 && out % 4 == 0, ET_ERR_UNSUPPORTED,
                "et_linear_dense_f32: in=%d must be a multiple of 16, out=%d of 4", in, out);
-    ET_REQUIRE(((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(X) | reinterpret_cast<uintptr_t>(Y)) & 15) == 0,
-               ET_ERR_UNSUPPORTED, "et_linear_dense_f32: W, X and Y must be 16-byte aligned");
+    ET_REQUIRE(aligned16(W) && aligned16(X) && aligned16(Y), ET_ERR_UNSUPPORTED,
+               "et_linear_dense_f32: W, X and Y must be 16-byte aligned");
+    if (T == 0) return ET_OK;
+    const LinearF32Args a{W, bias, X, Y, nullptr, nullptr, T, in, out, in, out};
+    return launch_linear_f32(a, act, false, kOutPlain, as_stream(stream));
+}
+
+int et_linear_rowpruned_f32(const float *rows, const int32_t *row_id, int nnz_row, const float *bias,
+                            const float *X, float *Y, int T, int in, int out, int act, et_stream stream) {
+    ET_REQUIRE(X && Y && (nnz_row == 0 || (rows && row_id)), ET_ERR_INVALID_ARG, "et_linear_rowpruned_f32: NULL pointer");
+    ET_REQUIRE(T >= 0 && in > 0 && out > 0 && nnz_row >= 0 && nnz_row <= out, ET_ERR_INVALID_ARG,
+               "et_linear_rowpruned_f32: T=%d in=%d out=%d nnz_row=%d", T, in, out, nnz_row);
+    ET_REQUIRE(act >= ET_ACT_NONE && act <= ET_ACT_GELU, ET_ERR_INVALID_ARG, "et_linear_rowpruned_f32: act=%d", act);
+    ET_REQUIRE(in % 16 == 0 && nnz_row % 4 == 0, ET_ERR_UNSUPPORTED,
+               "et_linear_rowpruned_f32: in=%d must be a multiple of 16, nnz_row=%d of 4", in, nnz_row);
+    ET_REQUIRE(aligned16(rows) && aligned16(X), ET_ERR_UNSUPPORTED,
+               "et_linear_rowpruned_f32: rows and X must be 16-byte aligned");
     if (T == 0) return ET_OK;
     hipStream_t st = as_stream(stream);
-    // 64 x 64 tiles once they give every compute unit a workgroup, 32 x 32 below that
-    const bool small = (long long)((out + 63) / 64) * ((T + 63) / 64) < 256;
-    const int tile = small ? 32 : 64;
-    const dim3 grid((out + tile - 1) / tile, (T + tile - 1) / tile);
-#define ET_F32_LINEAR(ACTV)                                                                        \
-    {                                                                                              \
-        if (small) linear_dense_f32_kernel<ACTV, 32><<<grid, 256, 0, st>>>(W, bias, X, Y, T, in, out); \
-        else linear_dense_f32_kernel<ACTV, 64><<<grid, 256, 0, st>>>(W, bias, X, Y, T, in, out);       \
-    }
-    switch (act) {
-        case ET_ACT_RELU: ET_F32_LINEAR(ET_ACT_RELU) break;
-        case ET_ACT_GELU: ET_F32_LINEAR(ET_ACT_GELU) break;
-        default: ET_F32_LINEAR(ET_ACT_NONE) break;
-    }
-#undef ET_F32_LINEAR
-    return check_launch("linear_dense_f32_kernel");
+    // pruned features: act(bias) — every column is written first, the surviving ones again below
+    const size_t n = (size_t)T * out;
+    fill_rows_bias_act_f32_kernel<<<(unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536), 256, 0, st>>>(
+        Y, bias, n, out, act);
+    const int s = check_launch("fill_rows_bias_act_f32_kernel");
+    if (s != ET_OK || nnz_row == 0) return s;
+    const LinearF32Args a{rows, bias, X, Y, nullptr, row_id, T, in, nnz_row, in, out};
+    return launch_linear_f32(a, act, false, kOutScatter, st);
+}
+
+int et_linear_rowpruned_compact_f32(const float *rows, const int32_t *row_id, int nnz_row, const float *bias,
+                                    const float *X, float *Yc, int T, int in, et_stream stream) {
+    ET_REQUIRE(rows && row_id && X && Yc, ET_ERR_INVALID_ARG, "et_linear_rowpruned_compact_f32: NULL pointer");
+    ET_REQUIRE(T >= 0 && in > 0 && nnz_row > 0, ET_ERR_INVALID_ARG,
+               "et_linear_rowpruned_compact_f32: T=%d in=%d nnz_row=%d", T, in, nnz_row);
+    ET_REQUIRE(in % 16 == 0 && nnz_row % 4 == 0, ET_ERR_UNSUPPORTED,
+               "et_linear_rowpruned_compact_f32: in=%d must be a multiple of 16, nnz_row=%d of 4", in, nnz_row);
+    ET_REQUIRE(aligned16(rows) && aligned16(X) && aligned16(Yc), ET_ERR_UNSUPPORTED,
+               "et_linear_rowpruned_compact_f32: rows, X and Yc must be 16-byte aligned");
+    if (T == 0) return ET_OK;
+    const LinearF32Args a{rows, bias, X, Yc, nullptr, row_id, T, in, nnz_row, in, nnz_row};
+    return launch_linear_f32(a, ET_ACT_NONE, false, bias ? kOutCompact : kOutPlain, as_stream(stream));
+}
+
+int et_linear_colpruned_f32(const float *cols, const int32_t *col_id, int nnz_col, const float *bias,
+                            const float *X, float *Y, int T, int in, int out, int act, et_stream stream) {
+    ET_REQUIRE(cols && col_id && X && Y, ET_ERR_INVALID_ARG, "et_linear_colpruned_f32: NULL pointer");
+    ET_REQUIRE(T >= 0 && in > 0 && out > 0 && nnz_col > 0 && nnz_col <= in, ET_ERR_INVALID_ARG,
+               "et_linear_colpruned_f32: T=%d in=%d out=%d nnz_col=%d", T, in, out, nnz_col);
+    ET_REQUIRE(act >= ET_ACT_NONE && act <= ET_ACT_GELU, ET_ERR_INVALID_ARG, "et_linear_colpruned_f32: act=%d", act);
+    ET_REQUIRE(nnz_col % 16 == 0 && out % 4 == 0, ET_ERR_UNSUPPORTED,
+               "et_linear_colpruned_f32: nnz_col=%d must be a multiple of 16, out=%d of 4", nnz_col, out);
+    ET_REQUIRE(aligned16(cols) && aligned16(col_id) && aligned16(Y), ET_ERR_UNSUPPORTED,
+               "et_linear_colpruned_f32: cols, col_id and Y must be 16-byte aligned");
+    if (T == 0) return ET_OK;
+    const LinearF32Args a{cols, bias, X, Y, col_id, nullptr, T, nnz_col, out, in, out};
+    return launch_linear_f32(a, act, true, kOutPlain, as_stream(stream));
 }
 
 int et_mha_fused_f32(const float *Q, const float *K, const float *V, int ldq, int ldk, int ldv, float *Z, int ldz,

@@ -156,3 +156,140 @@ def test_fp32_layer_with_biases_padding_and_batch(et):
                       t["g2"], t["be2"])
     want = L.encoder_layer(torch.from_numpy(x), P, L.LayerConfig(nh=nh, B=B, act="relu", lens=lens)).numpy()
     assert Hn.max_abs(y, want) <= TOL_F32
+
+
+# ---- binary32 twins over the sparse weight containers ---------------------------------------
+# Each is checked against the binary64 product with the dense image the format oracle builds
+# from the same structure arrays (oracle/formats.py), to the accumulation error of `inp` binary32
+# products.
+def _want64(x, Wd, b, act):
+    y = torch.from_numpy(x.astype(np.float64) @ Wd.astype(np.float64).T + (0 if b is None else b.astype(np.float64)))
+    return L.ACTS[ACT[act]](y).numpy()
+
+
+@pytest.mark.parametrize("T,inp,out,sp,act", [(128, 768, 2304, 0.8, 0), (1024, 768, 3072, 0.8, 2),
+                                              (2048, 3072, 768, 0.9, 0), (100, 48, 32, 0.5, 1), (1, 16, 16, 0.0, 0),
+                                              (77, 160, 144, 0.95, 2)])
+def test_linear_bsr16_f32(et, T, inp, out, sp, act):
+    from oracle import formats as F
+    row_ptr, col_idx = F.gen_tile_pattern(out, inp, sp, seed=31)
+    tiles = randf((max(len(col_idx), 1), 256), 32, 0.05)
+    Wd = F.bsr16_to_dense(row_ptr, col_idx, tiles[:len(col_idx)], inp)
+    b, x = randf((out,), 33, 0.1), randf((T, inp), 34)
+    d_y = et.DeviceBuffer.empty((T, out), np.float32)
+    ci = col_idx if len(col_idx) else np.zeros(1, np.int32)
+    et.check(et.lib().et_linear_bsr16_f32(up(et, row_ptr).ptr, up(et, ci).ptr, up(et, tiles).ptr, up(et, b).ptr,
+                                          up(et, x).ptr, d_y.ptr, T, inp, out, act, None))
+    assert Hn.max_abs(d_y.numpy(), _want64(x, Wd, b, act)) <= 5e-5
+
+
+def test_linear_bsr16_f32_closed_form_and_bad_args(et):
+    """All-ones tiles and inputs: every output is 16 x (tiles of its block-row) + bias, exactly."""
+    from oracle import formats as F
+    T, inp, out = 48, 256, 64
+    row_ptr, col_idx = F.gen_tile_pattern(out, inp, 0.6, seed=5)
+    tiles = np.ones((len(col_idx), 256), np.float32)
+    b = np.arange(out, dtype=np.float32)
+    d_y = et.DeviceBuffer.empty((T, out), np.float32)
+    args = (up(et, row_ptr).ptr, up(et, col_idx).ptr, up(et, tiles).ptr, up(et, b).ptr,
+            up(et, np.ones((T, inp), np.float32)).ptr, d_y.ptr)
+    et.check(et.lib().et_linear_bsr16_f32(*args, T, inp, out, 0, None))
+    want = np.repeat(16.0 * np.diff(row_ptr), 16)[None, :] + b[None, :]
+    assert np.array_equal(d_y.numpy(), np.broadcast_to(want, (T, out)).astype(np.float32))
+    assert et.lib().et_linear_bsr16_f32(*args, T, inp, 60, 0, None) == et.ET_ERR_UNSUPPORTED
+    assert et.lib().et_linear_bsr16_f32(*args, T, inp, out, 7, None) == et.ET_ERR_INVALID_ARG
+    assert et.lib().et_linear_bsr16_f32(None, *args[1:], T, inp, out, 0, None) == et.ET_ERR_INVALID_ARG
+
+
+@pytest.mark.parametrize("T,inp,out,sp,act", [(2048, 768, 768, 0.5, 0), (128, 768, 3072, 0.5, 2), (100, 48, 64, 0.3, 1),
+                                              (7, 3072, 768, 0.9, 0)])
+def test_linear_rowpruned_f32(et, T, inp, out, sp, act):
+    from oracle import formats as F
+    row_id = F.gen_row_ids(out, sp, seed=8)
+    rows, b, x = randf((len(row_id), inp), 35, 0.05), randf((out,), 36, 0.1), randf((T, inp), 37)
+    d_y = et.DeviceBuffer.from_numpy(np.full((T, out), np.nan, np.float32))  # every element must be written
+    et.check(et.lib().et_linear_rowpruned_f32(up(et, rows).ptr, up(et, row_id).ptr, len(row_id), up(et, b).ptr,
+                                              up(et, x).ptr, d_y.ptr, T, inp, out, act, None))
+    got = d_y.numpy()
+    assert Hn.max_abs(got, _want64(x, F.row_mat_to_dense(rows, row_id, out), b, act)) <= 5e-5
+    dead = np.setdiff1d(np.arange(out), row_id)
+    bias_only = L.ACTS[ACT[act]](torch.from_numpy(b).double()).numpy()
+    assert Hn.max_abs(got[:, dead], np.broadcast_to(bias_only[dead], (T, len(dead)))) <= 1e-6
+    d_c = et.DeviceBuffer.empty((T, len(row_id)), np.float32)
+    et.check(et.lib().et_linear_rowpruned_compact_f32(up(et, rows).ptr, up(et, row_id).ptr, len(row_id),
+                                                      up(et, b).ptr, up(et, x).ptr, d_c.ptr, T, inp, None))
+    assert Hn.max_abs(d_c.numpy(), _want64(x, rows, b[row_id], 0)) <= 5e-5
+    et.check(et.lib().et_linear_rowpruned_compact_f32(up(et, rows).ptr, up(et, row_id).ptr, len(row_id),
+                                                      None, up(et, x).ptr, d_c.ptr, T, inp, None))
+    assert Hn.max_abs(d_c.numpy(), _want64(x, rows, None, 0)) <= 5e-5
+
+
+@pytest.mark.parametrize("T,inp,out,sp,act", [(2048, 768, 768, 0.5, 0), (128, 768, 3072, 0.5, 2), (33, 160, 48, 0.3, 1),
+                                              (128, 3072, 768, 0.9, 0)])
+def test_linear_colpruned_f32(et, T, inp, out, sp, act):
+    from oracle import formats as F
+    col_id = F.gen_col_ids(inp, sp, seed=12)  # unsorted, as the reference generator leaves them
+    cols, b, x = randf((out, len(col_id)), 38, 0.05), randf((out,), 39, 0.1), randf((T, inp), 40)
+    d_y = et.DeviceBuffer.empty((T, out), np.float32)
+    et.check(et.lib().et_linear_colpruned_f32(up(et, cols).ptr, up(et, col_id).ptr, len(col_id), up(et, b).ptr,
+                                              up(et, x).ptr, d_y.ptr, T, inp, out, act, None))
+    assert Hn.max_abs(d_y.numpy(), _want64(x, F.col_mat_to_dense(cols, col_id, inp), b, act)) <= 5e-5
+
+
+@pytest.mark.parametrize("T,inp,out,sp,act", [(2048, 768, 768, 0.8, 0), (128, 768, 3072, 0.5, 2), (16, 32, 16, 0.0, 0),
+                                              (81, 3072, 64, 0.9, 1)])
+def test_linear_vec1x16_f32(et, T, inp, out, sp, act):
+    from oracle import formats as F
+    keep = np.repeat(torch.rand(out, inp // 16, generator=Hn.rng(16)).numpy() >= sp, 16, axis=1)
+    W = randf((out, inp), 41, 0.05) * keep
+    tile_idx, row_idx, data = F.dense_to_1x16(W)
+    data = np.ascontiguousarray(data, np.float32)
+    assert np.array_equal(F.mat1x16_to_dense(tile_idx, row_idx, data, out, inp), W)
+    b, x = randf((out,), 42, 0.1), randf((T, inp), 43)
+    d_y = et.DeviceBuffer.empty((T, out), np.float32)
+    row_idx_d = row_idx if len(row_idx) else np.zeros(1, np.int32)
+    data_d = data if data.size else np.zeros((16, 16), np.float32)
+    et.check(et.lib().et_linear_vec1x16_f32(up(et, tile_idx).ptr, up(et, row_idx_d).ptr, up(et, data_d).ptr,
+                                            up(et, b).ptr, up(et, x).ptr, d_y.ptr, T, inp, out, act, None))
+    assert Hn.max_abs(d_y.numpy(), _want64(x, W, b, act)) <= 5e-5
+
+
+def test_linear_vec1x16_f32_unsorted_rows_in_a_cell(et):
+    from oracle import formats as F
+    T, inp, out = 32, 64, 32
+    tile_idx, row_idx = F.gen_1x16_pattern(out, inp, 0.5, seed=3)  # keeps the permuted order inside a cell
+    data = randf((((len(row_idx) + 15) // 16) * 16, 16), 44, 0.1)
+    W = F.mat1x16_to_dense(tile_idx, row_idx, data, out, inp)
+    x = randf((T, inp), 45)
+    d_y = et.DeviceBuffer.empty((T, out), np.float32)
+    et.check(et.lib().et_linear_vec1x16_f32(up(et, tile_idx).ptr, up(et, row_idx).ptr, up(et, data).ptr, None,
+                                            up(et, x).ptr, d_y.ptr, T, inp, out, 0, None))
+    assert Hn.max_abs(d_y.numpy(), _want64(x, W, None, 0)) <= 1e-5
+
+
+@pytest.mark.parametrize("T,inp,out,sp,act", [(1024, 768, 768, 0.9, 0), (100, 768, 3072, 0.95, 2), (7, 40, 12, 0.5, 1),
+                                              (64, 40000, 16, 0.999, 0)])
+def test_linear_csr_f32(et, T, inp, out, sp, act):
+    from oracle import formats as F
+    mask = torch.rand(out, inp, generator=Hn.rng(22)).numpy() >= sp
+    W = randf((out, inp), 46, 0.05) * mask
+    indptr, indices, data = F.dense_to_csr(W)
+    data = np.ascontiguousarray(data, np.float32)
+    b, x = randf((out,), 47, 0.1), randf((T, inp), 48)
+    d_y = et.DeviceBuffer.from_numpy(np.full((T, out), np.nan, np.float32))
+    et.check(et.lib().et_linear_csr_f32(up(et, indptr).ptr, up(et, indices).ptr,
+                                        up(et, data if data.size else np.zeros(1, np.float32)).ptr,
+                                        up(et, b).ptr, up(et, x).ptr, d_y.ptr, T, inp, out, act, None))
+    assert Hn.max_abs(d_y.numpy(), _want64(x, W, b, act)) <= 5e-5
+
+
+def test_linear_csr_f32_reference_fixture(et):
+    """The reference's dense_4_3.csr (all ones): y = sum of the 3 inputs + bias."""
+    from oracle import formats as F
+    nrow, ncol, nnz, indptr, indices, data = F.read_csr(str(GOLDEN / "dense_4_3.csr"))
+    x = randf((5, ncol), 49)
+    b = np.array([0.5, -1, 2, 0], np.float32)
+    d_y = et.DeviceBuffer.empty((5, nrow), np.float32)
+    et.check(et.lib().et_linear_csr_f32(up(et, indptr).ptr, up(et, indices).ptr, up(et, data.astype(np.float32)).ptr,
+                                        up(et, b).ptr, up(et, x).ptr, d_y.ptr, 5, ncol, nrow, 0, None))
+    assert Hn.max_abs(d_y.numpy(), x.astype(np.float64).sum(1, keepdims=True) + b) <= 1e-6
