@@ -524,6 +524,32 @@ int et_mha_fused_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V,
                      const et_f16 *mask, const int32_t *lens, int B, int S,
                      int nh, int hd, float scale, int flags, et_stream stream);
 
+/* Fused attention and the tile-sparse output projection in ONE launch:
+ *   Z = attention as et_mha_fused_f16 (Z is written, [B*S x ldz]),
+ *   out[B*S x emdim] = Z[:, :nh*hd] * W_O^T + o_bias,
+ * W_O [emdim x nh*hd] as 16x16 tiles (o_row_ptr[emdim/16 + 1], o_col_idx,
+ * o_tiles as in et_linear_bsr16_f16; o_bias may be NULL).  Same values as
+ * et_mha_fused_f16 followed by et_linear_bsr16_f16 up to the order of the fp32
+ * accumulation.  The workgroup that completes the heads of a strip of tokens
+ * projects that strip; no workgroup waits for another.  hd a multiple of 8, at
+ * most 128; nh*hd and emdim multiples of 16; ldz % 8 == 0; Z and o_tiles
+ * 16-byte aligned.  Arrival counts live in a device array built into the
+ * library (allocates nothing): B*S/16 <= 16384, else ET_ERR_UNSUPPORTED, and
+ * two of these calls that overlap in time on one GPU (different streams) race
+ * on the counts — issue them on one stream.  Meant for few token rows (the
+ * reference's kernel takes one sequence): from a few thousand rows on the two
+ * separate launches are faster.
+ * Replaces Multihead_atttion_fuseO (Attention/kernel_fuseO.h:6-9, kernel
+ * Attention/kernel_fuseO.cu:138-243, host :254-290), which joins the two parts
+ * with a grid-wide barrier inside a cooperative launch. */
+int et_mha_fuseo_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V,
+                     int ldq, int ldk, int ldv, et_f16 *Z, int ldz,
+                     const et_f16 *mask, const int32_t *lens, int B, int S,
+                     int nh, int hd, float scale, int flags,
+                     const int32_t *o_row_ptr, const int32_t *o_col_idx,
+                     const et_f16 *o_tiles, const et_f16 *o_bias, et_f16 *out,
+                     int emdim, et_stream stream);
+
 /* Attention-aware pruning: W_V is row-pruned, so V arrives compact,
  * Vc[T x nnz_col] (row stride ldvc), holding only the surviving V columns.
  * v_col_id[nnz_col] (ascending) are their full-width positions and

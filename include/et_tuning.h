@@ -31,6 +31,17 @@ int et_bsr16_pack_create_geom(const int32_t *row_ptr, const int32_t *col_idx,
                               int flags, int mt, int ngroups, int nwave, int cap,
                               et_bsr_pack *pack);
 
+/* Tuning hook: et_mha_fuseo_f16 with an explicit number of waves per workgroup
+ * (1, 2 or 4: 16, 32 or 64 tokens per attention workgroup and projection strip;
+ * 0 picks as et_mha_fuseo_f16 does).  No reference counterpart. */
+int et_mha_fuseo_f16_geom(const et_f16 *Q, const et_f16 *K, const et_f16 *V,
+                          int ldq, int ldk, int ldv, et_f16 *Z, int ldz,
+                          const et_f16 *mask, const int32_t *lens, int B, int S,
+                          int nh, int hd, float scale, int flags,
+                          const int32_t *o_row_ptr, const int32_t *o_col_idx,
+                          const et_f16 *o_tiles, const et_f16 *o_bias,
+                          et_f16 *out, int emdim, int waves, et_stream stream);
+
 /* Machine probes (scpaper-2021_amd/kernel_bench.py --set machine): an empty launch of nwg
  * workgroups (what a kernel boundary costs inside a graph), and a launch in which every
  * workgroup requests vec_per_thread (4, 8, 16, 32) 16-byte vectors per thread, all before it

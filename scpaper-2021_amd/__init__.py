@@ -110,6 +110,10 @@ _SIGNATURES = {
     "et_linear_rowpruned_compact_f16": (_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _vp),
     "et_linear_colpruned_f16": (_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp),
     "et_mha_fused_f16": (_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _i, _vp),
+    "et_mha_fuseo_f16": (_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _i,
+                         _vp, _vp, _vp, _vp, _vp, _i, _vp),
+    "et_mha_fuseo_f16_geom": (_vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _i,
+                              _vp, _vp, _vp, _vp, _vp, _i, _i, _vp),
     "et_skip_layernorm_f16": (_vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp),
     "et_layernorm_f16": (_vp, _vp, _vp, _vp, _i, _i, _f, _vp),
     "et_gelu_f16": (_vp, _vp, _sz, _vp),
@@ -353,6 +357,17 @@ def gemm(A, B, Cm, M, N, K, lda, ldb, ldc, trans_b=True, batch=1, sa=0, sb=0, sc
 def mha_fused(Q, K, V, ldq, ldk, ldv, Z, ldz, mask, lens, B, S, nh, hd, scale, flags=0, stream=None):
     check(lib().et_mha_fused_f16(_ptr(Q), _ptr(K), _ptr(V), ldq, ldk, ldv, _ptr(Z), ldz, _ptr(mask),
                                  _ptr(lens), B, S, nh, hd, scale, flags, stream))
+
+
+def mha_fuseo(Q, K, V, ldq, ldk, ldv, Z, ldz, mask, lens, B, S, nh, hd, scale, flags, o_row_ptr, o_col_idx,
+              o_tiles, o_bias, out, emdim, waves=None, stream=None):
+    """Fused attention and the tile-sparse output projection in one launch (waves: the tuning form)."""
+    head = (_ptr(Q), _ptr(K), _ptr(V), ldq, ldk, ldv, _ptr(Z), ldz, _ptr(mask), _ptr(lens), B, S, nh, hd, scale,
+            flags, _ptr(o_row_ptr), _ptr(o_col_idx), _ptr(o_tiles), _ptr(o_bias), _ptr(out), emdim)
+    if waves is None:
+        check(lib().et_mha_fuseo_f16(*head, stream))
+    else:
+        check(lib().et_mha_fuseo_f16_geom(*head, waves, stream))
 
 
 def skip_layernorm(out, src, skip, gamma, beta, rows, H, eps=1e-5, stream=None):

@@ -21,7 +21,9 @@
 #include <math.h>
 
 #include <algorithm>
+#include <atomic>
 #include <memory>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -29,6 +31,7 @@
 
 #include "common.hip.h"
 #include "bsr_packed.hip.h"
+#include "../../include/et_tuning.h"
 
 namespace et {
 
@@ -101,6 +104,23 @@ template <int HD> __device__ __forceinline__ constexpr int vt_unit_keys(int kg) 
 // Some variants prefetch the next key block through registers (mha_prefetches).  The 4-wave one
 // is held to the 168 registers of three resident waves per SIMD; left alone the allocator takes
 // a few more and the third wave is lost, which costs more than the prefetch gains.
+// Eight bytes stored and sixteen bytes loaded at device scope: the access goes past the L2 of the issuing
+// accelerator die (each die has its own, and they are not kept coherent with one another inside a launch), so
+// a workgroup on another die reads what was written without either side writing back or invalidating a
+// whole cache.
+__device__ __forceinline__ void store_device_scope(_Float16 *p, h4 v) {
+    __hip_atomic_store(reinterpret_cast<unsigned long long *>(p), __builtin_bit_cast(unsigned long long, v), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ h8 load_device_scope(const _Float16 *p) {
+    typedef unsigned long long u2 __attribute__((ext_vector_type(2)));
+    const unsigned long long *q = reinterpret_cast<const unsigned long long *>(p);
+    u2 r;
+    r[0] = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    r[1] = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __builtin_bit_cast(h8, r);
+}
+
 template <int HD, int NW, bool COMPACT, int QT> constexpr bool mha_prefetches() {
     if (HD == 128 && !COMPACT && NW == 8 && QT == 1) return true;  // 202 registers: two waves per SIMD either way
     return HD <= 64 && !COMPACT && ((NW == 4 && QT == 1) || (NW == 8 && QT == 2));
@@ -113,301 +133,8 @@ template <int HD, bool COMPACT, int NW, int QT>
 __global__ __launch_bounds__(64 * NW)
     __attribute__((amdgpu_waves_per_eu(mha_three_waves<HD, NW, COMPACT, QT>() ? 3 : 1, mha_three_waves<HD, NW, COMPACT, QT>() ? 3 : 8))) void
     mha_fused_kernel(const MhaArgs a) {
-    using L = MhaLds<HD>;
-    constexpr int KS = HD / 32;  // K=32 MFMA steps over the head dimension
-    constexpr int DB = HD / 16;  // 16-wide output blocks of the head dimension
-    extern __shared__ __align__(16) unsigned char smem_raw[];
-    _Float16 *Ks = reinterpret_cast<_Float16 *>(smem_raw);
-    _Float16 *Vt = Ks + L::k_halfs;
-
-    const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
-    constexpr int nwave = NW;
-    constexpr int nthr = 64 * NW;
-    constexpr int kStripQ = 16 * NW * QT;  // queries per workgroup
-    const int r16 = lane & 15;
-    const int g = lane >> 4;
-    const int S = a.S;
-    // Workgroup id -> (sequence*head, query strip), XCD-aware: workgroups go to the 8
-    // XCDs round-robin by id, so the query strips of one (sequence, head) are given ids
-    // that land on the same XCD and share its K and V in that L2.
-    const int qstrips = (S + kStripQ - 1) / kStripQ;
-    const int xcd = blockIdx.x % kXcds, k_in_xcd = blockIdx.x / kXcds;
-    const int bh = xcd + kXcds * (k_in_xcd / qstrips);
-    if (bh >= a.nbh) return;  // padding of the last round (whole workgroup)
-    const int qstrip = k_in_xcd % qstrips;
-    const int b = bh / a.nh, h = bh - b * a.nh;
-    const size_t row0 = (size_t)b * S;  // first token row of this sequence
-    int q[QT];       // this lane's queries
-    bool q_ok[QT];
-#pragma unroll
-    for (int t = 0; t < QT; t++) {
-        q[t] = qstrip * kStripQ + (wave * QT + t) * 16 + r16;
-        q_ok[t] = q[t] < S;
-    }
-    int klimit = S;
-    if (a.lens) klimit = min(S, max(a.lens[b], 0));
-    // under a causal mask no query of this strip sees a key past the strip's last query
-    if (a.causal) klimit = min(klimit, (qstrip + 1) * kStripQ);
-    // compact-V: this head's surviving V columns
-    // head sizes between the template sizes: columns [hd, HD) of Q, K and V read as zero
-    // (no effect on scores or outputs) and are not written
-    const int hd = a.hd;
-    int vc0 = 0, vlive = hd;
-    bool v_vec = false;  // this head's compact columns can be read as aligned 16-byte vectors
-    if (COMPACT) {
-        vc0 = a.v_head_ptr[h];
-        vlive = min(a.v_head_ptr[h + 1] - vc0, hd);
-        v_vec = ((vc0 | vlive | a.ldv) & 7) == 0 && vlive > 0 && (reinterpret_cast<uintptr_t>(a.V) & 15) == 0;
-    }
-    // compact-V: the full-width positions of this head's surviving columns are requested now
-    // and used in the epilogue (kCid ids per thread cover the up to 128 columns of a head)
-    constexpr int kCid = COMPACT ? (128 + nthr - 1) / nthr : 1;
-    int my_cid[kCid];
-    if (COMPACT) {
-#pragma unroll
-        for (int i = 0; i < kCid; i++)
-            // clamped into the array also for a head without surviving columns that sits at its end
-            my_cid[i] = a.v_col_id[min(vc0 + min((int)threadIdx.x + i * nthr, max(vlive - 1, 0)), a.v_nnz - 1)];
-    }
-
-    // Q fragments: B operand, lane supplies Q[q][32*ks + 8g .. +7]
-    h8 qf[QT][KS];
-#pragma unroll
-    for (int t = 0; t < QT; t++) {
-        const _Float16 *qp = a.Q + (row0 + (q_ok[t] ? q[t] : 0)) * a.ldq + h * hd + 8 * g;
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            const bool live = q_ok[t] && 32 * ks + 8 * g < hd;
-            qf[t][ks] = *reinterpret_cast<const h8 *>(qp + (live ? 32 * ks : 0));
-            if (!live) qf[t][ks] = h8{0, 0, 0, 0, 0, 0, 0, 0};
-        }
-    }
-
-    f4 o[QT][DB];
-    float m_run[QT];   // running max of this lane's query (log2 domain)
-    float l_part[QT];  // this lane's share of the running row sum
-#pragma unroll
-    for (int t = 0; t < QT; t++) {
-#pragma unroll
-        for (int d = 0; d < DB; d++) o[t][d] = f4{0.f, 0.f, 0.f, 0.f};
-        m_run[t] = -INFINITY;
-        l_part[t] = 0.0f;
-    }
-
-    // ---- staging of one block of keys: K rows and V in units of 4 keys x 8 dims, which
-    // go to LDS transposed.  load_block issues every global load of a block (one memory
-    // round trip); store_block writes them to LDS.  The loads of block i+1 are issued
-    // before block i is multiplied.
-    constexpr int vec_per_row = HD / 8;
-    constexpr int KV = kKeyBlock * vec_per_row / nthr;  // K vectors per thread
-    constexpr int dgroups = HD / 8;
-    constexpr int v_units = (kKeyBlock / 4) * dgroups;  // V units of 4 keys x 8 dims
-    constexpr int VU = (v_units + nthr - 1) / nthr;       // ... per thread
-    static_assert(KV >= 1 && kKeyBlock * vec_per_row % nthr == 0, "K block must split evenly");
-    h8 kreg[KV];
-    h8 vreg[VU][4];
-    auto load_block = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < KV; i++) {
-            const int v = threadIdx.x + i * nthr;
-            const int r = v / vec_per_row, c = v - r * vec_per_row;
-            kreg[i] = h8{0, 0, 0, 0, 0, 0, 0, 0};
-            if (k0 + r < S && c * 8 < hd)
-                kreg[i] = *reinterpret_cast<const h8 *>(a.K + (row0 + k0 + r) * a.ldk + h * hd + c * 8);
-        }
-#pragma unroll
-        for (int j = 0; j < VU; j++) {
-            const int u = threadIdx.x + j * nthr;
-            const int dg = u % dgroups, kg = vt_unit_keys<HD>(u / dgroups);
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int key = (u < v_units) ? k0 + kg * 4 + i : S;  // surplus threads load nothing
-                vreg[j][i] = h8{0, 0, 0, 0, 0, 0, 0, 0};
-                if (COMPACT) {
-                    // Every load is unconditional, from a clamped address, and the value is
-                    // selected afterwards: a load under a branch gets a basic block of its own and
-                    // is waited for on the spot, one memory round trip per element.
-                    const bool key_ok = key < S;
-                    const _Float16 *vp = a.V + (row0 + (key_ok ? key : 0)) * a.ldv + (vlive > 0 ? vc0 : 0);
-                    if (v_vec) {  // workgroup-uniform: 16-byte vectors of surviving columns
-                        const bool live = key_ok && dg * 8 < vlive;
-                        const h8 t = *reinterpret_cast<const h8 *>(vp + (live ? dg * 8 : 0));
-                        vreg[j][i] = live ? t : h8{0, 0, 0, 0, 0, 0, 0, 0};
-                    } else {  // compact columns that start at an arbitrary element
-#pragma unroll
-                        for (int d = 0; d < 8; d++) {
-                            const bool live = key_ok && dg * 8 + d < vlive;
-                            const _Float16 t = vp[live ? dg * 8 + d : 0];
-                            vreg[j][i][d] = live ? t : (_Float16)0;
-                        }
-                    }
-                } else if (key < S && dg * 8 < hd) {
-                    vreg[j][i] = *reinterpret_cast<const h8 *>(a.V + (row0 + key) * a.ldv + h * hd + dg * 8);
-                }
-            }
-        }
-    };
-    auto store_block = [&]() {
-#pragma unroll
-        for (int i = 0; i < KV; i++) {
-            const int v = threadIdx.x + i * nthr;
-            const int r = v / vec_per_row, c = v - r * vec_per_row;
-            *reinterpret_cast<h8 *>(Ks + r * L::ldk + c * 8) = kreg[i];
-        }
-#pragma unroll
-        for (int j = 0; j < VU; j++) {
-            const int u = threadIdx.x + j * nthr;
-            const int dg = u % dgroups, kg = vt_unit_keys<HD>(u / dgroups);
-            if (u < v_units) {
-                // keys 4kg..4kg+3 = (s, a, g) = (kg / 8, (kg / 4) % 2, kg % 4); rows 8dg..8dg+7 share row / 16
-                const int pos = (32 * (kg >> 3) + 8 * (kg & 3) + 4 * ((kg >> 2) & 1)) ^ vt_swizzle<HD>(dg >> 1);
-#pragma unroll
-                for (int d = 0; d < 8; d++) {
-                    h4 col = {vreg[j][0][d], vreg[j][1][d], vreg[j][2][d], vreg[j][3][d]};
-                    *reinterpret_cast<h4 *>(Vt + (dg * 8 + d) * L::ldvt + pos) = col;
-                }
-            }
-        }
-    };
-
-    // Holding the next block's loads in registers through the multiplication costs 32 VGPRs: it
-    // is done where that still fits the resident waves the variant runs with anyway (3-4 % at
-    // 512 and 2048 keys); elsewhere it spills or loses a wave, and is off.
-    constexpr bool kPrefetch = mha_prefetches<HD, NW, COMPACT, QT>();
-    const int nblocks = (klimit + kKeyBlock - 1) / kKeyBlock;
-    if (kPrefetch && nblocks > 0) load_block(0);
-    for (int blk = 0; blk < nblocks; blk++) {
-        const int k0 = blk * kKeyBlock;
-        if (blk > 0) __syncthreads();  // every wave is done with the previous block
-        if (!kPrefetch) load_block(k0);
-        store_block();
-        __syncthreads();
-        if (kPrefetch && blk + 1 < nblocks) load_block(k0 + kKeyBlock);
-
-        // The multiplication of one staged block.  FAST (wave-uniform) = nothing is added to the
-        // scores and every key of the block is live for every query of the workgroup, or dead
-        // for every query (right padding):
-        // no per-16-key branches (the LDS reads of the whole block can be issued ahead of
-        // the MFMAs) and the softmax costs one max, one multiply-add, one exp2, half a
-        // conversion and half a dot-accumulate per score.
-#include "attention_core.inc"
-        const bool plain = a.mask == nullptr && a.scale_log2e > 0.0f &&
-                          (!a.causal || k0 + kKeyBlock <= qstrip * kStripQ + 1);
-        if (plain) multiply(std::true_type{});
-        else multiply(std::false_type{});
-    }
-
-    // ---- normalise and store: lane holds dims 16d + 4g..4g+3 of query r16
-    float inv[QT];
-#pragma unroll
-    for (int t = 0; t < QT; t++) {
-        float l = l_part[t];
-        l = rows_sum(l);
-        inv[t] = l > 0.0f ? 1.0f / l : 0.0f;
-    }
-    if (!COMPACT) {
-#pragma unroll
-        for (int t = 0; t < QT; t++) {
-            if (!q_ok[t]) continue;
-            _Float16 *zp = a.Z + (row0 + q[t]) * a.ldz + h * hd + 4 * g;
-#pragma unroll
-            for (int d = 0; d < DB; d++) {
-                if (16 * d >= hd) continue;  // wave-uniform
-                h4 out;
-#pragma unroll
-                for (int j = 0; j < 4; j++) out[j] = (_Float16)(o[t][d][j] * inv[t]);
-                // a head size that is a multiple of 8 only ends inside the last block: lanes past it store nothing
-                if (16 * d + 4 * g < hd) *reinterpret_cast<h4 *>(zp + 16 * d) = out;
-            }
-        }
-    }
-    if (COMPACT) {
-        // Full-width Z: surviving columns are scattered to v_col_id, the pruned columns of this
-        // head's slice get zeros.  Every element of the slice is written exactly once (the
-        // liveness mask tells the two sets apart), so no store has to be ordered against another.
-        // The column ids were requested at the start of the kernel; mask and compact-to-full map
-        // go through LDS here, where every wave of the workgroup arrives.
-        __shared__ unsigned live_mask[4];  // bit c: column c of this head's slice of Z survives
-        __shared__ int full_col[128];      // compact column -> column of Z
-        __shared__ int n_outside;          // surviving columns that lie outside this head's slice
-        if (threadIdx.x < 4) live_mask[threadIdx.x] = 0u;
-        if (threadIdx.x == 4) n_outside = 0;
-        __syncthreads();  // also: every wave is done with the staged K and V
-#pragma unroll
-        for (int i = 0; i < kCid; i++) {
-            const int j = threadIdx.x + i * nthr;
-            if (j < vlive) {
-                full_col[j] = my_cid[i];
-                const int c = my_cid[i] - h * hd;
-                if (c >= 0 && c < HD) atomicOr(&live_mask[c >> 5], 1u << (c & 31));
-                if (c < 0 || c >= hd) atomicAdd(&n_outside, 1);
-            }
-        }
-        __syncthreads();
-        if (n_outside == 0) {
-            // The usual case, every surviving column inside the head's own slice: the wave
-            // assembles its 16 queries x hd slice in LDS (zeros, then the surviving columns at
-            // their places) and stores whole 8-byte pieces of rows, 4 per lane and tile, instead
-            // of up to 32 two-byte stores.  One wave's LDS instructions complete in order, so
-            // the three steps need no barrier.
-            constexpr int ldt = HD + 8;
-            _Float16 *zt = Ks + wave * 16 * ldt;  // the K stage is free: NW * 16 rows <= 128
-            static_assert(NW * 16 <= kKeyBlock && HD + 8 <= MhaLds<HD>::ldk, "slice tiles fit the K stage");
-            int zl[DB][4];
-#pragma unroll
-            for (int d = 0; d < DB; d++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) zl[d][j] = full_col[min(d * 16 + 4 * g + j, 127)] - h * hd;
-#pragma unroll
-            for (int t = 0; t < QT; t++) {
-                const h4 zero4 = {0, 0, 0, 0};
-#pragma unroll
-                for (int i = 0; i < HD / 16; i++) {
-                    const int v = lane + 64 * i;  // 8-byte piece of the 16 x HD tile
-                    *reinterpret_cast<h4 *>(zt + (v / (HD / 4)) * ldt + (v % (HD / 4)) * 4) = zero4;
-                }
-#pragma unroll
-                for (int d = 0; d < DB; d++)
-#pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        if (d * 16 + 4 * g + j < vlive) zt[r16 * ldt + zl[d][j]] = (_Float16)(o[t][d][j] * inv[t]);
-                const int qbase = qstrip * kStripQ + (wave * QT + t) * 16;
-#pragma unroll
-                for (int i = 0; i < HD / 16; i++) {
-                    const int v = lane + 64 * i;
-                    const int rr = v / (HD / 4), cc = (v % (HD / 4)) * 4;
-                    const h4 piece = *reinterpret_cast<const h4 *>(zt + rr * ldt + cc);
-                    if (qbase + rr < S && cc < hd)
-                        *reinterpret_cast<h4 *>(a.Z + (row0 + qbase + rr) * a.ldz + h * hd + cc) = piece;
-                }
-            }
-            return;
-        }
-        int zc[DB][4];
-#pragma unroll
-        for (int d = 0; d < DB; d++)
-#pragma unroll
-            for (int j = 0; j < 4; j++) zc[d][j] = full_col[min(d * 16 + 4 * g + j, 127)];
-        unsigned live_w[4];
-#pragma unroll
-        for (int w = 0; w < 4; w++) live_w[w] = live_mask[w];
-#pragma unroll
-        for (int t = 0; t < QT; t++) {
-            if (q_ok[t]) {
-                _Float16 *zrow = a.Z + (row0 + q[t]) * a.ldz;
-#pragma unroll
-                for (int d = 0; d < DB; d++) {
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const int dc = d * 16 + 4 * g + j;  // as a compact index, and as a column of the slice
-                        if (dc < vlive) zrow[zc[d][j]] = (_Float16)(o[t][d][j] * inv[t]);
-                        if (dc < hd && !((live_w[dc >> 5] >> (dc & 31)) & 1u)) zrow[h * hd + dc] = (_Float16)0;
-                    }
-                }
-            }
-        }
-    }
+    constexpr bool kCoherentZ = false;
+#include "attention_body.inc"
 }
 
 template <int HD, bool COMPACT, int NW, int QT>
@@ -452,6 +179,305 @@ static int launch_mha(const MhaArgs &args, int B, hipStream_t stream) {
     if (qblocks % 4 == 0) return launch_mha_nw<HD, COMPACT, 4, 1>(args, stream);
     if (qblocks % 2 == 0) return launch_mha_nw<HD, COMPACT, 2, 1>(args, stream);
     return launch_mha_nw<HD, COMPACT, 1, 1>(args, stream);
+}
+
+
+// ---- attention and the tile-sparse output projection in one launch ------------------------------------
+// E.T.'s O-fused attention (Attention/kernel_fuseO.cu:138-243) runs the attention of every (head, query
+// strip), waits at a grid-wide barrier of a cooperative launch and then multiplies Z with the tile-sparse
+// W_O.  Here nothing waits: a workgroup runs the fused attention of its (sequence, head, query strip),
+// stores its slice of Z, and adds one to the arrival count of its (sequence, query strip).  The workgroup
+// whose addition completes the count — all heads of those tokens are in memory — stages the finished rows of
+// Z in LDS and multiplies them with W_O: a wave per block-row of the weight, two tiles per MFMA, the tile
+// fragments of the next three groups of six tile pairs on their way while a group is multiplied.  Every other
+// workgroup has left by then, so the launch needs no co-residency and no spinning, and the projection of
+// the first finished strips overlaps the attention of the rest.  The last arriver puts the count back to
+// zero: the counts are zero before and after every launch.
+// What bounds it: the projecting workgroup takes in the whole weight by itself (236 KB for 768 x 768 at 80 %
+// sparsity) and a compute unit takes in about 20 GB/s of lines its L2 does not hold, so the projection of a
+// strip costs 12 to 16 us wherever it runs, against 4 us for a launch of its own that spreads the weight over
+// a few hundred workgroups: 26 against 8 us for one sequence of 128 tokens, 29 against 9 us for eight.  The
+// class layer therefore keeps the two launches; this entry point is for callers that need one.
+struct FuseOArgs {
+    const int32_t *row_ptr, *col_idx;  // W_O [emdim x nh*hd] as 16x16 tiles (tile rows = output features)
+    const _Float16 *tiles;
+    const _Float16 *bias;              // [emdim] or nullptr
+    _Float16 *out;                     // [B*S x emdim]
+    int emdim;
+    unsigned *arrived;                 // [B * query strips]
+};
+
+constexpr int kFuseOPairs = 6;            // tile pairs of a block-row requested together
+constexpr int kFuseOCounters = 16384;     // arrival counts built into the library (per device)
+static __device__ __align__(256) unsigned fuseo_arrived[kFuseOCounters];
+
+template <int HD, int NW, int QT>
+__global__ __launch_bounds__(64 * NW) void mha_fuseo_kernel(const MhaArgs a, const FuseOArgs f) {
+    constexpr bool COMPACT = false;
+    constexpr bool kCoherentZ = true;
+#include "attention_body.inc"
+    // ---- arrival.  Z was stored at device scope, and such a store counts as complete only once it has
+    // reached the memory side: when every wave's stores are complete the count moves.  A device-wide fence
+    // would order the same, but it writes back the whole L2 of the die and invalidates it, 2.4 us for every
+    // workgroup of the launch, one after the other on a die.
+    __shared__ unsigned is_last;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // also: every wave is done with the staged K and V
+    if (threadIdx.x == 0) {
+        unsigned *cnt = f.arrived + (size_t)b * qstrips + qstrip;
+        const unsigned before = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = before + 1u == (unsigned)a.nh;
+        if (last) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        is_last = last ? 1u : 0u;
+    }
+    __syncthreads();
+    if (!is_last) return;
+
+    // ---- the projection of the strip.  Order of the requests: the wave's row pointers, the first rows of Z,
+    // the first tile fragments, the rest of Z; everything the first products need is then on its way at once.
+    constexpr int TT = NW * QT;  // 16-token tiles of the strip
+    constexpr int P = kFuseOPairs;
+    constexpr int ZU = 24;       // 16-byte vectors of Z a thread requests together (768-wide rows on 4 waves: all of them)
+    const int nbr = f.emdim / 16;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    // the wave owns block-rows wave, wave + NW, ...: its k-th row is wave + NW k.  The row pointers go to LDS
+    // behind the rows of Z: a load of them between the tile requests would have to be waited for, and the
+    // requests made before it with it (loads return in order).
+    const int nrows = nbr > wave_u ? (nbr - wave_u + NW - 1) / NW : 0;
+    const int ntile = f.row_ptr[nbr];
+
+    const int width = a.nh * hd;       // a multiple of 16
+    const int ldzs = width + 8;        // halfs; rows 16 bytes apart in the banks
+    _Float16 *Zs = reinterpret_cast<_Float16 *>(smem_raw);
+    const int vpr = width / 8;
+    const int nvec = kStripQ * vpr;
+    h8 zt[ZU];
+    auto z_request = [&](int v0) {
+#pragma unroll
+        for (int i = 0; i < ZU; i++) {
+            const int v = min(v0 + i * nthr + (int)threadIdx.x, nvec - 1);
+            const int r = v / vpr, c = v - r * vpr;
+            const int row = min(qstrip * kStripQ + r, S - 1);
+            zt[i] = load_device_scope(a.Z + (row0 + row) * a.ldz + c * 8);
+        }
+    };
+    auto z_place = [&](int v0) {  // rows past the sequence as zeros
+#pragma unroll
+        for (int i = 0; i < ZU; i++) {
+            const int v = v0 + i * nthr + (int)threadIdx.x;
+            const int r = v / vpr, c = v - r * vpr;
+            if (v < nvec)
+                *reinterpret_cast<h8 *>(Zs + r * ldzs + c * 8) =
+                    (qstrip * kStripQ + r < S) ? zt[i] : h8{0, 0, 0, 0, 0, 0, 0, 0};
+        }
+    };
+    int *rps = reinterpret_cast<int *>(Zs + kStripQ * ldzs);
+    for (int i0 = 0; i0 <= nbr; i0 += nthr) {  // one pass up to 64 NW - 1 block-rows
+        const int i = min(i0 + (int)threadIdx.x, nbr);
+        const int v = f.row_ptr[i];
+        if (i0 == 0) {
+            z_request(0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        rps[i] = v;
+    }
+    __syncthreads();
+
+    // a weight without tiles: the loads below go to valid dummy addresses and meet the zero operand
+    const _Float16 *tbase = ntile > 0 ? f.tiles : a.Z + row0 * a.ldz;
+    const int32_t *cbase = ntile > 0 ? f.col_idx : f.row_ptr;
+    const int jmax = max(ntile - 1, 0);
+    const int half_k = 8 * (g & 1), second = g >> 1;
+    const h8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    // chunk = up to P tile pairs of one block-row: (row of the wave, first tile, end of the row's tiles);
+    // three chunks are on their way while one is multiplied
+    struct Chunk {
+        int k, j, j1;
+    };
+    // (the row's bias comes with every chunk: requested where the row ends, it would be waited for on the
+    // spot, and with it every request made before it)
+    const _Float16 *bbase = f.bias ? f.bias + 4 * g : tbase;
+    const int bstep = f.bias ? 16 : 0;
+    auto request = [&](const Chunk &ch, h8 (&w)[P], int (&c)[P], h4 &bq) {
+        bq = *reinterpret_cast<const h4 *>(bbase + (size_t)min(wave_u + NW * ch.k, nbr - 1) * bstep);
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            const int jt = ch.j + 2 * p + second;
+            const int jc = min(jt, jmax);
+            c[p] = cbase[jc];
+            w[p] = *reinterpret_cast<const h8 *>(tbase + (size_t)jc * 256 + r16 * 16 + half_k);
+        }
+    };
+    auto after = [&](const Chunk &ch) {  // the rest of the row, or the start of the wave's next row
+        Chunk nx = {ch.k, ch.j + 2 * P, ch.j1};
+        if (nx.j >= ch.j1 && ch.k < nrows) {  // wave-uniform
+            nx.k = ch.k + 1;
+            if (nx.k < nrows) {
+                nx.j = __builtin_amdgcn_readfirstlane(rps[wave_u + NW * nx.k]);
+                nx.j1 = __builtin_amdgcn_readfirstlane(rps[wave_u + NW * nx.k + 1]);
+            } else {
+                nx.j = nx.j1 = ch.j1;  // past the end: requests that meet nothing
+            }
+        }
+        return nx;
+    };
+    h8 w0[P], w1[P], w2[P], w3[P];
+    int c0[P], c1[P], c2[P], c3[P];
+    h4 b0, b1, b2, b3;
+    Chunk ch0 = {0, 0, 0};
+    if (nrows > 0) {
+        ch0.j = __builtin_amdgcn_readfirstlane(rps[wave_u]);
+        ch0.j1 = __builtin_amdgcn_readfirstlane(rps[wave_u + 1]);
+    }
+    request(ch0, w0, c0, b0);
+    Chunk ch1 = after(ch0);
+    request(ch1, w1, c1, b1);
+    Chunk ch2 = after(ch1);
+    request(ch2, w2, c2, b2);
+    __builtin_amdgcn_sched_barrier(0);
+    z_place(0);
+    for (int v0 = ZU * nthr; v0 < nvec; v0 += ZU * nthr) {
+        z_request(v0);
+        z_place(v0);
+    }
+    __syncthreads();
+
+    // ---- out[token][16n + ..] = bias + sum over the tiles of block-row n
+    f4 acc[TT];
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++) acc[tt] = f4{0.f, 0.f, 0.f, 0.f};
+    auto multiply = [&](const Chunk &cur, const Chunk &nxt, const h8 (&w)[P], const int (&c)[P], const h4 &bq) {
+        // the Z fragments of half a chunk are read together and multiplied then: one wave per SIMD has
+        // nothing else to cover the LDS latency with, and read by read it adds up to most of the projection
+        constexpr int PH = P / 2;
+#pragma unroll
+        for (int p0 = 0; p0 < P; p0 += PH) {
+            h8 zf[PH][TT];
+#pragma unroll
+            for (int pp = 0; pp < PH; pp++) {
+                const bool live = cur.j + 2 * (p0 + pp) + second < cur.j1;
+                const _Float16 *zp = Zs + r16 * ldzs + (live ? c[p0 + pp] : 0) * 16 + half_k;
+#pragma unroll
+                for (int tt = 0; tt < TT; tt++) zf[pp][tt] = *reinterpret_cast<const h8 *>(zp + tt * 16 * ldzs);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int pp = 0; pp < PH; pp++) {
+                const bool live = cur.j + 2 * (p0 + pp) + second < cur.j1;
+                const h8 wf = live ? w[p0 + pp] : zero8;
+#pragma unroll
+                for (int tt = 0; tt < TT; tt++)
+                    acc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf, zf[pp][tt], acc[tt], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (nxt.k != cur.k) {  // the row is complete: lane holds features 16n + 4g .. +3 of token r16 of every tile
+            const int n = wave_u + NW * cur.k;
+            float bv[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) bv[j] = f.bias ? (float)bq[j] : 0.0f;
+#pragma unroll
+            for (int tt = 0; tt < TT; tt++) {
+                const int row = qstrip * kStripQ + tt * 16 + r16;
+                h4 o4;
+#pragma unroll
+                for (int j = 0; j < 4; j++) o4[j] = (_Float16)(acc[tt][j] + bv[j]);
+                if (row < S) *reinterpret_cast<h4 *>(f.out + (row0 + row) * f.emdim + n * 16 + 4 * g) = o4;
+                acc[tt] = f4{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+    };
+    // The four register sets take turns (a set is requested again right after it was multiplied); moving
+    // the fragments from set to set instead would make every turn wait for all of them.
+    Chunk ch3 = ch2;
+    // (scheduling barriers: left alone, the compiler moves requests down to where their values are used and
+    // then has to wait for all of them)
+    while (true) {  // every exit is wave-uniform
+        if (ch0.k >= nrows) break;
+        ch3 = after(ch2);
+        request(ch3, w3, c3, b3);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(ch0, ch1, w0, c0, b0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (ch1.k >= nrows) break;
+        ch0 = after(ch3);
+        request(ch0, w0, c0, b0);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(ch1, ch2, w1, c1, b1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (ch2.k >= nrows) break;
+        ch1 = after(ch0);
+        request(ch1, w1, c1, b1);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(ch2, ch3, w2, c2, b2);
+        __builtin_amdgcn_sched_barrier(0);
+        if (ch3.k >= nrows) break;
+        ch2 = after(ch1);
+        request(ch2, w2, c2, b2);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(ch3, ch0, w3, c3, b3);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+static std::mutex g_fuseo_mutex;
+static std::atomic<unsigned *> g_fuseo_counts[64];
+
+// Device address of the arrival counts on the current device (looked up on first use; the array is
+// zero when the library is loaded and every launch leaves it zero).
+static int fuseo_counts(unsigned **out) {
+    int dev = -1;
+    ET_HIP(hipGetDevice(&dev));
+    ET_REQUIRE(dev >= 0 && dev < 64, ET_ERR_UNSUPPORTED, "et_mha_fuseo_f16: device ordinal %d", dev);
+    unsigned *p = g_fuseo_counts[dev].load(std::memory_order_acquire);
+    if (!p) {
+        std::lock_guard<std::mutex> lock(g_fuseo_mutex);
+        p = g_fuseo_counts[dev].load(std::memory_order_relaxed);
+        if (!p) {
+            void *sym = nullptr;
+            ET_HIP(hipGetSymbolAddress(&sym, HIP_SYMBOL(fuseo_arrived)));
+            ET_REQUIRE(sym != nullptr, ET_ERR_LAUNCH, "et_mha_fuseo_f16: hipGetSymbolAddress returned NULL");
+            p = static_cast<unsigned *>(sym);
+            g_fuseo_counts[dev].store(p, std::memory_order_release);
+        }
+    }
+    *out = p;
+    return ET_OK;
+}
+
+constexpr size_t kLdsPerWorkgroup = 160 * 1024 - 256;  // the arrival flag is a static allocation of its own
+
+template <int HD, int NW>
+static int launch_fuseo_nw(const MhaArgs &args, const FuseOArgs &fo, hipStream_t stream) {
+    auto kernel = mha_fuseo_kernel<HD, NW, 1>;
+    const size_t strip = (size_t)16 * NW * (args.nh * args.hd + 8) * sizeof(_Float16) + (size_t)(fo.emdim / 16 + 1) * sizeof(int);
+    const size_t lds = std::max(MhaLds<HD>::bytes, strip);
+    ET_REQUIRE(lds <= kLdsPerWorkgroup, ET_ERR_UNSUPPORTED, "et_mha_fuseo_f16: a strip of %d rows of Z (%zu B) exceeds LDS",
+               16 * NW, strip);
+    static std::atomic<size_t> raised{64 * 1024};
+    if (lds > raised.load(std::memory_order_acquire)) {
+        ET_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   (int)kLdsPerWorkgroup));
+        raised.store(kLdsPerWorkgroup, std::memory_order_release);
+    }
+    const int qstrips = (args.S + 16 * NW - 1) / (16 * NW);
+    const int rounds = (args.nbh + kXcds - 1) / kXcds;
+    kernel<<<dim3((unsigned)(rounds * kXcds * qstrips)), 64 * NW, lds, stream>>>(args, fo);
+    return check_launch("mha_fuseo_kernel");
+}
+
+// waves: 0 picks; 1, 2 or 4 waves (16, 32 or 64 tokens per workgroup and projection strip)
+template <int HD>
+static int launch_fuseo(const MhaArgs &args, const FuseOArgs &fo, int waves, hipStream_t stream) {
+    const int qblocks = args.S / 16;
+    const size_t row_bytes = (size_t)(args.nh * args.hd + 8) * sizeof(_Float16);
+    if (waves == 0) {
+        waves = qblocks % 4 == 0 ? 4 : qblocks % 2 == 0 ? 2 : 1;
+        while (waves > 1 && 16 * waves * row_bytes + (fo.emdim / 16 + 1) * sizeof(int) > kLdsPerWorkgroup) waves >>= 1;
+    }
+    if (waves == 4) return launch_fuseo_nw<HD, 4>(args, fo, stream);
+    if (waves == 2) return launch_fuseo_nw<HD, 2>(args, fo, stream);
+    return launch_fuseo_nw<HD, 1>(args, fo, stream);
 }
 
 
@@ -875,6 +901,80 @@ int et_mha_fused_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V, int ldq,
     // register file (8 waves at 256 registers spill 68 bytes per lane); a strip shorter than 64 queries
     // leaves waves without queries, which stage and otherwise idle.
     return launch_mha_nw<256, false, 4, 1>(args, as_stream(stream));
+}
+
+int et_mha_fuseo_f16_geom(const et_f16 *Q, const et_f16 *K, const et_f16 *V, int ldq, int ldk, int ldv, et_f16 *Z,
+                          int ldz, const et_f16 *mask, const int32_t *lens, int B, int S, int nh, int hd,
+                          float scale, int flags, const int32_t *o_row_ptr, const int32_t *o_col_idx,
+                          const et_f16 *o_tiles, const et_f16 *o_bias, et_f16 *out, int emdim, int waves,
+                          et_stream stream) {
+    ET_REQUIRE(Q && K && V && Z && o_row_ptr && out, ET_ERR_INVALID_ARG, "et_mha_fuseo_f16: NULL pointer");
+    ET_REQUIRE(B >= 0 && S > 0 && nh > 0 && hd > 0 && emdim > 0, ET_ERR_INVALID_ARG,
+               "et_mha_fuseo_f16: B=%d S=%d nh=%d hd=%d emdim=%d", B, S, nh, hd, emdim);
+    ET_REQUIRE((flags & ~ET_MHA_CAUSAL) == 0, ET_ERR_INVALID_ARG, "et_mha_fuseo_f16: flags=%d", flags);
+    ET_REQUIRE(waves == 0 || waves == 1 || waves == 2 || waves == 4, ET_ERR_INVALID_ARG,
+               "et_mha_fuseo_f16: waves=%d", waves);
+    ET_REQUIRE(S % 16 == 0, ET_ERR_UNSUPPORTED, "et_mha_fuseo_f16: S=%d must be a multiple of 16", S);
+    ET_REQUIRE(hd % 8 == 0 && hd <= 128, ET_ERR_UNSUPPORTED,
+               "et_mha_fuseo_f16: head dim %d must be a multiple of 8, at most 128", hd);
+    const int width = nh * hd;
+    ET_REQUIRE(width % 16 == 0 && emdim % 16 == 0, ET_ERR_UNSUPPORTED,
+               "et_mha_fuseo_f16: nh*hd=%d and emdim=%d must be multiples of 16", width, emdim);
+    ET_REQUIRE(ldq >= width && ldk >= width && ldv >= width && ldz >= width, ET_ERR_INVALID_ARG,
+               "et_mha_fuseo_f16: row strides (%d %d %d %d) smaller than nh*hd=%d", ldq, ldk, ldv, ldz, width);
+    ET_REQUIRE(ldq % 8 == 0 && ldk % 8 == 0 && ldv % 8 == 0 && ldz % 8 == 0, ET_ERR_UNSUPPORTED,
+               "et_mha_fuseo_f16: row strides must keep 16-byte alignment");
+    ET_REQUIRE(((reinterpret_cast<uintptr_t>(Q) | reinterpret_cast<uintptr_t>(K) | reinterpret_cast<uintptr_t>(V) |
+                 reinterpret_cast<uintptr_t>(Z) | reinterpret_cast<uintptr_t>(o_tiles)) & 15) == 0 &&
+                   ((reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(o_bias)) & 7) == 0,
+               ET_ERR_UNSUPPORTED, "et_mha_fuseo_f16: operands must be 16-byte aligned (out, bias: 8)");
+    // one arrival count per (sequence, 16-query block) at most
+    ET_REQUIRE((long long)B * (S / 16) <= kFuseOCounters, ET_ERR_UNSUPPORTED,
+               "et_mha_fuseo_f16: B*S/16=%lld exceeds the %d arrival counts built into the library; run "
+               "et_mha_fused_f16 and et_linear_bsr16_f16 instead",
+               (long long)B * (S / 16), kFuseOCounters);
+    ET_REQUIRE((size_t)16 * (width + 8) * sizeof(_Float16) + (emdim / 16 + 1) * sizeof(int) <= kLdsPerWorkgroup, ET_ERR_UNSUPPORTED,
+               "et_mha_fuseo_f16: 16 rows of Z (%d wide) exceed LDS", width);
+    if (B == 0) return ET_OK;
+    MhaArgs args;
+    args.Q = reinterpret_cast<const _Float16 *>(Q);
+    args.K = reinterpret_cast<const _Float16 *>(K);
+    args.V = reinterpret_cast<const _Float16 *>(V);
+    args.Z = reinterpret_cast<_Float16 *>(Z);
+    args.mask = reinterpret_cast<const _Float16 *>(mask);
+    args.lens = lens;
+    args.ldq = ldq;
+    args.ldk = ldk;
+    args.ldv = ldv;
+    args.ldz = ldz;
+    args.S = S;
+    args.nh = nh;
+    args.hd = hd;
+    args.nbh = B * nh;
+    args.scale_log2e = scale * kLog2e;
+    args.causal = (flags & ET_MHA_CAUSAL) ? 1 : 0;
+    args.v_col_id = nullptr;
+    args.v_head_ptr = nullptr;
+    FuseOArgs fo;
+    fo.row_ptr = o_row_ptr;
+    fo.col_idx = o_col_idx;
+    fo.tiles = reinterpret_cast<const _Float16 *>(o_tiles);
+    fo.bias = reinterpret_cast<const _Float16 *>(o_bias);
+    fo.out = reinterpret_cast<_Float16 *>(out);
+    fo.emdim = emdim;
+    int st = fuseo_counts(&fo.arrived);
+    if (st != ET_OK) return st;
+    if (hd <= 32) return launch_fuseo<32>(args, fo, waves, as_stream(stream));
+    if (hd <= 64) return launch_fuseo<64>(args, fo, waves, as_stream(stream));
+    return launch_fuseo<128>(args, fo, waves, as_stream(stream));
+}
+
+int et_mha_fuseo_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *V, int ldq, int ldk, int ldv, et_f16 *Z,
+                     int ldz, const et_f16 *mask, const int32_t *lens, int B, int S, int nh, int hd, float scale,
+                     int flags, const int32_t *o_row_ptr, const int32_t *o_col_idx, const et_f16 *o_tiles,
+                     const et_f16 *o_bias, et_f16 *out, int emdim, et_stream stream) {
+    return et_mha_fuseo_f16_geom(Q, K, V, ldq, ldk, ldv, Z, ldz, mask, lens, B, S, nh, hd, scale, flags, o_row_ptr,
+                                 o_col_idx, o_tiles, o_bias, out, emdim, 0, stream);
 }
 
 int et_mha_compactv_f16(const et_f16 *Q, const et_f16 *K, const et_f16 *Vc, int ldq, int ldk, int ldvc,

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Per-kernel throughput against the roofline that bounds it, through the C ABI.
 
-    python scpaper-2021_amd/kernel_bench.py [--set configs|scale|vo|mha|plan|machine|all] [--json FILE]
+    python scpaper-2021_amd/kernel_bench.py [--set configs|scale|vo|mha|qkv|fuseo|plan|machine|all] [--json FILE]
 
 `configs` are the shapes of the benchmark configurations (attention block at batch
 1/4/16, the tile/row/column-pruned Linears at 2048 token rows, the BERT-large-shaped
@@ -184,6 +184,61 @@ class Bench:
         if destroy:
             et.check(destroy(handle))
         self.record(f"linear_bsr16 ({entry})", f"T{T} in{n_in} out{n_out} sparsity {sparsity}", us, 2 * 256 * ntile * T, "mfma")
+
+    def fuseo(self, B, S, sparsity, launches, nh=12, hd=64, nset=12):
+        """Fused attention followed by the tile-sparse output projection: the one launch (et_mha_fuseo_f16, with the
+        number of waves picked and forced) against the two launches it replaces (the projection through the plain
+        call and, where one exists for the shape, through a pack); every launch of a graph on another of `nset`
+        weight sets, as the layers of a stack."""
+        et, lib = self.et, self.lib
+        H, T = nh * hd, B * S
+        sets, ntile = [], 0
+        for i in range(nset):
+            row_ptr, col, ntile = self.tile_pattern(H, H, sparsity, 70 + i)
+            d_rp, d_col = self.dev(row_ptr), self.dev(col)
+            tiles = self.dev(self.rnd((max(ntile, 1), 256), 0.02))
+            pack = C.c_void_p()
+            if lib.et_bsr16_pack_create(d_rp.ptr, d_col.ptr, tiles.ptr, T, H, H, 0, 0, C.byref(pack)) != 0:
+                pack = None
+            sets.append((d_rp, d_col, tiles, pack))
+        bias = self.dev(np.zeros(H, np.float16))
+        qkv, z, out = self.dev(self.rnd((T, 3 * H))), self.empty((T, H)), self.empty((T, H))
+        scale, n = hd ** -0.5, {"i": 0}
+        q, k, v = qkv.ptr, qkv.offset(2 * H), qkv.offset(4 * H)
+
+        def one_launch(waves):
+            def fn():
+                s = sets[n["i"] % nset]
+                n["i"] += 1
+                et.check(lib.et_mha_fuseo_f16_geom(q, k, v, 3 * H, 3 * H, 3 * H, z.ptr, H, None, None, B, S, nh, hd, scale, 0,
+                                                   s[0].ptr, s[1].ptr, s[2].ptr, bias.ptr, out.ptr, H, waves, self.stream))
+            return fn
+
+        def two_launches(packed):
+            def fn():
+                s = sets[n["i"] % nset]
+                n["i"] += 1
+                et.check(lib.et_mha_fused_f16(q, k, v, 3 * H, 3 * H, 3 * H, z.ptr, H, None, None, B, S, nh, hd, scale, 0,
+                                              self.stream))
+                if packed:
+                    et.check(lib.et_linear_bsr16_packed_f16(s[3], bias.ptr, z.ptr, out.ptr, None, T, 0, self.stream))
+                else:
+                    et.check(lib.et_linear_bsr16_f16(s[0].ptr, s[1].ptr, s[2].ptr, bias.ptr, z.ptr, out.ptr, T, H, H, 0,
+                                                     self.stream))
+            return fn
+
+        work = 2 * 256 * ntile * T + 4 * B * S * S * hd * nh
+        shape = f"B{B} S{S} nh{nh} hd{hd} sparsity {sparsity}"
+        self.record("mha + O (two launches, plain)", shape, self.time_us(two_launches(False), launches), work, "mfma")
+        if all(s[3] is not None for s in sets):
+            self.record("mha + O (two launches, pack)", shape, self.time_us(two_launches(True), launches), work, "mfma")
+        self.record("mha + O (one launch)", shape, self.time_us(one_launch(0), launches), work, "mfma")
+        for waves in (1, 2, 4):
+            if (S // 16) % waves == 0:
+                self.record(f"mha + O (one launch, {waves} waves)", shape, self.time_us(one_launch(waves), launches), work, "mfma")
+        for s in sets:
+            if s[3] is not None:
+                et.check(lib.et_bsr16_pack_destroy(s[3]))
 
     def qkv_mha(self, B, S, sparsity, launches, nh=12, hd=64, nset=12):
         """The consumer QKV projection followed by the fused attention (two launches) against the attention kernel
@@ -491,7 +546,7 @@ def run_scale(b: Bench):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--set", choices=("configs", "scale", "vo", "mha", "qkv", "plan", "machine", "all"), default="all")
+    ap.add_argument("--set", choices=("configs", "scale", "vo", "mha", "qkv", "fuseo", "plan", "machine", "all"), default="all")
     ap.add_argument("--json", default=None, help="also write the rows as JSON to this file")
     args = ap.parse_args()
     b = Bench()
@@ -515,6 +570,11 @@ def main():
         for B, S, sp in ((4, 128, 0.8), (8, 128, 0.8), (8, 128, 0.9), (12, 128, 0.8), (16, 128, 0.8), (16, 128, 0.9), (24, 128, 0.8),
                          (32, 128, 0.8), (16, 64, 0.8), (32, 64, 0.8), (64, 32, 0.8)):
             b.qkv_mha(B, S, sp, 48)
+    if args.set == "fuseo":
+        print("# attention + tile-sparse output projection: one launch against the two it replaces (768-wide, 12 heads of 64)")
+        for B, S, sp in ((1, 128, 0.8), (1, 384, 0.8), (2, 128, 0.8), (4, 128, 0.8), (8, 128, 0.8), (8, 128, 0.9), (16, 128, 0.8),
+                         (32, 128, 0.8), (64, 128, 0.8), (4, 512, 0.8)):
+            b.fuseo(B, S, sp, 48)
     if args.set == "vo":
         print("# pre-computed-VO attention: probabilities through memory (mha_vo) and on chip (mha_vo_otf)")
         for B, N in ((1, 768), (4, 384), (8, 768), (16, 768)):
