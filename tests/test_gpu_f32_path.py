@@ -293,3 +293,56 @@ def test_linear_csr_f32_reference_fixture(et):
     et.check(et.lib().et_linear_csr_f32(up(et, indptr).ptr, up(et, indices).ptr, up(et, data.astype(np.float32)).ptr,
                                         up(et, b).ptr, up(et, x).ptr, d_y.ptr, 5, ncol, nrow, 0, None))
     assert Hn.max_abs(d_y.numpy(), x.astype(np.float64).sum(1, keepdims=True) + b) <= 1e-6
+
+
+def test_tile_sparse_fp32_encoder_stack(et):
+    """The benchmark's pruned encoder (BERT-base, 80 % 16x16 tile sparsity on Q/K/V/O and both FFN matrices, batch 8
+    of 128 tokens with right padding) composed from the binary32 entry points alone, three layers deep: tile-sparse
+    Linear, fused attention, SkipLayerNorm.  Against the oracle's binary32 forward, max-abs 2e-4."""
+    from oracle import formats as F
+    lib = et.lib()
+    H, nh, FF, S, B, depth = 768, 12, 3072, 128, 8, 3
+    T = B * S
+    lens = [128, 100, 64, 128, 17, 96, 128, 80]
+    d_l = up(et, np.asarray(lens, np.int32))
+    f = lambda shape: et.DeviceBuffer.empty(shape, np.float32)
+    qkv, z, a, y1, ff, f2 = f((T, 3 * H)), f((T, H)), f((T, H)), f((T, H)), f((T, FF)), f((T, H))
+
+    def sparse(out, inp, seed):
+        row_ptr, col_idx = F.gen_tile_pattern(out, inp, 0.8, seed=seed)
+        tiles = randf((len(col_idx), 256), seed + 1, 0.03)
+        b = randf((out,), seed + 2, 0.05)
+        dev = (up(et, row_ptr), up(et, col_idx), up(et, tiles), up(et, b))
+        return dev, torch.from_numpy(F.bsr16_to_dense(row_ptr, col_idx, tiles, inp)), torch.from_numpy(b)
+
+    x = randf((T, H), 900)
+    cur, want = up(et, x), torch.from_numpy(x)
+    for layer in range(depth):
+        s0 = 1000 + 50 * layer
+        (dq, Wq, bq), (do, Wo, bo) = sparse(3 * H, H, s0), sparse(H, H, s0 + 10)
+        (d1, W1, b1), (d2, W2, b2) = sparse(FF, H, s0 + 20), sparse(H, FF, s0 + 30)
+        g1, be1, g2, be2 = 1 + randf((H,), s0 + 40, 0.1), randf((H,), s0 + 41, 0.1), 1 + randf((H,), s0 + 42, 0.1), \
+            randf((H,), s0 + 43, 0.1)
+        dg1, dbe1, dg2, dbe2 = up(et, g1), up(et, be1), up(et, g2), up(et, be2)
+        lin = lambda w, src, dst, n_in, n_out, act: et.check(lib.et_linear_bsr16_f32(
+            w[0].ptr, w[1].ptr, w[2].ptr, w[3].ptr, src.ptr, dst.ptr, T, n_in, n_out, act, None))
+        out = f((T, H))
+        lin(dq, cur, qkv, H, 3 * H, 0)
+        et.check(lib.et_mha_fused_f32(qkv.ptr, qkv.offset(4 * H), qkv.offset(8 * H), 3 * H, 3 * H, 3 * H, z.ptr, H, None,
+                                      d_l.ptr, B, S, nh, H // nh, (H // nh) ** -0.5, 0, None))
+        lin(do, z, a, H, H, 0)
+        et.check(lib.et_skip_layernorm_f32(y1.ptr, a.ptr, cur.ptr, dg1.ptr, dbe1.ptr, T, H, 1e-5, None))
+        lin(d1, y1, ff, H, FF, 2)
+        lin(d2, ff, f2, FF, H, 0)
+        et.check(lib.et_skip_layernorm_f32(out.ptr, f2.ptr, y1.ptr, dg2.ptr, dbe2.ptr, T, H, 1e-5, None))
+        cur = out
+        t = torch.from_numpy
+        P = L.LayerParams(Wq, bq, Wo, bo, W1, b1, W2, b2, t(g1), t(be1), t(g2), t(be2))
+        want = L.encoder_layer(want, P, L.LayerConfig(nh=nh, B=B, act="gelu", lens=lens))
+    got, want = cur.numpy(), want.numpy()
+    for b in range(B):  # rows past a sequence's length are padding: not compared
+        got[b * S + lens[b]:(b + 1) * S] = 0
+        want[b * S + lens[b]:(b + 1) * S] = 0
+    err = Hn.max_abs(got, want)
+    print(f"tile-sparse fp32 stack, {depth} layers: max-abs vs oracle {err:.2e}")
+    assert err <= 2e-4
