@@ -193,11 +193,13 @@ static int launch_mha(const MhaArgs &args, int B, hipStream_t stream) {
 // workgroup has left by then, so the launch needs no co-residency and no spinning, and the projection of
 // the first finished strips overlaps the attention of the rest.  The last arriver puts the count back to
 // zero: the counts are zero before and after every launch.
-// What bounds it: the projecting workgroup takes in the whole weight by itself (236 KB for 768 x 768 at 80 %
-// sparsity) and a compute unit takes in about 20 GB/s of lines its L2 does not hold, so the projection of a
-// strip costs 12 to 16 us wherever it runs, against 4 us for a launch of its own that spreads the weight over
-// a few hundred workgroups: 26 against 8 us for one sequence of 128 tokens, 29 against 9 us for eight.  The
-// class layer therefore keeps the two launches; this entry point is for callers that need one.
+// What it costs: the projecting workgroup takes in the whole weight by itself (236 KB for 768 x 768 at 80 %
+// sparsity; a compute unit takes in 20 GB/s of lines its L2 does not hold, 90 GB/s of lines it does), and as
+// compiled the loop still waits for all of its requests once per turn of the four register sets, about one
+// memory round trip (1.1 us) per group of six tile pairs, 13 groups per wave: 16 us for the projection of a
+// strip, against 4 us for a launch of its own that spreads the weight over a few hundred workgroups.  26
+// against 8 us for one sequence of 128 tokens, 29 against 9 us for eight.  The class layer therefore keeps
+// the two launches; this entry point is for callers that need one.
 struct FuseOArgs {
     const int32_t *row_ptr, *col_idx;  // W_O [emdim x nh*hd] as 16x16 tiles (tile rows = output features)
     const _Float16 *tiles;
@@ -233,8 +235,8 @@ __global__ __launch_bounds__(64 * NW) void mha_fuseo_kernel(const MhaArgs a, con
     __syncthreads();
     if (!is_last) return;
 
-    // ---- the projection of the strip.  Order of the requests: the wave's row pointers, the first rows of Z,
-    // the first tile fragments, the rest of Z; everything the first products need is then on its way at once.
+    // ---- the projection of the strip.  Order of the requests: the row pointers, the rows of Z, then the first
+    // tile fragments.
     constexpr int TT = NW * QT;  // 16-token tiles of the strip
     constexpr int P = kFuseOPairs;
     constexpr int ZU = 24;       // 16-byte vectors of Z a thread requests together (768-wide rows on 4 waves: all of them)
@@ -329,17 +331,21 @@ __global__ __launch_bounds__(64 * NW) void mha_fuseo_kernel(const MhaArgs a, con
         ch0.j = __builtin_amdgcn_readfirstlane(rps[wave_u]);
         ch0.j1 = __builtin_amdgcn_readfirstlane(rps[wave_u + 1]);
     }
+    // (the first tile requests wait until the rows of Z are placed: with both in registers at once the
+    // kernel is out of registers, and the compiler then reuses a register a request is still due to fill,
+    // which it can only do after waiting for every request)
+    z_place(0);
+    for (int v0 = ZU * nthr; v0 < nvec; v0 += ZU * nthr) {
+        z_request(v0);
+        z_place(v0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     request(ch0, w0, c0, b0);
     Chunk ch1 = after(ch0);
     request(ch1, w1, c1, b1);
     Chunk ch2 = after(ch1);
     request(ch2, w2, c2, b2);
     __builtin_amdgcn_sched_barrier(0);
-    z_place(0);
-    for (int v0 = ZU * nthr; v0 < nvec; v0 += ZU * nthr) {
-        z_request(v0);
-        z_place(v0);
-    }
     __syncthreads();
 
     // ---- out[token][16n + ..] = bias + sum over the tiles of block-row n
@@ -347,9 +353,9 @@ __global__ __launch_bounds__(64 * NW) void mha_fuseo_kernel(const MhaArgs a, con
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) acc[tt] = f4{0.f, 0.f, 0.f, 0.f};
     auto multiply = [&](const Chunk &cur, const Chunk &nxt, const h8 (&w)[P], const int (&c)[P], const h4 &bq) {
-        // the Z fragments of half a chunk are read together and multiplied then: one wave per SIMD has
+        // the Z fragments of two tile pairs are read together and multiplied then: one wave per SIMD has
         // nothing else to cover the LDS latency with, and read by read it adds up to most of the projection
-        constexpr int PH = P / 2;
+        constexpr int PH = 2;
 #pragma unroll
         for (int p0 = 0; p0 < P; p0 += PH) {
             h8 zf[PH][TT];
