@@ -859,6 +859,30 @@ int et_model_sync(et_model m);
 int et_model_launches_per_layer(et_model m, int *launches);
 int et_model_destroy(et_model m);
 
+/* The same stack in binary32 from end to end: weights, activations, input and
+ * output are float; every layer is seven launches of the *_f32 entry points
+ * above (QKV, attention, O, SkipLayerNorm, linear1 + activation, linear2,
+ * SkipLayerNorm: Encoder/Encoder.h:81-96), replayed as one HIP graph when
+ * desc.use_graph != 0.  desc.mixed is ignored; kdim == vdim == emdim.  A
+ * layer's four matrices may each be dense or 16x16 tile-sparse.  No reference
+ * counterpart (the reference computes in binary16 only): the binary32 twin of
+ * et_model_*, for checking a pruned model's values without binary16 rounding.
+ * Argument meaning as in the et_model_* function of the same name. */
+typedef struct et_model_f32_s *et_model_f32;
+int et_model_f32_create(const et_model_desc *desc, et_model_f32 *out);
+int et_model_f32_set_bsr16(et_model_f32 m, int layer, int which, const int32_t *row_ptr,
+                           const int32_t *column, const float *data, int ntile,
+                           const float *bias);
+int et_model_f32_set_dense(et_model_f32 m, int layer, int which, const float *W,
+                           const float *bias);
+int et_model_f32_set_norm(et_model_f32 m, int layer, int which, const float *gamma,
+                          const float *beta);
+int et_model_f32_set_lens(et_model_f32 m, const int32_t *lens_host);
+int et_model_f32_finalize(et_model_f32 m);
+int et_model_f32_forward(et_model_f32 m, float *out, const float *in, et_stream stream);
+int et_model_f32_sync(et_model_f32 m);
+int et_model_f32_destroy(et_model_f32 m);
+
 /* ------------------------------------------------------------------------
  * Host-side construction of the sparse weight structures (integer work on
  * host pointers, usable without a GPU).  Outputs are caller-allocated; a

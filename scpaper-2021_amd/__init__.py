@@ -164,6 +164,15 @@ _SIGNATURES = {
     "et_model_sync": (_vp,),
     "et_model_launches_per_layer": (_vp, C.POINTER(_i)),
     "et_model_destroy": (_vp,),
+    "et_model_f32_create": (_vp, C.POINTER(_vp)),
+    "et_model_f32_set_bsr16": (_vp, _i, _i, _vp, _vp, _vp, _i, _vp),
+    "et_model_f32_set_dense": (_vp, _i, _i, _vp, _vp),
+    "et_model_f32_set_norm": (_vp, _i, _i, _vp, _vp),
+    "et_model_f32_set_lens": (_vp, _vp),
+    "et_model_f32_finalize": (_vp,),
+    "et_model_f32_forward": (_vp, _vp, _vp, _vp),
+    "et_model_f32_sync": (_vp,),
+    "et_model_f32_destroy": (_vp,),
     "et_fmt_permutation": (C.c_int64, C.c_uint64, _vp),
     "et_fmt_kept_count": (C.c_int64, _f),
     "et_fmt_tile_pattern": (_i, _i, _f, C.c_uint64, _vp, _vp, C.POINTER(_i)),

@@ -29,7 +29,7 @@ def header_declarations():
 
 
 def kind_of_c(param):
-    if "*" in param or re.match(r"(const\s+)?et_(stream|event|graph|model|bsr_plan|bsr_pack)\b", param):
+    if "*" in param or re.match(r"(const\s+)?et_(stream|event|graph|model_f32|model|bsr_plan|bsr_pack)\b", param):
         return "ptr"
     if re.match(r"(const\s+)?size_t\b", param):
         return "size"

@@ -1,6 +1,7 @@
 """binary32 twins on the GPU against the CPU oracle, and the dense fp32 encoder layer of the
 first benchmark configuration (one BERT-base layer, batch 1, seq 128) composed from them,
 to the fp32-path tolerance max-abs 1e-4."""
+import ctypes as C
 import importlib.util
 from pathlib import Path
 
@@ -346,3 +347,90 @@ def test_tile_sparse_fp32_encoder_stack(et):
     err = Hn.max_abs(got, want)
     print(f"tile-sparse fp32 stack, {depth} layers: max-abs vs oracle {err:.2e}")
     assert err <= 2e-4
+
+
+def _f32_model(et, H, nh, FF, S, B, nlayer, act, use_graph, causal=False):
+    desc = et.ModelDesc(H, H, S, nh, FF, H, nlayer, B, act, 1e-5, int(causal), int(use_graph), 0)
+    h = C.c_void_p()
+    et.check(et.lib().et_model_f32_create(C.byref(desc), C.byref(h)))
+    return h
+
+
+def _np(a):
+    return np.ascontiguousarray(a).ctypes.data
+
+
+@pytest.mark.parametrize("use_graph", [True, False])
+def test_fp32_model_handle_tile_sparse_stack(et, use_graph):
+    """et_model_f32_*: three pruned layers (80 % tiles; the last layer's FFN dense), batch 4 of 64 tokens with right
+    padding, GELU, against the oracle's binary32 forward; a second forward on the same buffers replays the graph."""
+    from oracle import formats as F
+    lib = et.lib()
+    H, nh, FF, S, B, depth = 256, 4, 512, 64, 4, 3
+    T = B * S
+    lens = np.array([64, 20, 33, 48], np.int32)
+    h = _f32_model(et, H, nh, FF, S, B, depth, et.ACT_GELU, use_graph)
+    want = torch.from_numpy(randf((T, H), 700))
+    x = want.numpy().copy()
+    shapes = {0: (3 * H, H), 1: (H, H), 2: (FF, H), 3: (H, FF)}
+    params = []
+    for layer in range(depth):
+        mats = []
+        for which, (out, inp) in shapes.items():
+            seed = 800 + 40 * layer + 7 * which
+            b = randf((out,), seed + 2, 0.05)
+            if layer == depth - 1 and which >= 2:  # dense
+                W = randf((out, inp), seed, 0.05)
+                et.check(lib.et_model_f32_set_dense(h, layer, which, _np(W), _np(b)))
+            else:
+                row_ptr, col_idx = F.gen_tile_pattern(out, inp, 0.8, seed=seed)
+                tiles = randf((len(col_idx), 256), seed + 1, 0.05)
+                W = F.bsr16_to_dense(row_ptr, col_idx, tiles, inp)
+                et.check(lib.et_model_f32_set_bsr16(h, layer, which, _np(row_ptr), _np(col_idx), _np(tiles), len(col_idx),
+                                                    _np(b)))
+            mats += [torch.from_numpy(W), torch.from_numpy(b)]
+        norms = []
+        for which in range(2):
+            g, be = 1 + randf((H,), 900 + 10 * layer + which, 0.1), randf((H,), 950 + 10 * layer + which, 0.1)
+            et.check(lib.et_model_f32_set_norm(h, layer, which, _np(g), _np(be)))
+            norms += [torch.from_numpy(g), torch.from_numpy(be)]
+        params.append(L.LayerParams(*mats, *norms))
+    et.check(lib.et_model_f32_set_lens(h, _np(lens)))
+    et.check(lib.et_model_f32_finalize(h))
+    assert lib.et_model_f32_set_norm(h, 0, 0, _np(x), _np(x)) == et.ET_ERR_INVALID_ARG  # frozen after finalize
+    d_x, d_y = up(et, x), et.DeviceBuffer.empty((T, H), np.float32)
+    for p in params:
+        want = L.encoder_layer(want, p, L.LayerConfig(nh=nh, B=B, act="gelu", lens=lens.tolist()))
+    want = want.numpy()
+    for rep in range(2):
+        nan = np.full((T, H), np.nan, np.float32)
+        et.check(lib.et_memcpy_h2d(d_y.ptr, _np(nan), nan.nbytes))
+        et.check(lib.et_model_f32_forward(h, d_y.ptr, d_x.ptr, None))
+        et.check(lib.et_model_f32_sync(h))
+        got = d_y.numpy()
+        for b in range(B):  # rows past a sequence's length are padding: not compared
+            got[b * S + lens[b]:(b + 1) * S] = 0
+            want[b * S + lens[b]:(b + 1) * S] = 0
+        err = Hn.max_abs(got, want)
+        print(f"fp32 model handle (graph={use_graph}) pass {rep}: max-abs vs oracle {err:.2e}")
+        assert err <= TOL_F32
+    et.check(lib.et_model_f32_destroy(h))
+
+
+def test_fp32_model_handle_rejects_bad_use(et):
+    lib = et.lib()
+    h = C.c_void_p()
+    bad = et.ModelDesc(256, 128, 64, 4, 512, 256, 1, 1, et.ACT_GELU, 1e-5, 0, 0, 0)  # kdim != vdim
+    assert lib.et_model_f32_create(C.byref(bad), C.byref(h)) == et.ET_ERR_INVALID_ARG
+    h = _f32_model(et, 64, 4, 128, 16, 1, 1, et.ACT_RELU, False)
+    assert lib.et_model_f32_finalize(h) == et.ET_ERR_INVALID_ARG  # weights never set
+    W = randf((192, 64), 1, 0.05)
+    assert lib.et_model_f32_set_dense(h, 1, 0, _np(W), None) == et.ET_ERR_INVALID_ARG  # layer out of range
+    assert lib.et_model_f32_set_dense(h, 0, 4, _np(W), None) == et.ET_ERR_INVALID_ARG  # bad selector
+    rp = np.zeros(13, np.int32)
+    rp[1:] = 1
+    assert lib.et_model_f32_set_bsr16(h, 0, 0, _np(rp), _np(np.array([9], np.int32)), _np(randf((1, 256), 2)), 1,
+                                      None) != et.ET_OK  # column tile outside the matrix
+    x = np.zeros((16, 64), np.float32)
+    assert lib.et_model_f32_forward(h, _np(x), _np(x), None) == et.ET_ERR_INVALID_ARG  # not finalized
+    et.check(lib.et_model_f32_destroy(h))
