@@ -368,6 +368,13 @@ static int run_attn_variants(const std::string &dir) {
                                 wo.data.get(), bo.get(), para, OUT.get(), run);
         etChk(et_device_sync());
         save_half(dir + "/out_fuseO_free.npy", OUT, (std::size_t)rows, (std::size_t)H);
+        // ... and as one launch
+        et::DeviceBuffer<half> Z1((std::size_t)rows * H), OUT1((std::size_t)rows * H);
+        run.one_launch = true;
+        Multihead_atttion_fuseO(X.get(), X.get(), X.get(), nullptr, Z1.get(), wo.row_ptr.get(), wo.row_offset.get(),
+                                wo.data.get(), bo.get(), para, OUT1.get(), run);
+        etChk(et_device_sync());
+        save_half(dir + "/out_fuseO_one_launch.npy", OUT1, (std::size_t)rows, (std::size_t)H);
     }
     return 0;
 }

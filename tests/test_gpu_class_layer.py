@@ -198,6 +198,7 @@ def test_attention_tags_with_separate_projections(tmp_path):
     # free function: attention over Q = K = V = x without projections, no padding, then the O projection
     z0 = L.mha(xf, xf, xf, nh, B, store=st)
     assert Hn.max_abs(np.load(tmp_path / "out_fuseO_free.npy"), lin("o", z0).numpy()) <= 6e-3
+    assert Hn.max_abs(np.load(tmp_path / "out_fuseO_one_launch.npy"), lin("o", z0).numpy()) <= 6e-3
 
 
 def test_encoder_fuse_class(tmp_path):
