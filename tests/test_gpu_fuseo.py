@@ -119,3 +119,50 @@ def test_fuseo_rejects_what_it_cannot_do(et):
     assert call(**args(emdim=200)) == et.ET_ERR_UNSUPPORTED
     assert call(**args(B=20000)) == et.ET_ERR_UNSUPPORTED       # more strips than arrival counts
     assert call(**args(B=0)) == et.ET_OK
+
+
+def test_fuseo_interleaved_qkv_and_strided_z(et):
+    """Q, K and V as column slices of one [T x 3H] buffer and Z inside a wider buffer (row stride H + 64): the
+    projection reads Z through its stride; the columns beside Z stay untouched."""
+    B, S, nh, hd, emdim = 3, 64, 6, 32, 192
+    H, T = nh * hd, B * S
+    qkv = Hn.randn((T, 3 * H), 41)
+    d_qkv = up(et, qkv)
+    w = Hn.BsrWeight(emdim, H, 0.6, seed=45, std=0.05, bias_std=0.1).upload(et)
+    ldz = H + 64
+    zbuf = np.full((T, ldz), 7.0, np.float16)
+    d_z = up(et, zbuf)
+    d_out = et.DeviceBuffer.empty((T, emdim), np.float16)
+    et.mha_fuseo(d_qkv.ptr, d_qkv.offset(2 * H), d_qkv.offset(4 * H), 3 * H, 3 * H, 3 * H, d_z, ldz, None, None, B, S, nh,
+                 hd, 1.0 / math.sqrt(hd), 0, w.d_row_ptr, w.d_col_idx, w.d_tiles, w.d_bias, d_out, emdim)
+    q, k, v = qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:]
+    z_want = L.mha(Hn.f32(q), Hn.f32(k), Hn.f32(v), nh, B, store=torch.float16)
+    out_want = L.linear(z_want.float(), Hn.f32(w.dense), Hn.f32(w.bias), None, torch.float16)
+    z_got = d_z.numpy()
+    assert Hn.max_abs(z_got[:, :H], z_want.numpy()) <= 2e-3
+    assert (z_got[:, H:] == 7.0).all()
+    assert Hn.max_abs(d_out.numpy(), out_want.numpy()) <= 1.2e-2
+
+
+def _random_fuseo_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        S = 16 * int(rng.integers(1, 17))
+        B, nh = int(rng.integers(1, 6)), int(rng.integers(1, 9))
+        hd = 8 * int(rng.integers(1, 17))
+        while (nh * hd) % 16:
+            hd += 8
+        emdim = 16 * int(rng.integers(1, 40))
+        kind = int(rng.integers(0, 3))  # 0 plain, 1 right padding, 2 causal
+        cases.append((B, S, nh, hd, emdim, round(float(rng.uniform(0.0, 0.95)), 2), kind, int(rng.integers(1, 1 << 20))))
+    return cases
+
+
+@pytest.mark.parametrize("B,S,nh,hd,emdim,sp,kind,seed", _random_fuseo_cases(16, 20211117))
+def test_fuseo_random_shapes(et, B, S, nh, hd, emdim, sp, kind, seed):
+    rng = np.random.default_rng(seed)
+    lens = rng.integers(0, S + 1, B).astype(np.int32) if kind == 1 else None
+    got, two, want = run_fuseo(et, B, S, nh, hd, emdim, sp, seed=seed & 0xFFFF, lens=lens, causal=kind == 2,
+                               waves=[None, 1, 2, 4][seed % 4] if (S // 16) % 4 == 0 else None)
+    compare(B, S, lens, got, two, want)
