@@ -188,18 +188,19 @@ static int launch_mha(const MhaArgs &args, int B, hipStream_t stream) {
 // W_O.  Here nothing waits: a workgroup runs the fused attention of its (sequence, head, query strip),
 // stores its slice of Z, and adds one to the arrival count of its (sequence, query strip).  The workgroup
 // whose addition completes the count — all heads of those tokens are in memory — stages the finished rows of
-// Z in LDS and multiplies them with W_O: a wave per block-row of the weight, two tiles per MFMA, the tile
+// Z (and the weight's row pointers and column indices) in LDS and multiplies them with W_O: a wave per block-row
+// of the weight, two tiles per MFMA, the tile
 // fragments of the next three groups of six tile pairs on their way while a group is multiplied.  Every other
 // workgroup has left by then, so the launch needs no co-residency and no spinning, and the projection of
 // the first finished strips overlaps the attention of the rest.  The last arriver puts the count back to
 // zero: the counts are zero before and after every launch.
 // What it costs: the projecting workgroup takes in the whole weight by itself (236 KB for 768 x 768 at 80 %
-// sparsity; a compute unit takes in 20 GB/s of lines its L2 does not hold, 90 GB/s of lines it does), and as
-// compiled the loop still waits for all of its requests once per turn of the four register sets, about one
-// memory round trip (1.1 us) per group of six tile pairs, 13 groups per wave: 16 us for the projection of a
-// strip, against 4 us for a launch of its own that spreads the weight over a few hundred workgroups.  26
-// against 8 us for one sequence of 128 tokens, 29 against 9 us for eight.  The class layer therefore keeps
-// the two launches; this entry point is for callers that need one.
+// sparsity; a compute unit takes in 20 GB/s of lines its L2 does not hold, 90 GB/s of lines it does), and the
+// loop measures 1.1 us per group of six tile pairs whatever the number of live tiles in it, 13 groups per wave
+// (as compiled it still waits for all of its requests once per turn of the four register sets): 14 us for the
+// projection of a strip, against 4 us for a launch of its own that spreads the weight over a few hundred
+// workgroups.  25 against 8 us for one sequence of 128 tokens, 28 against 9 us for eight.  The class layer
+// therefore keeps the two launches; this entry point is for callers that need one.
 struct FuseOArgs {
     const int32_t *row_ptr, *col_idx;  // W_O [emdim x nh*hd] as 16x16 tiles (tile rows = output features)
     const _Float16 *tiles;
@@ -246,7 +247,6 @@ __global__ __launch_bounds__(64 * NW) void mha_fuseo_kernel(const MhaArgs a, con
     // behind the rows of Z: a load of them between the tile requests would have to be waited for, and the
     // requests made before it with it (loads return in order).
     const int nrows = nbr > wave_u ? (nbr - wave_u + NW - 1) / NW : 0;
-    const int ntile = f.row_ptr[nbr];
 
     const int width = a.nh * hd;       // a multiple of 16
     const int ldzs = width + 8;        // halfs; rows 16 bytes apart in the banks
@@ -263,14 +263,16 @@ __global__ __launch_bounds__(64 * NW) void mha_fuseo_kernel(const MhaArgs a, con
             zt[i] = load_device_scope(a.Z + (row0 + row) * a.ldz + c * 8);
         }
     };
-    auto z_place = [&](int v0) {  // rows past the sequence as zeros
+    // rows past the sequence as zeros.  Every store is unconditional (surplus threads repeat the last vector):
+    // a store under a branch leaves its load unwaited on the other path as far as the compiler can tell, and
+    // the first write to that register in the projection loop then waits for every outstanding request.
+    auto z_place = [&](int v0) {
 #pragma unroll
         for (int i = 0; i < ZU; i++) {
-            const int v = v0 + i * nthr + (int)threadIdx.x;
+            const int v = min(v0 + i * nthr + (int)threadIdx.x, nvec - 1);
             const int r = v / vpr, c = v - r * vpr;
-            if (v < nvec)
-                *reinterpret_cast<h8 *>(Zs + r * ldzs + c * 8) =
-                    (qstrip * kStripQ + r < S) ? zt[i] : h8{0, 0, 0, 0, 0, 0, 0, 0};
+            *reinterpret_cast<h8 *>(Zs + r * ldzs + c * 8) =
+                (qstrip * kStripQ + r < S) ? zt[i] : h8{0, 0, 0, 0, 0, 0, 0, 0};
         }
     };
     int *rps = reinterpret_cast<int *>(Zs + kStripQ * ldzs);
@@ -284,10 +286,15 @@ __global__ __launch_bounds__(64 * NW) void mha_fuseo_kernel(const MhaArgs a, con
         rps[i] = v;
     }
     __syncthreads();
+    // ... and the column indices behind them (room for every tile of a full weight): read from LDS where they
+    // are used, they do not take part in the count of outstanding memory requests
+    int *cols = rps + nbr + 1;
+    const int ntile = min(rps[nbr], nbr * (width / 16));
+    for (int i = threadIdx.x; i < ntile; i += nthr) cols[i] = f.col_idx[i];
+    if (ntile == 0 && threadIdx.x == 0) cols[0] = 0;
 
     // a weight without tiles: the loads below go to valid dummy addresses and meet the zero operand
     const _Float16 *tbase = ntile > 0 ? f.tiles : a.Z + row0 * a.ldz;
-    const int32_t *cbase = ntile > 0 ? f.col_idx : f.row_ptr;
     const int jmax = max(ntile - 1, 0);
     const int half_k = 8 * (g & 1), second = g >> 1;
     const h8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -300,13 +307,12 @@ __global__ __launch_bounds__(64 * NW) void mha_fuseo_kernel(const MhaArgs a, con
     // spot, and with it every request made before it)
     const _Float16 *bbase = f.bias ? f.bias + 4 * g : tbase;
     const int bstep = f.bias ? 16 : 0;
-    auto request = [&](const Chunk &ch, h8 (&w)[P], int (&c)[P], h4 &bq) {
+    auto request = [&](const Chunk &ch, h8 (&w)[P], h4 &bq) {
         bq = *reinterpret_cast<const h4 *>(bbase + (size_t)min(wave_u + NW * ch.k, nbr - 1) * bstep);
 #pragma unroll
         for (int p = 0; p < P; p++) {
             const int jt = ch.j + 2 * p + second;
             const int jc = min(jt, jmax);
-            c[p] = cbase[jc];
             w[p] = *reinterpret_cast<const h8 *>(tbase + (size_t)jc * 256 + r16 * 16 + half_k);
         }
     };
@@ -324,7 +330,6 @@ __global__ __launch_bounds__(64 * NW) void mha_fuseo_kernel(const MhaArgs a, con
         return nx;
     };
     h8 w0[P], w1[P], w2[P], w3[P];
-    int c0[P], c1[P], c2[P], c3[P];
     h4 b0, b1, b2, b3;
     Chunk ch0 = {0, 0, 0};
     if (nrows > 0) {
@@ -340,11 +345,11 @@ __global__ __launch_bounds__(64 * NW) void mha_fuseo_kernel(const MhaArgs a, con
         z_place(v0);
     }
     __builtin_amdgcn_sched_barrier(0);
-    request(ch0, w0, c0, b0);
+    request(ch0, w0, b0);
     Chunk ch1 = after(ch0);
-    request(ch1, w1, c1, b1);
+    request(ch1, w1, b1);
     Chunk ch2 = after(ch1);
-    request(ch2, w2, c2, b2);
+    request(ch2, w2, b2);
     __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
 
@@ -352,7 +357,7 @@ __global__ __launch_bounds__(64 * NW) void mha_fuseo_kernel(const MhaArgs a, con
     f4 acc[TT];
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) acc[tt] = f4{0.f, 0.f, 0.f, 0.f};
-    auto multiply = [&](const Chunk &cur, const Chunk &nxt, const h8 (&w)[P], const int (&c)[P], const h4 &bq) {
+    auto multiply = [&](const Chunk &cur, const Chunk &nxt, const h8 (&w)[P], const h4 &bq) {
         // the Z fragments of two tile pairs are read together and multiplied then: one wave per SIMD has
         // nothing else to cover the LDS latency with, and read by read it adds up to most of the projection
         constexpr int PH = 2;
@@ -362,7 +367,8 @@ __global__ __launch_bounds__(64 * NW) void mha_fuseo_kernel(const MhaArgs a, con
 #pragma unroll
             for (int pp = 0; pp < PH; pp++) {
                 const bool live = cur.j + 2 * (p0 + pp) + second < cur.j1;
-                const _Float16 *zp = Zs + r16 * ldzs + (live ? c[p0 + pp] : 0) * 16 + half_k;
+                const int col = cols[min(cur.j + 2 * (p0 + pp) + second, jmax)];
+                const _Float16 *zp = Zs + r16 * ldzs + col * 16 + half_k;
 #pragma unroll
                 for (int tt = 0; tt < TT; tt++) zf[pp][tt] = *reinterpret_cast<const h8 *>(zp + tt * 16 * ldzs);
             }
@@ -401,27 +407,27 @@ __global__ __launch_bounds__(64 * NW) void mha_fuseo_kernel(const MhaArgs a, con
     while (true) {  // every exit is wave-uniform
         if (ch0.k >= nrows) break;
         ch3 = after(ch2);
-        request(ch3, w3, c3, b3);
+        request(ch3, w3, b3);
         __builtin_amdgcn_sched_barrier(0);
-        multiply(ch0, ch1, w0, c0, b0);
+        multiply(ch0, ch1, w0, b0);
         __builtin_amdgcn_sched_barrier(0);
         if (ch1.k >= nrows) break;
         ch0 = after(ch3);
-        request(ch0, w0, c0, b0);
+        request(ch0, w0, b0);
         __builtin_amdgcn_sched_barrier(0);
-        multiply(ch1, ch2, w1, c1, b1);
+        multiply(ch1, ch2, w1, b1);
         __builtin_amdgcn_sched_barrier(0);
         if (ch2.k >= nrows) break;
         ch1 = after(ch0);
-        request(ch1, w1, c1, b1);
+        request(ch1, w1, b1);
         __builtin_amdgcn_sched_barrier(0);
-        multiply(ch2, ch3, w2, c2, b2);
+        multiply(ch2, ch3, w2, b2);
         __builtin_amdgcn_sched_barrier(0);
         if (ch3.k >= nrows) break;
         ch2 = after(ch1);
-        request(ch2, w2, c2, b2);
+        request(ch2, w2, b2);
         __builtin_amdgcn_sched_barrier(0);
-        multiply(ch3, ch0, w3, c3, b3);
+        multiply(ch3, ch0, w3, b3);
         __builtin_amdgcn_sched_barrier(0);
     }
 }
@@ -451,12 +457,16 @@ static int fuseo_counts(unsigned **out) {
     return ET_OK;
 }
 
+// row pointers and (room for) the column index of every tile of a full weight, kept in LDS behind the rows of Z
+static size_t fuseo_index_bytes(int width, int emdim) {
+    return ((size_t)(emdim / 16) + 1 + (size_t)(emdim / 16) * (width / 16)) * sizeof(int);
+}
 constexpr size_t kLdsPerWorkgroup = 160 * 1024 - 256;  // the arrival flag is a static allocation of its own
 
 template <int HD, int NW>
 static int launch_fuseo_nw(const MhaArgs &args, const FuseOArgs &fo, hipStream_t stream) {
     auto kernel = mha_fuseo_kernel<HD, NW, 1>;
-    const size_t strip = (size_t)16 * NW * (args.nh * args.hd + 8) * sizeof(_Float16) + (size_t)(fo.emdim / 16 + 1) * sizeof(int);
+    const size_t strip = (size_t)16 * NW * (args.nh * args.hd + 8) * sizeof(_Float16) + fuseo_index_bytes(args.nh * args.hd, fo.emdim);
     const size_t lds = std::max(MhaLds<HD>::bytes, strip);
     ET_REQUIRE(lds <= kLdsPerWorkgroup, ET_ERR_UNSUPPORTED, "et_mha_fuseo_f16: a strip of %d rows of Z (%zu B) exceeds LDS",
                16 * NW, strip);
@@ -479,7 +489,7 @@ static int launch_fuseo(const MhaArgs &args, const FuseOArgs &fo, int waves, hip
     const size_t row_bytes = (size_t)(args.nh * args.hd + 8) * sizeof(_Float16);
     if (waves == 0) {
         waves = qblocks % 4 == 0 ? 4 : qblocks % 2 == 0 ? 2 : 1;
-        while (waves > 1 && 16 * waves * row_bytes + (fo.emdim / 16 + 1) * sizeof(int) > kLdsPerWorkgroup) waves >>= 1;
+        while (waves > 1 && 16 * waves * row_bytes + fuseo_index_bytes(args.nh * args.hd, fo.emdim) > kLdsPerWorkgroup) waves >>= 1;
     }
     if (waves == 4) return launch_fuseo_nw<HD, 4>(args, fo, stream);
     if (waves == 2) return launch_fuseo_nw<HD, 2>(args, fo, stream);
@@ -939,8 +949,8 @@ int et_mha_fuseo_f16_geom(const et_f16 *Q, const et_f16 *K, const et_f16 *V, int
                "et_mha_fuseo_f16: B*S/16=%lld exceeds the %d arrival counts built into the library; run "
                "et_mha_fused_f16 and et_linear_bsr16_f16 instead",
                (long long)B * (S / 16), kFuseOCounters);
-    ET_REQUIRE((size_t)16 * (width + 8) * sizeof(_Float16) + (emdim / 16 + 1) * sizeof(int) <= kLdsPerWorkgroup, ET_ERR_UNSUPPORTED,
-               "et_mha_fuseo_f16: 16 rows of Z (%d wide) exceed LDS", width);
+    ET_REQUIRE((size_t)16 * (width + 8) * sizeof(_Float16) + fuseo_index_bytes(width, emdim) <= kLdsPerWorkgroup, ET_ERR_UNSUPPORTED,
+               "et_mha_fuseo_f16: 16 rows of Z and the index arrays of a %d x %d weight exceed LDS", emdim, width);
     if (B == 0) return ET_OK;
     MhaArgs args;
     args.Q = reinterpret_cast<const _Float16 *>(Q);
