@@ -122,7 +122,7 @@ void Multihead_atttion(ptr_t *mat_q, ptr_t *mat_k, col_mat *mat_v, ptr_t *mat_qk
 // (Attention/kernel_fuseO.h:6-9, Attention/kernel_fuseO.cu:254-290).  The
 // reference joins the two with a grid-wide barrier inside one cooperative
 // launch; here they are two back-to-back launches on one stream, which is the
-// faster form on this device (8 against 26 us for one sequence of 128 tokens),
+// faster form on this device (8 against 25 us for one sequence of 128 tokens),
 // or, with run.one_launch, the one launch of et_mha_fuseo_f16.
 inline void Multihead_atttion_fuseO(half *mat_q, half *mat_k, half *mat_v, const half *mask, half *mat_z,
                                     const int *row_ptr, const int *row_offset, const half *data,
